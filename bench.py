@@ -1,0 +1,233 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X int8 path: one JSON line on stdout.
+
+A step is one pass of the hot path over one batch of synthetic input that is
+already resident in GPU memory: by default the MatMulInteger of the BERT-base
+FFN-up projection (M=4096, K=768, N=3072, uint8 activations x int8 weights,
+per-column fp32 dequantisation fused into the store) -- the shape the int8
+target is quoted on.  The same line carries, under "extras", the
+QuantizeLinear / DequantizeLinear / DynamicQuantizeLinear rates at
+[8192, 32768] and the other GEMM shapes.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+
+Every entry point is called through the C-ABI (include/om_mi355x.h).  Kernel
+time is measured with HIP events recorded on the runtime's own stream around
+the timed region; whole-job time with the host clock around the same region.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "onnx-mlir_amd"))
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK_GBS = 8000.0        # MI355X published HBM3E bandwidth
+INT8_PEAK_TOPS = 5000.0      # MI355X published dense int8 MFMA rate (no sparsity)
+
+METRIC = "int8 MatMulInteger TOPS (% MFMA peak) + Q/DQ GB/s (% HBM), 1 MI355X"
+
+
+def timed(rt, fn, steps, warmup):
+    """Returns (host seconds per step, event milliseconds per step)."""
+    for _ in range(warmup):
+        fn()
+    rt.synchronize()
+    t0 = time.perf_counter()
+    rt.timer_start()
+    for _ in range(steps):
+        fn()
+    ev_ms = rt.timer_stop()          # waits for the last launch
+    rt.synchronize()
+    host = time.perf_counter() - t0
+    return host / steps, ev_ms / steps
+
+
+def gemm_case(rt, wl, name, M, K, N, w_i8, w_scale, steps, warmup, epilogue="f32"):
+    rng = np.random.default_rng(0xC0FFEE00 + M + K + N)
+    A = rng.integers(0, 256, (M, K), dtype=np.uint8)
+    dA = rt.DeviceArray.from_numpy(A)
+    dW = rt.DeviceArray.from_numpy(w_i8)
+    dS = rt.DeviceArray.from_numpy(w_scale)
+    dAs = rt.DeviceArray.from_numpy(np.array(0.0173, np.float32))
+    dAz = rt.DeviceArray.from_numpy(np.array(131, np.uint8))
+    rt.mark_constant(dW)             # weights: packed once, like any model constant
+    if epilogue == "f32":
+        dY = rt.DeviceArray((M, N), np.float32)
+        fn = lambda: rt.MatMulIntegerDequant(dA, dW, dAz, None, dAs, dS, out=dY)
+    else:
+        dY = rt.DeviceArray((M, N), np.int32)
+        fn = lambda: rt.MatMulInteger(dA, dW, dAz, None, out=dY)
+    host_s, ev_ms = timed(rt, fn, steps, warmup)
+    ops = 2.0 * M * N * K
+    res = {"name": name, "M": M, "K": K, "N": N, "epilogue": epilogue,
+           "ms_per_step": host_s * 1e3, "kernel_ms": ev_ms,
+           "tops": ops / host_s / 1e12, "kernel_tops": ops / (ev_ms * 1e-3) / 1e12,
+           "ops": ops, "hbm_bytes_algorithmic": M * K + K * N + 4 * M * N}
+    for d in (dA, dW, dS, dAs, dAz, dY):
+        d.free()
+    return res
+
+
+def decode_case(rt, wl, M, steps, warmup):
+    c = wl.config5("up", M=M)
+    K, N = c["W"].shape
+    dX = rt.DeviceArray.from_numpy(c["X"])
+    dW = rt.DeviceArray.from_numpy(c["W"])
+    dS = rt.DeviceArray.from_numpy(c["w_scale"])
+    dY = rt.DeviceArray((M, N), np.float32)
+    rt.mark_constant(dW)
+    fn = lambda: rt.DynQuantMatMulDequant(dX, dW, None, dS, out=dY)
+    host_s, ev_ms = timed(rt, fn, steps, warmup)
+    nbytes = K * N + M * K + 4 * M * N
+    res = {"name": f"config5 decode M={M}", "M": M, "K": K, "N": N, "ms_per_step": host_s * 1e3,
+           "kernel_ms": ev_ms, "gbs": nbytes / (ev_ms * 1e-3) / 1e9, "bytes": nbytes,
+           "hbm_frac": nbytes / (ev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+    for d in (dX, dW, dS, dY):
+        d.free()
+    return res
+
+
+def qdq_cases(rt, wl, rows, cols, steps, warmup):
+    c = wl.config2(rows, cols)
+    n = rows * cols
+    dX = rt.DeviceArray.from_numpy(c["X"])
+    dS = rt.DeviceArray.from_numpy(c["scale"])
+    dZ = rt.DeviceArray.from_numpy(c["zp"])
+    dQ = rt.DeviceArray((rows, cols), np.uint8)
+    dD = rt.DeviceArray((rows, cols), np.float32)
+    dys = rt.DeviceArray((), np.float32)
+    dyz = rt.DeviceArray((), np.uint8)
+    s1 = rt.DeviceArray.from_numpy(np.array(0.02, np.float32))
+    z1 = rt.DeviceArray.from_numpy(np.array(128, np.uint8))
+    out = {}
+
+    def run(name, fn, nbytes):
+        host_s, ev_ms = timed(rt, fn, steps, warmup)
+        out[name] = {"ms_per_step": host_s * 1e3, "kernel_ms": ev_ms, "bytes": nbytes,
+                     "gbs": nbytes / (ev_ms * 1e-3) / 1e9,
+                     "hbm_frac": nbytes / (ev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+
+    run("quantize_per_axis", lambda: rt.QuantizeLinear(dX, dS, dZ, axis=1, out=dQ), 5 * n)
+    run("dequantize_per_axis", lambda: rt.DequantizeLinear(dQ, dS, dZ, axis=1, out=dD), 5 * n)
+    run("quantize_per_tensor", lambda: rt.QuantizeLinear(dX, s1, z1, out=dQ), 5 * n)
+    run("dequantize_per_tensor", lambda: rt.DequantizeLinear(dQ, s1, z1, out=dD), 5 * n)
+    # two reads of X (min/max, then quantize) + one write: the tensor is far
+    # larger than any on-chip cache
+    run("dynamic_quantize", lambda: rt.DynamicQuantizeLinear(dX, out=(dQ, dys, dyz)), 9 * n)
+    for d in (dX, dS, dZ, dQ, dD, dys, dyz, s1, z1):
+        d.free()
+    return out
+
+
+def cpu_baseline_gemm(oracle, wl, M, K, N, budget_s=20.0):
+    """The oracle's restatement of the reference's CPU pass structure for the
+    same MatMulInteger + Cast + Mul, timed on this host's cores."""
+    c = wl.config4("ffn_up", M=M)
+    rng = np.random.default_rng(7)
+    A = rng.integers(0, 256, (M, K), dtype=np.uint8)
+    az = np.array(131, np.uint8)
+    t0 = time.perf_counter()
+    acc = oracle.matmul_integer(A, c["W"], az, None, passes=True)
+    oracle.dequant_epilogue(acc, np.float32(0.0173), c["w_scale"])
+    first = time.perf_counter() - t0
+    reps = int(max(1, min(10, budget_s / max(first, 1e-3) - 1)))
+    times = [first]
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        acc = oracle.matmul_integer(A, c["W"], az, None, passes=True)
+        oracle.dequant_epilogue(acc, np.float32(0.0173), c["w_scale"])
+        times.append(time.perf_counter() - t0)
+    best = float(np.median(times))
+    return {"value": 2.0 * M * N * K / best / 1e12, "unit": "TOPS", "cores": oracle.num_threads(),
+            "kind": "port",
+            "sample": f"full M={M} K={K} N={N} MatMulInteger+Cast+Mul, median of {len(times)} runs of the "
+                      "oracle's restatement of the reference's CPU passes (int32 copies, zero-point "
+                      "passes, 4x8x8-blocked int32 GEMM, OpenMP over row tiles); not onnx-mlir codegen",
+            "seconds_per_step": best}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="config4_ffn_up",
+                    choices=["config4_ffn_up", "config4_ffn_up_i32"])
+    ap.add_argument("--no-extras", action="store_true", help="skip the Q/DQ and other-shape measurements")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import om_mi355x as rt
+    from om_mi355x import workloads as wl
+    rt.load()                       # raises if the HIP library is not built
+    info = rt.device_info()         # raises if there is no gfx950 device
+
+    M, K, N = 4096, 768, 3072
+    c = wl.config4("ffn_up", M=8)   # weights and scales only; activations are made in gemm_case
+    epi = "f32" if args.workload == "config4_ffn_up" else "i32"
+    main_res = gemm_case(rt, wl, "config4 FFN-up", M, K, N, c["W"], c["w_scale"],
+                         args.steps, args.warmup, epi)
+
+    extras = {}
+    if not args.no_extras:
+        gemms = []
+        for name, (k, n) in wl.CONFIG4_SHAPES.items():
+            cc = wl.config4(name, M=8)
+            gemms.append(gemm_case(rt, wl, f"config4 {name}", 4096, k, n, cc["W"], cc["w_scale"],
+                                   args.steps, args.warmup, "f32"))
+        gemms.append(gemm_case(rt, wl, "config4 FFN-up int32 out", M, K, N, c["W"], c["w_scale"],
+                               args.steps, args.warmup, "i32"))
+        for name, (k, n) in wl.CONFIG5_SHAPES.items():
+            cc = wl.config5(name, M=8)
+            gemms.append(gemm_case(rt, wl, f"config5 prefill {name}", 2048, k, n, cc["W"], cc["w_scale"],
+                                   max(10, args.steps // 10), max(2, args.warmup // 10), "f32"))
+        extras["gemm"] = gemms
+        extras["decode"] = [decode_case(rt, wl, m, args.steps, args.warmup) for m in (1, 4, 16)]
+        qsteps = max(5, args.steps // 10)
+        extras["qdq_8192x32768"] = qdq_cases(rt, wl, 8192, 32768, qsteps, max(2, args.warmup // 10))
+        extras["qdq_8191x32767"] = qdq_cases(rt, wl, 8191, 32767, qsteps, max(2, args.warmup // 10))
+
+    cpu = None
+    if not args.no_cpu:
+        import oracle_lib
+        cpu = cpu_baseline_gemm(oracle_lib.load(), wl, M, K, N)
+
+    line = {
+        "metric": METRIC,
+        "value": main_res["tops"],
+        "unit": "TOPS",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": main_res["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int8",
+        "data": "synthetic",
+        "config": {"workload": f"config4 FFN-up MatMulInteger M={M} K={K} N={N}, uint8 activations x int8 "
+                               f"weights, a_zp scalar, {'per-column fp32 dequant' if epi == 'f32' else 'int32'} "
+                               "output, operands resident in HBM, weights packed once"},
+        "roofline": {"bound": "mfma", "achieved": main_res["kernel_tops"], "peak": INT8_PEAK_TOPS,
+                     "unit": "TOP/s", "frac": main_res["kernel_tops"] / INT8_PEAK_TOPS,
+                     "traffic": None, "kernel": "k_gemm_i8", "kernel_ms": main_res["kernel_ms"],
+                     "hbm_bound_tops": main_res["ops"] / (main_res["hbm_bytes_algorithmic"] / (HBM_PEAK_GBS * 1e9)) / 1e12},
+        "cpu_baseline": cpu,
+        "device": info,
+        "extras": extras,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

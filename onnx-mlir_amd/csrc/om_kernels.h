@@ -1,0 +1,89 @@
+// Internal interface between the runtime (OMTensor marshalling, residency)
+// and the gfx950 kernels.  Everything here works on GPU pointers only.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace om {
+
+enum QKind : int { kU8 = 0, kI8 = 1, kI32 = 2 };
+enum Epilogue : int { kEpiI32 = 0, kEpiF32 = 1, kEpiQ8 = 2 };
+enum NarrowMode : int { kWrap = 0, kSaturate = 1 };
+
+// ---- quantize / dequantize (HBM-bound streaming kernels) ------------------
+// The tensor is viewed as [outer, channels, inner]; scale / zp have `channels`
+// entries.  channels == 1 is the per-tensor case.  zp may be null.
+hipError_t launch_quantize(hipStream_t s, const float *x, int64_t outer,
+    int64_t channels, int64_t inner, const float *scale, const void *zp,
+    bool is_signed, void *y);
+
+hipError_t launch_dequantize(hipStream_t s, const void *x, QKind xkind,
+    int64_t outer, int64_t channels, int64_t inner, const float *scale,
+    const void *zp, float *y);
+
+// Scratch a DynamicQuantizeLinear launch needs: per-block partial min / max
+// and an arrival counter that must be zero before the first launch (the
+// kernel leaves it zero).
+struct DqlScratch {
+  float *partial_min; // [kDqlMaxBlocks]
+  float *partial_max; // [kDqlMaxBlocks]
+  unsigned *counter;  // [1]
+};
+constexpr int kDqlMaxBlocks = 4096;
+
+// y u8[n], scale f32[1], zp u8[1].  If y_shift is true the stored bytes are
+// y ^ 0x80 (the value minus 128 as int8), the form the GEMM consumes, and
+// row sums are not needed because they are not produced here.
+hipError_t launch_dynamic_quantize(hipStream_t s, const DqlScratch &scratch,
+    const float *x, int64_t n, uint8_t *y, float *scale, uint8_t *zp,
+    bool y_shift);
+
+// ---- int8 GEMM ------------------------------------------------------------
+// B [K,N] row-major (u8 or i8) -> Bt [Npad, Kpad] int8, K-contiguous, with
+// u8 shifted to int8 by -128, zero filled outside [N,K]; colsum[n] = sum_k of
+// the int8 values written (int32), colsum has Npad entries.
+constexpr int kGemmBK = 64;    // K granularity of the packed operand
+constexpr int kGemmBN = 128;   // N granularity of the packed operand
+inline int64_t round_up(int64_t v, int64_t m) { return (v + m - 1) / m * m; }
+
+hipError_t launch_pack_b(hipStream_t s, const void *B, bool b_unsigned,
+    int64_t K, int64_t N, int8_t *Bt, int32_t *colsum);
+
+// rowsum[m] = sum_k (A[m,k] - (a_unsigned ? 128 : 0)).
+hipError_t launch_rowsum_a(hipStream_t s, const void *A, bool a_unsigned,
+    int64_t M, int64_t K, int32_t *rowsum);
+
+struct GemmArgs {
+  const void *A;       // [M,K] row-major, u8 or i8
+  bool a_unsigned;     // A holds u8
+  bool a_preshifted;   // A already holds (u8 - 128) as int8; offsets as for u8
+  const int8_t *Bt;    // packed [Npad,Kpad]
+  bool b_unsigned;     // original B was u8 (packed values are B - 128)
+  int64_t M, K, N;
+  const void *a_zp;    // element type follows A; may be null
+  int64_t a_zp_len;    // 0, 1 or M
+  const void *b_zp;    // element type follows B; may be null
+  int64_t b_zp_len;    // 0, 1 or N
+  const int32_t *rowsum; // sum_k A' per row; may be null when B offset is 0
+  const int32_t *colsum; // sum_k B' per column (Npad entries)
+  Epilogue epi;
+  // kEpiF32: out = f32(acc) * (a_scale[0] * b_scale[j or 0])
+  // kEpiQ8 : s = (a_scale[0]*b_scale[0]) / y_scale[0];
+  //          out = narrow(i32(rne(f32(acc) * s)) + y_zp)
+  const float *a_scale;
+  const float *b_scale;
+  int64_t b_scale_len; // 1 or N
+  const float *y_scale;
+  const void *y_zp;
+  bool y_unsigned;
+  NarrowMode narrow;
+  void *out;           // i32 / f32 / u8|i8 [M,N]
+};
+
+hipError_t launch_gemm(hipStream_t s, const GemmArgs &g);
+
+// Fill n 32-bit words with v.
+hipError_t launch_fill_u32(hipStream_t s, uint32_t *p, int64_t n, uint32_t v);
+
+} // namespace om

@@ -1,0 +1,701 @@
+// QuantizeLinear / DequantizeLinear / DynamicQuantizeLinear for gfx950.
+//
+// All three are HBM-bound streaming kernels: every lane moves 16 bytes per
+// memory instruction on the wide side (float4) and 4 bytes on the narrow side
+// (four packed 8-bit values), consecutive lanes touch consecutive addresses,
+// and several loads are issued before the first use so that enough bytes are
+// in flight to cover HBM latency.
+//
+// Arithmetic follows the reference's generated code operation for operation
+// (src/Conversion/ONNXToKrnl/Quantization/QuantizeLinear.cpp:119-144):
+//   t = x / scale          IEEE-754 correctly rounded divide (never rcp*mul)
+//   r = roundEven(t)       v_rndne_f32 == the reference's floor-based
+//                          emulation (src/Dialect/Mlir/DialectBuilder.cpp
+//                          :291-332) for every input, up to the sign of zero
+//   r = r + zp             separate add (no FMA contraction: -ffp-contract=off)
+//   c = min(max(r,lo),hi)  maxnum then minnum: NaN -> lo
+//   y = trunc_i8(fpto[us]i(c))
+// Denormals are kept (the file is built with -fno-gpu-flush-denormals-to-zero).
+
+#include "om_kernels.h"
+
+namespace om {
+
+namespace {
+
+constexpr int kThreads = 256;
+
+typedef float f4a __attribute__((ext_vector_type(4)));
+typedef float f4u __attribute__((ext_vector_type(4), aligned(4)));
+typedef uint32_t u32_a1 __attribute__((aligned(1)));
+typedef int32_t i4u __attribute__((ext_vector_type(4), aligned(4)));
+
+template <bool SIGNED>
+__device__ __forceinline__ float load_zp_f32(const void *zp, int64_t i) {
+  // int -> f32 through a 32-bit integer of the same signedness
+  // (src/Dialect/Mlir/DialectBuilder.cpp:979-995).
+  if (SIGNED)
+    return (float)(int32_t)((const int8_t *)zp)[i];
+  return (float)(uint32_t)((const uint8_t *)zp)[i];
+}
+
+template <bool SIGNED, bool HAS_ZP>
+__device__ __forceinline__ uint32_t quant_one(float x, float s, float zpf) {
+  float t = x / s;
+  float r = __builtin_rintf(t);
+  if (HAS_ZP)
+    r = r + zpf;
+  if (SIGNED) {
+    float c = __builtin_fminf(__builtin_fmaxf(r, -128.0f), 127.0f);
+    return (uint32_t)((int32_t)c) & 0xFFu;
+  }
+  float c = __builtin_fminf(__builtin_fmaxf(r, 0.0f), 255.0f);
+  return (uint32_t)c;
+}
+
+template <bool SIGNED, bool HAS_ZP>
+__device__ __forceinline__ uint32_t quant_four(
+    f4a v, float s, float zpf, uint32_t flip) {
+  uint32_t b0 = quant_one<SIGNED, HAS_ZP>(v.x, s, zpf);
+  uint32_t b1 = quant_one<SIGNED, HAS_ZP>(v.y, s, zpf);
+  uint32_t b2 = quant_one<SIGNED, HAS_ZP>(v.z, s, zpf);
+  uint32_t b3 = quant_one<SIGNED, HAS_ZP>(v.w, s, zpf);
+  return (b0 | (b1 << 8) | (b2 << 16) | (b3 << 24)) ^ flip;
+}
+
+// ---- per-tensor quantize over a flat array -------------------------------
+// x must be 16-byte aligned and y 4-byte aligned.  Each block handles
+// kThreads*UNROLL float4 per step; `flip` is 0, or 0x80808080 to store the
+// result minus 128 as int8.
+constexpr int kUnroll = 4;
+
+template <bool SIGNED, bool HAS_ZP>
+__global__ __launch_bounds__(kThreads) void k_quant_flat(
+    const float *__restrict__ x, uint8_t *__restrict__ y, int64_t n,
+    const float *__restrict__ scale_p, const void *__restrict__ zp_p,
+    uint32_t flip) {
+  const float s = scale_p[0];
+  const float zpf = HAS_ZP ? load_zp_f32<SIGNED>(zp_p, 0) : 0.0f;
+  const int64_t nvec = n >> 2;
+  const f4a *__restrict__ x4 = (const f4a *)x;
+  uint32_t *__restrict__ y4 = (uint32_t *)y;
+  const int64_t step = (int64_t)gridDim.x * (kThreads * kUnroll);
+  for (int64_t base = (int64_t)blockIdx.x * (kThreads * kUnroll); base < nvec;
+       base += step) {
+    f4a v[kUnroll];
+    int64_t idx[kUnroll];
+#pragma unroll
+    for (int j = 0; j < kUnroll; ++j) {
+      idx[j] = base + j * kThreads + threadIdx.x;
+      if (idx[j] < nvec)
+        v[j] = __builtin_nontemporal_load(&x4[idx[j]]);
+    }
+#pragma unroll
+    for (int j = 0; j < kUnroll; ++j) {
+      if (idx[j] < nvec)
+        __builtin_nontemporal_store(
+            quant_four<SIGNED, HAS_ZP>(v[j], s, zpf, flip), &y4[idx[j]]);
+    }
+  }
+  // Up to three trailing elements.
+  if (blockIdx.x == 0) {
+    int64_t e = (nvec << 2) + threadIdx.x;
+    if (e < n)
+      y[e] = (uint8_t)(quant_one<SIGNED, HAS_ZP>(x[e], s, zpf) ^ (flip & 0xFFu));
+  }
+}
+
+// ---- per-axis quantize, axis is the innermost dimension -------------------
+// View [rows, C]; each thread owns four fixed columns, keeps their scale and
+// zero point in registers and walks down `rows_per_block` rows.  Row starts
+// need not be 16-byte aligned (C % 4 != 0): loads are dword-aligned float4,
+// the 4-byte store may sit at any byte address.
+template <bool SIGNED, bool HAS_ZP>
+__global__ __launch_bounds__(kThreads) void k_quant_lastaxis(
+    const float *__restrict__ x, uint8_t *__restrict__ y, int64_t rows,
+    int64_t C, const float *__restrict__ scale, const void *__restrict__ zp,
+    int rows_per_block) {
+  const int64_t c0 = ((int64_t)blockIdx.x * kThreads + threadIdx.x) * 4;
+  if (c0 >= C)
+    return;
+  const int ncol = (C - c0 >= 4) ? 4 : (int)(C - c0);
+  float s[4], z[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int64_t c = c0 + (j < ncol ? j : 0);
+    s[j] = scale[c];
+    z[j] = HAS_ZP ? load_zp_f32<SIGNED>(zp, c) : 0.0f;
+  }
+  const int64_t r_begin = (int64_t)blockIdx.y * rows_per_block;
+  const int64_t r_end =
+      (r_begin + rows_per_block < rows) ? r_begin + rows_per_block : rows;
+  if (ncol == 4) {
+    int64_t r = r_begin;
+    for (; r + kUnroll <= r_end; r += kUnroll) {
+      f4u v[kUnroll];
+#pragma unroll
+      for (int j = 0; j < kUnroll; ++j)
+        v[j] = __builtin_nontemporal_load((const f4u *)(x + (r + j) * C + c0));
+#pragma unroll
+      for (int j = 0; j < kUnroll; ++j) {
+        uint32_t b0 = quant_one<SIGNED, HAS_ZP>(v[j].x, s[0], z[0]);
+        uint32_t b1 = quant_one<SIGNED, HAS_ZP>(v[j].y, s[1], z[1]);
+        uint32_t b2 = quant_one<SIGNED, HAS_ZP>(v[j].z, s[2], z[2]);
+        uint32_t b3 = quant_one<SIGNED, HAS_ZP>(v[j].w, s[3], z[3]);
+        *(u32_a1 *)(y + (r + j) * C + c0) =
+            b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
+      }
+    }
+    for (; r < r_end; ++r) {
+      f4u v = *(const f4u *)(x + r * C + c0);
+      uint32_t b0 = quant_one<SIGNED, HAS_ZP>(v.x, s[0], z[0]);
+      uint32_t b1 = quant_one<SIGNED, HAS_ZP>(v.y, s[1], z[1]);
+      uint32_t b2 = quant_one<SIGNED, HAS_ZP>(v.z, s[2], z[2]);
+      uint32_t b3 = quant_one<SIGNED, HAS_ZP>(v.w, s[3], z[3]);
+      *(u32_a1 *)(y + r * C + c0) = b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
+    }
+  } else {
+    for (int64_t r = r_begin; r < r_end; ++r)
+      for (int j = 0; j < ncol; ++j)
+        y[r * C + c0 + j] =
+            (uint8_t)quant_one<SIGNED, HAS_ZP>(x[r * C + c0 + j], s[j], z[j]);
+  }
+}
+
+// ---- general [outer, channels, inner] quantize ---------------------------
+// One block row per (outer, channel) pair; the scale is uniform over a run of
+// `inner` elements.  Used when the axis is not the innermost dimension, and as
+// the fallback for misaligned per-tensor buffers.
+template <bool SIGNED, bool HAS_ZP>
+__global__ __launch_bounds__(kThreads) void k_quant_general(
+    const float *__restrict__ x, uint8_t *__restrict__ y, int64_t channels,
+    int64_t inner, const float *__restrict__ scale,
+    const void *__restrict__ zp, int64_t oc_total) {
+  for (int64_t oc = blockIdx.y; oc < oc_total; oc += gridDim.y) {
+    const int64_t c = oc % channels;
+    const float s = scale[c];
+    const float zpf = HAS_ZP ? load_zp_f32<SIGNED>(zp, c) : 0.0f;
+    const float *__restrict__ xr = x + oc * inner;
+    uint8_t *__restrict__ yr = y + oc * inner;
+    for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < inner;
+         i += (int64_t)gridDim.x * kThreads)
+      yr[i] = (uint8_t)quant_one<SIGNED, HAS_ZP>(xr[i], s, zpf);
+  }
+}
+
+// ---- dequantize -----------------------------------------------------------
+// y = (f32(x) - f32(zp)) * scale  (src/Conversion/ONNXToKrnl/Math/
+// Elementwise.cpp:1439-1461): int->f32 conversion, subtract, multiply, each
+// rounded once.
+template <int KIND>
+__device__ __forceinline__ float q_to_f32(uint32_t byte_or_word) {
+  if (KIND == kU8)
+    return (float)(byte_or_word & 0xFFu);
+  if (KIND == kI8)
+    return (float)(int32_t)(int8_t)(byte_or_word & 0xFFu);
+  return (float)(int32_t)byte_or_word;
+}
+
+template <int KIND>
+__device__ __forceinline__ float load_q_zp_f32(const void *zp, int64_t i) {
+  if (KIND == kU8)
+    return (float)(uint32_t)((const uint8_t *)zp)[i];
+  if (KIND == kI8)
+    return (float)(int32_t)((const int8_t *)zp)[i];
+  return (float)((const int32_t *)zp)[i];
+}
+
+template <bool HAS_ZP>
+__device__ __forceinline__ float dq_one(float xf, float s, float zpf) {
+  if (HAS_ZP)
+    xf = xf - zpf;
+  return xf * s;
+}
+
+// 8-bit input, flat: each lane reads one dword (4 values) and writes one
+// float4; x 4-byte aligned, y 16-byte aligned.
+template <int KIND, bool HAS_ZP>
+__global__ __launch_bounds__(kThreads) void k_dequant8_flat(
+    const uint8_t *__restrict__ x, float *__restrict__ y, int64_t n,
+    const float *__restrict__ scale_p, const void *__restrict__ zp_p) {
+  const float s = scale_p[0];
+  const float zpf = HAS_ZP ? load_q_zp_f32<KIND>(zp_p, 0) : 0.0f;
+  const int64_t nvec = n >> 2;
+  const uint32_t *__restrict__ x4 = (const uint32_t *)x;
+  f4a *__restrict__ y4 = (f4a *)y;
+  const int64_t step = (int64_t)gridDim.x * (kThreads * kUnroll);
+  for (int64_t base = (int64_t)blockIdx.x * (kThreads * kUnroll); base < nvec;
+       base += step) {
+    uint32_t w[kUnroll];
+    int64_t idx[kUnroll];
+#pragma unroll
+    for (int j = 0; j < kUnroll; ++j) {
+      idx[j] = base + j * kThreads + threadIdx.x;
+      if (idx[j] < nvec)
+        w[j] = __builtin_nontemporal_load(&x4[idx[j]]);
+    }
+#pragma unroll
+    for (int j = 0; j < kUnroll; ++j) {
+      if (idx[j] < nvec) {
+        f4a o;
+        o.x = dq_one<HAS_ZP>(q_to_f32<KIND>(w[j]), s, zpf);
+        o.y = dq_one<HAS_ZP>(q_to_f32<KIND>(w[j] >> 8), s, zpf);
+        o.z = dq_one<HAS_ZP>(q_to_f32<KIND>(w[j] >> 16), s, zpf);
+        o.w = dq_one<HAS_ZP>(q_to_f32<KIND>(w[j] >> 24), s, zpf);
+        __builtin_nontemporal_store(o, &y4[idx[j]]);
+      }
+    }
+  }
+  if (blockIdx.x == 0) {
+    int64_t e = (nvec << 2) + threadIdx.x;
+    if (e < n)
+      y[e] = dq_one<HAS_ZP>(q_to_f32<KIND>(x[e]), s, zpf);
+  }
+}
+
+// Axis innermost: four fixed columns per thread.  8-bit input is read as one
+// dword at any byte address, 32-bit input as a dword-aligned int4.
+template <int KIND>
+__device__ __forceinline__ void load_four_q(
+    const void *x, int64_t elem, uint32_t (&q)[4]) {
+  if (KIND == kI32) {
+    i4u v = __builtin_nontemporal_load((const i4u *)((const int32_t *)x + elem));
+    q[0] = (uint32_t)v.x;
+    q[1] = (uint32_t)v.y;
+    q[2] = (uint32_t)v.z;
+    q[3] = (uint32_t)v.w;
+  } else {
+    uint32_t w =
+        __builtin_nontemporal_load((const u32_a1 *)((const uint8_t *)x + elem));
+    q[0] = w & 0xFFu;
+    q[1] = (w >> 8) & 0xFFu;
+    q[2] = (w >> 16) & 0xFFu;
+    q[3] = w >> 24;
+  }
+}
+
+template <int KIND>
+__device__ __forceinline__ uint32_t load_one_q(const void *x, int64_t elem) {
+  if (KIND == kI32)
+    return (uint32_t)((const int32_t *)x)[elem];
+  return ((const uint8_t *)x)[elem];
+}
+
+template <int KIND, bool HAS_ZP>
+__global__ __launch_bounds__(kThreads) void k_dequant_lastaxis(
+    const void *__restrict__ x, float *__restrict__ y, int64_t rows, int64_t C,
+    const float *__restrict__ scale, const void *__restrict__ zp,
+    int rows_per_block) {
+  const int64_t c0 = ((int64_t)blockIdx.x * kThreads + threadIdx.x) * 4;
+  if (c0 >= C)
+    return;
+  const int ncol = (C - c0 >= 4) ? 4 : (int)(C - c0);
+  float s[4], z[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int64_t c = c0 + (j < ncol ? j : 0);
+    s[j] = scale[c];
+    z[j] = HAS_ZP ? load_q_zp_f32<KIND>(zp, c) : 0.0f;
+  }
+  const int64_t r_begin = (int64_t)blockIdx.y * rows_per_block;
+  const int64_t r_end =
+      (r_begin + rows_per_block < rows) ? r_begin + rows_per_block : rows;
+  if (ncol == 4) {
+    int64_t r = r_begin;
+    for (; r + kUnroll <= r_end; r += kUnroll) {
+      uint32_t q[kUnroll][4];
+#pragma unroll
+      for (int j = 0; j < kUnroll; ++j)
+        load_four_q<KIND>(x, (r + j) * C + c0, q[j]);
+#pragma unroll
+      for (int j = 0; j < kUnroll; ++j) {
+        f4u o;
+        o.x = dq_one<HAS_ZP>(q_to_f32<KIND>(q[j][0]), s[0], z[0]);
+        o.y = dq_one<HAS_ZP>(q_to_f32<KIND>(q[j][1]), s[1], z[1]);
+        o.z = dq_one<HAS_ZP>(q_to_f32<KIND>(q[j][2]), s[2], z[2]);
+        o.w = dq_one<HAS_ZP>(q_to_f32<KIND>(q[j][3]), s[3], z[3]);
+        *(f4u *)(y + (r + j) * C + c0) = o;
+      }
+    }
+    for (; r < r_end; ++r) {
+      uint32_t q[4];
+      load_four_q<KIND>(x, r * C + c0, q);
+      f4u o;
+      o.x = dq_one<HAS_ZP>(q_to_f32<KIND>(q[0]), s[0], z[0]);
+      o.y = dq_one<HAS_ZP>(q_to_f32<KIND>(q[1]), s[1], z[1]);
+      o.z = dq_one<HAS_ZP>(q_to_f32<KIND>(q[2]), s[2], z[2]);
+      o.w = dq_one<HAS_ZP>(q_to_f32<KIND>(q[3]), s[3], z[3]);
+      *(f4u *)(y + r * C + c0) = o;
+    }
+  } else {
+    for (int64_t r = r_begin; r < r_end; ++r)
+      for (int j = 0; j < ncol; ++j)
+        y[r * C + c0 + j] = dq_one<HAS_ZP>(
+            q_to_f32<KIND>(load_one_q<KIND>(x, r * C + c0 + j)), s[j], z[j]);
+  }
+}
+
+// Any element kind, [outer, channels, inner]: one element per lane.
+template <int KIND, bool HAS_ZP>
+__global__ __launch_bounds__(kThreads) void k_dequant_general(
+    const void *__restrict__ x, float *__restrict__ y, int64_t channels,
+    int64_t inner, const float *__restrict__ scale,
+    const void *__restrict__ zp, int64_t oc_total) {
+  for (int64_t oc = blockIdx.y; oc < oc_total; oc += gridDim.y) {
+    const int64_t c = oc % channels;
+    const float s = scale[c];
+    const float zpf = HAS_ZP ? load_q_zp_f32<KIND>(zp, c) : 0.0f;
+    float *__restrict__ yr = y + oc * inner;
+    for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < inner;
+         i += (int64_t)gridDim.x * kThreads) {
+      uint32_t raw;
+      if (KIND == kI32)
+        raw = (uint32_t)((const int32_t *)x)[oc * inner + i];
+      else
+        raw = ((const uint8_t *)x)[oc * inner + i];
+      yr[i] = dq_one<HAS_ZP>(q_to_f32<KIND>(raw), s, zpf);
+    }
+  }
+}
+
+// ---- DynamicQuantizeLinear: min / max reduction ---------------------------
+// minnum / maxnum from +inf / -inf (src/Conversion/ONNXToKrnl/Math/
+// Reduction.cpp:529-548); the order of a min / max reduction does not change
+// its value, so lanes, waves and blocks may combine in any order.
+__device__ __forceinline__ float wave_min(float v) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1)
+    v = __builtin_fminf(v, __shfl_xor(v, off, 64));
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1)
+    v = __builtin_fmaxf(v, __shfl_xor(v, off, 64));
+  return v;
+}
+
+__device__ __forceinline__ void block_minmax(float &lo, float &hi) {
+  __shared__ float s_lo[kThreads / 64], s_hi[kThreads / 64];
+  lo = wave_min(lo);
+  hi = wave_max(hi);
+  const int wave = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) {
+    s_lo[wave] = lo;
+    s_hi[wave] = hi;
+  }
+  __syncthreads();
+  lo = s_lo[0];
+  hi = s_hi[0];
+#pragma unroll
+  for (int w = 1; w < kThreads / 64; ++w) {
+    lo = __builtin_fminf(lo, s_lo[w]);
+    hi = __builtin_fmaxf(hi, s_hi[w]);
+  }
+  __syncthreads();
+}
+
+// Scale and zero point from min / max
+// (src/Conversion/ONNXToKrnl/Quantization/DynamicQuantizeLinear.cpp:43-84).
+__device__ __forceinline__ void dynamic_params(
+    float xmin, float xmax, float &scale, float &zpf) {
+  const float mx = __builtin_fmaxf(xmax, 0.0f);
+  const float mn = __builtin_fminf(xmin, 0.0f);
+  const float xdiff = mx - mn;
+  const float bound = 255.0f - 0.0f;
+  scale = xdiff / bound;
+  const float inter = 0.0f - mn / scale;
+  const float sat = __builtin_fminf(__builtin_fmaxf(inter, 0.0f), 255.0f);
+  zpf = __builtin_rintf(sat);
+}
+
+__global__ __launch_bounds__(kThreads) void k_minmax_params(
+    const float *__restrict__ x, int64_t n, float *partial_min,
+    float *partial_max, unsigned *counter, float *__restrict__ scale_out,
+    uint8_t *__restrict__ zp_out) {
+  float lo = __builtin_inff(), hi = -__builtin_inff();
+  const int64_t nvec = n >> 2;
+  const float4 *__restrict__ x4 = (const float4 *)x;
+  const bool aligned = (((uintptr_t)x) & 15) == 0;
+  if (aligned) {
+    const int64_t step = (int64_t)gridDim.x * (kThreads * kUnroll);
+    for (int64_t base = (int64_t)blockIdx.x * (kThreads * kUnroll);
+         base < nvec; base += step) {
+      float4 v[kUnroll];
+#pragma unroll
+      for (int j = 0; j < kUnroll; ++j) {
+        const int64_t idx = base + j * kThreads + threadIdx.x;
+        if (idx < nvec)
+          v[j] = x4[idx];
+        else
+          v[j] = make_float4(__builtin_nanf(""), __builtin_nanf(""),
+              __builtin_nanf(""), __builtin_nanf(""));
+      }
+#pragma unroll
+      for (int j = 0; j < kUnroll; ++j) {
+        // The NaN filler above is neutral: minnum / maxnum ignore NaN.
+        lo = __builtin_fminf(lo, __builtin_fminf(__builtin_fminf(v[j].x, v[j].y),
+                                     __builtin_fminf(v[j].z, v[j].w)));
+        hi = __builtin_fmaxf(hi, __builtin_fmaxf(__builtin_fmaxf(v[j].x, v[j].y),
+                                     __builtin_fmaxf(v[j].z, v[j].w)));
+      }
+    }
+    if (blockIdx.x == 0) {
+      const int64_t e = (nvec << 2) + threadIdx.x;
+      if (e < n) {
+        lo = __builtin_fminf(lo, x[e]);
+        hi = __builtin_fmaxf(hi, x[e]);
+      }
+    }
+  } else {
+    for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < n;
+         i += (int64_t)gridDim.x * kThreads) {
+      lo = __builtin_fminf(lo, x[i]);
+      hi = __builtin_fmaxf(hi, x[i]);
+    }
+  }
+  block_minmax(lo, hi);
+
+  __shared__ bool s_last;
+  if (threadIdx.x == 0) {
+    __hip_atomic_store(&partial_min[blockIdx.x], lo, __ATOMIC_RELAXED,
+        __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(&partial_max[blockIdx.x], hi, __ATOMIC_RELAXED,
+        __HIP_MEMORY_SCOPE_AGENT);
+    const unsigned ticket = __hip_atomic_fetch_add(
+        counter, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+    s_last = (ticket == gridDim.x - 1);
+  }
+  __syncthreads();
+  if (!s_last)
+    return;
+  // Last block to arrive: every partial is visible (release on each block's
+  // ticket, acquire on ours).  Fold them and derive the parameters.
+  lo = __builtin_inff();
+  hi = -__builtin_inff();
+  for (unsigned i = threadIdx.x; i < gridDim.x; i += kThreads) {
+    lo = __builtin_fminf(lo, __hip_atomic_load(&partial_min[i],
+                                 __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+    hi = __builtin_fmaxf(hi, __hip_atomic_load(&partial_max[i],
+                                 __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+  }
+  block_minmax(lo, hi);
+  if (threadIdx.x == 0) {
+    float scale, zpf;
+    dynamic_params(lo, hi, scale, zpf);
+    scale_out[0] = scale;
+    zp_out[0] = (uint8_t)(uint32_t)zpf;
+    __hip_atomic_store(
+        counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
+__global__ __launch_bounds__(kThreads) void k_fill_u32(
+    uint32_t *__restrict__ p, int64_t n, uint32_t v) {
+  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < n;
+       i += (int64_t)gridDim.x * kThreads)
+    p[i] = v;
+}
+
+inline int stream_grid(int64_t work_items, int64_t per_block) {
+  // Enough blocks to keep 256 CUs busy with several resident blocks each,
+  // never more than the work needs.
+  int64_t need = (work_items + per_block - 1) / per_block;
+  if (need < 1)
+    need = 1;
+  const int64_t cap = 256 * 16;
+  return (int)(need < cap ? need : cap);
+}
+
+template <bool SIGNED>
+hipError_t quantize_dispatch(hipStream_t st, const float *x, int64_t outer,
+    int64_t channels, int64_t inner, const float *scale, const void *zp,
+    void *y, uint32_t flip) {
+  const int64_t n = outer * channels * inner;
+  if (n == 0)
+    return hipSuccess;
+  uint8_t *yo = (uint8_t *)y;
+  const bool has_zp = zp != nullptr;
+  if (channels == 1) {
+    const bool aligned =
+        ((((uintptr_t)x) & 15) == 0) && ((((uintptr_t)y) & 3) == 0);
+    if (aligned) {
+      const int grid = stream_grid(n >> 2, kThreads * kUnroll);
+      if (has_zp)
+        k_quant_flat<SIGNED, true>
+            <<<grid, kThreads, 0, st>>>(x, yo, n, scale, zp, flip);
+      else
+        k_quant_flat<SIGNED, false>
+            <<<grid, kThreads, 0, st>>>(x, yo, n, scale, zp, flip);
+      return hipGetLastError();
+    }
+    if (flip != 0)
+      return hipErrorInvalidValue;
+    // Misaligned buffers: treat as one long run.
+    outer = 1;
+    inner = n;
+  }
+  if (flip != 0)
+    return hipErrorInvalidValue;
+  if (inner == 1 && channels > 1) {
+    const int64_t rows = outer, C = channels;
+    const int64_t col_blocks = (C + kThreads * 4 - 1) / (kThreads * 4);
+    // Aim for ~4096 blocks in total; at least 16 rows per block.
+    int64_t row_blocks = 4096 / col_blocks;
+    if (row_blocks < 1)
+      row_blocks = 1;
+    int64_t rpb = (rows + row_blocks - 1) / row_blocks;
+    if (rpb < 16)
+      rpb = 16;
+    row_blocks = (rows + rpb - 1) / rpb;
+    if (row_blocks > 65535) {
+      rpb = (rows + 65534) / 65535;
+      row_blocks = (rows + rpb - 1) / rpb;
+    }
+    dim3 grid((unsigned)col_blocks, (unsigned)row_blocks);
+    if (has_zp)
+      k_quant_lastaxis<SIGNED, true>
+          <<<grid, kThreads, 0, st>>>(x, yo, rows, C, scale, zp, (int)rpb);
+    else
+      k_quant_lastaxis<SIGNED, false>
+          <<<grid, kThreads, 0, st>>>(x, yo, rows, C, scale, zp, (int)rpb);
+    return hipGetLastError();
+  }
+  // General [outer, channels, inner].
+  const int64_t oc = outer * channels;
+  const int64_t gy = oc < 4096 ? oc : 4096;
+  int64_t gx = (inner + kThreads - 1) / kThreads;
+  const int64_t cap = (4096 + gy - 1) / gy;
+  if (gx > cap)
+    gx = cap;
+  if (gx < 1)
+    gx = 1;
+  dim3 grid((unsigned)gx, (unsigned)gy);
+  if (has_zp)
+    k_quant_general<SIGNED, true>
+        <<<grid, kThreads, 0, st>>>(x, yo, channels, inner, scale, zp, oc);
+  else
+    k_quant_general<SIGNED, false>
+        <<<grid, kThreads, 0, st>>>(x, yo, channels, inner, scale, zp, oc);
+  return hipGetLastError();
+}
+
+template <int KIND>
+hipError_t dequantize_dispatch(hipStream_t st, const void *x, int64_t outer,
+    int64_t channels, int64_t inner, const float *scale, const void *zp,
+    float *y) {
+  const int64_t n = outer * channels * inner;
+  if (n == 0)
+    return hipSuccess;
+  const bool has_zp = zp != nullptr;
+  if (KIND != kI32 && channels == 1 && ((((uintptr_t)x) & 3) == 0) &&
+      ((((uintptr_t)y) & 15) == 0)) {
+    const uint8_t *xi = (const uint8_t *)x;
+    const int grid = stream_grid(n >> 2, kThreads * kUnroll);
+    if (has_zp)
+      k_dequant8_flat<KIND, true>
+          <<<grid, kThreads, 0, st>>>(xi, y, n, scale, zp);
+    else
+      k_dequant8_flat<KIND, false>
+          <<<grid, kThreads, 0, st>>>(xi, y, n, scale, zp);
+    return hipGetLastError();
+  }
+  if (inner == 1 && channels > 1) {
+    const int64_t rows = outer, C = channels;
+    const int64_t col_blocks = (C + kThreads * 4 - 1) / (kThreads * 4);
+    int64_t row_blocks = 4096 / col_blocks;
+    if (row_blocks < 1)
+      row_blocks = 1;
+    int64_t rpb = (rows + row_blocks - 1) / row_blocks;
+    if (rpb < 16)
+      rpb = 16;
+    row_blocks = (rows + rpb - 1) / rpb;
+    if (row_blocks > 65535) {
+      rpb = (rows + 65534) / 65535;
+      row_blocks = (rows + rpb - 1) / rpb;
+    }
+    dim3 grid((unsigned)col_blocks, (unsigned)row_blocks);
+    if (has_zp)
+      k_dequant_lastaxis<KIND, true>
+          <<<grid, kThreads, 0, st>>>(x, y, rows, C, scale, zp, (int)rpb);
+    else
+      k_dequant_lastaxis<KIND, false>
+          <<<grid, kThreads, 0, st>>>(x, y, rows, C, scale, zp, (int)rpb);
+    return hipGetLastError();
+  }
+  if (channels == 1) {
+    outer = 1;
+    inner = n;
+  }
+  const int64_t oc = outer * channels;
+  const int64_t gy = oc < 4096 ? oc : 4096;
+  int64_t gx = (inner + kThreads - 1) / kThreads;
+  const int64_t cap = (4096 + gy - 1) / gy;
+  if (gx > cap)
+    gx = cap;
+  if (gx < 1)
+    gx = 1;
+  dim3 grid((unsigned)gx, (unsigned)gy);
+  if (has_zp)
+    k_dequant_general<KIND, true>
+        <<<grid, kThreads, 0, st>>>(x, y, channels, inner, scale, zp, oc);
+  else
+    k_dequant_general<KIND, false>
+        <<<grid, kThreads, 0, st>>>(x, y, channels, inner, scale, zp, oc);
+  return hipGetLastError();
+}
+
+} // namespace
+
+hipError_t launch_quantize(hipStream_t s, const float *x, int64_t outer,
+    int64_t channels, int64_t inner, const float *scale, const void *zp,
+    bool is_signed, void *y) {
+  if (is_signed)
+    return quantize_dispatch<true>(
+        s, x, outer, channels, inner, scale, zp, y, 0u);
+  return quantize_dispatch<false>(
+      s, x, outer, channels, inner, scale, zp, y, 0u);
+}
+
+hipError_t launch_dequantize(hipStream_t s, const void *x, QKind xkind,
+    int64_t outer, int64_t channels, int64_t inner, const float *scale,
+    const void *zp, float *y) {
+  switch (xkind) {
+  case kU8:
+    return dequantize_dispatch<kU8>(s, x, outer, channels, inner, scale, zp, y);
+  case kI8:
+    return dequantize_dispatch<kI8>(s, x, outer, channels, inner, scale, zp, y);
+  default:
+    return dequantize_dispatch<kI32>(
+        s, x, outer, channels, inner, scale, zp, y);
+  }
+}
+
+hipError_t launch_dynamic_quantize(hipStream_t s, const DqlScratch &scratch,
+    const float *x, int64_t n, uint8_t *y, float *scale, uint8_t *zp,
+    bool y_shift) {
+  if (n == 0)
+    return hipSuccess;
+  int grid = stream_grid(n >> 2, kThreads * kUnroll);
+  if (grid > kDqlMaxBlocks)
+    grid = kDqlMaxBlocks;
+  k_minmax_params<<<grid, kThreads, 0, s>>>(x, n, scratch.partial_min,
+      scratch.partial_max, scratch.counter, scale, zp);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess)
+    return e;
+  // Second pass: the ordinary per-tensor quantize with the parameters just
+  // written (the u8 zero point converted back to f32 is the float zero point
+  // the reference adds: it is an integer in [0, 255]).
+  return quantize_dispatch<false>(
+      s, x, 1, 1, n, scale, zp, y, y_shift ? 0x80808080u : 0u);
+}
+
+hipError_t launch_fill_u32(hipStream_t s, uint32_t *p, int64_t n, uint32_t v) {
+  if (n == 0)
+    return hipSuccess;
+  k_fill_u32<<<stream_grid(n, kThreads * 4), kThreads, 0, s>>>(p, n, v);
+  return hipGetLastError();
+}
+
+} // namespace om

@@ -1,0 +1,1072 @@
+// C-ABI runtime of the MI355X accelerator for onnx-mlir's int8 path:
+// accelerator life cycle, OMTensor marshalling, GPU residency and the op
+// entry points declared in include/om_mi355x.h.
+//
+// An entry point receives OMTensor wrappers exactly as KrnlCallOpLowering
+// builds them (src/Conversion/KrnlToLLVM/KrnlCall.cpp:34-102).  A tensor whose
+// data pointer is GPU memory is used in place; a host tensor is staged into a
+// per-thread pool of GPU buffers (inputs copied in before the kernels, outputs
+// copied back after them, one stream synchronisation per call).  Host buffers
+// declared constant are uploaded once; a constant matmul right-hand side is
+// also packed and column-summed once.
+//
+// There is no CPU implementation behind these entry points: without a gfx950
+// device they fail (errno, stderr, om_mi355x_last_error).
+
+#include <errno.h>
+#include <pthread.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <map>
+#include <mutex>
+#include <string>
+#include <unordered_map>
+#include <unordered_set>
+#include <vector>
+
+#include "om_kernels.h"
+#include "om_mi355x.h"
+
+using namespace om;
+
+// ---------------------------------------------------------------------------
+// errors
+// ---------------------------------------------------------------------------
+namespace {
+
+thread_local std::string t_last_error;
+thread_local std::string t_last_error_returned;
+
+void fail(int err, const char *fmt, ...) {
+  char buf[512];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof buf, fmt, ap);
+  va_end(ap);
+  t_last_error = buf;
+  fprintf(stderr, "om_mi355x: %s\n", buf);
+  errno = err;
+}
+
+#define HIP_OK(expr)                                                           \
+  do {                                                                         \
+    hipError_t e_ = (expr);                                                    \
+    if (e_ != hipSuccess) {                                                    \
+      fail(EIO, "%s failed: %s (%s:%d)", #expr, hipGetErrorString(e_),        \
+          __FILE__, __LINE__);                                                 \
+      return false;                                                            \
+    }                                                                          \
+  } while (0)
+
+// ---------------------------------------------------------------------------
+// device state
+// ---------------------------------------------------------------------------
+pthread_mutex_t g_init_mutex = PTHREAD_MUTEX_INITIALIZER;
+bool g_device_ok = false;
+std::string g_device_why;
+
+std::mutex g_mem_mutex;
+// GPU allocations handed out by om_mi355x_malloc: start -> bytes.
+std::map<uintptr_t, size_t> g_user_allocs;
+// Host buffers declared constant, and their GPU copies.
+std::unordered_set<const void *> g_constants;
+struct DevCopy {
+  void *dev;
+  size_t bytes;
+};
+std::unordered_map<const void *, DevCopy> g_const_copies;
+// Packed right-hand sides of constant B, keyed by B's data pointer.
+struct PackedB {
+  int8_t *bt;
+  int32_t *colsum;
+  int64_t K, N;
+  bool is_unsigned;
+};
+std::unordered_map<const void *, PackedB> g_packed;
+
+bool probe_device() {
+  int count = 0;
+  hipError_t e = hipGetDeviceCount(&count);
+  if (e != hipSuccess || count < 1) {
+    (void)hipGetLastError();
+    g_device_why = "no HIP device visible";
+    return false;
+  }
+  hipDeviceProp_t prop;
+  if (hipGetDeviceProperties(&prop, 0) != hipSuccess) {
+    (void)hipGetLastError();
+    g_device_why = "hipGetDeviceProperties failed";
+    return false;
+  }
+  if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+    g_device_why = std::string("device 0 is ") + prop.gcnArchName +
+                   ", the kernels are built for gfx950 only";
+    return false;
+  }
+  if (hipSetDevice(0) != hipSuccess) {
+    (void)hipGetLastError();
+    g_device_why = "hipSetDevice(0) failed";
+    return false;
+  }
+  return true;
+}
+
+// Per-thread execution context: one stream (default priority), the scratch of
+// DynamicQuantizeLinear, a pool of reusable GPU buffers and timer events.
+// Buffers of the pool are only ever used by work on this stream, so handing a
+// buffer to the next call without waiting is safe: stream order serialises
+// the uses.
+struct Ctx {
+  bool ready = false;
+  hipStream_t stream = nullptr;
+  DqlScratch dql = {nullptr, nullptr, nullptr};
+  float *dql_scale = nullptr; // scale / zero point of the fused path
+  uint8_t *dql_zp = nullptr;
+  std::multimap<size_t, void *> pool;
+  hipEvent_t ev0 = nullptr, ev1 = nullptr;
+
+  bool init() {
+    if (ready)
+      return true;
+    OMInitAccelMI355X();
+    if (!g_device_ok) {
+      fail(EIO, "accelerator unavailable: %s", g_device_why.c_str());
+      return false;
+    }
+    HIP_OK(hipSetDevice(0));
+    HIP_OK(hipStreamCreateWithFlags(&stream, hipStreamNonBlocking));
+    void *p = nullptr;
+    HIP_OK(hipMalloc(&p, sizeof(float) * 2 * kDqlMaxBlocks + 256));
+    dql.partial_min = (float *)p;
+    dql.partial_max = dql.partial_min + kDqlMaxBlocks;
+    dql.counter = (unsigned *)(dql.partial_max + kDqlMaxBlocks);
+    dql_scale = (float *)(dql.counter + 16);
+    dql_zp = (uint8_t *)(dql.counter + 32);
+    HIP_OK(hipMemset(dql.counter, 0, 256));
+    HIP_OK(hipEventCreate(&ev0));
+    HIP_OK(hipEventCreate(&ev1));
+    ready = true;
+    return true;
+  }
+
+  void *take(size_t bytes) {
+    if (bytes == 0)
+      bytes = 16;
+    bytes = (bytes + 255) & ~(size_t)255;
+    auto it = pool.lower_bound(bytes);
+    if (it != pool.end() && it->first <= bytes * 2) {
+      void *p = it->second;
+      taken[p] = it->first;
+      pool.erase(it);
+      return p;
+    }
+    void *p = nullptr;
+    hipError_t e = hipMalloc(&p, bytes);
+    if (e != hipSuccess) {
+      // Give cached buffers back to the driver and retry once.
+      for (auto &kv : pool)
+        (void)hipFree(kv.second);
+      pool.clear();
+      e = hipMalloc(&p, bytes);
+    }
+    if (e != hipSuccess) {
+      fail(EIO, "hipMalloc(%zu) failed: %s", bytes, hipGetErrorString(e));
+      return nullptr;
+    }
+    taken[p] = bytes;
+    return p;
+  }
+  void give(void *p) {
+    auto it = taken.find(p);
+    if (it == taken.end())
+      return;
+    pool.emplace(it->second, p);
+    taken.erase(it);
+  }
+  void drop_pool() {
+    for (auto &kv : pool)
+      (void)hipFree(kv.second);
+    pool.clear();
+  }
+  std::unordered_map<void *, size_t> taken;
+};
+
+thread_local Ctx t_ctx;
+
+bool is_device_ptr(const void *p) {
+  {
+    std::lock_guard<std::mutex> lk(g_mem_mutex);
+    auto it = g_user_allocs.upper_bound((uintptr_t)p);
+    if (it != g_user_allocs.begin()) {
+      --it;
+      if ((uintptr_t)p < it->first + it->second)
+        return true;
+    }
+  }
+  hipPointerAttribute_t attr;
+  hipError_t e = hipPointerGetAttributes(&attr, p);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  return attr.type == hipMemoryTypeDevice;
+}
+
+// ---------------------------------------------------------------------------
+// tensor views
+// ---------------------------------------------------------------------------
+struct View {
+  void *data = nullptr;
+  int dtype = 0;
+  int64_t rank = 0;
+  const int64_t *shape = nullptr;
+  int64_t numel = 0;
+  size_t bytes = 0;
+};
+
+size_t dtype_bytes(int dt) {
+  switch (dt) {
+  case OM_MI355X_TYPE_FLOAT:
+  case OM_MI355X_TYPE_INT32:
+    return 4;
+  case OM_MI355X_TYPE_UINT8:
+  case OM_MI355X_TYPE_INT8:
+    return 1;
+  default:
+    return 0;
+  }
+}
+
+bool view_of(const OMTensor *t, const char *name, View &v) {
+  if (!t) {
+    fail(EINVAL, "%s: tensor is NULL", name);
+    return false;
+  }
+  v.data = omTensorGetDataPtr(t);
+  v.dtype = omTensorGetDataType(t);
+  v.rank = omTensorGetRank(t);
+  v.shape = omTensorGetShape(t);
+  const int64_t *strides = omTensorGetStrides(t);
+  v.numel = 1;
+  for (int64_t i = 0; i < v.rank; ++i)
+    v.numel *= v.shape[i];
+  // Row-major contiguous is what memref.alloc and the entry-point wrapper
+  // produce (src/Runtime/OMTensor.inc:185-192); anything else is refused.
+  int64_t expect = 1;
+  for (int64_t i = v.rank - 1; i >= 0; --i) {
+    if (v.shape[i] != 1 && strides[i] != expect) {
+      fail(EINVAL, "%s: tensor is not row-major contiguous", name);
+      return false;
+    }
+    expect *= v.shape[i];
+  }
+  if (dtype_bytes(v.dtype) == 0) {
+    fail(EINVAL, "%s: unsupported element type %d", name, v.dtype);
+    return false;
+  }
+  v.bytes = (size_t)v.numel * dtype_bytes(v.dtype);
+  if (v.numel > 0 && !v.data) {
+    fail(EINVAL, "%s: data pointer is NULL", name);
+    return false;
+  }
+  return true;
+}
+
+// One entry-point invocation: resolves tensors to GPU pointers, remembers
+// which host outputs need copying back and which pool buffers to return.
+struct Call {
+  Ctx &c;
+  bool ok = true;
+  bool touched_host = false;
+  struct Back {
+    void *host;
+    void *dev;
+    size_t bytes;
+  };
+  std::vector<Back> backs;
+  std::vector<void *> temps;
+
+  explicit Call(Ctx &ctx) : c(ctx) { ok = c.init(); }
+
+  void *temp(size_t bytes) {
+    void *p = c.take(bytes);
+    if (!p)
+      ok = false;
+    else
+      temps.push_back(p);
+    return p;
+  }
+
+  const void *in(const View &v) {
+    if (!ok || v.numel == 0)
+      return v.data;
+    if (is_device_ptr(v.data))
+      return v.data;
+    {
+      std::lock_guard<std::mutex> lk(g_mem_mutex);
+      if (g_constants.count(v.data)) {
+        auto it = g_const_copies.find(v.data);
+        if (it != g_const_copies.end() && it->second.bytes == v.bytes)
+          return it->second.dev;
+      }
+    }
+    bool constant;
+    {
+      std::lock_guard<std::mutex> lk(g_mem_mutex);
+      constant = g_constants.count(v.data) != 0;
+    }
+    void *d = nullptr;
+    if (constant) {
+      if (hipMalloc(&d, v.bytes ? v.bytes : 16) != hipSuccess) {
+        fail(EIO, "hipMalloc(%zu) for a constant failed", v.bytes);
+        ok = false;
+        return nullptr;
+      }
+      if (hipMemcpy(d, v.data, v.bytes, hipMemcpyHostToDevice) != hipSuccess) {
+        fail(EIO, "upload of a constant failed");
+        ok = false;
+        return nullptr;
+      }
+      std::lock_guard<std::mutex> lk(g_mem_mutex);
+      auto ins = g_const_copies.emplace(v.data, DevCopy{d, v.bytes});
+      if (!ins.second) { // another thread won, or the size changed
+        if (ins.first->second.bytes == v.bytes) {
+          (void)hipFree(d);
+          return ins.first->second.dev;
+        }
+        (void)hipFree(ins.first->second.dev);
+        ins.first->second = DevCopy{d, v.bytes};
+      }
+      return d;
+    }
+    d = temp(v.bytes);
+    if (!d)
+      return nullptr;
+    hipError_t e =
+        hipMemcpyAsync(d, v.data, v.bytes, hipMemcpyHostToDevice, c.stream);
+    if (e != hipSuccess) {
+      fail(EIO, "host-to-device copy failed: %s", hipGetErrorString(e));
+      ok = false;
+      return nullptr;
+    }
+    touched_host = true;
+    return d;
+  }
+
+  void *out(const View &v) {
+    if (!ok || v.numel == 0)
+      return v.data;
+    if (is_device_ptr(v.data))
+      return v.data;
+    void *d = temp(v.bytes);
+    if (!d)
+      return nullptr;
+    backs.push_back(Back{v.data, d, v.bytes});
+    touched_host = true;
+    return d;
+  }
+
+  void check(hipError_t e, const char *what) {
+    if (e != hipSuccess) {
+      fail(EIO, "%s failed: %s", what, hipGetErrorString(e));
+      ok = false;
+    }
+  }
+
+  void finish() {
+    if (ok) {
+      for (const Back &b : backs) {
+        hipError_t e = hipMemcpyAsync(
+            b.host, b.dev, b.bytes, hipMemcpyDeviceToHost, c.stream);
+        if (e != hipSuccess) {
+          fail(EIO, "device-to-host copy failed: %s", hipGetErrorString(e));
+          ok = false;
+          break;
+        }
+      }
+    }
+    if (touched_host && c.ready) {
+      hipError_t e = hipStreamSynchronize(c.stream);
+      if (e != hipSuccess && ok)
+        fail(EIO, "stream synchronisation failed: %s", hipGetErrorString(e));
+    }
+    for (void *p : temps)
+      c.give(p);
+    temps.clear();
+  }
+};
+
+bool is_q8(int dt) {
+  return dt == OM_MI355X_TYPE_UINT8 || dt == OM_MI355X_TYPE_INT8;
+}
+
+// Splits `shape` around `axis` for a scale of `scale_numel` entries.
+bool axis_split(const View &x, int64_t scale_numel, int64_t axis,
+    const char *op, int64_t &outer, int64_t &channels, int64_t &inner) {
+  if (scale_numel == 1) {
+    outer = 1;
+    channels = 1;
+    inner = x.numel;
+    return true;
+  }
+  if (axis < 0)
+    axis += x.rank;
+  if (axis < 0 || axis >= x.rank) {
+    fail(EINVAL, "%s: axis out of range", op);
+    return false;
+  }
+  if (x.shape[axis] != scale_numel) {
+    fail(EINVAL, "%s: scale has %lld entries, dimension %lld has %lld", op,
+        (long long)scale_numel, (long long)axis, (long long)x.shape[axis]);
+    return false;
+  }
+  outer = 1;
+  inner = 1;
+  for (int64_t i = 0; i < axis; ++i)
+    outer *= x.shape[i];
+  for (int64_t i = axis + 1; i < x.rank; ++i)
+    inner *= x.shape[i];
+  channels = scale_numel;
+  return true;
+}
+
+// A [.., M, K] (leading dimensions folded into M) times B [K, N].
+bool matmul_dims(const View &a, const View &b, const char *op, int64_t &M,
+    int64_t &K, int64_t &N) {
+  if (b.rank != 2 || a.rank < 1) {
+    fail(EINVAL, "%s: expected A [..,M,K] and a 2-D B [K,N]", op);
+    return false;
+  }
+  K = a.shape[a.rank - 1];
+  M = (K == 0) ? 0 : a.numel / K;
+  if (a.rank >= 2 && K == 0) {
+    M = 1;
+    for (int64_t i = 0; i + 1 < a.rank; ++i)
+      M *= a.shape[i];
+  }
+  if (b.shape[0] != K) {
+    fail(EINVAL, "%s: inner dimensions differ (%lld vs %lld)", op,
+        (long long)K, (long long)b.shape[0]);
+    return false;
+  }
+  N = b.shape[1];
+  return true;
+}
+
+// Packed form of B: from the cache when B was declared constant, otherwise
+// packed into pool buffers for this call only.
+bool packed_b(Call &call, const View &b, int64_t K, int64_t N,
+    const int8_t *&bt, const int32_t *&colsum) {
+  const bool uns = b.dtype == OM_MI355X_TYPE_UINT8;
+  const int64_t Kpad = round_up(K > 0 ? K : 1, kGemmBK);
+  const int64_t Npad = round_up(N, kGemmBN);
+  bool constant;
+  {
+    std::lock_guard<std::mutex> lk(g_mem_mutex);
+    constant = g_constants.count(b.data) != 0;
+    if (constant) {
+      auto it = g_packed.find(b.data);
+      if (it != g_packed.end() && it->second.K == K && it->second.N == N &&
+          it->second.is_unsigned == uns) {
+        bt = it->second.bt;
+        colsum = it->second.colsum;
+        return true;
+      }
+    }
+  }
+  const void *db = call.in(b);
+  if (!call.ok)
+    return false;
+  int8_t *pbt;
+  int32_t *pcs;
+  if (constant) {
+    void *p = nullptr, *q = nullptr;
+    if (hipMalloc(&p, (size_t)Kpad * Npad) != hipSuccess ||
+        hipMalloc(&q, (size_t)Npad * 4) != hipSuccess) {
+      fail(EIO, "hipMalloc for a packed constant failed");
+      call.ok = false;
+      return false;
+    }
+    pbt = (int8_t *)p;
+    pcs = (int32_t *)q;
+  } else {
+    pbt = (int8_t *)call.temp((size_t)Kpad * Npad);
+    pcs = (int32_t *)call.temp((size_t)Npad * 4);
+    if (!call.ok)
+      return false;
+  }
+  call.check(launch_pack_b(call.c.stream, db, uns, K, N, pbt, pcs), "pack B");
+  if (!call.ok)
+    return false;
+  if (constant) {
+    // Other threads use their own streams: make the packed data final first.
+    call.check(hipStreamSynchronize(call.c.stream), "pack B synchronise");
+    std::lock_guard<std::mutex> lk(g_mem_mutex);
+    auto ins = g_packed.emplace(b.data, PackedB{pbt, pcs, K, N, uns});
+    if (!ins.second) {
+      (void)hipFree(ins.first->second.bt);
+      (void)hipFree(ins.first->second.colsum);
+      ins.first->second = PackedB{pbt, pcs, K, N, uns};
+    }
+  }
+  bt = pbt;
+  colsum = pcs;
+  return true;
+}
+
+bool zp_len_ok(const View *zp, int64_t full, const char *op, const char *name,
+    int64_t &len) {
+  if (!zp) {
+    len = 0;
+    return true;
+  }
+  if (zp->numel == 1)
+    len = 1;
+  else if (zp->numel == full)
+    len = full;
+  else {
+    fail(EINVAL, "%s: %s has %lld entries, expected 1 or %lld", op, name,
+        (long long)zp->numel, (long long)full);
+    return false;
+  }
+  return true;
+}
+
+// Shared body of MatMulInteger, MatMulIntegerDequant and QLinearMatMul.
+struct MatmulSpec {
+  const char *op;
+  Epilogue epi;
+  const OMTensor *y, *a, *b, *a_zp, *b_zp;
+  const OMTensor *a_scale = nullptr, *b_scale = nullptr, *y_scale = nullptr,
+                 *y_zp = nullptr;
+  NarrowMode narrow = kWrap;
+};
+
+void run_matmul(const MatmulSpec &sp) {
+  View y, a, b, azp, bzp, as, bs, ys, yzp;
+  if (!view_of(sp.y, "y", y) || !view_of(sp.a, "a", a) ||
+      !view_of(sp.b, "b", b))
+    return;
+  if (sp.a_zp && !view_of(sp.a_zp, "a_zero_point", azp))
+    return;
+  if (sp.b_zp && !view_of(sp.b_zp, "b_zero_point", bzp))
+    return;
+  if (!is_q8(a.dtype) || !is_q8(b.dtype)) {
+    fail(EINVAL, "%s: A and B must be uint8 or int8", sp.op);
+    return;
+  }
+  if ((sp.a_zp && azp.dtype != a.dtype) || (sp.b_zp && bzp.dtype != b.dtype)) {
+    fail(EINVAL, "%s: a zero point's type differs from its tensor's", sp.op);
+    return;
+  }
+  int64_t M, K, N;
+  if (!matmul_dims(a, b, sp.op, M, K, N))
+    return;
+  if (y.numel != M * N) {
+    fail(EINVAL, "%s: output has %lld elements, expected %lld", sp.op,
+        (long long)y.numel, (long long)(M * N));
+    return;
+  }
+  const int want_y = sp.epi == kEpiI32   ? OM_MI355X_TYPE_INT32
+                     : sp.epi == kEpiF32 ? OM_MI355X_TYPE_FLOAT
+                                         : 0;
+  if ((want_y && y.dtype != want_y) || (!want_y && !is_q8(y.dtype))) {
+    fail(EINVAL, "%s: output element type %d is wrong", sp.op, y.dtype);
+    return;
+  }
+  int64_t azl, bzl;
+  if (!zp_len_ok(sp.a_zp ? &azp : nullptr, M, sp.op, "a_zero_point", azl) ||
+      !zp_len_ok(sp.b_zp ? &bzp : nullptr, N, sp.op, "b_zero_point", bzl))
+    return;
+  if (sp.epi != kEpiI32) {
+    if (!view_of(sp.a_scale, "a_scale", as) ||
+        !view_of(sp.b_scale, "b_scale", bs))
+      return;
+    if (as.dtype != OM_MI355X_TYPE_FLOAT || bs.dtype != OM_MI355X_TYPE_FLOAT ||
+        as.numel != 1 || (bs.numel != 1 && bs.numel != N)) {
+      fail(EINVAL, "%s: scales must be f32, a_scale scalar, b_scale scalar "
+                   "or [N]", sp.op);
+      return;
+    }
+  }
+  if (sp.epi == kEpiQ8) {
+    if (!view_of(sp.y_scale, "y_scale", ys) ||
+        !view_of(sp.y_zp, "y_zero_point", yzp))
+      return;
+    if (ys.dtype != OM_MI355X_TYPE_FLOAT || ys.numel != 1 ||
+        yzp.numel != 1 || yzp.dtype != y.dtype) {
+      fail(EINVAL, "%s: y_scale must be an f32 scalar and y_zero_point a "
+                   "scalar of the output type", sp.op);
+      return;
+    }
+  }
+  if (M == 0 || N == 0)
+    return;
+
+  Call call(t_ctx);
+  if (!call.ok)
+    return;
+  const bool a_uns = a.dtype == OM_MI355X_TYPE_UINT8;
+  const bool b_uns = b.dtype == OM_MI355X_TYPE_UINT8;
+  GemmArgs g = {};
+  g.A = call.in(a);
+  g.a_unsigned = a_uns;
+  g.a_preshifted = false;
+  g.b_unsigned = b_uns;
+  g.M = M;
+  g.K = K;
+  g.N = N;
+  const int32_t *colsum = nullptr;
+  if (!packed_b(call, b, K, N, g.Bt, colsum)) {
+    call.finish();
+    return;
+  }
+  g.colsum = colsum;
+  g.a_zp = sp.a_zp ? call.in(azp) : nullptr;
+  g.a_zp_len = azl;
+  g.b_zp = sp.b_zp ? call.in(bzp) : nullptr;
+  g.b_zp_len = bzl;
+  // Row sums of A are only needed when B carries an offset.
+  g.rowsum = nullptr;
+  if (b_uns || sp.b_zp) {
+    int32_t *rs = (int32_t *)call.temp((size_t)M * 4);
+    if (call.ok)
+      call.check(
+          launch_rowsum_a(call.c.stream, g.A, a_uns, M, K, rs), "row sums");
+    g.rowsum = rs;
+  }
+  g.epi = sp.epi;
+  if (sp.epi != kEpiI32) {
+    g.a_scale = (const float *)call.in(as);
+    g.b_scale = (const float *)call.in(bs);
+    g.b_scale_len = bs.numel;
+  }
+  if (sp.epi == kEpiQ8) {
+    g.y_scale = (const float *)call.in(ys);
+    g.y_zp = call.in(yzp);
+    g.y_unsigned = y.dtype == OM_MI355X_TYPE_UINT8;
+    g.narrow = sp.narrow;
+  }
+  g.out = call.out(y);
+  if (call.ok)
+    call.check(launch_gemm(call.c.stream, g), sp.op);
+  call.finish();
+}
+
+} // namespace
+
+// ---------------------------------------------------------------------------
+// accelerator life cycle
+// ---------------------------------------------------------------------------
+extern "C" {
+
+long OMIsInitAccelMI355X = 0;
+
+void OMInitAccelMI355X(void) {
+  if (!OMIsInitAccelMI355X) {
+    pthread_mutex_lock(&g_init_mutex);
+    if (!OMIsInitAccelMI355X) {
+      g_device_ok = probe_device();
+      OMIsInitAccelMI355X = 1;
+    }
+    pthread_mutex_unlock(&g_init_mutex);
+  }
+}
+
+uint64_t OMInitCompatibleAccelMI355X(uint64_t versionNum) {
+  OMInitAccelMI355X();
+  // A model runs here when it was compiled for this major version or an
+  // older minor one, and device 0 is a gfx950.
+  const uint64_t major = (versionNum >> 16) & 0xFF;
+  const uint64_t mine_major = (OM_MI355X_VERSION >> 16) & 0xFF;
+  if (major != mine_major ||
+      (versionNum & 0xFFFF) > (OM_MI355X_VERSION & 0xFFFF)) {
+    fprintf(stderr,
+        "om_mi355x: model needs runtime version 0x%llx, this runtime is "
+        "0x%llx\n",
+        (unsigned long long)versionNum,
+        (unsigned long long)OM_MI355X_VERSION);
+    errno = EPERM;
+    return 0;
+  }
+  if (!g_device_ok) {
+    fprintf(stderr,
+        "om_mi355x: this model was compiled for the MI355X accelerator: %s\n",
+        g_device_why.c_str());
+    errno = EPERM;
+    return 0;
+  }
+  return 1;
+}
+
+void OMShutdownAccelMI355X(void) {
+  if (OMIsInitAccelMI355X) {
+    pthread_mutex_lock(&g_init_mutex);
+    OMIsInitAccelMI355X = 0;
+    pthread_mutex_unlock(&g_init_mutex);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// ops
+// ---------------------------------------------------------------------------
+void om_mi355x_QuantizeLinear(OMTensor *y_t, const OMTensor *x_t,
+    const OMTensor *scale_t, const OMTensor *zp_t, int64_t axis,
+    int64_t saturate) {
+  (void)saturate;
+  View y, x, sc, zp;
+  if (!view_of(y_t, "y", y) || !view_of(x_t, "x", x) ||
+      !view_of(scale_t, "y_scale", sc))
+    return;
+  if (zp_t && !view_of(zp_t, "y_zero_point", zp))
+    return;
+  if (x.dtype != OM_MI355X_TYPE_FLOAT || sc.dtype != OM_MI355X_TYPE_FLOAT ||
+      !is_q8(y.dtype) || y.numel != x.numel ||
+      (zp_t && (zp.dtype != y.dtype || zp.numel != sc.numel))) {
+    fail(EINVAL, "QuantizeLinear: expected f32 x and scale, ui8/i8 y with a "
+                 "zero point of y's type and the scale's shape");
+    return;
+  }
+  int64_t outer, channels, inner;
+  if (!axis_split(x, sc.numel, axis, "QuantizeLinear", outer, channels, inner))
+    return;
+  if (x.numel == 0)
+    return;
+  Call call(t_ctx);
+  if (!call.ok)
+    return;
+  const float *dx = (const float *)call.in(x);
+  const float *ds = (const float *)call.in(sc);
+  const void *dz = zp_t ? call.in(zp) : nullptr;
+  void *dy = call.out(y);
+  if (call.ok)
+    call.check(launch_quantize(call.c.stream, dx, outer, channels, inner, ds,
+                   dz, y.dtype == OM_MI355X_TYPE_INT8, dy),
+        "QuantizeLinear");
+  call.finish();
+}
+
+void om_mi355x_DequantizeLinear(OMTensor *y_t, const OMTensor *x_t,
+    const OMTensor *scale_t, const OMTensor *zp_t, int64_t axis) {
+  View y, x, sc, zp;
+  if (!view_of(y_t, "y", y) || !view_of(x_t, "x", x) ||
+      !view_of(scale_t, "x_scale", sc))
+    return;
+  if (zp_t && !view_of(zp_t, "x_zero_point", zp))
+    return;
+  const bool x_ok = is_q8(x.dtype) || x.dtype == OM_MI355X_TYPE_INT32;
+  if (!x_ok || y.dtype != OM_MI355X_TYPE_FLOAT ||
+      sc.dtype != OM_MI355X_TYPE_FLOAT || y.numel != x.numel ||
+      (zp_t && (zp.dtype != x.dtype || zp.numel != sc.numel))) {
+    fail(EINVAL, "DequantizeLinear: expected ui8/i8/i32 x, f32 scale and y, a "
+                 "zero point of x's type and the scale's shape");
+    return;
+  }
+  int64_t outer, channels, inner;
+  if (!axis_split(
+          x, sc.numel, axis, "DequantizeLinear", outer, channels, inner))
+    return;
+  if (x.numel == 0)
+    return;
+  Call call(t_ctx);
+  if (!call.ok)
+    return;
+  const void *dx = call.in(x);
+  const float *ds = (const float *)call.in(sc);
+  const void *dz = zp_t ? call.in(zp) : nullptr;
+  float *dy = (float *)call.out(y);
+  const QKind kind = x.dtype == OM_MI355X_TYPE_UINT8  ? kU8
+                     : x.dtype == OM_MI355X_TYPE_INT8 ? kI8
+                                                      : kI32;
+  if (call.ok)
+    call.check(launch_dequantize(call.c.stream, dx, kind, outer, channels,
+                   inner, ds, dz, dy),
+        "DequantizeLinear");
+  call.finish();
+}
+
+void om_mi355x_DynamicQuantizeLinear(OMTensor *y_t, OMTensor *scale_t,
+    OMTensor *zp_t, const OMTensor *x_t) {
+  View y, sc, zp, x;
+  if (!view_of(y_t, "y", y) || !view_of(scale_t, "y_scale", sc) ||
+      !view_of(zp_t, "y_zero_point", zp) || !view_of(x_t, "x", x))
+    return;
+  if (x.dtype != OM_MI355X_TYPE_FLOAT || y.dtype != OM_MI355X_TYPE_UINT8 ||
+      sc.dtype != OM_MI355X_TYPE_FLOAT || zp.dtype != OM_MI355X_TYPE_UINT8 ||
+      sc.numel != 1 || zp.numel != 1 || y.numel != x.numel) {
+    fail(EINVAL, "DynamicQuantizeLinear: expected f32 x, ui8 y of x's shape, "
+                 "scalar f32 scale and scalar ui8 zero point");
+    return;
+  }
+  if (x.numel == 0)
+    return;
+  Call call(t_ctx);
+  if (!call.ok)
+    return;
+  const float *dx = (const float *)call.in(x);
+  uint8_t *dy = (uint8_t *)call.out(y);
+  float *ds = (float *)call.out(sc);
+  uint8_t *dz = (uint8_t *)call.out(zp);
+  if (call.ok)
+    call.check(launch_dynamic_quantize(
+                   call.c.stream, call.c.dql, dx, x.numel, dy, ds, dz, false),
+        "DynamicQuantizeLinear");
+  call.finish();
+}
+
+void om_mi355x_MatMulInteger(OMTensor *y, const OMTensor *a,
+    const OMTensor *b, const OMTensor *a_zp, const OMTensor *b_zp) {
+  MatmulSpec sp = {"MatMulInteger", kEpiI32, y, a, b, a_zp, b_zp};
+  run_matmul(sp);
+}
+
+void om_mi355x_MatMulIntegerDequant(OMTensor *y, const OMTensor *a,
+    const OMTensor *b, const OMTensor *a_zp, const OMTensor *b_zp,
+    const OMTensor *a_scale, const OMTensor *b_scale) {
+  MatmulSpec sp = {"MatMulIntegerDequant", kEpiF32, y, a, b, a_zp, b_zp};
+  sp.a_scale = a_scale;
+  sp.b_scale = b_scale;
+  run_matmul(sp);
+}
+
+void om_mi355x_QLinearMatMul(OMTensor *y, const OMTensor *a,
+    const OMTensor *a_scale, const OMTensor *a_zp, const OMTensor *b,
+    const OMTensor *b_scale, const OMTensor *b_zp, const OMTensor *y_scale,
+    const OMTensor *y_zp, int64_t narrow_mode) {
+  if (!a_zp || !b_zp || !y_zp) {
+    fail(EINVAL, "QLinearMatMul: zero points are required operands");
+    return;
+  }
+  MatmulSpec sp = {"QLinearMatMul", kEpiQ8, y, a, b, a_zp, b_zp};
+  sp.a_scale = a_scale;
+  sp.b_scale = b_scale;
+  sp.y_scale = y_scale;
+  sp.y_zp = y_zp;
+  sp.narrow = narrow_mode ? kSaturate : kWrap;
+  run_matmul(sp);
+}
+
+void om_mi355x_DynQuantMatMulDequant(OMTensor *y_t, const OMTensor *x_t,
+    const OMTensor *b_t, const OMTensor *bzp_t, const OMTensor *bscale_t) {
+  const char *op = "DynQuantMatMulDequant";
+  View y, x, b, bzp, bs;
+  if (!view_of(y_t, "y", y) || !view_of(x_t, "x", x) ||
+      !view_of(b_t, "b", b) || !view_of(bscale_t, "b_scale", bs))
+    return;
+  if (bzp_t && !view_of(bzp_t, "b_zero_point", bzp))
+    return;
+  if (x.dtype != OM_MI355X_TYPE_FLOAT || y.dtype != OM_MI355X_TYPE_FLOAT ||
+      !is_q8(b.dtype) || bs.dtype != OM_MI355X_TYPE_FLOAT ||
+      (bzp_t && bzp.dtype != b.dtype)) {
+    fail(EINVAL, "%s: expected f32 x and y, ui8/i8 b, f32 b_scale", op);
+    return;
+  }
+  int64_t M, K, N;
+  if (!matmul_dims(x, b, op, M, K, N))
+    return;
+  int64_t bzl;
+  if (!zp_len_ok(bzp_t ? &bzp : nullptr, N, op, "b_zero_point", bzl))
+    return;
+  if (y.numel != M * N || (bs.numel != 1 && bs.numel != N)) {
+    fail(EINVAL, "%s: output or b_scale shape is wrong", op);
+    return;
+  }
+  if (M == 0 || N == 0)
+    return;
+  Call call(t_ctx);
+  if (!call.ok)
+    return;
+  const float *dx = (const float *)call.in(x);
+  // Quantized activations stay on the GPU, stored as (u8 - 128) so the GEMM
+  // stages them without a per-byte fix-up.
+  uint8_t *aq = (uint8_t *)call.temp((size_t)M * K);
+  if (call.ok)
+    call.check(launch_dynamic_quantize(call.c.stream, call.c.dql, dx, M * K,
+                   aq, call.c.dql_scale, call.c.dql_zp, true),
+        "dynamic quantize");
+  GemmArgs g = {};
+  g.A = aq;
+  g.a_unsigned = true;
+  g.a_preshifted = true;
+  g.b_unsigned = b.dtype == OM_MI355X_TYPE_UINT8;
+  g.M = M;
+  g.K = K;
+  g.N = N;
+  const int32_t *colsum = nullptr;
+  if (!call.ok || !packed_b(call, b, K, N, g.Bt, colsum)) {
+    call.finish();
+    return;
+  }
+  g.colsum = colsum;
+  g.a_zp = call.c.dql_zp;
+  g.a_zp_len = 1;
+  g.b_zp = bzp_t ? call.in(bzp) : nullptr;
+  g.b_zp_len = bzl;
+  g.rowsum = nullptr;
+  if (g.b_unsigned || bzp_t) {
+    int32_t *rs = (int32_t *)call.temp((size_t)M * 4);
+    // Row sums of the shifted bytes are the int8 sums.
+    if (call.ok)
+      call.check(
+          launch_rowsum_a(call.c.stream, aq, false, M, K, rs), "row sums");
+    g.rowsum = rs;
+  }
+  g.epi = kEpiF32;
+  g.a_scale = call.c.dql_scale;
+  g.b_scale = (const float *)call.in(bs);
+  g.b_scale_len = bs.numel;
+  g.out = call.out(y);
+  if (call.ok)
+    call.check(launch_gemm(call.c.stream, g), op);
+  call.finish();
+}
+
+// ---------------------------------------------------------------------------
+// residency, memory, measurement
+// ---------------------------------------------------------------------------
+void om_mi355x_MarkConstant(const OMTensor *t) {
+  if (!t)
+    return;
+  const void *p = omTensorGetDataPtr(t);
+  std::lock_guard<std::mutex> lk(g_mem_mutex);
+  g_constants.insert(p);
+}
+
+void om_mi355x_ClearCache(void) {
+  if (t_ctx.ready)
+    (void)hipStreamSynchronize(t_ctx.stream);
+  std::lock_guard<std::mutex> lk(g_mem_mutex);
+  for (auto &kv : g_const_copies)
+    (void)hipFree(kv.second.dev);
+  g_const_copies.clear();
+  for (auto &kv : g_packed) {
+    (void)hipFree(kv.second.bt);
+    (void)hipFree(kv.second.colsum);
+  }
+  g_packed.clear();
+  g_constants.clear();
+  t_ctx.drop_pool();
+}
+
+void *om_mi355x_malloc(size_t bytes) {
+  if (!t_ctx.init())
+    return nullptr;
+  void *p = nullptr;
+  hipError_t e = hipMalloc(&p, bytes ? bytes : 16);
+  if (e != hipSuccess) {
+    fail(EIO, "hipMalloc(%zu) failed: %s", bytes, hipGetErrorString(e));
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lk(g_mem_mutex);
+  g_user_allocs[(uintptr_t)p] = bytes ? bytes : 16;
+  return p;
+}
+
+void om_mi355x_free(void *p) {
+  if (!p)
+    return;
+  if (t_ctx.ready)
+    (void)hipStreamSynchronize(t_ctx.stream);
+  {
+    std::lock_guard<std::mutex> lk(g_mem_mutex);
+    g_user_allocs.erase((uintptr_t)p);
+    g_constants.erase(p);
+    auto it = g_packed.find(p);
+    if (it != g_packed.end()) {
+      (void)hipFree(it->second.bt);
+      (void)hipFree(it->second.colsum);
+      g_packed.erase(it);
+    }
+  }
+  (void)hipFree(p);
+}
+
+int om_mi355x_memcpy_h2d(void *dst, const void *src, size_t bytes) {
+  if (!t_ctx.init())
+    return -1;
+  hipError_t e = hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice,
+      t_ctx.stream);
+  if (e == hipSuccess)
+    e = hipStreamSynchronize(t_ctx.stream);
+  if (e != hipSuccess) {
+    fail(EIO, "host-to-device copy failed: %s", hipGetErrorString(e));
+    return -1;
+  }
+  return 0;
+}
+
+int om_mi355x_memcpy_d2h(void *dst, const void *src, size_t bytes) {
+  if (!t_ctx.init())
+    return -1;
+  hipError_t e = hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost,
+      t_ctx.stream);
+  if (e == hipSuccess)
+    e = hipStreamSynchronize(t_ctx.stream);
+  if (e != hipSuccess) {
+    fail(EIO, "device-to-host copy failed: %s", hipGetErrorString(e));
+    return -1;
+  }
+  return 0;
+}
+
+int om_mi355x_synchronize(void) {
+  if (!t_ctx.init())
+    return -1;
+  hipError_t e = hipStreamSynchronize(t_ctx.stream);
+  if (e != hipSuccess) {
+    fail(EIO, "stream synchronisation failed: %s", hipGetErrorString(e));
+    return -1;
+  }
+  return 0;
+}
+
+int om_mi355x_timer_start(void) {
+  if (!t_ctx.init())
+    return -1;
+  hipError_t e = hipEventRecord(t_ctx.ev0, t_ctx.stream);
+  if (e != hipSuccess) {
+    fail(EIO, "hipEventRecord failed: %s", hipGetErrorString(e));
+    return -1;
+  }
+  return 0;
+}
+
+float om_mi355x_timer_stop(void) {
+  if (!t_ctx.init())
+    return -1.0f;
+  hipError_t e = hipEventRecord(t_ctx.ev1, t_ctx.stream);
+  if (e == hipSuccess)
+    e = hipEventSynchronize(t_ctx.ev1);
+  float ms = -1.0f;
+  if (e == hipSuccess)
+    e = hipEventElapsedTime(&ms, t_ctx.ev0, t_ctx.ev1);
+  if (e != hipSuccess) {
+    fail(EIO, "event timing failed: %s", hipGetErrorString(e));
+    return -1.0f;
+  }
+  return ms;
+}
+
+const char *om_mi355x_last_error(void) {
+  t_last_error_returned.swap(t_last_error);
+  t_last_error.clear();
+  return t_last_error_returned.c_str();
+}
+
+int om_mi355x_device_info(char *buf, size_t len) {
+  if (!t_ctx.init())
+    return -1;
+  hipDeviceProp_t prop;
+  if (hipGetDeviceProperties(&prop, 0) != hipSuccess) {
+    (void)hipGetLastError();
+    return -1;
+  }
+  snprintf(buf, len, "%s|%s|%d|%d|%.1f", prop.name, prop.gcnArchName,
+      prop.multiProcessorCount, prop.clockRate / 1000,
+      (double)prop.totalGlobalMem / (1024.0 * 1024.0 * 1024.0));
+  return 0;
+}
+
+} // extern "C"

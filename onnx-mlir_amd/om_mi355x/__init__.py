@@ -1,0 +1,375 @@
+"""Host-side binding of the MI355X runtime for onnx-mlir's int8 path.
+
+The functions mirror the ONNX operators the reference lowers on its CPU path
+(QuantizeLinear, DequantizeLinear, DynamicQuantizeLinear, MatMulInteger,
+QLinearMatMul; src/Conversion/ONNXToKrnl/ConvertONNXToKrnl.cpp:226-241) and
+call the C-ABI entry points of ``include/om_mi355x.h`` exactly as a compiled
+model's ``krnl.call`` would: outputs first, then inputs, then integer
+attributes, every tensor wrapped in an ``OMTensor``
+(src/Conversion/KrnlToLLVM/KrnlCall.cpp:34-102).
+
+Operands may be numpy arrays (host memory: the runtime stages them through the
+GPU and copies results back) or :class:`DeviceArray` (GPU memory owned by the
+runtime: used in place, results stay on the GPU).
+
+There is no CPU implementation here.  If the HIP library is missing or no
+gfx950 device is present the calls raise.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import Optional, Sequence, Tuple, Union
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_CSRC = os.path.normpath(os.path.join(_HERE, "..", "csrc"))
+LIB_PATH = os.path.join(_CSRC, "libom_mi355x.so")
+SHIM_PATH = os.path.join(_CSRC, "libom_tensor_shim.so")
+
+# ONNX element-type codes (include/onnx-mlir/Runtime/OnnxDataTypeMetaData.inc:22-44)
+ONNX_FLOAT, ONNX_UINT8, ONNX_INT8, ONNX_INT32 = 1, 2, 3, 6
+_NP_TO_ONNX = {
+    np.dtype(np.float32): ONNX_FLOAT,
+    np.dtype(np.uint8): ONNX_UINT8,
+    np.dtype(np.int8): ONNX_INT8,
+    np.dtype(np.int32): ONNX_INT32,
+}
+
+WRAP, SATURATE = 0, 1
+
+
+class RuntimeError_(RuntimeError):
+    """An entry point reported an error (errno + message)."""
+
+
+_lib = None
+_shim = None
+
+
+def library_present() -> bool:
+    return os.path.exists(LIB_PATH) and os.path.exists(SHIM_PATH)
+
+
+def load(tensor_runtime: Optional[str] = None):
+    """Load the runtime.  ``tensor_runtime`` names an alternative provider of
+    the ``omTensor*`` accessors (e.g. the reference's own C runtime); it is
+    loaded with RTLD_GLOBAL first so that it wins symbol resolution."""
+    global _lib, _shim
+    if _lib is not None:
+        return _lib
+    if not library_present():
+        raise FileNotFoundError(
+            f"{LIB_PATH} is not built; run __graft_entry__.build() "
+            "(make -C onnx-mlir_amd/csrc)")
+    provider = tensor_runtime or SHIM_PATH
+    _shim = ctypes.CDLL(provider, mode=ctypes.RTLD_GLOBAL)
+    _lib = ctypes.CDLL(LIB_PATH, mode=ctypes.RTLD_GLOBAL)
+    _declare(_lib, _shim)
+    return _lib
+
+
+def _declare(lib, shim):
+    P, I64, SZ = ctypes.c_void_p, ctypes.c_int64, ctypes.c_size_t
+    shim.omTensorCreate.restype = P
+    shim.omTensorCreate.argtypes = [P, ctypes.POINTER(I64), I64, ctypes.c_int]
+    shim.omTensorDestroy.restype = None
+    shim.omTensorDestroy.argtypes = [P]
+    sigs = {
+        "om_mi355x_QuantizeLinear": [P, P, P, P, I64, I64],
+        "om_mi355x_DequantizeLinear": [P, P, P, P, I64],
+        "om_mi355x_DynamicQuantizeLinear": [P, P, P, P],
+        "om_mi355x_MatMulInteger": [P, P, P, P, P],
+        "om_mi355x_MatMulIntegerDequant": [P, P, P, P, P, P, P],
+        "om_mi355x_QLinearMatMul": [P, P, P, P, P, P, P, P, P, I64],
+        "om_mi355x_DynQuantMatMulDequant": [P, P, P, P, P],
+        "om_mi355x_MarkConstant": [P],
+        "om_mi355x_ClearCache": [],
+        "OMInitAccelMI355X": [],
+        "OMShutdownAccelMI355X": [],
+    }
+    for name, args in sigs.items():
+        fn = getattr(lib, name)
+        fn.restype = None
+        fn.argtypes = args
+    lib.OMInitCompatibleAccelMI355X.restype = ctypes.c_uint64
+    lib.OMInitCompatibleAccelMI355X.argtypes = [ctypes.c_uint64]
+    lib.om_mi355x_malloc.restype = P
+    lib.om_mi355x_malloc.argtypes = [SZ]
+    lib.om_mi355x_free.restype = None
+    lib.om_mi355x_free.argtypes = [P]
+    lib.om_mi355x_memcpy_h2d.restype = ctypes.c_int
+    lib.om_mi355x_memcpy_h2d.argtypes = [P, P, SZ]
+    lib.om_mi355x_memcpy_d2h.restype = ctypes.c_int
+    lib.om_mi355x_memcpy_d2h.argtypes = [P, P, SZ]
+    lib.om_mi355x_synchronize.restype = ctypes.c_int
+    lib.om_mi355x_timer_start.restype = ctypes.c_int
+    lib.om_mi355x_timer_stop.restype = ctypes.c_float
+    lib.om_mi355x_last_error.restype = ctypes.c_char_p
+    lib.om_mi355x_device_info.restype = ctypes.c_int
+    lib.om_mi355x_device_info.argtypes = [ctypes.c_char_p, SZ]
+
+
+def _check():
+    msg = _lib.om_mi355x_last_error()
+    if msg:
+        raise RuntimeError_(msg.decode())
+
+
+def device_info() -> dict:
+    load()
+    buf = ctypes.create_string_buffer(256)
+    if _lib.om_mi355x_device_info(buf, 256) != 0:
+        _check()
+        raise RuntimeError_("no device")
+    name, arch, cus, mhz, gib = buf.value.decode().split("|")
+    return {"name": name, "arch": arch, "cus": int(cus), "clock_mhz": int(mhz),
+            "mem_gib": float(gib)}
+
+
+def init_compatible(version: int = 0x100) -> bool:
+    load()
+    return bool(_lib.OMInitCompatibleAccelMI355X(version))
+
+
+class DeviceArray:
+    """A row-major tensor in GPU memory obtained from the runtime."""
+
+    def __init__(self, shape: Sequence[int], dtype):
+        load()
+        self.shape = tuple(int(s) for s in shape)
+        self.dtype = np.dtype(dtype)
+        self.size = int(np.prod(self.shape, dtype=np.int64)) if self.shape else 1
+        self.nbytes = self.size * self.dtype.itemsize
+        self.ptr = _lib.om_mi355x_malloc(max(self.nbytes, 16))
+        if not self.ptr:
+            _check()
+            raise MemoryError("om_mi355x_malloc failed")
+
+    @classmethod
+    def from_numpy(cls, a: np.ndarray) -> "DeviceArray":
+        a = np.ascontiguousarray(a)
+        d = cls(a.shape, a.dtype)
+        if a.nbytes and _lib.om_mi355x_memcpy_h2d(
+                d.ptr, a.ctypes.data_as(ctypes.c_void_p), a.nbytes) != 0:
+            _check()
+        return d
+
+    @classmethod
+    def view_of(cls, owner: "DeviceArray", offset_elems: int, shape) -> "DeviceArray":
+        """A window into ``owner``'s memory starting ``offset_elems`` elements in."""
+        v = cls.__new__(cls)
+        v.shape = tuple(int(s) for s in shape)
+        v.dtype = owner.dtype
+        v.size = int(np.prod(v.shape, dtype=np.int64)) if v.shape else 1
+        v.nbytes = v.size * v.dtype.itemsize
+        assert offset_elems * v.dtype.itemsize + v.nbytes <= owner.nbytes
+        v.ptr = owner.ptr + offset_elems * v.dtype.itemsize
+        v.owner = owner
+        return v
+
+    def numpy(self) -> np.ndarray:
+        out = np.empty(self.shape, self.dtype)
+        if self.nbytes and _lib.om_mi355x_memcpy_d2h(
+                out.ctypes.data_as(ctypes.c_void_p), self.ptr, self.nbytes) != 0:
+            _check()
+        return out
+
+    def free(self):
+        if getattr(self, "owner", None) is not None:
+            self.ptr = None
+            return
+        if self.ptr:
+            _lib.om_mi355x_free(self.ptr)
+            self.ptr = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+Tensor = Union[np.ndarray, DeviceArray]
+
+
+class _OMT:
+    """A non-owning OMTensor wrapper around a numpy array or DeviceArray, made
+    the way the generated code makes one per krnl.call operand."""
+
+    def __init__(self, t: Optional[Tensor]):
+        self.handle = None
+        self.keep = t
+        if t is None:
+            return
+        if isinstance(t, DeviceArray):
+            ptr, shape, dt = t.ptr, t.shape, t.dtype
+        else:
+            if not t.flags["C_CONTIGUOUS"]:
+                raise ValueError("host tensors must be C-contiguous")
+            ptr, shape, dt = t.ctypes.data, t.shape, t.dtype
+        code = _NP_TO_ONNX.get(np.dtype(dt))
+        if code is None:
+            raise TypeError(f"unsupported element type {dt}")
+        arr = (ctypes.c_int64 * max(len(shape), 1))(*shape)
+        self.handle = _shim.omTensorCreate(ptr, arr, len(shape), code)
+        if not self.handle:
+            raise MemoryError("omTensorCreate failed")
+
+    def __enter__(self):
+        return self.handle
+
+    def __exit__(self, *exc):
+        if self.handle:
+            _shim.omTensorDestroy(self.handle)
+            self.handle = None
+
+
+def _like(template: Tensor, shape, dtype) -> Tensor:
+    if isinstance(template, DeviceArray):
+        return DeviceArray(shape, dtype)
+    return np.empty(shape, dtype)
+
+
+def _host(a, dtype=None) -> Tensor:
+    if isinstance(a, DeviceArray):
+        return a
+    a = np.asarray(a) if dtype is None else np.asarray(a, dtype=dtype)
+    return np.ascontiguousarray(a)
+
+
+def mark_constant(t: Tensor):
+    """Declare that ``t`` never changes (a model constant)."""
+    load()
+    with _OMT(t) as h:
+        _lib.om_mi355x_MarkConstant(h)
+
+
+def clear_cache():
+    load()
+    _lib.om_mi355x_ClearCache()
+
+
+def synchronize():
+    load()
+    if _lib.om_mi355x_synchronize() != 0:
+        _check()
+
+
+def timer_start():
+    if _lib.om_mi355x_timer_start() != 0:
+        _check()
+
+
+def timer_stop() -> float:
+    ms = float(_lib.om_mi355x_timer_stop())
+    if ms < 0:
+        _check()
+    return ms
+
+
+def QuantizeLinear(x: Tensor, y_scale: Tensor, y_zero_point: Optional[Tensor] = None,
+                   axis: int = 1, saturate: int = 1, out: Optional[Tensor] = None) -> Tensor:
+    load()
+    x, y_scale = _host(x), _host(y_scale, np.float32)
+    ydt = np.uint8 if y_zero_point is None else _host(y_zero_point).dtype
+    if y_zero_point is not None:
+        y_zero_point = _host(y_zero_point)
+    y = out if out is not None else _like(x, x.shape, ydt)
+    with _OMT(y) as hy, _OMT(x) as hx, _OMT(y_scale) as hs, _OMT(y_zero_point) as hz:
+        _lib.om_mi355x_QuantizeLinear(hy, hx, hs, hz, axis, saturate)
+    _check()
+    return y
+
+
+def DequantizeLinear(x: Tensor, x_scale: Tensor, x_zero_point: Optional[Tensor] = None,
+                     axis: int = 1, out: Optional[Tensor] = None) -> Tensor:
+    load()
+    x, x_scale = _host(x), _host(x_scale, np.float32)
+    if x_zero_point is not None:
+        x_zero_point = _host(x_zero_point)
+    y = out if out is not None else _like(x, x.shape, np.float32)
+    with _OMT(y) as hy, _OMT(x) as hx, _OMT(x_scale) as hs, _OMT(x_zero_point) as hz:
+        _lib.om_mi355x_DequantizeLinear(hy, hx, hs, hz, axis)
+    _check()
+    return y
+
+
+def DynamicQuantizeLinear(x: Tensor, out: Optional[Tuple[Tensor, Tensor, Tensor]] = None
+                          ) -> Tuple[Tensor, Tensor, Tensor]:
+    load()
+    x = _host(x)
+    if out is not None:
+        y, s, z = out
+    else:
+        y = _like(x, x.shape, np.uint8)
+        s = _like(x, (), np.float32)
+        z = _like(x, (), np.uint8)
+    with _OMT(y) as hy, _OMT(s) as hs, _OMT(z) as hz, _OMT(x) as hx:
+        _lib.om_mi355x_DynamicQuantizeLinear(hy, hs, hz, hx)
+    _check()
+    return y, s, z
+
+
+def _mm_shape(a: Tensor, b: Tensor):
+    return tuple(a.shape[:-1]) + (b.shape[-1],)
+
+
+def MatMulInteger(a: Tensor, b: Tensor, a_zero_point: Optional[Tensor] = None,
+                  b_zero_point: Optional[Tensor] = None, out: Optional[Tensor] = None) -> Tensor:
+    load()
+    a, b = _host(a), _host(b)
+    az = None if a_zero_point is None else _host(a_zero_point)
+    bz = None if b_zero_point is None else _host(b_zero_point)
+    y = out if out is not None else _like(a, _mm_shape(a, b), np.int32)
+    with _OMT(y) as hy, _OMT(a) as ha, _OMT(b) as hb, _OMT(az) as haz, _OMT(bz) as hbz:
+        _lib.om_mi355x_MatMulInteger(hy, ha, hb, haz, hbz)
+    _check()
+    return y
+
+
+def MatMulIntegerDequant(a: Tensor, b: Tensor, a_zero_point: Optional[Tensor],
+                         b_zero_point: Optional[Tensor], a_scale: Tensor, b_scale: Tensor,
+                         out: Optional[Tensor] = None) -> Tensor:
+    load()
+    a, b = _host(a), _host(b)
+    a_scale, b_scale = _host(a_scale, np.float32), _host(b_scale, np.float32)
+    az = None if a_zero_point is None else _host(a_zero_point)
+    bz = None if b_zero_point is None else _host(b_zero_point)
+    y = out if out is not None else _like(a, _mm_shape(a, b), np.float32)
+    with _OMT(y) as hy, _OMT(a) as ha, _OMT(b) as hb, _OMT(az) as haz, _OMT(bz) as hbz, \
+            _OMT(a_scale) as has, _OMT(b_scale) as hbs:
+        _lib.om_mi355x_MatMulIntegerDequant(hy, ha, hb, haz, hbz, has, hbs)
+    _check()
+    return y
+
+
+def QLinearMatMul(a: Tensor, a_scale: Tensor, a_zero_point: Tensor, b: Tensor,
+                  b_scale: Tensor, b_zero_point: Tensor, y_scale: Tensor,
+                  y_zero_point: Tensor, narrow_mode: int = WRAP,
+                  out: Optional[Tensor] = None) -> Tensor:
+    load()
+    a, b = _host(a), _host(b)
+    a_scale, b_scale = _host(a_scale, np.float32), _host(b_scale, np.float32)
+    y_scale = _host(y_scale, np.float32)
+    az, bz, yz = _host(a_zero_point), _host(b_zero_point), _host(y_zero_point)
+    y = out if out is not None else _like(a, _mm_shape(a, b), yz.dtype)
+    with _OMT(y) as hy, _OMT(a) as ha, _OMT(a_scale) as has, _OMT(az) as haz, \
+            _OMT(b) as hb, _OMT(b_scale) as hbs, _OMT(bz) as hbz, \
+            _OMT(y_scale) as hys, _OMT(yz) as hyz:
+        _lib.om_mi355x_QLinearMatMul(hy, ha, has, haz, hb, hbs, hbz, hys, hyz, narrow_mode)
+    _check()
+    return y
+
+
+def DynQuantMatMulDequant(x: Tensor, b: Tensor, b_zero_point: Optional[Tensor],
+                          b_scale: Tensor, out: Optional[Tensor] = None) -> Tensor:
+    load()
+    x, b, b_scale = _host(x), _host(b), _host(b_scale, np.float32)
+    bz = None if b_zero_point is None else _host(b_zero_point)
+    y = out if out is not None else _like(x, _mm_shape(x, b), np.float32)
+    with _OMT(y) as hy, _OMT(x) as hx, _OMT(b) as hb, _OMT(bz) as hbz, _OMT(b_scale) as hbs:
+        _lib.om_mi355x_DynQuantMatMulDequant(hy, hx, hb, hbz, hbs)
+    _check()
+    return y

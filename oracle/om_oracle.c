@@ -1,0 +1,438 @@
+/*
+ * CPU oracle for the onnx-mlir int8 quantized-inference path: a restatement of
+ * the arithmetic the reference's ONNX->Krnl lowering generates.
+ *
+ * TEST INFRASTRUCTURE ONLY -- see om_oracle.h.  Build with
+ *   gcc -O2 -ffp-contract=off -fno-fast-math (-fopenmp)
+ * so that no operation is fused, re-associated or replaced by a reciprocal.
+ *
+ * What pins each function (beyond following the cited lowering op for op):
+ *  - om_oracle_rne: swept against nearbyintf over a dense set of binary32
+ *    values (all exponents, tie cases); equal except the sign of zero on
+ *    (-0.5, 0), which no caller can observe.
+ *  - quantize / dequantize per-tensor, dynamic quantize, matmul integer,
+ *    qlinear matmul: the ONNX node-test vectors the reference enables in
+ *    test/backend/inference_backend.py (test_quantizelinear_cpu :2531,
+ *    test_dequantizelinear_cpu :880, test_dynamicquantizelinear*_cpu :932-957,
+ *    test_matmulinteger_cpu :2047, test_qlinearmatmul_2D_*_cpu :2539-2554),
+ *    the constant-propagation answers in test/mlir/onnx/onnx_constprop.mlir
+ *    :1175-1300, brute force on tiny shapes and algebraic identities.
+ *  - per-axis quantize / dequantize: PARITY UNPINNED (the reference asserts
+ *    on per-axis, src/Conversion/ONNXToKrnl/Quantization/QuantizeLinear.cpp
+ *    :192-195); checked only against the ONNX specification's axis vectors.
+ */
+#include "om_oracle.h"
+
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+int om_oracle_num_threads(void) {
+#ifdef _OPENMP
+  return omp_get_max_threads();
+#else
+  return 1;
+#endif
+}
+
+/* Round half to even through floor, the numpy rint algorithm.
+ * Follows MathBuilder::roundEvenEmulation,
+ * src/Dialect/Mlir/DialectBuilder.cpp:291-332, which KrnlBuilder::roundEven
+ * (src/Dialect/Krnl/DialectBuilder.cpp:460-501) selects on non-Z targets. */
+float om_oracle_rne(float x) {
+  float y = floorf(x);
+  float r = x - y;
+  float y1 = (r > 0.5f) ? (y + 1.0f) : y;
+  float h = floorf(0.5f * y);
+  float rr = y - h * 2.0f;
+  float y2 = (rr == 1.0f) ? (y + 1.0f) : y;
+  return (r == 0.5f) ? y2 : y1;
+}
+
+/* MathBuilder::clip = max then min, both the NaN-ignoring "num" flavours,
+ * src/Dialect/Mlir/DialectBuilder.cpp:355-360,462-484. */
+static inline float clipf(float v, float lo, float hi) {
+  return fminf(fmaxf(v, lo), hi);
+}
+
+static inline float load_q_as_f32(const void *p, int kind, int64_t i) {
+  /* MathBuilder::cast int->float widens to a 32-bit int of the same
+   * signedness first, then uitofp / sitofp
+   * (src/Dialect/Mlir/DialectBuilder.cpp:979-995,1044-1054). */
+  switch (kind) {
+  case OM_ORACLE_U8:
+    return (float)(uint32_t)((const uint8_t *)p)[i];
+  case OM_ORACLE_I8:
+    return (float)(int32_t)((const int8_t *)p)[i];
+  default:
+    return (float)((const int32_t *)p)[i];
+  }
+}
+
+/* One element of emitQuantizationLinearScalarParameters,
+ * src/Conversion/ONNXToKrnl/Quantization/QuantizeLinear.cpp:119-144:
+ * divf, roundEven, addf (if zero point), maxnumf, minnumf, fptoui/fptosi to
+ * i32, trunci to i8. */
+static inline uint8_t quant_one(
+    float x, float scale, float zpf, int has_zp, int qkind) {
+  float t = x / scale;
+  float r = om_oracle_rne(t);
+  if (has_zp)
+    r = r + zpf;
+  if (qkind == OM_ORACLE_U8) {
+    float c = clipf(r, 0.0f, 255.0f);
+    return (uint8_t)(uint32_t)c;
+  }
+  float c = clipf(r, -128.0f, 127.0f);
+  return (uint8_t)(int8_t)(int32_t)c;
+}
+
+/* ONNXQuantizeLinearOpLowering,
+ * src/Conversion/ONNXToKrnl/Quantization/QuantizeLinear.cpp:155-246
+ * (bounds :211-218, zero point cast to f32 :223-230).  channels > 1 applies
+ * the same scalar formula with scale[c], zp[c] (per-axis: parity unpinned). */
+void om_oracle_quantize_linear(const float *x, int64_t outer, int64_t channels,
+    int64_t inner, const float *scale, const void *zp, int qkind, void *y) {
+  uint8_t *out = (uint8_t *)y;
+  for (int64_t o = 0; o < outer; ++o)
+    for (int64_t c = 0; c < channels; ++c) {
+      float s = scale[c];
+      float zpf = zp ? load_q_as_f32(zp, qkind, c) : 0.0f;
+      int64_t base = (o * channels + c) * inner;
+      for (int64_t i = 0; i < inner; ++i)
+        out[base + i] = quant_one(x[base + i], s, zpf, zp != NULL, qkind);
+    }
+}
+
+void om_oracle_quantize_linear_omp(const float *x, int64_t outer,
+    int64_t channels, int64_t inner, const float *scale, const void *zp,
+    int qkind, void *y) {
+  uint8_t *out = (uint8_t *)y;
+  if (channels == 1) {
+    float s = scale[0];
+    float zpf = zp ? load_q_as_f32(zp, qkind, 0) : 0.0f;
+    int64_t n = outer * inner;
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < n; ++i)
+      out[i] = quant_one(x[i], s, zpf, zp != NULL, qkind);
+    return;
+  }
+  int64_t rows = outer * channels;
+#pragma omp parallel for schedule(static)
+  for (int64_t rc = 0; rc < rows; ++rc) {
+    int64_t c = rc % channels;
+    float s = scale[c];
+    float zpf = zp ? load_q_as_f32(zp, qkind, c) : 0.0f;
+    int64_t base = rc * inner;
+    for (int64_t i = 0; i < inner; ++i)
+      out[base + i] = quant_one(x[base + i], s, zpf, zp != NULL, qkind);
+  }
+}
+
+/* emitScalarOpFor<ONNXDequantizeLinearOp>,
+ * src/Conversion/ONNXToKrnl/Math/Elementwise.cpp:1439-1461:
+ * cast to f32, subf zero point (if present), mulf scale. */
+void om_oracle_dequantize_linear(const void *x, int xkind, int64_t outer,
+    int64_t channels, int64_t inner, const float *scale, const void *zp,
+    float *y) {
+  for (int64_t o = 0; o < outer; ++o)
+    for (int64_t c = 0; c < channels; ++c) {
+      float s = scale[c];
+      float zpf = zp ? load_q_as_f32(zp, xkind, c) : 0.0f;
+      int64_t base = (o * channels + c) * inner;
+      for (int64_t i = 0; i < inner; ++i) {
+        float xf = load_q_as_f32(x, xkind, base + i);
+        if (zp)
+          xf = xf - zpf;
+        y[base + i] = xf * s;
+      }
+    }
+}
+
+void om_oracle_dequantize_linear_omp(const void *x, int xkind, int64_t outer,
+    int64_t channels, int64_t inner, const float *scale, const void *zp,
+    float *y) {
+  int64_t rows = outer * channels;
+  if (channels == 1) {
+    float s = scale[0];
+    float zpf = zp ? load_q_as_f32(zp, xkind, 0) : 0.0f;
+    int64_t n = outer * inner;
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < n; ++i) {
+      float xf = load_q_as_f32(x, xkind, i);
+      if (zp)
+        xf = xf - zpf;
+      y[i] = xf * s;
+    }
+    return;
+  }
+#pragma omp parallel for schedule(static)
+  for (int64_t rc = 0; rc < rows; ++rc) {
+    int64_t c = rc % channels;
+    float s = scale[c];
+    float zpf = zp ? load_q_as_f32(zp, xkind, c) : 0.0f;
+    int64_t base = rc * inner;
+    for (int64_t i = 0; i < inner; ++i) {
+      float xf = load_q_as_f32(x, xkind, base + i);
+      if (zp)
+        xf = xf - zpf;
+      y[base + i] = xf * s;
+    }
+  }
+}
+
+/* emitMinMaxReductionToScalar,
+ * src/Conversion/ONNXToKrnl/Math/Reduction.cpp:529-548: minnumf / maxnumf
+ * reductions from +inf / -inf.  The order of a min/max reduction does not
+ * change its value. */
+void om_oracle_minmax(const float *x, int64_t n, float *mn, float *mx) {
+  float lo = INFINITY, hi = -INFINITY;
+  for (int64_t i = 0; i < n; ++i) {
+    lo = fminf(lo, x[i]);
+    hi = fmaxf(hi, x[i]);
+  }
+  *mn = lo;
+  *mx = hi;
+}
+
+/* emitDynamicQuantizationLinearScalarParametersFromMinMax,
+ * src/Conversion/ONNXToKrnl/Quantization/DynamicQuantizeLinear.cpp:43-84. */
+void om_oracle_dynamic_params(
+    float xmin, float xmax, float *scale, float *zp_f32, uint8_t *zp_u8) {
+  const float qmin = 0.0f, qmax = 255.0f;
+  float mx = fmaxf(xmax, 0.0f);
+  float mn = fminf(xmin, 0.0f);
+  float xdiff = mx - mn;
+  float bound = qmax - qmin;
+  float s = xdiff / bound;
+  float inter = qmin - mn / s;
+  float sat = clipf(inter, qmin, qmax); /* saturate, then round */
+  float z = om_oracle_rne(sat);
+  *scale = s;
+  *zp_f32 = z;
+  *zp_u8 = (uint8_t)(uint32_t)z;
+}
+
+/* ONNXDynamicQuantizeLinearOpLowering,
+ * src/Conversion/ONNXToKrnl/Quantization/DynamicQuantizeLinear.cpp:86-158:
+ * min/max, parameters, then the shared quantize loop with the FLOAT zero
+ * point (:149-152). */
+void om_oracle_dynamic_quantize_linear(
+    const float *x, int64_t n, uint8_t *y, float *scale, uint8_t *zp) {
+  float mn, mx, s, zf;
+  om_oracle_minmax(x, n, &mn, &mx);
+  om_oracle_dynamic_params(mn, mx, &s, &zf, zp);
+  *scale = s;
+  for (int64_t i = 0; i < n; ++i)
+    y[i] = quant_one(x[i], s, zf, 1, OM_ORACLE_U8);
+}
+
+/* The reference with --parallel reduces in 8 chunks and then across the 8
+ * partial results (tNum = 8, src/Conversion/ONNXToKrnl/Math/Reduction.cpp
+ * :466-515); the quantize loop is one more parallel pass over X. */
+void om_oracle_dynamic_quantize_linear_omp(
+    const float *x, int64_t n, uint8_t *y, float *scale, uint8_t *zp) {
+  enum { T = 8 };
+  float lo[T], hi[T];
+  int64_t chunk = (n + T - 1) / T;
+#pragma omp parallel for schedule(static)
+  for (int t = 0; t < T; ++t) {
+    int64_t b = t * chunk, e = b + chunk < n ? b + chunk : n;
+    float l = INFINITY, h = -INFINITY;
+    for (int64_t i = b; i < e; ++i) {
+      l = fminf(l, x[i]);
+      h = fmaxf(h, x[i]);
+    }
+    lo[t] = l;
+    hi[t] = h;
+  }
+  float mn = INFINITY, mx = -INFINITY;
+  for (int t = 0; t < T; ++t) {
+    mn = fminf(mn, lo[t]);
+    mx = fmaxf(mx, hi[t]);
+  }
+  float s, zf;
+  om_oracle_dynamic_params(mn, mx, &s, &zf, zp);
+  *scale = s;
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < n; ++i)
+    y[i] = quant_one(x[i], s, zf, 1, OM_ORACLE_U8);
+}
+
+static inline int32_t load_q_as_i32(const void *p, int kind, int64_t i) {
+  return kind == OM_ORACLE_U8 ? (int32_t)((const uint8_t *)p)[i]
+                              : (int32_t)((const int8_t *)p)[i];
+}
+
+static inline int32_t zp_at(
+    const void *zp, int kind, int64_t len, int64_t i) {
+  if (!zp || len == 0)
+    return 0;
+  return load_q_as_i32(zp, kind, len == 1 ? 0 : i);
+}
+
+/* ONNXMatMulIntegerOpLowering,
+ * src/Conversion/ONNXToKrnl/Math/MatMulInteger.cpp:59-90: cast to i32 (zext
+ * ui8 / sext i8), subtract zero points (per-row a_zp unsqueezed to [M,1]
+ * :66-75, per-column b_zp broadcast over K :79-84), int32 MatMul.  All
+ * arithmetic is modulo 2^32 (done in uint32_t to keep C defined). */
+void om_oracle_matmul_integer(const void *A, int akind, const void *B,
+    int bkind, int64_t M, int64_t K, int64_t N, const void *a_zp,
+    int64_t a_zp_len, const void *b_zp, int64_t b_zp_len, int32_t *Y) {
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < M; ++i) {
+    int32_t az = zp_at(a_zp, akind, a_zp_len, i);
+    for (int64_t j = 0; j < N; ++j) {
+      int32_t bz = zp_at(b_zp, bkind, b_zp_len, j);
+      uint32_t acc = 0;
+      for (int64_t k = 0; k < K; ++k) {
+        uint32_t a = (uint32_t)(load_q_as_i32(A, akind, i * K + k) - az);
+        uint32_t b = (uint32_t)(load_q_as_i32(B, bkind, k * N + j) - bz);
+        acc += a * b;
+      }
+      Y[i * N + j] = (int32_t)acc;
+    }
+  }
+}
+
+/* Pass structure of the reference's CPU code for the same op: the casts and
+ * subtractions are separate full-tensor passes
+ * (src/Conversion/ONNXToKrnl/Math/MatMulInteger.cpp:59-84), the result is
+ * memset and the int32 MatMul is blocked I/J/K = 4/8/8 with the I tiles in
+ * parallel (src/Conversion/ONNXToKrnl/Math/MatMul.cpp:143-150,278-327). */
+void om_oracle_matmul_integer_passes(const void *A, int akind, const void *B,
+    int bkind, int64_t M, int64_t K, int64_t N, const void *a_zp,
+    int64_t a_zp_len, const void *b_zp, int64_t b_zp_len, int32_t *Y) {
+  uint32_t *A32 = (uint32_t *)malloc((size_t)M * K * sizeof(uint32_t));
+  uint32_t *B32 = (uint32_t *)malloc((size_t)K * N * sizeof(uint32_t));
+  uint32_t *C = (uint32_t *)Y;
+  int64_t i, k;
+#pragma omp parallel for schedule(static)
+  for (i = 0; i < M * K; ++i)
+    A32[i] = (uint32_t)load_q_as_i32(A, akind, i);
+  if (a_zp && a_zp_len > 0) {
+#pragma omp parallel for schedule(static)
+    for (i = 0; i < M; ++i) {
+      uint32_t az = (uint32_t)zp_at(a_zp, akind, a_zp_len, i);
+      for (int64_t kk = 0; kk < K; ++kk)
+        A32[i * K + kk] -= az;
+    }
+  }
+#pragma omp parallel for schedule(static)
+  for (i = 0; i < K * N; ++i)
+    B32[i] = (uint32_t)load_q_as_i32(B, bkind, i);
+  if (b_zp && b_zp_len > 0) {
+#pragma omp parallel for schedule(static)
+    for (k = 0; k < K; ++k)
+      for (int64_t j = 0; j < N; ++j)
+        B32[k * N + j] -= (uint32_t)zp_at(b_zp, bkind, b_zp_len, j);
+  }
+  memset(C, 0, (size_t)M * N * sizeof(uint32_t));
+  enum { TI = 4, TJ = 8, TK = 8 };
+#pragma omp parallel for schedule(static)
+  for (int64_t i0 = 0; i0 < M; i0 += TI) {
+    int64_t ie = i0 + TI < M ? i0 + TI : M;
+    for (int64_t j0 = 0; j0 < N; j0 += TJ) {
+      int64_t je = j0 + TJ < N ? j0 + TJ : N;
+      for (int64_t k0 = 0; k0 < K; k0 += TK) {
+        int64_t ke = k0 + TK < K ? k0 + TK : K;
+        if (ie - i0 == TI && je - j0 == TJ && ke - k0 == TK) {
+          uint32_t c[TI][TJ];
+          for (int ii = 0; ii < TI; ++ii)
+            for (int jj = 0; jj < TJ; ++jj)
+              c[ii][jj] = C[(i0 + ii) * N + j0 + jj];
+          for (int kk = 0; kk < TK; ++kk)
+            for (int ii = 0; ii < TI; ++ii) {
+              uint32_t a = A32[(i0 + ii) * K + k0 + kk];
+              for (int jj = 0; jj < TJ; ++jj)
+                c[ii][jj] += a * B32[(k0 + kk) * N + j0 + jj];
+            }
+          for (int ii = 0; ii < TI; ++ii)
+            for (int jj = 0; jj < TJ; ++jj)
+              C[(i0 + ii) * N + j0 + jj] = c[ii][jj];
+        } else {
+          for (int64_t ii = i0; ii < ie; ++ii)
+            for (int64_t kk = k0; kk < ke; ++kk) {
+              uint32_t a = A32[ii * K + kk];
+              for (int64_t jj = j0; jj < je; ++jj)
+                C[ii * N + jj] += a * B32[kk * N + jj];
+            }
+        }
+      }
+    }
+  }
+  free(A32);
+  free(B32);
+}
+
+/* OnnxBuilder::getOrCastToI8, src/Dialect/ONNX/DialectBuilder.cpp:916-933:
+ * ui8 v -> i8(i16(v) - 128); i8 unchanged. */
+static inline int32_t to_i8_domain(const void *p, int kind, int64_t i) {
+  if (kind == OM_ORACLE_U8) {
+    int16_t v = (int16_t)((const uint8_t *)p)[i];
+    return (int32_t)(int8_t)(v - 128);
+  }
+  return (int32_t)((const int8_t *)p)[i];
+}
+
+/* ONNXQLinearMatMulOpLowering,
+ * src/Conversion/ONNXToKrnl/Math/QLinearMatMul.cpp:88-138:
+ * everything is moved to the i8 domain, widened to i32, zero points
+ * subtracted, int32 MatMul, sitofp, mulf by (a_scale*b_scale)/y_scale,
+ * roundEven, fptosi, addi y_zp, and for ui8 results addi 128 then trunci to
+ * i8, then a reinterpreting cast: NO clip, the narrowing wraps.  SATURATE is
+ * the ONNX specification's behaviour instead of the trunci. */
+void om_oracle_qlinear_matmul(const void *A, int akind, float a_scale,
+    const void *a_zp, int64_t a_zp_len, const void *B, int bkind,
+    float b_scale, const void *b_zp, int64_t b_zp_len, float y_scale,
+    const void *y_zp, int ykind, int64_t M, int64_t K, int64_t N, int mode,
+    void *Y) {
+  float s = (a_scale * b_scale) / y_scale;
+  int32_t yz = to_i8_domain(y_zp, ykind, 0);
+  uint8_t *out = (uint8_t *)Y;
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < M; ++i) {
+    int32_t az = to_i8_domain(a_zp, akind, a_zp_len == 1 ? 0 : i);
+    for (int64_t j = 0; j < N; ++j) {
+      int32_t bz = to_i8_domain(b_zp, bkind, b_zp_len == 1 ? 0 : j);
+      uint32_t acc = 0;
+      for (int64_t k = 0; k < K; ++k) {
+        uint32_t a = (uint32_t)(to_i8_domain(A, akind, i * K + k) - az);
+        uint32_t b = (uint32_t)(to_i8_domain(B, bkind, k * N + j) - bz);
+        acc += a * b;
+      }
+      float f = (float)(int32_t)acc * s;
+      int32_t q = (int32_t)om_oracle_rne(f);
+      uint32_t r = (uint32_t)q + (uint32_t)yz;
+      if (ykind == OM_ORACLE_U8)
+        r += 128u;
+      if (mode == OM_ORACLE_WRAP) {
+        out[i * N + j] = (uint8_t)(r & 0xFFu);
+      } else {
+        int32_t v = (int32_t)r;
+        if (ykind == OM_ORACLE_U8)
+          v = v < 0 ? 0 : (v > 255 ? 255 : v);
+        else
+          v = v < -128 ? -128 : (v > 127 ? 127 : v);
+        out[i * N + j] = (uint8_t)v;
+      }
+    }
+  }
+}
+
+/* Graph-level epilogue Cast(i32->f32) then Mul by the product of the scales:
+ * out = sitofp(acc) * (a_scale * b_scale[j]); the two graph shapes the
+ * reference recognises are listed at
+ * src/Accelerators/NNPA/Conversion/ONNXToZHigh/ONNXToZHigh.cpp:1021-1060. */
+void om_oracle_dequant_epilogue(const int32_t *acc, int64_t M, int64_t N,
+    float a_scale, const float *b_scale, int64_t b_scale_len, float *out) {
+  for (int64_t i = 0; i < M; ++i)
+    for (int64_t j = 0; j < N; ++j) {
+      float s = a_scale * b_scale[b_scale_len == 1 ? 0 : j];
+      out[i * N + j] = (float)acc[i * N + j] * s;
+    }
+}

@@ -1,0 +1,127 @@
+"""Boundary checks that need no GPU: the C-ABI library loads and exports every
+symbol the headers declare, the OMTensor layout is the reference's, arguments
+are validated, and without a device the entry points fail loudly (there is no
+CPU path behind them)."""
+import ctypes
+import errno
+import os
+import re
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+INCLUDE = os.path.join(ROOT, "include")
+REF_RUNTIME = os.path.join(ROOT, "oracle", "_ref", "libomruntime_ref.so")
+
+
+def _declared(header, pattern):
+    text = open(os.path.join(INCLUDE, header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(pattern, text)))
+
+
+def test_library_exports_every_declared_symbol(rt):
+    lib = rt.load()
+    names = _declared("om_mi355x.h", r"\b(om_mi355x_\w+|OM\w+AccelMI355X)\s*\(")
+    assert len(names) >= 18
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in om_mi355x.h but not exported"
+    assert ctypes.c_long.in_dll(lib, "OMIsInitAccelMI355X") is not None
+    shim = ctypes.CDLL(rt.SHIM_PATH)
+    for n in _declared("om_tensor_abi.h", r"\b(omTensor\w+)\s*\("):
+        assert hasattr(shim, n), f"{n} declared in om_tensor_abi.h but not exported"
+
+
+def test_runtime_library_does_not_define_tensor_accessors(rt):
+    # A compiled model brings the omTensor* symbols from libcruntime; the runtime
+    # library must only reference them, or the model link would see duplicates.
+    import subprocess
+    out = subprocess.check_output(["nm", "-D", "--defined-only", rt.LIB_PATH], text=True)
+    assert "omTensorGetDataPtr" not in out
+    und = subprocess.check_output(["nm", "-D", "--undefined-only", rt.LIB_PATH], text=True)
+    assert "omTensorGetDataPtr" in und
+
+
+@pytest.mark.skipif(not os.path.exists(REF_RUNTIME), reason="oracle/_ref not built (no reference tree)")
+def test_omtensor_layout_matches_reference_runtime(rt):
+    """A tensor built by the reference's own C runtime is read correctly by our
+    accessors and vice versa (struct of src/Runtime/OMTensor.inc:125-140)."""
+    ref = ctypes.CDLL(REF_RUNTIME)
+    shim = ctypes.CDLL(rt.SHIM_PATH)
+    P, I64 = ctypes.c_void_p, ctypes.c_int64
+    for lib in (ref, shim):
+        lib.omTensorCreate.restype = P
+        lib.omTensorCreate.argtypes = [P, ctypes.POINTER(I64), I64, ctypes.c_int]
+        lib.omTensorDestroy.argtypes = [P]
+        lib.omTensorGetDataPtr.restype = P
+        lib.omTensorGetDataPtr.argtypes = [P]
+        lib.omTensorGetShape.restype = ctypes.POINTER(I64)
+        lib.omTensorGetShape.argtypes = [P]
+        lib.omTensorGetStrides.restype = ctypes.POINTER(I64)
+        lib.omTensorGetStrides.argtypes = [P]
+        lib.omTensorGetRank.restype = I64
+        lib.omTensorGetRank.argtypes = [P]
+        lib.omTensorGetDataType.restype = ctypes.c_int
+        lib.omTensorGetDataType.argtypes = [P]
+        lib.omTensorGetNumElems.restype = I64
+        lib.omTensorGetNumElems.argtypes = [P]
+        lib.omTensorGetBufferSize.restype = I64
+        lib.omTensorGetBufferSize.argtypes = [P]
+    data = np.arange(2 * 3 * 5, dtype=np.int32)
+    shape = (I64 * 3)(2, 3, 5)
+    for maker, reader in ((ref, shim), (shim, ref)):
+        for dtype_code, itemsize in ((6, 4), (1, 4), (2, 1), (3, 1)):
+            t = maker.omTensorCreate(data.ctypes.data, shape, 3, dtype_code)
+            assert reader.omTensorGetDataPtr(t) == data.ctypes.data
+            assert reader.omTensorGetRank(t) == 3
+            assert [reader.omTensorGetShape(t)[i] for i in range(3)] == [2, 3, 5]
+            assert [reader.omTensorGetStrides(t)[i] for i in range(3)] == [15, 5, 1]
+            assert reader.omTensorGetDataType(t) == dtype_code
+            assert reader.omTensorGetNumElems(t) == 30
+            assert reader.omTensorGetBufferSize(t) == 30 * itemsize
+            maker.omTensorDestroy(t)
+    # rank 0 (scalars such as y_scale)
+    t = ref.omTensorCreate(data.ctypes.data, shape, 0, 1)
+    assert shim.omTensorGetRank(t) == 0 and shim.omTensorGetNumElems(t) == 1
+    ref.omTensorDestroy(t)
+
+
+def _no_gpu():
+    return not os.path.exists("/dev/kfd")
+
+
+def test_argument_validation_sets_einval(rt):
+    x = np.zeros((4, 6), np.float32)
+    with pytest.raises(rt.RuntimeError_, match="scale has 5 entries"):
+        rt.QuantizeLinear(x, np.ones(5, np.float32), np.zeros(5, np.uint8), axis=1)
+    assert ctypes.get_errno() in (0, errno.EINVAL)
+    with pytest.raises(rt.RuntimeError_, match="zero point"):
+        rt.QuantizeLinear(x, np.ones(6, np.float32), np.zeros(3, np.uint8), axis=1)
+    with pytest.raises(rt.RuntimeError_, match="inner dimensions differ"):
+        rt.MatMulInteger(np.zeros((4, 6), np.uint8), np.zeros((5, 3), np.int8))
+    with pytest.raises(rt.RuntimeError_, match="zero point's type"):
+        rt.MatMulInteger(np.zeros((4, 6), np.uint8), np.zeros((6, 3), np.int8),
+                         np.zeros((), np.int8), None)
+    with pytest.raises(rt.RuntimeError_, match="expected 1 or 3"):
+        rt.MatMulInteger(np.zeros((4, 6), np.uint8), np.zeros((6, 3), np.int8),
+                         None, np.zeros(2, np.int8))
+    with pytest.raises(rt.RuntimeError_, match="expected f32 x"):
+        rt.DynamicQuantizeLinear(np.zeros(4, np.int32))
+
+
+def test_incompatible_version_is_refused(rt):
+    lib = rt.load()
+    assert lib.OMInitCompatibleAccelMI355X(0x00020000) == 0   # newer major
+    assert lib.OMInitCompatibleAccelMI355X(0x00000101) == 0   # newer minor
+    rt._lib.om_mi355x_last_error()
+
+
+@pytest.mark.skipif(not _no_gpu(), reason="only meaningful on a box without a GPU")
+def test_without_a_gpu_the_ops_fail_loudly(rt):
+    lib = rt.load()
+    assert lib.OMInitCompatibleAccelMI355X(0x100) == 0    # run_main_graph would return NULL
+    with pytest.raises(rt.RuntimeError_, match="accelerator unavailable"):
+        rt.QuantizeLinear(np.ones(8, np.float32), np.float32(0.5), np.array(3, np.uint8))
+    with pytest.raises(rt.RuntimeError_, match="accelerator unavailable"):
+        rt.MatMulInteger(np.ones((2, 2), np.uint8), np.ones((2, 2), np.int8))

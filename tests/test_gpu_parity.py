@@ -1,0 +1,425 @@
+"""Parity of the HIP path with the CPU oracle, through the C-ABI.
+
+Integer, byte and index results must be bit-exact.  fp32 results are produced
+by the same sequence of correctly rounded binary32 operations as the oracle's,
+so they are compared bit-exactly too (the stated tolerance, 1e-6 relative /
+1 ulp, is therefore met with zero slack).
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+
+import oracle_lib
+from om_mi355x import workloads as wl
+
+pytestmark = pytest.mark.gpu
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+with open(os.path.join(HERE, "golden", "onnx_node_vectors.json")) as f:
+    GOLD = json.load(f)
+
+
+def bits(a):
+    return np.ascontiguousarray(a).view(np.uint32)
+
+
+def same_f32(a, b):
+    """Bit-equal, except that NaN payloads are not compared."""
+    a, b = np.asarray(a, np.float32), np.asarray(b, np.float32)
+    return a.shape == b.shape and bool(np.all((bits(a) == bits(b)) | (np.isnan(a) & np.isnan(b))))
+
+
+# --------------------------------------------------------------------------
+# golden vectors through the GPU
+# --------------------------------------------------------------------------
+def test_device_is_gfx950(rt):
+    info = rt.device_info()
+    print("device:", info, flush=True)
+    assert info["arch"].startswith("gfx950")
+    assert rt.init_compatible(0x100)
+
+
+def test_golden_vectors_on_gpu(rt):
+    g = GOLD["quantizelinear"]
+    y = rt.QuantizeLinear(np.array(g["x"], np.float32), np.float32(g["scale"]), np.array(g["zp"], np.uint8))
+    assert y.tolist() == g["y"]
+    g = GOLD["quantizelinear_axis"]
+    y = rt.QuantizeLinear(np.array(g["x"], np.float32).reshape(g["x_shape"]), np.array(g["scale"], np.float32),
+                          np.array(g["zp"], np.uint8), axis=1)
+    assert y.reshape(-1).tolist() == g["y"]
+    g = GOLD["dequantizelinear"]
+    y = rt.DequantizeLinear(np.array(g["x"], np.uint8), np.float32(g["scale"]), np.array(g["zp"], np.uint8))
+    assert y.tolist() == g["y"]
+    g = GOLD["dequantizelinear_axis"]
+    y = rt.DequantizeLinear(np.array(g["x"], np.uint8).reshape(g["x_shape"]), np.array(g["scale"], np.float32),
+                            np.array(g["zp"], np.uint8), axis=1)
+    assert y.reshape(-1).tolist() == g["y"]
+    for name in ("dynamicquantizelinear", "dynamicquantizelinear_max_adjusted",
+                 "dynamicquantizelinear_min_adjusted"):
+        g = GOLD[name]
+        y, s, z = rt.DynamicQuantizeLinear(np.array(g["x"], np.float32))
+        assert y.tolist() == g["y"] and int(z) == g["zp"] and np.float32(s) == np.float32(g["scale"])
+    g = GOLD["matmulinteger"]
+    y = rt.MatMulInteger(np.array(g["A"], np.uint8), np.array(g["B"], np.uint8),
+                         np.array(g["a_zp"], np.uint8), np.array(g["b_zp"], np.uint8))
+    assert y.tolist() == g["Y"]
+    for name, dt in (("qlinearmatmul_2D_uint8_float32", np.uint8), ("qlinearmatmul_2D_int8_float32", np.int8)):
+        g = GOLD[name]
+        for mode in (rt.WRAP, rt.SATURATE):
+            y = rt.QLinearMatMul(np.array(g["a"], dt), np.float32(g["a_scale"]), np.array(g["a_zp"], dt),
+                                 np.array(g["b"], dt), np.float32(g["b_scale"]), np.array(g["b_zp"], dt),
+                                 np.float32(g["y_scale"]), np.array(g["y_zp"], dt), mode)
+            assert y.dtype == dt and y.tolist() == g["y"]
+
+
+# --------------------------------------------------------------------------
+# QuantizeLinear / DequantizeLinear
+# --------------------------------------------------------------------------
+SPECIALS = np.array([np.nan, np.inf, -np.inf, 1e30, -1e30, 0.0, -0.0, 1e-40, -1e-40,
+                     0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 127.5, 128.5, 254.5, 255.5], np.float32)
+
+
+@pytest.mark.parametrize("n", [1, 3, 4, 5, 255, 1023, 1024, 4097, 1 << 20, (1 << 20) + 3])
+@pytest.mark.parametrize("qdt", [np.uint8, np.int8])
+def test_quantize_per_tensor(rt, oracle, n, qdt):
+    rng = np.random.default_rng(n)
+    x = rng.normal(0, 2, n).astype(np.float32)
+    x[: min(n, SPECIALS.size)] = SPECIALS[: min(n, SPECIALS.size)]
+    if n > 4000:                       # exact ties: x/s lands on k + 0.5
+        x[100:1100] = (np.arange(1000, dtype=np.float32) - 500 + 0.5) * np.float32(0.25)
+    for s, zp in [(0.02, 128 if qdt == np.uint8 else -3), (0.25, 0), (1e-38, 7)]:
+        zpa = np.array(zp, qdt)
+        want = oracle.quantize_linear(x, np.float32(s), zpa)
+        got = rt.QuantizeLinear(x, np.float32(s), zpa)
+        assert got.dtype == qdt and np.array_equal(got, want), (n, s, zp)
+    if qdt == np.uint8:
+        assert np.array_equal(rt.QuantizeLinear(x, np.float32(0.02), None),
+                              oracle.quantize_linear(x, np.float32(0.02), None))
+
+
+def test_quantize_zero_and_denormal_scale(rt, oracle):
+    x = np.array([0.0, -0.0, 1.0, -1.0, np.nan, 3e-45, -3e-45], np.float32)
+    for s in (0.0, 1e-45, 1e-39):
+        want = oracle.quantize_linear(x, np.float32(s), np.array(9, np.uint8))
+        assert np.array_equal(rt.QuantizeLinear(x, np.float32(s), np.array(9, np.uint8)), want), s
+
+
+@pytest.mark.parametrize("shape,axis", [((64, 1000), 1), ((37, 1023), 1), ((5, 7), 1), ((129, 4096), -1),
+                                        ((3, 5, 64, 33), 1), ((6, 100), 0), ((2, 3, 4, 5), 2),
+                                        ((1, 3, 3, 2), 1), ((300, 2), 1)])
+@pytest.mark.parametrize("qdt", [np.uint8, np.int8])
+def test_quantize_dequantize_per_axis(rt, oracle, shape, axis, qdt):
+    # per-axis: the oracle applies the reference's per-tensor formula per channel
+    # (parity unpinned by the reference itself, which asserts on per-axis)
+    rng = np.random.default_rng(abs(hash((shape, axis))) % 2**32)
+    x = rng.normal(0, 2, shape).astype(np.float32)
+    C = shape[axis]
+    sc = rng.uniform(0.005, 0.05, C).astype(np.float32)
+    info = np.iinfo(qdt)
+    zp = rng.integers(info.min, info.max + 1, C).astype(qdt)
+    want = oracle.quantize_linear(x, sc, zp, axis=axis)
+    got = rt.QuantizeLinear(x, sc, zp, axis=axis)
+    assert np.array_equal(got, want)
+    got_nozp = rt.QuantizeLinear(x, sc, None, axis=axis)
+    assert np.array_equal(got_nozp, oracle.quantize_linear(x, sc, None, axis=axis))
+    wd = oracle.dequantize_linear(want, sc, zp, axis=axis)
+    gd = rt.DequantizeLinear(want, sc, zp, axis=axis)
+    assert same_f32(gd, wd)
+    assert same_f32(rt.DequantizeLinear(want, sc, None, axis=axis),
+                    oracle.dequantize_linear(want, sc, None, axis=axis))
+
+
+@pytest.mark.parametrize("n", [1, 2, 3, 4, 7, 1024, 4099, (1 << 20) + 1])
+@pytest.mark.parametrize("xdt", [np.uint8, np.int8, np.int32])
+def test_dequantize_per_tensor(rt, oracle, n, xdt):
+    rng = np.random.default_rng(n + 17)
+    info = np.iinfo(xdt)
+    x = rng.integers(info.min, info.max, n, dtype=np.int64).astype(xdt)
+    zp = np.array(info.max // 2 - 3, xdt)
+    s = np.float32(0.0371)
+    assert same_f32(rt.DequantizeLinear(x, s, zp), oracle.dequantize_linear(x, s, zp))
+    assert same_f32(rt.DequantizeLinear(x, s, None), oracle.dequantize_linear(x, s, None))
+
+
+def test_dequantize_int32_per_column(rt, oracle):
+    rng = np.random.default_rng(23)
+    acc = rng.integers(-2**31, 2**31 - 1, (70, 1027), dtype=np.int64).astype(np.int32)
+    sc = rng.uniform(1e-5, 1e-3, 1027).astype(np.float32)
+    zp = rng.integers(-1000, 1000, 1027).astype(np.int32)
+    assert same_f32(rt.DequantizeLinear(acc, sc, zp, axis=1), oracle.dequantize_linear(acc, sc, zp, axis=1))
+
+
+def test_misaligned_device_views_are_handled(rt, oracle):
+    # tensors that start 4 bytes (x) / 1 byte (y) into a GPU allocation: the
+    # 16-byte and 4-byte alignment the fast kernels rely on is lost
+    rng = np.random.default_rng(31)
+    x = rng.normal(0, 2, 5001).astype(np.float32)
+    s, zp = np.float32(0.03), np.array(100, np.uint8)
+    dx = rt.DeviceArray.from_numpy(x)
+    dy = rt.DeviceArray((6000,), np.uint8)
+    xv = rt.DeviceArray.view_of(dx, 1, (5000,))
+    yv = rt.DeviceArray.view_of(dy, 1, (5000,))
+    rt.QuantizeLinear(xv, s, zp, out=yv)
+    want = oracle.quantize_linear(x[1:], s, zp)
+    assert np.array_equal(yv.numpy(), want)
+    dd = rt.DeviceArray((5004,), np.float32)
+    dv = rt.DeviceArray.view_of(dd, 1, (5000,))
+    rt.DequantizeLinear(yv, s, zp, out=dv)
+    assert same_f32(dv.numpy(), oracle.dequantize_linear(want, s, zp))
+    gy, gs, gz = rt.DynamicQuantizeLinear(xv)
+    wy, ws, wz = oracle.dynamic_quantize_linear(x[1:])
+    assert np.array_equal(gy.numpy(), wy) and gs.numpy().reshape(()) == ws
+    # matmul with A starting at an odd address and K not a multiple of 16
+    A = rng.integers(0, 256, 40 * 50 + 1).astype(np.uint8)
+    B = rng.integers(-128, 128, (50, 30)).astype(np.int8)
+    dA = rt.DeviceArray.from_numpy(A)
+    Av = rt.DeviceArray.view_of(dA, 1, (40, 50))
+    got = rt.MatMulInteger(Av, rt.DeviceArray.from_numpy(B), None, None)
+    assert np.array_equal(got.numpy(), oracle.matmul_integer(A[1:].reshape(40, 50), B))
+
+
+# --------------------------------------------------------------------------
+# DynamicQuantizeLinear
+# --------------------------------------------------------------------------
+@pytest.mark.parametrize("shape", [(1,), (6,), (3, 4), (1023,), (128, 768), (257, 1031), (4096, 768)])
+def test_dynamic_quantize(rt, oracle, shape):
+    rng = np.random.default_rng(int(np.prod(shape)))
+    x = rng.normal(0, 1, shape).astype(np.float32)
+    wy, ws, wz = oracle.dynamic_quantize_linear(x)
+    gy, gs, gz = rt.DynamicQuantizeLinear(x)
+    assert np.float32(gs).view(np.uint32) == np.float32(ws).view(np.uint32)
+    assert int(gz) == int(wz)
+    assert np.array_equal(gy, wy)
+
+
+def test_dynamic_quantize_edge_inputs(rt, oracle):
+    cases = [np.zeros(100, np.float32),                         # scale 0 -> NaN paths -> all 0
+             np.full(77, 3.25, np.float32),                     # all positive: min widened to 0
+             np.full(77, -3.25, np.float32),                    # all negative: zp 255
+             np.array([np.nan, 1.0, -2.0, np.nan, 0.5], np.float32),   # NaN ignored by min/max, NaN -> 0
+             np.array([1e-42, -1e-43, 0.0], np.float32),        # denormals kept
+             np.array([3e38, -3e38], np.float32)]               # max - min overflows to inf
+    for x in cases:
+        wy, ws, wz = oracle.dynamic_quantize_linear(x)
+        gy, gs, gz = rt.DynamicQuantizeLinear(x)
+        assert same_f32(np.float32(gs), np.float32(ws)), x[:4]
+        assert int(gz) == int(wz) and np.array_equal(gy, wy), x[:4]
+
+
+def test_dynamic_quantize_invariants_large(rt):
+    # properties that hold at any size: zp in range, the extremes map to 0 / 255
+    x = wl.normal_f32(2, 0, (2048, 4099), 2.0)
+    y, s, z = rt.DynamicQuantizeLinear(x)
+    assert 0 <= int(z) <= 255
+    assert y[np.unravel_index(np.argmin(x), x.shape)] == 0
+    assert y[np.unravel_index(np.argmax(x), x.shape)] == 255
+    assert np.float32(s) == (np.float32(x.max()) - np.float32(x.min())) / np.float32(255)
+
+
+# --------------------------------------------------------------------------
+# MatMulInteger
+# --------------------------------------------------------------------------
+def _rand_q(rng, dt, shape):
+    info = np.iinfo(dt)
+    return rng.integers(info.min, info.max + 1, shape).astype(dt)
+
+
+@pytest.mark.parametrize("adt,bdt", [(np.uint8, np.int8), (np.int8, np.uint8), (np.uint8, np.uint8), (np.int8, np.int8)])
+def test_matmulinteger_small_exhaustive_shapes(rt, oracle, adt, bdt):
+    rng = np.random.default_rng(41)
+    for M in (1, 2, 3, 5, 8):
+        for K in (1, 2, 7, 16, 33):
+            for N in (1, 3, 8):
+                A, B = _rand_q(rng, adt, (M, K)), _rand_q(rng, bdt, (K, N))
+                for az, bz in ((None, None), (_rand_q(rng, adt, ()), _rand_q(rng, bdt, ())),
+                               (_rand_q(rng, adt, (M,)), _rand_q(rng, bdt, (N,)))):
+                    want = oracle.matmul_integer(A, B, az, bz)
+                    got = rt.MatMulInteger(A, B, az, bz)
+                    assert np.array_equal(got, want), (M, K, N, adt, bdt)
+
+
+@pytest.mark.parametrize("M,K,N", [(128, 768, 768), (130, 200, 260), (257, 1000, 129), (64, 4096, 192),
+                                   (1, 4096, 1000), (4, 640, 11008), (16, 333, 77), (500, 48, 500)])
+def test_matmulinteger_shapes(rt, oracle, M, K, N):
+    rng = np.random.default_rng(M * 7 + K * 3 + N)
+    A, B = _rand_q(rng, np.uint8, (M, K)), _rand_q(rng, np.int8, (K, N))
+    az = _rand_q(rng, np.uint8, ())
+    want = oracle.matmul_integer(A, B, az, None)
+    assert np.array_equal(rt.MatMulInteger(A, B, az, None), want)
+    azr, bzc = _rand_q(rng, np.uint8, (M,)), _rand_q(rng, np.int8, (N,))
+    want = oracle.matmul_integer(A, B, azr, bzc)
+    assert np.array_equal(rt.MatMulInteger(A, B, azr, bzc), want)
+
+
+def test_matmulinteger_extreme_values_wrap(rt, oracle):
+    # all-255 x all-(-128) with large K: the int32 accumulator must wrap, not saturate
+    M, K, N = 64, 70000, 64
+    A = np.full((M, K), 255, np.uint8)
+    B = np.full((K, N), -128, np.int8)
+    az = np.array(0, np.uint8)
+    want = oracle.matmul_integer(A, B, az, None)
+    assert want[0, 0] == np.int32((255 * -128 * K + 2**31) % 2**32 - 2**31)
+    assert np.array_equal(rt.MatMulInteger(A, B, az, None), want)
+
+
+def test_matmulinteger_zero_point_identity(rt):
+    # Y(A, B, az, bz) == Y(A - az, B - bz, 0, 0) whenever the differences fit in int8
+    rng = np.random.default_rng(43)
+    A = rng.integers(-50, 50, (100, 300)).astype(np.int8)
+    B = rng.integers(-50, 50, (300, 140)).astype(np.int8)
+    az, bz = np.array(20, np.int8), rng.integers(-30, 30, 140).astype(np.int8)
+    y1 = rt.MatMulInteger(A, B, az, bz)
+    y2 = rt.MatMulInteger((A - 20).astype(np.int8), (B - bz[None, :]).astype(np.int8), None, None)
+    assert np.array_equal(y1, y2)
+
+
+def test_matmulinteger_batched_a(rt, oracle):
+    rng = np.random.default_rng(44)
+    A, B = _rand_q(rng, np.uint8, (3, 5, 64)), _rand_q(rng, np.int8, (64, 24))
+    az = _rand_q(rng, np.uint8, ())
+    got = rt.MatMulInteger(A, B, az, None)
+    assert got.shape == (3, 5, 24) and np.array_equal(got, oracle.matmul_integer(A, B, az, None))
+
+
+def test_constant_weights_are_packed_once_and_stay_correct(rt, oracle):
+    rng = np.random.default_rng(45)
+    B = _rand_q(rng, np.int8, (256, 384))
+    rt.mark_constant(B)
+    try:
+        for seed in range(3):
+            A = _rand_q(np.random.default_rng(seed), np.uint8, (100, 256))
+            az = np.array(seed * 40, np.uint8)
+            assert np.array_equal(rt.MatMulInteger(A, B, az, None), oracle.matmul_integer(A, B, az, None))
+    finally:
+        rt.clear_cache()
+
+
+# --------------------------------------------------------------------------
+# QLinearMatMul and the fused layers at the benchmark configurations
+# --------------------------------------------------------------------------
+@pytest.mark.parametrize("mode", ["wrap", "saturate"])
+def test_config3_qlinearmatmul(rt, oracle, mode):
+    c = wl.config3()
+    m_rt, m_or = (rt.WRAP, oracle_lib.WRAP) if mode == "wrap" else (rt.SATURATE, oracle_lib.SATURATE)
+    want = oracle.qlinear_matmul(c["A"], c["a_scale"], c["a_zp"], c["B"], c["b_scale"], c["b_zp"],
+                                 c["y_scale"], c["y_zp"], m_or)
+    got = rt.QLinearMatMul(c["A"], c["a_scale"], c["a_zp"], c["B"], c["b_scale"], c["b_zp"],
+                           c["y_scale"], c["y_zp"], m_rt)
+    assert got.dtype == np.uint8 and np.array_equal(got, want)
+
+
+def test_qlinearmatmul_int8_and_per_row_column_zero_points(rt, oracle):
+    rng = np.random.default_rng(51)
+    a, b = _rand_q(rng, np.int8, (70, 130)), _rand_q(rng, np.int8, (130, 90))
+    az, bz = _rand_q(rng, np.int8, (70,)), _rand_q(rng, np.int8, (90,))
+    for mode_rt, mode_or in ((rt.WRAP, oracle_lib.WRAP), (rt.SATURATE, oracle_lib.SATURATE)):
+        want = oracle.qlinear_matmul(a, 0.02, az, b, 0.01, bz, 0.3, np.array(-7, np.int8), mode_or)
+        got = rt.QLinearMatMul(a, np.float32(0.02), az, b, np.float32(0.01), bz, np.float32(0.3),
+                               np.array(-7, np.int8), mode_rt)
+        assert got.dtype == np.int8 and np.array_equal(got, want)
+
+
+def test_config1_graph_separate_ops_and_fused(rt, oracle):
+    c = wl.config1()
+    aq, a_s, a_zp = oracle.dynamic_quantize_linear(c["A"])
+    acc = oracle.matmul_integer(aq, c["B"], a_zp, c["b_zp"])
+    want = oracle.dequant_epilogue(acc, a_s, c["b_scale"])
+    # the graph as the reference compiles it: three ops, host tensors between them
+    gq, gs, gz = rt.DynamicQuantizeLinear(c["A"])
+    assert np.array_equal(gq, aq) and np.float32(gs) == a_s and int(gz) == int(a_zp)
+    gacc = rt.MatMulInteger(gq, c["B"], gz, c["b_zp"])
+    assert np.array_equal(gacc, acc)
+    assert same_f32(rt.MatMulIntegerDequant(gq, c["B"], gz, c["b_zp"], gs, c["b_scale"]), want)
+    # the fused layer
+    assert same_f32(rt.DynQuantMatMulDequant(c["A"], c["B"], c["b_zp"], c["b_scale"]), want)
+    assert same_f32(rt.DynQuantMatMulDequant(c["A"], c["B"], None, c["b_scale"]), want)
+
+
+@pytest.mark.parametrize("name", list(wl.CONFIG4_SHAPES))
+def test_config4_layers_reduced_m(rt, oracle, name):
+    c = wl.config4(name, M=384)
+    aq, a_s, a_zp = oracle.dynamic_quantize_linear(c["X"])
+    acc = oracle.matmul_integer(aq, c["W"], a_zp, None)
+    want = oracle.dequant_epilogue(acc, a_s, c["w_scale"])
+    assert same_f32(rt.DynQuantMatMulDequant(c["X"], c["W"], None, c["w_scale"]), want)
+
+
+@pytest.mark.parametrize("M", [1, 4, 16])
+def test_config5_decode_shapes(rt, oracle, M):
+    c = wl.config5("up", M=M)
+    aq, a_s, a_zp = oracle.dynamic_quantize_linear(c["X"])
+    acc = oracle.matmul_integer(aq, c["W"], a_zp, None)
+    want = oracle.dequant_epilogue(acc, a_s, c["w_scale"])
+    assert same_f32(rt.DynQuantMatMulDequant(c["X"], c["W"], None, c["w_scale"]), want)
+
+
+def test_fused_layer_with_unsigned_weights_and_zero_points(rt, oracle):
+    rng = np.random.default_rng(61)
+    x = rng.normal(0, 1, (200, 320)).astype(np.float32)
+    W = _rand_q(rng, np.uint8, (320, 150))
+    wz = _rand_q(rng, np.uint8, (150,))
+    ws = rng.uniform(1e-3, 1e-2, 150).astype(np.float32)
+    aq, a_s, a_zp = oracle.dynamic_quantize_linear(x)
+    want = oracle.dequant_epilogue(oracle.matmul_integer(aq, W, a_zp, wz), a_s, ws)
+    assert same_f32(rt.DynQuantMatMulDequant(x, W, wz, ws), want)
+
+
+# --------------------------------------------------------------------------
+# device-resident operands: used in place, results stay on the GPU
+# --------------------------------------------------------------------------
+def test_device_resident_chain(rt, oracle):
+    c = wl.config4("out", M=512)
+    dX = rt.DeviceArray.from_numpy(c["X"])
+    dW = rt.DeviceArray.from_numpy(c["W"])
+    dS = rt.DeviceArray.from_numpy(c["w_scale"])
+    rt.mark_constant(dW)
+    try:
+        dq, ds, dz = rt.DynamicQuantizeLinear(dX)
+        assert isinstance(dq, rt.DeviceArray)
+        dacc = rt.MatMulInteger(dq, dW, dz, None)
+        dout = rt.MatMulIntegerDequant(dq, dW, dz, None, ds, dS)
+        dfused = rt.DynQuantMatMulDequant(dX, dW, None, dS)
+        rt.synchronize()
+        aq, a_s, a_zp = oracle.dynamic_quantize_linear(c["X"])
+        acc = oracle.matmul_integer(aq, c["W"], a_zp, None)
+        want = oracle.dequant_epilogue(acc, a_s, c["w_scale"])
+        assert np.array_equal(dq.numpy(), aq)
+        assert np.array_equal(dacc.numpy(), acc)
+        assert same_f32(dout.numpy(), want) and same_f32(dfused.numpy(), want)
+    finally:
+        rt.clear_cache()
+
+
+# --------------------------------------------------------------------------
+# full benchmark sizes: size-independent properties + sampled oracle rows
+# --------------------------------------------------------------------------
+@pytest.mark.parametrize("rows,cols", [(8192, 32768), (8191, 32767)])
+def test_config2_full_size(rt, oracle, rows, cols):
+    c = wl.config2(rows, cols)
+    dX = rt.DeviceArray.from_numpy(c["X"])
+    dS = rt.DeviceArray.from_numpy(c["scale"])
+    dZ = rt.DeviceArray.from_numpy(c["zp"])
+    dQ = rt.QuantizeLinear(dX, dS, dZ, axis=1)
+    dD = rt.DequantizeLinear(dQ, dS, dZ, axis=1)
+    dQ2 = rt.QuantizeLinear(dD, dS, dZ, axis=1)        # Q(DQ(q)) == q on the 8-bit lattice
+    q = dQ.numpy()
+    assert np.array_equal(q, dQ2.numpy())
+    sample = np.r_[0:8, rows // 2:rows // 2 + 8, rows - 8:rows]
+    want = oracle.quantize_linear(c["X"][sample], c["scale"], c["zp"], axis=1)
+    assert np.array_equal(q[sample], want)
+    d = dD.numpy()
+    assert same_f32(d[sample], oracle.dequantize_linear(want, c["scale"], c["zp"], axis=1))
+    del d, dD, dQ2
+    # dynamic quantisation of the same tensor: parameters from numpy's min / max
+    dY, ds, dz = rt.DynamicQuantizeLinear(dX)
+    mn, mx = np.float32(min(c["X"].min(), 0)), np.float32(max(c["X"].max(), 0))
+    s, zf, z = oracle.dynamic_params(float(c["X"].min()), float(c["X"].max()))
+    assert ds.numpy().reshape(()) == s and int(dz.numpy().reshape(())) == int(z)
+    y = dY.numpy()
+    assert np.array_equal(y[sample], oracle.quantize_linear(c["X"][sample], s, np.array(z, np.uint8)))
+    # per-tensor quantize / dequantize at full size against the oracle's OpenMP twin
+    dQt = rt.QuantizeLinear(dX, np.float32(0.02), np.array(128, np.uint8))
+    wq = oracle.quantize_linear(c["X"], np.float32(0.02), np.array(128, np.uint8), omp=True)
+    assert np.array_equal(dQt.numpy(), wq)
