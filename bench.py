@@ -59,11 +59,13 @@ def gemm_case(rt, wl, name, M, K, N, w_i8, w_scale, steps, warmup, epilogue="f32
     rt.mark_constant(dW)             # weights: packed once, like any model constant
     if epilogue == "f32":
         dY = rt.DeviceArray((M, N), np.float32)
-        fn = lambda: rt.MatMulIntegerDequant(dA, dW, dAz, None, dAs, dS, out=dY)
+        fn = rt.PreparedCall("om_mi355x_MatMulIntegerDequant", dY, dA, dW, dAz, None, dAs, dS)
     else:
         dY = rt.DeviceArray((M, N), np.int32)
-        fn = lambda: rt.MatMulInteger(dA, dW, dAz, None, out=dY)
+        fn = rt.PreparedCall("om_mi355x_MatMulInteger", dY, dA, dW, dAz, None)
     host_s, ev_ms = timed(rt, fn, steps, warmup)
+    fn.check()
+    fn.close()
     ops = 2.0 * M * N * K
     res = {"name": name, "M": M, "K": K, "N": N, "epilogue": epilogue,
            "ms_per_step": host_s * 1e3, "kernel_ms": ev_ms,
@@ -82,8 +84,10 @@ def decode_case(rt, wl, M, steps, warmup):
     dS = rt.DeviceArray.from_numpy(c["w_scale"])
     dY = rt.DeviceArray((M, N), np.float32)
     rt.mark_constant(dW)
-    fn = lambda: rt.DynQuantMatMulDequant(dX, dW, None, dS, out=dY)
+    fn = rt.PreparedCall("om_mi355x_DynQuantMatMulDequant", dY, dX, dW, None, dS)
     host_s, ev_ms = timed(rt, fn, steps, warmup)
+    fn.check()
+    fn.close()
     nbytes = K * N + M * K + 4 * M * N
     res = {"name": f"config5 decode M={M}", "M": M, "K": K, "N": N, "ms_per_step": host_s * 1e3,
            "kernel_ms": ev_ms, "gbs": nbytes / (ev_ms * 1e-3) / 1e9, "bytes": nbytes,
@@ -109,17 +113,20 @@ def qdq_cases(rt, wl, rows, cols, steps, warmup):
 
     def run(name, fn, nbytes):
         host_s, ev_ms = timed(rt, fn, steps, warmup)
+        fn.check()
+        fn.close()
         out[name] = {"ms_per_step": host_s * 1e3, "kernel_ms": ev_ms, "bytes": nbytes,
                      "gbs": nbytes / (ev_ms * 1e-3) / 1e9,
                      "hbm_frac": nbytes / (ev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
 
-    run("quantize_per_axis", lambda: rt.QuantizeLinear(dX, dS, dZ, axis=1, out=dQ), 5 * n)
-    run("dequantize_per_axis", lambda: rt.DequantizeLinear(dQ, dS, dZ, axis=1, out=dD), 5 * n)
-    run("quantize_per_tensor", lambda: rt.QuantizeLinear(dX, s1, z1, out=dQ), 5 * n)
-    run("dequantize_per_tensor", lambda: rt.DequantizeLinear(dQ, s1, z1, out=dD), 5 * n)
+    P = rt.PreparedCall
+    run("quantize_per_axis", P("om_mi355x_QuantizeLinear", dQ, dX, dS, dZ, 1, 1), 5 * n)
+    run("dequantize_per_axis", P("om_mi355x_DequantizeLinear", dD, dQ, dS, dZ, 1), 5 * n)
+    run("quantize_per_tensor", P("om_mi355x_QuantizeLinear", dQ, dX, s1, z1, 1, 1), 5 * n)
+    run("dequantize_per_tensor", P("om_mi355x_DequantizeLinear", dD, dQ, s1, z1, 1), 5 * n)
     # two reads of X (min/max, then quantize) + one write: the tensor is far
     # larger than any on-chip cache
-    run("dynamic_quantize", lambda: rt.DynamicQuantizeLinear(dX, out=(dQ, dys, dyz)), 9 * n)
+    run("dynamic_quantize", P("om_mi355x_DynamicQuantizeLinear", dQ, dys, dyz, dX), 9 * n)
     for d in (dX, dS, dZ, dQ, dD, dys, dyz, s1, z1):
         d.free()
     return out
@@ -160,6 +167,7 @@ def main():
     ap.add_argument("--workload", default="config4_ffn_up",
                     choices=["config4_ffn_up", "config4_ffn_up_i32"])
     ap.add_argument("--no-extras", action="store_true", help="skip the Q/DQ and other-shape measurements")
+    ap.add_argument("--extras", default="gemm,decode,qdq", help="which extra groups to measure")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -179,7 +187,8 @@ def main():
                          args.steps, args.warmup, epi)
 
     extras = {}
-    if not args.no_extras:
+    groups = set() if args.no_extras else set(args.extras.split(","))
+    if "gemm" in groups:
         gemms = []
         for name, (k, n) in wl.CONFIG4_SHAPES.items():
             cc = wl.config4(name, M=8)
@@ -192,7 +201,9 @@ def main():
             gemms.append(gemm_case(rt, wl, f"config5 prefill {name}", 2048, k, n, cc["W"], cc["w_scale"],
                                    max(10, args.steps // 10), max(2, args.warmup // 10), "f32"))
         extras["gemm"] = gemms
+    if "decode" in groups:
         extras["decode"] = [decode_case(rt, wl, m, args.steps, args.warmup) for m in (1, 4, 16)]
+    if "qdq" in groups:
         qsteps = max(5, args.steps // 10)
         extras["qdq_8192x32768"] = qdq_cases(rt, wl, 8192, 32768, qsteps, max(2, args.warmup // 10))
         extras["qdq_8191x32767"] = qdq_cases(rt, wl, 8191, 32767, qsteps, max(2, args.warmup // 10))

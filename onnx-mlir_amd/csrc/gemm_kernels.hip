@@ -15,11 +15,19 @@
 //
 // Layout: A is used as given ([M,K] row-major, K contiguous).  B is packed
 // once into Bt [Npad,Kpad] int8 (K contiguous, zero filled), so both MFMA
-// operands are read as 16 consecutive K bytes per lane.  Tiles go through LDS
-// with an XOR swizzle of the 16-byte chunk index so that ds_read_b128 and
-// ds_write_b128 are bank-conflict free.
+// operands are read as 16 consecutive K bytes per lane.
+//
+// Pipeline: a block owns a BM x BN tile of Y and walks K in steps of 64 bytes.
+// Global loads run two steps ahead of the MFMAs in registers (two register
+// sets), LDS is double buffered, and the block barrier only orders LDS traffic
+// so the global loads stay in flight across it.  LDS rows are 64 bytes; the
+// 16-byte chunk index is XOR-swizzled with bits 2..3 of the row so that both
+// ds_write_b128 (staging) and ds_read_b128 (MFMA operands) are bank-conflict
+// free.
 
 #include "om_kernels.h"
+
+#include <stdlib.h>
 
 namespace om {
 
@@ -28,13 +36,19 @@ namespace {
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 
-constexpr int BM = 128, BN = kGemmBN, BK = kGemmBK;
-constexpr int kGemmThreads = 256;
+constexpr int BK = kGemmBK;
 
 // Byte offset of 16-byte chunk `c` (0..3) of tile row `r` (row = 64 bytes).
-// Rows r, r+4, r+8, r+12 share a bank group; XOR with (r>>2)&3 spreads them.
 __device__ __forceinline__ int lds_off(int r, int c) {
   return r * BK + ((c ^ ((r >> 2) & 3)) << 4);
+}
+
+// Barrier that orders LDS accesses only; global loads already issued keep
+// flying across it.
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
 struct EpiParams {
@@ -61,182 +75,277 @@ __device__ __forceinline__ int32_t load_zp_i32(
                      : (int32_t)((const int8_t *)p)[i];
 }
 
+// BM x BN block tile, WGM x WGN waves, each wave a (BM/WGM) x (BN/WGN) tile
+// made of 32x32 MFMA tiles.
 // A_MODE: 0 = int8 as is, 1 = uint8 (XOR 0x80 while staging), 2 = already
 // shifted (stored as u8-128) -- offsets as for uint8, no XOR.
-// ALIGNED: K % 16 == 0 and A 16-byte aligned (vector loads), else byte loads.
-template <int A_MODE, int EPI, bool ALIGNED>
-__global__ __launch_bounds__(kGemmThreads) void k_gemm_i8(
+// ALIGNED: K % 64 == 0 and A 16-byte aligned (vector loads), else byte loads.
+template <int BM, int BN, int WGM, int WGN, int MINB, int A_MODE, int EPI,
+    bool ALIGNED>
+__global__ __launch_bounds__(WGM *WGN * 64, MINB) void k_gemm_i8(
     const uint8_t *__restrict__ A, const int8_t *__restrict__ Bt, int M, int N,
     int K, int Kpad, EpiParams ep, int tiles_m, int tiles_n) {
-  const bool B_UNSIGNED = ep.b_unsigned;
-  const bool Y_UNSIGNED = ep.y_unsigned;
-  const int NARROW = ep.narrow;
+  constexpr int THREADS = WGM * WGN * 64;
+  constexpr int WTM = BM / WGM, WTN = BN / WGN; // wave tile
+  constexpr int TM = WTM / 32, TN = WTN / 32;   // MFMA tiles per wave
+  constexpr int CH_A = BM * 4 / THREADS;        // 16-byte chunks per thread
+  constexpr int CH_B = BN * 4 / THREADS;
+  static_assert(BM * 4 % THREADS == 0 && BN * 4 % THREADS == 0, "tile/threads");
+
   __shared__ __attribute__((aligned(16))) uint8_t sA[2][BM * BK];
   __shared__ __attribute__((aligned(16))) uint8_t sB[2][BN * BK];
 
-  // Tile order: consecutive blocks walk down M inside a band of N, so the
-  // blocks resident at one time share a few Bt tiles and the A panel.
-  const int pid = blockIdx.x;
-  const int tm = pid % tiles_m;
-  const int tn = pid / tiles_m;
+  // Tile order.  Consecutive workgroup ids are dealt round-robin to the 8
+  // XCDs, each with its own L2; renumber so that one XCD gets a contiguous
+  // range, then walk that range in groups of 8 tile rows so the tiles resident
+  // on an XCD share a few A panels and Bt panels.
+  int pid = blockIdx.x;
+  {
+    const int nb = gridDim.x;
+    const int per = nb >> 3;
+    if (per > 0 && pid < per * 8)
+      pid = (pid & 7) * per + (pid >> 3);
+  }
+  constexpr int GROUP = 8;
+  const int in_group = GROUP * tiles_n;
+  const int group = pid / in_group;
+  const int first_m = group * GROUP;
+  const int gsize = (tiles_m - first_m < GROUP) ? tiles_m - first_m : GROUP;
+  const int tm = first_m + (pid % in_group) % gsize;
+  const int tn = (pid % in_group) / gsize;
   const int m0 = tm * BM, n0 = tn * BN;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1; // 2 x 2 waves, 64 x 64 each
+  const int wm = wave / WGN, wn = wave % WGN;
 
-  // Staging map: thread -> (row, 16-byte chunk) twice per operand.
-  const int lc = tid & 3;
-  const int lr = tid >> 2; // 0..63
+  constexpr int kFill = (A_MODE == 1) ? (int)0x80808080 : 0;
 
-  v4i ra[2], rb[2];
-
-  auto load_global = [&](int k0) {
+  // Global loads only fetch; uint8 data is shifted to int8 after it is read
+  // back from LDS.  In the byte-wise path chunks outside [M,K] are filled with
+  // the byte that the shift maps to 0.
+  auto load_global = [&](int k0, v4i(&ra)[CH_A], v4i(&rb)[CH_B]) {
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const int r = lr + h * 64;
+    for (int h = 0; h < CH_A; ++h) {
+      const int q = tid + h * THREADS;
+      const int r = q >> 2, c = q & 3;
       const int gm = m0 + r;
-      const int gk = k0 + lc * 16;
-      v4i v = {0, 0, 0, 0};
+      const int gk = k0 + c * 16;
+      v4i v = {kFill, kFill, kFill, kFill};
       if (ALIGNED) {
-        // K % 16 == 0: a chunk is either wholly inside the row or absent.
-        // Absent chunks and rows >= M stay 0 in the int8 domain.
-        if (gm < M && gk < K) {
-          v = *(const v4i *)(A + (int64_t)gm * K + gk);
-          if (A_MODE == 1)
-            v ^= (v4i){(int)0x80808080, (int)0x80808080, (int)0x80808080,
-                (int)0x80808080};
-        }
+        // K % 64 == 0, so every chunk lies inside its row.  Rows past M are
+        // clamped to the last row: they only feed output rows that are never
+        // stored, and an unconditional load lets the hardware counter of
+        // outstanding loads be waited on exactly (a load under a branch
+        // would force a full drain).
+        const int gmc = gm < M ? gm : M - 1;
+        v = *(const v4i *)(A + (int64_t)gmc * K + gk);
       } else {
         uint32_t w[4] = {0, 0, 0, 0};
-        if (gm < M) {
 #pragma unroll
-          for (int b = 0; b < 16; ++b) {
-            const int kk = gk + b;
-            uint32_t byte = 0;
-            if (kk < K) {
-              byte = A[(int64_t)gm * K + kk];
-              if (A_MODE == 1)
-                byte ^= 0x80u;
-            }
-            w[b >> 2] |= byte << ((b & 3) * 8);
-          }
+        for (int b = 0; b < 16; ++b) {
+          const int kk = gk + b;
+          uint32_t byte = (uint32_t)kFill & 0xFFu;
+          if (gm < M && kk < K)
+            byte = A[(int64_t)gm * K + kk];
+          w[b >> 2] |= byte << ((b & 3) * 8);
         }
         v = (v4i){(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
       }
       ra[h] = v;
+    }
+#pragma unroll
+    for (int h = 0; h < CH_B; ++h) {
+      const int q = tid + h * THREADS;
+      const int r = q >> 2, c = q & 3;
       // Bt is padded to [Npad, Kpad]: always in bounds and aligned.
-      rb[h] = *(const v4i *)(Bt + (int64_t)(n0 + r) * Kpad + gk);
+      rb[h] = *(const v4i *)(Bt + (int64_t)(n0 + r) * Kpad + k0 + c * 16);
     }
   };
-  auto store_lds = [&](int buf) {
+  auto store_lds = [&](int buf, const v4i(&ra)[CH_A], const v4i(&rb)[CH_B]) {
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const int r = lr + h * 64;
-      *(v4i *)(&sA[buf][lds_off(r, lc)]) = ra[h];
-      *(v4i *)(&sB[buf][lds_off(r, lc)]) = rb[h];
+    for (int h = 0; h < CH_A; ++h) {
+      const int q = tid + h * THREADS;
+      *(v4i *)(&sA[buf][lds_off(q >> 2, q & 3)]) = ra[h];
+    }
+#pragma unroll
+    for (int h = 0; h < CH_B; ++h) {
+      const int q = tid + h * THREADS;
+      *(v4i *)(&sB[buf][lds_off(q >> 2, q & 3)]) = rb[h];
     }
   };
 
-  v16i acc[2][2];
+  v16i acc[TM][TN];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r)
         acc[i][j][r] = 0;
 
-  const int kt_total = Kpad / BK;
-  load_global(0);
-  store_lds(0);
-  __syncthreads();
-
   const int l32 = lane & 31;
   const int lh = lane >> 5;
 
-  for (int kt = 0; kt < kt_total; ++kt) {
-    const int buf = kt & 1;
-    if (kt + 1 < kt_total)
-      load_global((kt + 1) * BK);
+  auto compute = [&](int buf) {
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
       const int c = s * 2 + lh;
-      v4i fa[2], fb[2];
+      v4i fa[TM], fb[TN];
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
-        fa[i] = *(const v4i *)(&sA[buf][lds_off(wm * 64 + i * 32 + l32, c)]);
+      for (int i = 0; i < TM; ++i) {
+        fa[i] = *(const v4i *)(&sA[buf][lds_off(wm * WTM + i * 32 + l32, c)]);
+        // uint8 -> int8 (minus 128) on the operand registers: VALU work that
+        // runs beside the MFMAs and keeps the staging path free of any use
+        // of freshly loaded data.
+        if (A_MODE == 1)
+          fa[i] ^= (v4i){(int)0x80808080, (int)0x80808080, (int)0x80808080,
+              (int)0x80808080};
+      }
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
-        fb[j] = *(const v4i *)(&sB[buf][lds_off(wn * 64 + j * 32 + l32, c)]);
+      for (int j = 0; j < TN; ++j)
+        fb[j] = *(const v4i *)(&sB[buf][lds_off(wn * WTN + j * 32 + l32, c)]);
+#if defined(OM_EXP) && (OM_EXP & 2)
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < TN; ++j)
+          acc[i][j][0] += fa[i].x ^ fb[j].y;
+#else
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
               fa[i], fb[j], acc[i][j], 0, 0, 0);
+#endif
     }
-    if (kt + 1 < kt_total)
-      store_lds(buf ^ 1);
-    __syncthreads();
+  };
+
+  // Every load and LDS store below is unconditional (steps past the end are
+  // clamped to the last step and their data is never consumed): with no
+  // branch around a load the compiler can wait for exactly the register set
+  // it is about to store and leave the other set's loads in flight.
+  const int KT = Kpad / BK;
+  const int klast = (KT - 1) * BK;
+  auto kclamp = [&](int step) { return step < KT ? step * BK : klast; };
+  v4i ra0[CH_A], rb0[CH_B], ra1[CH_A], rb1[CH_B];
+  load_global(0, ra0, rb0);
+  load_global(kclamp(1), ra1, rb1);
+  store_lds(0, ra0, rb0);
+  load_global(kclamp(2), ra0, rb0);
+  lds_barrier();
+
+  int kt = 0;
+  while (true) {
+    // even step: MFMAs on buffer 0; step kt+1 goes to buffer 1 from set 1,
+    // then set 1 fetches step kt+3.
+    compute(0);
+    __builtin_amdgcn_sched_barrier(0);
+    store_lds(1, ra1, rb1);
+#if !(defined(OM_EXP) && (OM_EXP & 1))
+    load_global(kclamp(kt + 3), ra1, rb1);
+#endif
+    lds_barrier();
+    if (++kt >= KT)
+      break;
+    compute(1);
+    __builtin_amdgcn_sched_barrier(0);
+    store_lds(0, ra0, rb0);
+#if !(defined(OM_EXP) && (OM_EXP & 1))
+    load_global(kclamp(kt + 3), ra0, rb0);
+#endif
+    lds_barrier();
+    if (++kt >= KT)
+      break;
   }
 
   // ---- epilogue ----------------------------------------------------------
   // 32x32 accumulator layout: lane holds column (lane & 31); register r holds
   // row 8*(r/4) + 4*(lane/32) + (r%4).
+  const bool B_UNSIGNED = ep.b_unsigned;
+  const bool Y_UNSIGNED = ep.y_unsigned;
+  const int NARROW = ep.narrow;
   constexpr bool A_OFF = (A_MODE != 0);
   const int32_t oa = A_OFF ? 128 : 0;
   const int32_t ob = B_UNSIGNED ? 128 : 0;
   const bool a_uns = A_OFF;
 
-  float s_q = 0.0f;
   int32_t yz = 0;
   float a_scale = 0.0f;
-  if (EPI == kEpiQ8) {
-    // (a_scale * b_scale) / y_scale: two roundings, in this order
-    // (src/Conversion/ONNXToKrnl/Math/QLinearMatMul.cpp:127).
-    s_q = (ep.a_scale[0] * ep.b_scale[0]) / ep.y_scale[0];
+  if (EPI == kEpiQ8)
     yz = load_zp_i32(ep.y_zp, Y_UNSIGNED, 0);
-  }
   if (EPI == kEpiF32)
     a_scale = ep.a_scale[0];
 
+  // Everything the epilogue reads is loaded into registers before the first
+  // store: a load placed after a store to possibly aliasing memory would have
+  // to wait for it.
+  int n_[TN];
+  bool n_ok[TN];
+  int32_t db[TN], cs[TN];
+  float sj[TN];
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    const int n = n0 + wn * 64 + j * 32 + l32;
-    const bool n_ok = n < N;
-    int32_t db = ob, cs = 0;
-    float sj = 0.0f;
-    if (n_ok) {
+  for (int j = 0; j < TN; ++j) {
+    n_[j] = n0 + wn * WTN + j * 32 + l32;
+    n_ok[j] = n_[j] < N;
+    db[j] = ob;
+    cs[j] = 0;
+    sj[j] = 0.0f;
+    if (n_ok[j]) {
       if (ep.b_zp_len > 0)
-        db = ob - load_zp_i32(ep.b_zp, B_UNSIGNED, ep.b_zp_len == 1 ? 0 : n);
-      cs = ep.colsum[n];
+        db[j] = ob - load_zp_i32(
+                         ep.b_zp, B_UNSIGNED, ep.b_zp_len == 1 ? 0 : n_[j]);
+      cs[j] = ep.colsum[n_[j]];
+      // a_scale * b_scale[j] first, then one multiply per element; for the
+      // requantize (a_scale * b_scale) / y_scale, in this order
+      // (src/Conversion/ONNXToKrnl/Math/QLinearMatMul.cpp:127).
       if (EPI == kEpiF32)
-        sj = a_scale * ep.b_scale[ep.b_scale_len == 1 ? 0 : n];
+        sj[j] = a_scale * ep.b_scale[ep.b_scale_len == 1 ? 0 : n_[j]];
+      if (EPI == kEpiQ8)
+        sj[j] = (ep.a_scale[0] * ep.b_scale[ep.b_scale_len == 1 ? 0 : n_[j]]) /
+                ep.y_scale[0];
+    }
+  }
+  const int32_t az0 = ep.a_zp_len > 0 ? load_zp_i32(ep.a_zp, a_uns, 0) : 0;
+  const bool per_row = ep.a_zp_len > 1;
+  const bool has_rs = ep.rowsum != nullptr;
+
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const int mbase = m0 + wm * WTM + i * 32 + 4 * lh;
+    int32_t da[16], rs[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int m = mbase + 8 * (r >> 2) + (r & 3);
+      da[r] = oa - az0;
+      rs[r] = 0;
+      if (m < M) {
+        if (per_row)
+          da[r] = oa - load_zp_i32(ep.a_zp, a_uns, m);
+        if (has_rs)
+          rs[r] = ep.rowsum[m];
+      }
     }
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int j = 0; j < TN; ++j) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const int m = m0 + wm * 64 + i * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
-        if (!(n_ok && m < M))
+        const int m = mbase + 8 * (r >> 2) + (r & 3);
+        if (!(n_ok[j] && m < M))
           continue;
-        int32_t da = oa;
-        if (ep.a_zp_len > 0)
-          da = oa - load_zp_i32(ep.a_zp, a_uns, ep.a_zp_len == 1 ? 0 : m);
         uint32_t y = (uint32_t)acc[i][j][r];
-        y += (uint32_t)da * (uint32_t)cs;
-        if (ep.rowsum)
-          y += (uint32_t)db * (uint32_t)ep.rowsum[m];
-        y += (uint32_t)K * (uint32_t)da * (uint32_t)db;
-        const int64_t o = (int64_t)m * N + n;
+        y += (uint32_t)da[r] * (uint32_t)cs[j];
+        y += (uint32_t)db[j] * (uint32_t)rs[r];
+        y += (uint32_t)K * (uint32_t)da[r] * (uint32_t)db[j];
+        const int64_t o = (int64_t)m * N + n_[j];
         if (EPI == kEpiI32) {
           ((int32_t *)ep.out)[o] = (int32_t)y;
         } else if (EPI == kEpiF32) {
-          ((float *)ep.out)[o] = (float)(int32_t)y * sj;
+          ((float *)ep.out)[o] = (float)(int32_t)y * sj[j];
         } else {
-          const float f = (float)(int32_t)y * s_q;
+          const float f = (float)(int32_t)y * sj[j];
           const int32_t q = (int32_t)__builtin_rintf(f);
           int32_t v = (int32_t)((uint32_t)q + (uint32_t)yz);
           if (NARROW == kSaturate) {
@@ -329,35 +438,71 @@ __global__ __launch_bounds__(256) void k_rowsum_a(
     rowsum[m] = sum;
 }
 
-template <int A_MODE, int EPI>
-hipError_t gemm_launch_aligned(hipStream_t st, const GemmArgs &g,
-    const EpiParams &ep, int Kpad, int tiles_m, int tiles_n) {
-  const bool aligned = (g.K % 16 == 0) && ((((uintptr_t)g.A) & 15) == 0);
+// ---- launch ---------------------------------------------------------------
+enum TileCfg : int { kT128x128 = 0, kT256x128 = 1, kT256x256 = 2 };
+
+template <int BM, int BN, int WGM, int WGN, int MINB, int A_MODE, int EPI>
+hipError_t gemm_launch_tile(
+    hipStream_t st, const GemmArgs &g, const EpiParams &ep, int Kpad) {
+  const int tiles_m = (int)((g.M + BM - 1) / BM);
+  const int tiles_n = (int)((g.N + BN - 1) / BN);
   const dim3 grid((unsigned)(tiles_m * tiles_n));
-  if (aligned)
-    k_gemm_i8<A_MODE, EPI, true><<<grid, kGemmThreads, 0, st>>>(
-        (const uint8_t *)g.A, g.Bt, (int)g.M, (int)g.N, (int)g.K, Kpad, ep,
-        tiles_m, tiles_n);
-  else
-    k_gemm_i8<A_MODE, EPI, false><<<grid, kGemmThreads, 0, st>>>(
-        (const uint8_t *)g.A, g.Bt, (int)g.M, (int)g.N, (int)g.K, Kpad, ep,
-        tiles_m, tiles_n);
+  constexpr int threads = WGM * WGN * 64;
+  static const char *pad_env = getenv("OM_MI355X_GEMM_LDS_PAD");
+  const size_t pad = pad_env ? (size_t)atoi(pad_env) : 0;
+  k_gemm_i8<BM, BN, WGM, WGN, MINB, A_MODE, EPI, true>
+      <<<grid, threads, pad, st>>>((const uint8_t *)g.A, g.Bt, (int)g.M,
+          (int)g.N, (int)g.K, Kpad, ep, tiles_m, tiles_n);
   return hipGetLastError();
 }
 
+// Tile choice.  Small-K or small problems want many small tiles (several
+// resident per CU hide each other's latency and store phases); large problems
+// want the big tiles' higher MFMA-per-LDS-byte ratio.
+int choose_tile(const GemmArgs &g) {
+  static const char *force = getenv("OM_MI355X_GEMM_TILE");
+  if (force && force[0] >= '0' && force[0] <= '2')
+    return force[0] - '0';
+  const int64_t t128 = ((g.M + 127) / 128) * ((g.N + 127) / 128);
+  if (t128 < 3 * 256 || g.K < 1024)
+    return kT128x128;
+  return kT256x128;
+}
+
+template <int A_MODE, int EPI>
+hipError_t gemm_launch_cfg(
+    hipStream_t st, const GemmArgs &g, const EpiParams &ep, int Kpad) {
+  const bool aligned = (g.K % 64 == 0) && ((((uintptr_t)g.A) & 15) == 0);
+  if (!aligned) {
+    // Byte-wise staging of A for odd K or a misaligned A.
+    const int tiles_m = (int)((g.M + 127) / 128);
+    const int tiles_n = (int)((g.N + 127) / 128);
+    k_gemm_i8<128, 128, 2, 2, 2, A_MODE, EPI, false>
+        <<<dim3((unsigned)(tiles_m * tiles_n)), 256, 0, st>>>(
+            (const uint8_t *)g.A, g.Bt, (int)g.M, (int)g.N, (int)g.K, Kpad, ep,
+            tiles_m, tiles_n);
+    return hipGetLastError();
+  }
+  switch (choose_tile(g)) {
+  case kT256x256:
+    return gemm_launch_tile<256, 256, 2, 4, 1, A_MODE, EPI>(st, g, ep, Kpad);
+  case kT256x128:
+    return gemm_launch_tile<256, 128, 2, 2, 2, A_MODE, EPI>(st, g, ep, Kpad);
+  default:
+    return gemm_launch_tile<128, 128, 2, 2, 3, A_MODE, EPI>(st, g, ep, Kpad);
+  }
+}
+
 template <int A_MODE>
-hipError_t gemm_launch_epi(hipStream_t st, const GemmArgs &g,
-    const EpiParams &ep, int Kpad, int tiles_m, int tiles_n) {
+hipError_t gemm_launch_epi(
+    hipStream_t st, const GemmArgs &g, const EpiParams &ep, int Kpad) {
   switch (g.epi) {
   case kEpiI32:
-    return gemm_launch_aligned<A_MODE, kEpiI32>(
-        st, g, ep, Kpad, tiles_m, tiles_n);
+    return gemm_launch_cfg<A_MODE, kEpiI32>(st, g, ep, Kpad);
   case kEpiF32:
-    return gemm_launch_aligned<A_MODE, kEpiF32>(
-        st, g, ep, Kpad, tiles_m, tiles_n);
+    return gemm_launch_cfg<A_MODE, kEpiF32>(st, g, ep, Kpad);
   default:
-    return gemm_launch_aligned<A_MODE, kEpiQ8>(
-        st, g, ep, Kpad, tiles_m, tiles_n);
+    return gemm_launch_cfg<A_MODE, kEpiQ8>(st, g, ep, Kpad);
   }
 }
 
@@ -401,8 +546,6 @@ hipError_t launch_gemm(hipStream_t s, const GemmArgs &g) {
       g.M * g.N > ((int64_t)1 << 40))
     return hipErrorInvalidValue;
   const int Kpad = (int)round_up(g.K > 0 ? g.K : 1, kGemmBK);
-  const int tiles_m = (int)((g.M + BM - 1) / BM);
-  const int tiles_n = (int)((g.N + BN - 1) / BN);
   EpiParams ep;
   ep.a_zp = g.a_zp;
   ep.a_zp_len = g.a_zp ? g.a_zp_len : 0;
@@ -422,11 +565,11 @@ hipError_t launch_gemm(hipStream_t s, const GemmArgs &g) {
   const int a_mode = g.a_preshifted ? 2 : (g.a_unsigned ? 1 : 0);
   switch (a_mode) {
   case 0:
-    return gemm_launch_epi<0>(s, g, ep, Kpad, tiles_m, tiles_n);
+    return gemm_launch_epi<0>(s, g, ep, Kpad);
   case 1:
-    return gemm_launch_epi<1>(s, g, ep, Kpad, tiles_m, tiles_n);
+    return gemm_launch_epi<1>(s, g, ep, Kpad);
   default:
-    return gemm_launch_epi<2>(s, g, ep, Kpad, tiles_m, tiles_n);
+    return gemm_launch_epi<2>(s, g, ep, Kpad);
   }
 }
 

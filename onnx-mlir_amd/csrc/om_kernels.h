@@ -44,7 +44,7 @@ hipError_t launch_dynamic_quantize(hipStream_t s, const DqlScratch &scratch,
 // u8 shifted to int8 by -128, zero filled outside [N,K]; colsum[n] = sum_k of
 // the int8 values written (int32), colsum has Npad entries.
 constexpr int kGemmBK = 64;    // K granularity of the packed operand
-constexpr int kGemmBN = 128;   // N granularity of the packed operand
+constexpr int kGemmBN = 256;   // N granularity of the packed operand (largest tile)
 inline int64_t round_up(int64_t v, int64_t m) { return (v + m - 1) / m * m; }
 
 hipError_t launch_pack_b(hipStream_t s, const void *B, bool b_unsigned,

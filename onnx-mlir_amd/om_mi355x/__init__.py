@@ -373,3 +373,34 @@ def DynQuantMatMulDequant(x: Tensor, b: Tensor, b_zero_point: Optional[Tensor],
         _lib.om_mi355x_DynQuantMatMulDequant(hy, hx, hb, hbz, hbs)
     _check()
     return y
+
+
+class PreparedCall:
+    """An entry point bound once to fixed operands: the OMTensor wrappers are
+    built a single time, so that calling it costs one C call (what a compiled
+    model pays), not a Python marshalling pass.  ``operands`` follow the C
+    signature: tensors (or None) first, then integer attributes."""
+
+    def __init__(self, entry: str, *operands):
+        load()
+        self._fn = getattr(_lib, entry)
+        self._wrappers = []
+        self._args = []
+        for o in operands:
+            if isinstance(o, (int, np.integer)) and not isinstance(o, np.ndarray):
+                self._args.append(int(o))
+            else:
+                w = _OMT(o)
+                self._wrappers.append(w)
+                self._args.append(w.handle)
+
+    def __call__(self):
+        self._fn(*self._args)
+
+    def check(self):
+        _check()
+
+    def close(self):
+        for w in self._wrappers:
+            w.__exit__()
+        self._wrappers = []
