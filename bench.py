@@ -97,7 +97,7 @@ def decode_case(rt, wl, M, steps, warmup):
     return res
 
 
-def qdq_cases(rt, wl, rows, cols, steps, warmup):
+def qdq_cases(rt, wl, rows, cols, steps, warmup, only=None):
     c = wl.config2(rows, cols)
     n = rows * cols
     dX = rt.DeviceArray.from_numpy(c["X"])
@@ -112,6 +112,9 @@ def qdq_cases(rt, wl, rows, cols, steps, warmup):
     out = {}
 
     def run(name, fn, nbytes):
+        if only is not None and name != only:
+            fn.close()
+            return
         host_s, ev_ms = timed(rt, fn, steps, warmup)
         fn.check()
         fn.close()
@@ -130,6 +133,32 @@ def qdq_cases(rt, wl, rows, cols, steps, warmup):
     for d in (dX, dS, dZ, dQ, dD, dys, dyz, s1, z1):
         d.free()
     return out
+
+
+def only_mode(rt, wl, what, steps, warmup):
+    """One kernel, `steps` launches, nothing else on the GPU: the target of the
+    rocprofv3 counter runs whose summaries are kept under profiles/."""
+    import ctypes
+    if what == "copy":
+        # plain device-to-device copy of known size: calibrates FETCH_SIZE / WRITE_SIZE
+        n = 1 << 30
+        a, b = rt.DeviceArray((n,), np.uint8), rt.DeviceArray((n,), np.uint8)
+        hip = ctypes.CDLL("libamdhip64.so")
+        hip.hipMemcpy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
+        for _ in range(steps):
+            assert hip.hipMemcpy(b.ptr, a.ptr, n, 3) == 0
+        hip.hipDeviceSynchronize()
+        return {"only": what, "bytes_read": n, "bytes_written": n, "launches": steps}
+    if what == "gemm_ffn_up":
+        c = wl.config4("ffn_up", M=8)
+        r = gemm_case(rt, wl, "config4 FFN-up", 4096, 768, 3072, c["W"], c["w_scale"], steps, warmup, "f32")
+        return {"only": what, **r}
+    if what == "gemm_prefill_up":
+        c = wl.config5("up", M=8)
+        r = gemm_case(rt, wl, "config5 prefill up", 2048, 4096, 11008, c["W"], c["w_scale"], steps, warmup, "f32")
+        return {"only": what, **r}
+    r = qdq_cases(rt, wl, 8192, 32768, steps, warmup, only=what)
+    return {"only": what, **r[what]}
 
 
 def cpu_baseline_gemm(oracle, wl, M, K, N, budget_s=20.0):
@@ -169,6 +198,10 @@ def main():
     ap.add_argument("--no-extras", action="store_true", help="skip the Q/DQ and other-shape measurements")
     ap.add_argument("--extras", default="gemm,decode,qdq", help="which extra groups to measure")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--only", default=None,
+                    choices=["copy", "gemm_ffn_up", "gemm_prefill_up", "quantize_per_axis", "dequantize_per_axis",
+                             "quantize_per_tensor", "dequantize_per_tensor", "dynamic_quantize"],
+                    help="launch just this kernel --steps times (for rocprofv3 counter runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1",
@@ -179,6 +212,9 @@ def main():
     from om_mi355x import workloads as wl
     rt.load()                       # raises if the HIP library is not built
     info = rt.device_info()         # raises if there is no gfx950 device
+    if args.only:
+        print(json.dumps(only_mode(rt, wl, args.only, args.steps, args.warmup)))
+        return
 
     M, K, N = 4096, 768, 3072
     c = wl.config4("ffn_up", M=8)   # weights and scales only; activations are made in gemm_case

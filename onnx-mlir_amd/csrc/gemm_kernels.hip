@@ -67,12 +67,164 @@ struct EpiParams {
   bool b_unsigned;
   bool y_unsigned;
   int narrow;
+  int group;   // tile rows per scheduling group
+  int xcd;     // renumber workgroups per XCD
 };
 
 __device__ __forceinline__ int32_t load_zp_i32(
     const void *p, bool is_unsigned, int64_t i) {
   return is_unsigned ? (int32_t)((const uint8_t *)p)[i]
                      : (int32_t)((const int8_t *)p)[i];
+}
+
+// Epilogue shared by the GEMM kernels: applies the zero-point correction and
+// the op's output conversion to a wave's TM x TN grid of 32x32 accumulator
+// tiles whose top-left element is (mrow0, ncol0).
+// 32x32 accumulator layout: lane holds column (lane & 31); register r holds
+// row 8*(r/4) + 4*(lane/32) + (r%4).
+//
+// The code is kept free of branches around memory operations: every load is
+// unconditional (indices clamped, absent operands redirected to valid memory
+// and masked afterwards) and all loads precede the stores, so the stores can
+// be issued back to back without waiting on one another.
+template <int EPI>
+__device__ __forceinline__ void store_one(const EpiParams &ep, int64_t o,
+    uint32_t y, float sj, int32_t yz) {
+  if (EPI == kEpiI32) {
+    ((int32_t *)ep.out)[o] = (int32_t)y;
+  } else if (EPI == kEpiF32) {
+    ((float *)ep.out)[o] = (float)(int32_t)y * sj;
+  } else {
+    const float f = (float)(int32_t)y * sj;
+    const int32_t q = (int32_t)__builtin_rintf(f);
+    int32_t v = (int32_t)((uint32_t)q + (uint32_t)yz);
+    if (ep.narrow == kSaturate) {
+      const int32_t lo = ep.y_unsigned ? 0 : -128;
+      const int32_t hi = ep.y_unsigned ? 255 : 127;
+      v = v < lo ? lo : (v > hi ? hi : v);
+    }
+    ((uint8_t *)ep.out)[o] = (uint8_t)(v & 0xFF);
+  }
+}
+
+template <int TM, int TN, int A_MODE, int EPI>
+__device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TM][TN], int mrow0,
+    int ncol0, int M, int N, int K, const EpiParams &ep) {
+  const int lane = threadIdx.x & 63;
+  const int l32 = lane & 31;
+  const int lh = lane >> 5;
+  const bool B_UNSIGNED = ep.b_unsigned;
+  constexpr bool A_OFF = (A_MODE != 0);
+  const int32_t oa = A_OFF ? 128 : 0;
+  const int32_t ob = B_UNSIGNED ? 128 : 0;
+
+  int32_t yz = 0;
+  float a_scale = 0.0f, y_scale = 1.0f;
+  if (EPI == kEpiQ8) {
+    yz = load_zp_i32(ep.y_zp, ep.y_unsigned, 0);
+    y_scale = ep.y_scale[0];
+  }
+  if (EPI != kEpiI32)
+    a_scale = ep.a_scale[0];
+
+  // Absent operands read from colsum (always valid) and are masked to zero.
+  const bool has_bzp = ep.b_zp_len > 0;
+  const void *bzp_ptr = has_bzp ? ep.b_zp : (const void *)ep.colsum;
+  const bool has_azp = ep.a_zp_len > 0;
+  const void *azp_ptr = has_azp ? ep.a_zp : (const void *)ep.colsum;
+  const bool per_row = ep.a_zp_len > 1;
+  const bool has_rs = ep.rowsum != nullptr;
+  const int32_t *rs_ptr = has_rs ? ep.rowsum : ep.colsum;
+
+  int n_[TN];
+  int32_t db[TN], cs[TN];
+  float sj[TN];
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    n_[j] = ncol0 + j * 32 + l32;
+    const int nc = n_[j] < N ? n_[j] : N - 1;
+    const int32_t bz =
+        load_zp_i32(bzp_ptr, B_UNSIGNED, ep.b_zp_len > 1 ? nc : 0);
+    db[j] = ob - (has_bzp ? bz : 0);
+    cs[j] = ep.colsum[nc];
+    sj[j] = 0.0f;
+    // a_scale * b_scale[j] first, then one multiply per element; for the
+    // requantize (a_scale * b_scale) / y_scale, in this order
+    // (src/Conversion/ONNXToKrnl/Math/QLinearMatMul.cpp:127).
+    if (EPI != kEpiI32) {
+      sj[j] = a_scale * ep.b_scale[ep.b_scale_len == 1 ? 0 : nc];
+      if (EPI == kEpiQ8)
+        sj[j] = sj[j] / y_scale;
+    }
+  }
+
+  // Wave-uniform: the whole TM x TN grid lies inside the matrix.
+  const bool full = (mrow0 + 32 * TM <= M) && (ncol0 + 32 * TN <= N);
+
+  const int32_t az0 = load_zp_i32(azp_ptr, A_OFF, 0);
+  const int32_t da0 = oa - (has_azp ? az0 : 0);
+  __builtin_amdgcn_sched_barrier(0);
+
+  if (!per_row && !has_rs) {
+    // Common case: one zero point for all rows and no offset on B, so no
+    // per-row operand exists and nothing is loaded between the stores.
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int mbase = mrow0 + i * 32 + 4 * lh;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = mbase + 8 * (r >> 2) + (r & 3);
+        const int64_t orow = (int64_t)m * N;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          uint32_t y = (uint32_t)acc[i][j][r];
+          y += (uint32_t)da0 * (uint32_t)cs[j];
+          y += (uint32_t)K * (uint32_t)da0 * (uint32_t)db[j];
+          if (full) {
+            store_one<EPI>(ep, orow + n_[j], y, sj[j], yz);
+          } else if (m < M && n_[j] < N) {
+            store_one<EPI>(ep, orow + n_[j], y, sj[j], yz);
+          }
+        }
+      }
+    }
+    return;
+  }
+
+  // Per-row zero points and / or row sums: four rows at a time, to keep the
+  // register footprint of this rarely taken path small.
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const int mbase = mrow0 + i * 32 + 4 * lh;
+#pragma unroll
+    for (int rg = 0; rg < 4; ++rg) {
+      int32_t da[4], rs[4];
+#pragma unroll
+      for (int rr = 0; rr < 4; ++rr) {
+        const int m = mbase + 8 * rg + rr;
+        const int mc = m < M ? m : M - 1;
+        const int32_t az = load_zp_i32(azp_ptr, A_OFF, per_row ? mc : 0);
+        da[rr] = oa - (has_azp ? az : 0);
+        const int32_t rv = rs_ptr[has_rs ? mc : 0];
+        rs[rr] = has_rs ? rv : 0;
+      }
+#pragma unroll
+      for (int rr = 0; rr < 4; ++rr) {
+        const int r = rg * 4 + rr;
+        const int m = mbase + 8 * rg + rr;
+        const int64_t orow = (int64_t)m * N;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          uint32_t y = (uint32_t)acc[i][j][r];
+          y += (uint32_t)da[rr] * (uint32_t)cs[j];
+          y += (uint32_t)db[j] * (uint32_t)rs[rr];
+          y += (uint32_t)K * (uint32_t)da[rr] * (uint32_t)db[j];
+          if (m < M && n_[j] < N)
+            store_one<EPI>(ep, orow + n_[j], y, sj[j], yz);
+        }
+      }
+    }
+  }
 }
 
 // BM x BN block tile, WGM x WGN waves, each wave a (BM/WGM) x (BN/WGN) tile
@@ -206,20 +358,12 @@ __global__ __launch_bounds__(WGM *WGN * 64, MINB) void k_gemm_i8(
 #pragma unroll
       for (int j = 0; j < TN; ++j)
         fb[j] = *(const v4i *)(&sB[buf][lds_off(wn * WTN + j * 32 + l32, c)]);
-#if defined(OM_EXP) && (OM_EXP & 2)
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-          acc[i][j][0] += fa[i].x ^ fb[j].y;
-#else
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
               fa[i], fb[j], acc[i][j], 0, 0, 0);
-#endif
     }
   };
 
@@ -244,121 +388,207 @@ __global__ __launch_bounds__(WGM *WGN * 64, MINB) void k_gemm_i8(
     compute(0);
     __builtin_amdgcn_sched_barrier(0);
     store_lds(1, ra1, rb1);
-#if !(defined(OM_EXP) && (OM_EXP & 1))
     load_global(kclamp(kt + 3), ra1, rb1);
-#endif
     lds_barrier();
     if (++kt >= KT)
       break;
     compute(1);
     __builtin_amdgcn_sched_barrier(0);
     store_lds(0, ra0, rb0);
-#if !(defined(OM_EXP) && (OM_EXP & 1))
     load_global(kclamp(kt + 3), ra0, rb0);
-#endif
     lds_barrier();
     if (++kt >= KT)
       break;
   }
 
-  // ---- epilogue ----------------------------------------------------------
-  // 32x32 accumulator layout: lane holds column (lane & 31); register r holds
-  // row 8*(r/4) + 4*(lane/32) + (r%4).
-  const bool B_UNSIGNED = ep.b_unsigned;
-  const bool Y_UNSIGNED = ep.y_unsigned;
-  const int NARROW = ep.narrow;
-  constexpr bool A_OFF = (A_MODE != 0);
-  const int32_t oa = A_OFF ? 128 : 0;
-  const int32_t ob = B_UNSIGNED ? 128 : 0;
-  const bool a_uns = A_OFF;
+  gemm_epilogue<TM, TN, A_MODE, EPI>(
+      acc, m0 + wm * WTM, n0 + wn * WTN, M, N, K, ep);
+}
 
-  int32_t yz = 0;
-  float a_scale = 0.0f;
-  if (EPI == kEpiQ8)
-    yz = load_zp_i32(ep.y_zp, Y_UNSIGNED, 0);
-  if (EPI == kEpiF32)
-    a_scale = ep.a_scale[0];
+// ---- GEMM, A streamed to registers ----------------------------------------
+// LDS stores are the scarcest on-chip resource of a CU (about a third of the
+// LDS read rate), so this kernel keeps A out of LDS altogether.  The four
+// waves of a block are stacked along M: a wave owns 32*TM rows that no other
+// wave needs, and reads its A operands straight from global memory in MFMA
+// operand layout (lane = row, 16 K-bytes per lane).  Only the Bt tile, which
+// all four waves share, goes through LDS: a ring of three 64-byte-deep stages.
+//
+// Global loads run D steps ahead in registers (D register sets, loop unrolled
+// by D so that every set is addressed statically).  Per K step (64 bytes) a
+// wave issues, in this order,
+//   ds_read  B operands of sub-step 1 (this step's stage)
+//   MFMAs of sub-step 0; A registers of sub-step 0 are refilled for step +D
+//   ds_write the staged Bt chunk of step +2 into its stage; refetch step +2+D
+//   ds_read  B operands of sub-step 0 of step +1 (stage published one barrier
+//            ago -- this is what the third stage buys: nothing waits on LDS
+//            right after the barrier)
+//   MFMAs of sub-step 1; A registers of sub-step 1 are refilled for step +D
+//   one LDS-only barrier
+// All loads are unconditional (clamped), so every wait is an exact count.
+template <int TM, int TN, int D, int A_MODE, int EPI>
+__global__ __launch_bounds__(256, (TM == 1 ? 2 : 1)) void k_gemm_i8_stream(
+    const uint8_t *__restrict__ Ap, const int8_t *__restrict__ Bt, int M, int N,
+    int K, int Kpad, EpiParams ep, int tiles_m, int tiles_n) {
+  constexpr int BM = 4 * 32 * TM, BN = 32 * TN;
+  constexpr int CH_B = BN * 4 / 256; // 16-byte chunks of Bt per thread, per step
+  static_assert(BN * 4 % 256 == 0, "BN must be a multiple of 64");
+  constexpr int STAGE = BN * BK;
 
-  // Everything the epilogue reads is loaded into registers before the first
-  // store: a load placed after a store to possibly aliasing memory would have
-  // to wait for it.
-  int n_[TN];
-  bool n_ok[TN];
-  int32_t db[TN], cs[TN];
-  float sj[TN];
+  __shared__ __attribute__((aligned(16))) uint8_t sB[3 * STAGE];
+
+  int pid = blockIdx.x;
+  if (ep.xcd) {
+    const int nb = gridDim.x;
+    const int per = nb >> 3;
+    if (per > 0 && pid < per * 8)
+      pid = (pid & 7) * per + (pid >> 3);
+  }
+  const int GROUP = ep.group;
+  const int in_group = GROUP * tiles_n;
+  const int group = pid / in_group;
+  const int first_m = group * GROUP;
+  const int gsize = (tiles_m - first_m < GROUP) ? tiles_m - first_m : GROUP;
+  const int tm = first_m + (pid % in_group) % gsize;
+  const int tn = (pid % in_group) / gsize;
+  const int m0 = tm * BM, n0 = tn * BN;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int l32 = lane & 31;
+  const int lh = lane >> 5;
+  const int mrow0 = m0 + wave * 32 * TM;
+
+  const int KT = Kpad / BK;
+  const int klast = (KT - 1) * BK;
+  auto kclamp = [&](int step) { return step < KT ? step * BK : klast; };
+
+  // A operand pointers into the fragment-packed copy of A (see k_pack_a): the
+  // operand of MFMA row tile mt, step ks, half step sub is one contiguous KiB,
+  // 16 bytes per lane.  Row tiles past the last one are clamped (they only
+  // feed output rows that are never stored).
+  const uint8_t *__restrict__ arow[TM];
+  {
+    const int mt_max = (M + 31) / 32 - 1;
 #pragma unroll
-  for (int j = 0; j < TN; ++j) {
-    n_[j] = n0 + wn * WTN + j * 32 + l32;
-    n_ok[j] = n_[j] < N;
-    db[j] = ob;
-    cs[j] = 0;
-    sj[j] = 0.0f;
-    if (n_ok[j]) {
-      if (ep.b_zp_len > 0)
-        db[j] = ob - load_zp_i32(
-                         ep.b_zp, B_UNSIGNED, ep.b_zp_len == 1 ? 0 : n_[j]);
-      cs[j] = ep.colsum[n_[j]];
-      // a_scale * b_scale[j] first, then one multiply per element; for the
-      // requantize (a_scale * b_scale) / y_scale, in this order
-      // (src/Conversion/ONNXToKrnl/Math/QLinearMatMul.cpp:127).
-      if (EPI == kEpiF32)
-        sj[j] = a_scale * ep.b_scale[ep.b_scale_len == 1 ? 0 : n_[j]];
-      if (EPI == kEpiQ8)
-        sj[j] = (ep.a_scale[0] * ep.b_scale[ep.b_scale_len == 1 ? 0 : n_[j]]) /
-                ep.y_scale[0];
+    for (int i = 0; i < TM; ++i) {
+      int mt = (mrow0 >> 5) + i;
+      mt = mt < mt_max ? mt : mt_max;
+      arow[i] = Ap + (int64_t)mt * KT * 2048 + lane * 16;
     }
   }
-  const int32_t az0 = ep.a_zp_len > 0 ? load_zp_i32(ep.a_zp, a_uns, 0) : 0;
-  const bool per_row = ep.a_zp_len > 1;
-  const bool has_rs = ep.rowsum != nullptr;
+  // Bt staging pointers: chunk q -> row q>>2, 16-byte chunk q&3.
+  const int8_t *__restrict__ brow[CH_B];
+  int bdst[CH_B];
+#pragma unroll
+  for (int h = 0; h < CH_B; ++h) {
+    const int q = tid + h * 256;
+    // Bt has round_up(N, kGemmBN) rows; a tile whose width does not divide
+    // that may reach past it: clamp (those columns are never stored).
+    const int npad = (N + kGemmBN - 1) / kGemmBN * kGemmBN;
+    int bn = n0 + (q >> 2);
+    bn = bn < npad ? bn : npad - 1;
+    brow[h] = Bt + (int64_t)bn * Kpad + (q & 3) * 16;
+    bdst[h] = lds_off(q >> 2, q & 3);
+  }
 
+  // k0 is a byte offset along K (64 per step); a step of packed A is 2 KiB.
+  auto load_a = [&](int k0, int sub, v4i(&ra)[TM]) {
 #pragma unroll
-  for (int i = 0; i < TM; ++i) {
-    const int mbase = m0 + wm * WTM + i * 32 + 4 * lh;
-    int32_t da[16], rs[16];
+    for (int i = 0; i < TM; ++i)
+      ra[i] = *(const v4i *)(arow[i] + k0 * 32 + sub * 1024);
+  };
+  auto load_b = [&](int k0, v4i(&rb)[CH_B]) {
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int m = mbase + 8 * (r >> 2) + (r & 3);
-      da[r] = oa - az0;
-      rs[r] = 0;
-      if (m < M) {
-        if (per_row)
-          da[r] = oa - load_zp_i32(ep.a_zp, a_uns, m);
-        if (has_rs)
-          rs[r] = ep.rowsum[m];
-      }
+    for (int h = 0; h < CH_B; ++h)
+      rb[h] = *(const v4i *)(brow[h] + k0);
+  };
+  auto write_b = [&](int stage, const v4i(&rb)[CH_B]) {
+#pragma unroll
+    for (int h = 0; h < CH_B; ++h)
+      *(v4i *)(&sB[stage * STAGE + bdst[h]]) = rb[h];
+  };
+  auto read_frag = [&](int stage, int sub, v4i(&fb)[TN]) {
+    const int c = sub * 2 + lh;
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+      fb[j] = *(const v4i *)(&sB[stage * STAGE + lds_off(j * 32 + l32, c)]);
+  };
+
+  v16i acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        acc[i][j][r] = 0;
+
+  auto mfma_sub = [&](const v4i(&ra)[TM], const v4i(&fb)[TN]) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
+            ra[i], fb[j], acc[i][j], 0, 0, 0);
     }
+  };
+
+  // D register sets: as[u][sub] holds A of a step with (step % D) == u;
+  // bs[u] holds the staged Bt chunk of the step two ahead of that.
+  v4i as[D][2][TM];
+  v4i bs[D][CH_B];
+  v4i f0[TN], f1[TN];
+
+  // Prologue.  Bt of steps 0 and 1 goes to stages 0 and 1 through bs[0],
+  // bs[1]; then bs[u] is filled with step 2+u.  as[u] is filled with step u.
+  load_b(0, bs[0]);
+  load_b(kclamp(1), bs[D > 1 ? 1 : 0]);
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
+  for (int u = 0; u < D; ++u) {
+    load_a(kclamp(u), 0, as[u][0]);
+    load_a(kclamp(u), 1, as[u][1]);
+  }
+  write_b(0, bs[0]);
+  if (D > 1)
+    write_b(1, bs[1]);
+  else {
+    load_b(kclamp(1), bs[0]);
+    write_b(1, bs[0]);
+  }
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int m = mbase + 8 * (r >> 2) + (r & 3);
-        if (!(n_ok[j] && m < M))
-          continue;
-        uint32_t y = (uint32_t)acc[i][j][r];
-        y += (uint32_t)da[r] * (uint32_t)cs[j];
-        y += (uint32_t)db[j] * (uint32_t)rs[r];
-        y += (uint32_t)K * (uint32_t)da[r] * (uint32_t)db[j];
-        const int64_t o = (int64_t)m * N + n_[j];
-        if (EPI == kEpiI32) {
-          ((int32_t *)ep.out)[o] = (int32_t)y;
-        } else if (EPI == kEpiF32) {
-          ((float *)ep.out)[o] = (float)(int32_t)y * sj[j];
-        } else {
-          const float f = (float)(int32_t)y * sj[j];
-          const int32_t q = (int32_t)__builtin_rintf(f);
-          int32_t v = (int32_t)((uint32_t)q + (uint32_t)yz);
-          if (NARROW == kSaturate) {
-            if (Y_UNSIGNED)
-              v = v < 0 ? 0 : (v > 255 ? 255 : v);
-            else
-              v = v < -128 ? -128 : (v > 127 ? 127 : v);
-          }
-          ((uint8_t *)ep.out)[o] = (uint8_t)(v & 0xFF);
-        }
+  for (int u = 0; u < D; ++u)
+    load_b(kclamp(2 + u), bs[u]);
+  lds_barrier();
+  read_frag(0, 0, f0);
+
+  int kt = 0;
+  int st0 = 0, st1 = 1, st2 = 2; // stages of steps kt, kt+1, kt+2
+  bool done = false;
+  while (!done) {
+#pragma unroll
+    for (int u = 0; u < D; ++u) {
+      read_frag(st0, 1, f1);
+      mfma_sub(as[u][0], f0);
+      load_a(kclamp(kt + D), 0, as[u][0]);
+      write_b(st2, bs[u]);
+      load_b(kclamp(kt + 2 + D), bs[u]);
+      read_frag(st1, 0, f0);
+      mfma_sub(as[u][1], f1);
+      load_a(kclamp(kt + D), 1, as[u][1]);
+      lds_barrier();
+      if (++kt >= KT) {
+        done = true;
+        break;
       }
+      const int t = st0;
+      st0 = st1;
+      st1 = st2;
+      st2 = t;
     }
   }
+
+  gemm_epilogue<TM, TN, A_MODE, EPI>(acc, mrow0, n0, M, N, K, ep);
 }
 
 // ---- pack B ---------------------------------------------------------------
@@ -416,6 +646,61 @@ __global__ __launch_bounds__(256) void k_pack_b(const uint8_t *__restrict__ B,
   }
 }
 
+// ---- pack A ---------------------------------------------------------------
+// Rewrites A [M,K] (row-major) in MFMA operand order for k_gemm_i8_stream:
+//   Ap[mt][ks][sub][lane][16 bytes],  lane = half*32 + row,
+//   bytes = A[mt*32 + row][ks*64 + (sub*2 + half)*16 .. +16]
+// so that a wave fetches one operand (32 rows x 32 K-bytes... x 2 halves) as a
+// single contiguous KiB.  uint8 is moved to int8 (minus 128) on the way and
+// everything outside [M,K] is zero in that domain, which also makes K that is
+// not a multiple of 64 (or 16) legal for the fast kernel.
+// A block handles one 32-row tile and four K steps (256 bytes of each row):
+// eight consecutive threads read 128 contiguous bytes of a row.
+template <bool A_UNSIGNED, bool ALIGNED>
+__global__ __launch_bounds__(256) void k_pack_a(const uint8_t *__restrict__ A,
+    int64_t M, int64_t K, int KT, uint8_t *__restrict__ Ap) {
+  const int mt = blockIdx.y;
+  const int ks0 = blockIdx.x * 4;
+  const int tid = threadIdx.x;
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int row = tid >> 3;
+    const int c16 = (tid & 7) + 8 * h; // 16-byte chunk within the 256 bytes
+    const int ks = ks0 + (c16 >> 2);
+    if (ks >= KT)
+      continue;
+    const int c = c16 & 3;
+    const int64_t m = (int64_t)mt * 32 + row;
+    const int64_t k = (int64_t)ks * 64 + c * 16;
+    v4i v = {0, 0, 0, 0};
+    if (ALIGNED) {
+      if (m < M && k < K) {
+        v = *(const v4i *)(A + m * K + k);
+        if (A_UNSIGNED)
+          v ^= (v4i){(int)0x80808080, (int)0x80808080, (int)0x80808080,
+              (int)0x80808080};
+      }
+    } else {
+      uint32_t w[4] = {0, 0, 0, 0};
+#pragma unroll
+      for (int b = 0; b < 16; ++b) {
+        uint32_t byte = 0;
+        if (m < M && k + b < K) {
+          byte = A[m * K + k + b];
+          if (A_UNSIGNED)
+            byte ^= 0x80u;
+        }
+        w[b >> 2] |= byte << ((b & 3) * 8);
+      }
+      v = (v4i){(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+    }
+    const int sub = c >> 1, half = c & 1;
+    const int64_t o =
+        ((((int64_t)mt * KT + ks) * 2 + sub) * 64 + half * 32 + row) * 16;
+    *(v4i *)(Ap + o) = v;
+  }
+}
+
 // rowsum[m] = sum_k A'[m,k]; one wave per row.
 template <bool A_UNSIGNED>
 __global__ __launch_bounds__(256) void k_rowsum_a(
@@ -439,7 +724,6 @@ __global__ __launch_bounds__(256) void k_rowsum_a(
 }
 
 // ---- launch ---------------------------------------------------------------
-enum TileCfg : int { kT128x128 = 0, kT256x128 = 1, kT256x256 = 2 };
 
 template <int BM, int BN, int WGM, int WGN, int MINB, int A_MODE, int EPI>
 hipError_t gemm_launch_tile(
@@ -448,30 +732,122 @@ hipError_t gemm_launch_tile(
   const int tiles_n = (int)((g.N + BN - 1) / BN);
   const dim3 grid((unsigned)(tiles_m * tiles_n));
   constexpr int threads = WGM * WGN * 64;
-  static const char *pad_env = getenv("OM_MI355X_GEMM_LDS_PAD");
-  const size_t pad = pad_env ? (size_t)atoi(pad_env) : 0;
   k_gemm_i8<BM, BN, WGM, WGN, MINB, A_MODE, EPI, true>
-      <<<grid, threads, pad, st>>>((const uint8_t *)g.A, g.Bt, (int)g.M,
+      <<<grid, threads, 0, st>>>((const uint8_t *)g.A, g.Bt, (int)g.M,
           (int)g.N, (int)g.K, Kpad, ep, tiles_m, tiles_n);
   return hipGetLastError();
 }
 
-// Tile choice.  Small-K or small problems want many small tiles (several
-// resident per CU hide each other's latency and store phases); large problems
-// want the big tiles' higher MFMA-per-LDS-byte ratio.
+hipError_t launch_pack_a(hipStream_t st, const void *A, bool a_unsigned,
+    int64_t M, int64_t K, uint8_t *Ap) {
+  const int KT = (int)(round_up(K > 0 ? K : 1, kGemmBK) / kGemmBK);
+  const int MT = (int)((M + 31) / 32);
+  const bool aligned = (K % 16 == 0) && ((((uintptr_t)A) & 15) == 0);
+  dim3 grid((unsigned)((KT + 3) / 4), (unsigned)MT);
+  if (a_unsigned) {
+    if (aligned)
+      k_pack_a<true, true><<<grid, 256, 0, st>>>(
+          (const uint8_t *)A, M, K, KT, Ap);
+    else
+      k_pack_a<true, false><<<grid, 256, 0, st>>>(
+          (const uint8_t *)A, M, K, KT, Ap);
+  } else {
+    if (aligned)
+      k_pack_a<false, true><<<grid, 256, 0, st>>>(
+          (const uint8_t *)A, M, K, KT, Ap);
+    else
+      k_pack_a<false, false><<<grid, 256, 0, st>>>(
+          (const uint8_t *)A, M, K, KT, Ap);
+  }
+  return hipGetLastError();
+}
+
+template <int TM, int TN, int D, int A_MODE, int EPI>
+hipError_t gemm_launch_stream(
+    hipStream_t st, const GemmArgs &g, const EpiParams &ep, int Kpad) {
+  constexpr int BM = 4 * 32 * TM, BN = 32 * TN;
+  const int tiles_m = (int)((g.M + BM - 1) / BM);
+  const int tiles_n = (int)((g.N + BN - 1) / BN);
+  k_gemm_i8_stream<TM, TN, D, A_MODE, EPI>
+      <<<dim3((unsigned)(tiles_m * tiles_n)), 256, 0, st>>>(g.a_pack, g.Bt,
+          (int)g.M, (int)g.N, (int)g.K, Kpad, ep, tiles_m, tiles_n);
+  return hipGetLastError();
+}
+
+// Kernel / tile configurations.
+enum TileCfg : int {
+  kT128x128 = 0, // k_gemm_i8, BM x BN
+  kT256x128 = 1,
+  kS256x192 = 2, // k_gemm_i8_stream (needs the packed copy of A)
+  kS256x128 = 3,
+  kS128x192 = 4,
+  kS128x128 = 5,
+  kNumCfg = 6
+};
+
+bool cfg_is_stream(int c) {
+  return c == kS256x192 || c == kS256x128 || c == kS128x192 || c == kS128x128;
+}
+
+// Tile choice.  Each configuration is costed as (rounds of tiles over the 256
+// CUs) x (tile area), i.e. matrix-core time including the idle tail of the
+// last round; among near-equal costs the larger tile wins (fewer LDS and L2
+// bytes per MFMA).  The streamed-A kernels are only eligible when the caller
+// provided the buffer for the packed copy of A.
 int choose_tile(const GemmArgs &g) {
-  static const char *force = getenv("OM_MI355X_GEMM_TILE");
-  if (force && force[0] >= '0' && force[0] <= '2')
-    return force[0] - '0';
-  const int64_t t128 = ((g.M + 127) / 128) * ((g.N + 127) / 128);
-  if (t128 < 3 * 256 || g.K < 1024)
+  // Override for tests and tuning: OM_MI355X_GEMM_TILE=<TileCfg value>.
+  const char *force = getenv("OM_MI355X_GEMM_TILE");
+  if (force && force[0]) {
+    const int c = atoi(force);
+    if (c >= 0 && c < kNumCfg && (!cfg_is_stream(c) || g.a_pack))
+      return c;
+  }
+  struct Cand {
+    int cfg, bm, bn, per_cu;
+  };
+  static const Cand cands[] = {{kS256x192, 256, 192, 1}, {kS256x128, 256, 128, 1},
+      {kS128x192, 128, 192, 2}, {kS128x128, 128, 128, 2}};
+  if (!g.a_pack)
     return kT128x128;
-  return kT256x128;
+  int best = kS128x128;
+  double best_cost = 1e300;
+  for (const Cand &c : cands) {
+    const int64_t tiles =
+        ((g.M + c.bm - 1) / c.bm) * ((g.N + c.bn - 1) / c.bn);
+    const int64_t slots = 256 * c.per_cu;
+    const int64_t rounds = (tiles + slots - 1) / slots;
+    // two co-resident tiles share a CU's matrix cores
+    double cost = (double)rounds * c.per_cu * c.bm * c.bn;
+    // small tiles pay more LDS / L2 traffic per MFMA
+    cost *= 1.0 + 24.0 / c.bm + 24.0 / c.bn;
+    if (cost < best_cost) {
+      best_cost = cost;
+      best = c.cfg;
+    }
+  }
+  return best;
 }
 
 template <int A_MODE, int EPI>
 hipError_t gemm_launch_cfg(
     hipStream_t st, const GemmArgs &g, const EpiParams &ep, int Kpad) {
+  const int cfg = choose_tile(g);
+  if (cfg_is_stream(cfg)) {
+    // A_MODE 1 (raw uint8) is shifted to int8 by the pack; 0 and 2 are copied.
+    hipError_t e = launch_pack_a(st, g.A, A_MODE == 1, g.M, g.K, g.a_pack);
+    if (e != hipSuccess)
+      return e;
+    switch (cfg) {
+    case kS256x192:
+      return gemm_launch_stream<2, 6, 3, A_MODE, EPI>(st, g, ep, Kpad);
+    case kS256x128:
+      return gemm_launch_stream<2, 4, 3, A_MODE, EPI>(st, g, ep, Kpad);
+    case kS128x192:
+      return gemm_launch_stream<1, 6, 4, A_MODE, EPI>(st, g, ep, Kpad);
+    default:
+      return gemm_launch_stream<1, 4, 4, A_MODE, EPI>(st, g, ep, Kpad);
+    }
+  }
   const bool aligned = (g.K % 64 == 0) && ((((uintptr_t)g.A) & 15) == 0);
   if (!aligned) {
     // Byte-wise staging of A for odd K or a misaligned A.
@@ -483,14 +859,9 @@ hipError_t gemm_launch_cfg(
             tiles_m, tiles_n);
     return hipGetLastError();
   }
-  switch (choose_tile(g)) {
-  case kT256x256:
-    return gemm_launch_tile<256, 256, 2, 4, 1, A_MODE, EPI>(st, g, ep, Kpad);
-  case kT256x128:
+  if (cfg == kT256x128)
     return gemm_launch_tile<256, 128, 2, 2, 2, A_MODE, EPI>(st, g, ep, Kpad);
-  default:
-    return gemm_launch_tile<128, 128, 2, 2, 3, A_MODE, EPI>(st, g, ep, Kpad);
-  }
+  return gemm_launch_tile<128, 128, 2, 2, 3, A_MODE, EPI>(st, g, ep, Kpad);
 }
 
 template <int A_MODE>
@@ -525,6 +896,21 @@ hipError_t launch_pack_b(hipStream_t s, const void *B, bool b_unsigned,
     k_pack_b<false><<<grid, 256, 0, s>>>(
         (const uint8_t *)B, K, N, Kpad, Bt, colsum);
   return hipGetLastError();
+}
+
+size_t gemm_a_pack_bytes(int64_t M, int64_t K, int64_t N) {
+  // The packed copy pays off once there are enough rows and columns for the
+  // large tiles; below that the kernels that stage A through LDS are used.
+  if (M < 128 || N < 128 || K < 64)
+    return 0;
+  // Measured on MI355X: below ~3e10 multiply-accumulates the extra pass over A
+  // and the single round of large tiles cost more than they save.
+  const char *force = getenv("OM_MI355X_GEMM_TILE");
+  if (!(force && force[0]) && (double)M * (double)N * (double)K < 3e10)
+    return 0;
+  const int64_t KT = round_up(K, kGemmBK) / kGemmBK;
+  const int64_t MT = (M + 31) / 32;
+  return (size_t)(MT * KT * 2048);
 }
 
 hipError_t launch_rowsum_a(hipStream_t s, const void *A, bool a_unsigned,
@@ -562,6 +948,8 @@ hipError_t launch_gemm(hipStream_t s, const GemmArgs &g) {
   ep.b_unsigned = g.b_unsigned;
   ep.y_unsigned = g.y_unsigned;
   ep.narrow = (int)g.narrow;
+  ep.group = 8;
+  ep.xcd = 1;
   const int a_mode = g.a_preshifted ? 2 : (g.a_unsigned ? 1 : 0);
   switch (a_mode) {
   case 0:

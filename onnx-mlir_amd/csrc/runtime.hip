@@ -650,6 +650,8 @@ void run_matmul(const MatmulSpec &sp) {
     g.narrow = sp.narrow;
   }
   g.out = call.out(y);
+  if (const size_t pb = gemm_a_pack_bytes(M, K, N))
+    g.a_pack = (uint8_t *)call.temp(pb);
   if (call.ok)
     call.check(launch_gemm(call.c.stream, g), sp.op);
   call.finish();
@@ -918,6 +920,8 @@ void om_mi355x_DynQuantMatMulDequant(OMTensor *y_t, const OMTensor *x_t,
   g.b_scale = (const float *)call.in(bs);
   g.b_scale_len = bs.numel;
   g.out = call.out(y);
+  if (const size_t pb = gemm_a_pack_bytes(M, K, N))
+    g.a_pack = (uint8_t *)call.temp(pb);
   if (call.ok)
     call.check(launch_gemm(call.c.stream, g), op);
   call.finish();

@@ -253,6 +253,41 @@ def test_matmulinteger_shapes(rt, oracle, M, K, N):
     assert np.array_equal(rt.MatMulInteger(A, B, azr, bzc), want)
 
 
+@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 4, 5])
+def test_every_gemm_kernel_configuration(rt, oracle, cfg, monkeypatch):
+    """The tile / kernel choice is a heuristic; force each configuration in turn
+    (0-1 stage A through LDS, 2-5 stream a fragment-packed copy of A) on shapes
+    with ragged edges, every operand type and all zero-point forms."""
+    monkeypatch.setenv("OM_MI355X_GEMM_TILE", str(cfg))
+    rng = np.random.default_rng(100 + cfg)
+    for (M, K, N), adt, bdt in (((300, 200, 500), np.uint8, np.int8), ((129, 64, 193), np.int8, np.uint8),
+                                ((513, 1000, 257), np.uint8, np.uint8), ((256, 192, 384), np.int8, np.int8)):
+        A, B = _rand_q(rng, adt, (M, K)), _rand_q(rng, bdt, (K, N))
+        az, bz = _rand_q(rng, adt, (M,)), _rand_q(rng, bdt, (N,))
+        assert np.array_equal(rt.MatMulInteger(A, B, az, bz), oracle.matmul_integer(A, B, az, bz))
+        assert np.array_equal(rt.MatMulInteger(A, B, az[:1], None), oracle.matmul_integer(A, B, az[:1], None))
+    c = wl.config3(300, 256, 520)
+    want = oracle.qlinear_matmul(c["A"], c["a_scale"], c["a_zp"], c["B"], c["b_scale"], c["b_zp"],
+                                 c["y_scale"], c["y_zp"], oracle_lib.WRAP)
+    assert np.array_equal(rt.QLinearMatMul(c["A"], c["a_scale"], c["a_zp"], c["B"], c["b_scale"], c["b_zp"],
+                                           c["y_scale"], c["y_zp"], rt.WRAP), want)
+    x = rng.normal(0, 1, (260, 320)).astype(np.float32)
+    W = _rand_q(rng, np.int8, (320, 200))
+    ws = rng.uniform(1e-3, 1e-2, 200).astype(np.float32)
+    aq, a_s, a_zp = oracle.dynamic_quantize_linear(x)
+    wantf = oracle.dequant_epilogue(oracle.matmul_integer(aq, W, a_zp, None), a_s, ws)
+    assert same_f32(rt.DynQuantMatMulDequant(x, W, None, ws), wantf)
+
+
+def test_large_gemm_takes_the_streamed_path(rt, oracle):
+    # big enough for the heuristic to pick the packed-A kernels on its own
+    rng = np.random.default_rng(77)
+    M, K, N = 1024, 2048, 16000
+    A, B = _rand_q(rng, np.uint8, (M, K)), _rand_q(rng, np.int8, (K, N))
+    az = _rand_q(rng, np.uint8, ())
+    assert np.array_equal(rt.MatMulInteger(A, B, az, None), oracle.matmul_integer(A, B, az, None, passes=True))
+
+
 def test_matmulinteger_extreme_values_wrap(rt, oracle):
     # all-255 x all-(-128) with large K: the int32 accumulator must wrap, not saturate
     M, K, N = 64, 70000, 64
