@@ -591,6 +591,121 @@ __global__ __launch_bounds__(256, (TM == 1 ? 2 : 1)) void k_gemm_i8_stream(
   gemm_epilogue<TM, TN, A_MODE, EPI>(acc, mrow0, n0, M, N, K, ep);
 }
 
+// ---- skinny GEMM (M <= 16): weight streaming -------------------------------
+// With at most 16 rows the product is bound by reading the weights once, so
+// the kernel is organised around keeping many KiB of Bt in flight per CU and
+// nothing else: a block owns 32 output columns, its 8 waves split K between
+// them, and each wave streams its slice of the 32 Bt rows straight from
+// global memory into v_mfma_i32_16x16x64_i8 operands (lane = column, 16
+// K-bytes per lane; a wave instruction reads 16 rows x 64 contiguous bytes).
+// The tiny A operand (rows padded to 16 with zeros) comes from L2.  The eight
+// partial 16x32 results are summed through LDS and the usual epilogue runs on
+// the sum.  No LDS staging, no barrier in the K loop.
+template <int NG, int A_MODE, int EPI>
+__global__ __launch_bounds__(512) void k_gemm_i8_skinny(
+    const uint8_t *__restrict__ A, const int8_t *__restrict__ Bt, int M, int N,
+    int K, int Kpad, EpiParams ep) {
+  constexpr int WAVES = 8, U = 8;
+  __shared__ int32_t part[WAVES][NG][4][64];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int l16 = lane & 15;
+  const int lq = lane >> 4; // K quarter of the 64-byte step
+  const int n0 = blockIdx.x * 16 * NG;
+
+  const int KT = Kpad / BK;
+  const int per = (KT + WAVES - 1) / WAVES;
+  const int kt_begin = wave * per;
+  const int kt_end = (kt_begin + per < KT) ? kt_begin + per : KT;
+
+  // Row l16 of A (clamped; rows >= M are zeroed after the load).
+  const bool row_ok = l16 < M;
+  const uint8_t *__restrict__ ap =
+      A + (int64_t)(row_ok ? l16 : 0) * K + (lq * 16 < K ? lq * 16 : 0);
+  const int8_t *__restrict__ bp0 = Bt + (int64_t)(n0 + l16) * Kpad + lq * 16;
+  const int8_t *__restrict__ bp1 = bp0 + (int64_t)(NG > 1 ? 16 : 0) * Kpad;
+  const int klim = K - lq * 16; // chunks starting at or past this are absent
+
+  v4i acc0 = {0, 0, 0, 0}, acc1 = {0, 0, 0, 0};
+  constexpr int kFill = (A_MODE == 1) ? (int)0x80808080 : 0;
+  for (int kt = kt_begin; kt < kt_end; kt += U) {
+    v4i a[U], b0[U], b1[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      // steps past this wave's slice reload its last step and are discarded
+      const int s = (kt + u < kt_end) ? kt + u : kt_end - 1;
+      const int k0 = s * BK;
+      const int ka = (k0 < klim) ? k0 : 0; // in bounds whatever K is
+      a[u] = *(const v4i *)(ap + ka);
+      if (!(row_ok && k0 < klim))
+        a[u] = (v4i){kFill, kFill, kFill, kFill};
+      b0[u] = *(const v4i *)(bp0 + k0);
+      if (NG > 1)
+        b1[u] = *(const v4i *)(bp1 + k0);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (kt + u < kt_end) {
+        v4i av = a[u];
+        if (A_MODE == 1)
+          av ^= (v4i){(int)0x80808080, (int)0x80808080, (int)0x80808080,
+              (int)0x80808080};
+        acc0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, b0[u], acc0, 0, 0, 0);
+        if (NG > 1)
+          acc1 =
+              __builtin_amdgcn_mfma_i32_16x16x64_i8(av, b1[u], acc1, 0, 0, 0);
+      }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    part[wave][0][r][lane] = acc0[r];
+    if (NG > 1)
+      part[wave][1][r][lane] = acc1[r];
+  }
+  __syncthreads();
+
+  // 16x16 accumulator layout: lane holds column (lane & 15); register r holds
+  // row 4*(lane/16) + r.  Thread t finishes element (g, r, lane) = t.
+  const int g = tid >> 8, r = (tid >> 6) & 3;
+  if (g >= NG)
+    return;
+  uint32_t y = 0;
+#pragma unroll
+  for (int w = 0; w < WAVES; ++w)
+    y += (uint32_t)part[w][g][r][lane];
+  const int m = 4 * lq + r;
+  const int n = n0 + g * 16 + l16;
+  if (m >= M || n >= N)
+    return;
+
+  constexpr bool A_OFF = (A_MODE != 0);
+  const int32_t oa = A_OFF ? 128 : 0;
+  const int32_t ob = ep.b_unsigned ? 128 : 0;
+  int32_t da = oa, db = ob, rs = 0;
+  if (ep.a_zp_len > 0)
+    da = oa - load_zp_i32(ep.a_zp, A_OFF, ep.a_zp_len > 1 ? m : 0);
+  if (ep.b_zp_len > 0)
+    db = ob - load_zp_i32(ep.b_zp, ep.b_unsigned, ep.b_zp_len > 1 ? n : 0);
+  if (ep.rowsum)
+    rs = ep.rowsum[m];
+  y += (uint32_t)da * (uint32_t)ep.colsum[n];
+  y += (uint32_t)db * (uint32_t)rs;
+  y += (uint32_t)K * (uint32_t)da * (uint32_t)db;
+  float sj = 0.0f;
+  int32_t yz = 0;
+  if (EPI != kEpiI32) {
+    sj = ep.a_scale[0] * ep.b_scale[ep.b_scale_len == 1 ? 0 : n];
+    if (EPI == kEpiQ8) {
+      sj = sj / ep.y_scale[0];
+      yz = load_zp_i32(ep.y_zp, ep.y_unsigned, 0);
+    }
+  }
+  store_one<EPI>(ep, (int64_t)m * N + n, y, sj, yz);
+}
+
 // ---- pack B ---------------------------------------------------------------
 // One block transposes a 64(k) x 64(n) tile through LDS and adds the tile's
 // column sums into colsum with int32 atomics (integer adds commute, so the
@@ -831,6 +946,23 @@ int choose_tile(const GemmArgs &g) {
 template <int A_MODE, int EPI>
 hipError_t gemm_launch_cfg(
     hipStream_t st, const GemmArgs &g, const EpiParams &ep, int Kpad) {
+  const char *force = getenv("OM_MI355X_GEMM_TILE");
+  if (g.M <= 16 && g.K % 16 == 0 && ((((uintptr_t)g.A) & 15) == 0) &&
+      !(force && force[0])) {
+    // 32 columns per block halves the reads of A (measured faster whenever
+    // that still gives every CU a block); 16 columns for narrower outputs.
+    if ((g.N + 31) / 32 >= 256)
+      k_gemm_i8_skinny<2, A_MODE, EPI>
+          <<<dim3((unsigned)((g.N + 31) / 32)), 512, 0, st>>>(
+              (const uint8_t *)g.A, g.Bt, (int)g.M, (int)g.N, (int)g.K, Kpad,
+              ep);
+    else
+      k_gemm_i8_skinny<1, A_MODE, EPI>
+          <<<dim3((unsigned)((g.N + 15) / 16)), 512, 0, st>>>(
+              (const uint8_t *)g.A, g.Bt, (int)g.M, (int)g.N, (int)g.K, Kpad,
+              ep);
+    return hipGetLastError();
+  }
   const int cfg = choose_tile(g);
   if (cfg_is_stream(cfg)) {
     // A_MODE 1 (raw uint8) is shifted to int8 by the pack; 0 and 2 are copied.

@@ -490,6 +490,55 @@ __global__ __launch_bounds__(kThreads) void k_minmax_params(
   }
 }
 
+// Small tensors (the activations of a decode step): one block does the whole
+// op -- every thread keeps its elements in registers across the min / max
+// reduction, so x is read once and there is a single launch.
+constexpr int kSmallThreads = 1024;
+constexpr int kSmallPerThread = 16; // float4 x 4
+constexpr int64_t kSmallMax = (int64_t)kSmallThreads * kSmallPerThread;
+
+__global__ __launch_bounds__(kSmallThreads) void k_dql_small(
+    const float *__restrict__ x, int64_t n, uint8_t *__restrict__ y,
+    float *__restrict__ scale_out, uint8_t *__restrict__ zp_out,
+    uint32_t flip) {
+  __shared__ float s_lo[kSmallThreads / 64], s_hi[kSmallThreads / 64];
+  float v[kSmallPerThread];
+  float lo = __builtin_inff(), hi = -__builtin_inff();
+#pragma unroll
+  for (int j = 0; j < kSmallPerThread; ++j) {
+    const int64_t e = (int64_t)j * kSmallThreads + threadIdx.x;
+    v[j] = e < n ? x[e] : __builtin_nanf(""); // NaN is neutral for minnum/maxnum
+    lo = __builtin_fminf(lo, v[j]);
+    hi = __builtin_fmaxf(hi, v[j]);
+  }
+  lo = wave_min(lo);
+  hi = wave_max(hi);
+  if ((threadIdx.x & 63) == 0) {
+    s_lo[threadIdx.x >> 6] = lo;
+    s_hi[threadIdx.x >> 6] = hi;
+  }
+  __syncthreads();
+  lo = s_lo[0];
+  hi = s_hi[0];
+#pragma unroll
+  for (int w = 1; w < kSmallThreads / 64; ++w) {
+    lo = __builtin_fminf(lo, s_lo[w]);
+    hi = __builtin_fmaxf(hi, s_hi[w]);
+  }
+  float scale, zpf;
+  dynamic_params(lo, hi, scale, zpf);
+  if (threadIdx.x == 0) {
+    scale_out[0] = scale;
+    zp_out[0] = (uint8_t)(uint32_t)zpf;
+  }
+#pragma unroll
+  for (int j = 0; j < kSmallPerThread; ++j) {
+    const int64_t e = (int64_t)j * kSmallThreads + threadIdx.x;
+    if (e < n)
+      y[e] = (uint8_t)(quant_one<false, true>(v[j], scale, zpf) ^ (flip & 0xFFu));
+  }
+}
+
 __global__ __launch_bounds__(kThreads) void k_fill_u32(
     uint32_t *__restrict__ p, int64_t n, uint32_t v) {
   for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < n;
@@ -676,6 +725,11 @@ hipError_t launch_dynamic_quantize(hipStream_t s, const DqlScratch &scratch,
     bool y_shift) {
   if (n == 0)
     return hipSuccess;
+  if (n <= kSmallMax) {
+    k_dql_small<<<1, kSmallThreads, 0, s>>>(
+        x, n, y, scale, zp, y_shift ? 0x80808080u : 0u);
+    return hipGetLastError();
+  }
   int grid = stream_grid(n >> 2, kThreads * kUnroll);
   if (grid > kDqlMaxBlocks)
     grid = kDqlMaxBlocks;
