@@ -19,6 +19,8 @@
 
 #include "om_kernels.h"
 
+#include <stdlib.h>
+
 namespace om {
 
 namespace {
@@ -159,6 +161,89 @@ __global__ __launch_bounds__(kThreads) void k_quant_lastaxis(
       for (int j = 0; j < ncol; ++j)
         y[r * C + c0 + j] =
             (uint8_t)quant_one<SIGNED, HAS_ZP>(x[r * C + c0 + j], s[j], z[j]);
+  }
+}
+
+// ---- per-axis quantize, innermost axis, rows not 16-byte aligned -----------
+// When C % 4 != 0 the rows of a [rows, C] tensor start at odd alignments and
+// the row-walking kernel above would issue misaligned 16-byte loads and
+// misaligned 4-byte stores.  This kernel walks the flat array instead, so
+// every data access is aligned, and carries the column of each float4 along
+// incrementally (one modulo per thread at the start, then add-and-wrap).
+// Scale and zero point are fetched per float4 from L1 / L2 (they are tiny);
+// the rare float4 that straddles the end of a row takes a scalar path.
+template <bool SIGNED, bool HAS_ZP>
+__global__ __launch_bounds__(kThreads) void k_quant_flat_axis(
+    const float *__restrict__ x, uint8_t *__restrict__ y, int64_t n, uint32_t C,
+    const float *__restrict__ scale, const void *__restrict__ zp) {
+  const int64_t nvec = n >> 2;
+  const f4a *__restrict__ x4 = (const f4a *)x;
+  uint32_t *__restrict__ y4 = (uint32_t *)y;
+  const int64_t step = (int64_t)gridDim.x * (kThreads * kUnroll);
+  const uint32_t dstep = (uint32_t)((step * 4) % C);
+  const uint32_t dj = (uint32_t)((kThreads * 4) % C);
+  int64_t base = (int64_t)blockIdx.x * (kThreads * kUnroll);
+  uint32_t c0 = (uint32_t)(((base + threadIdx.x) * 4) % C);
+  const uint8_t *__restrict__ zpb = (const uint8_t *)zp;
+  for (; base < nvec; base += step) {
+    f4a v[kUnroll];
+    int64_t idx[kUnroll];
+    uint32_t c[kUnroll];
+    uint32_t cj = c0;
+#pragma unroll
+    for (int j = 0; j < kUnroll; ++j) {
+      idx[j] = base + j * kThreads + threadIdx.x;
+      c[j] = cj;
+      cj += dj;
+      cj -= (cj >= C) ? C : 0;
+      if (idx[j] < nvec)
+        v[j] = __builtin_nontemporal_load(&x4[idx[j]]);
+    }
+#pragma unroll
+    for (int j = 0; j < kUnroll; ++j) {
+      if (idx[j] >= nvec)
+        continue;
+      float s[4], z[4];
+      if (c[j] + 4 <= C) {
+        const f4u sv = *(const f4u *)(scale + c[j]);
+        s[0] = sv.x; s[1] = sv.y; s[2] = sv.z; s[3] = sv.w;
+        if (HAS_ZP) {
+          const uint32_t zw = *(const u32_a1 *)(zpb + c[j]);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const uint32_t b = (zw >> (8 * e)) & 0xFFu;
+            z[e] = SIGNED ? (float)(int32_t)(int8_t)b : (float)b;
+          }
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          uint32_t ce = c[j] + e;
+          ce -= (ce >= C) ? C : 0;
+          s[e] = scale[ce];
+          if (HAS_ZP)
+            z[e] = load_zp_f32<SIGNED>(zp, ce);
+        }
+      }
+      if (!HAS_ZP)
+        z[0] = z[1] = z[2] = z[3] = 0.0f;
+      const uint32_t b0 = quant_one<SIGNED, HAS_ZP>(v[j].x, s[0], z[0]);
+      const uint32_t b1 = quant_one<SIGNED, HAS_ZP>(v[j].y, s[1], z[1]);
+      const uint32_t b2 = quant_one<SIGNED, HAS_ZP>(v[j].z, s[2], z[2]);
+      const uint32_t b3 = quant_one<SIGNED, HAS_ZP>(v[j].w, s[3], z[3]);
+      __builtin_nontemporal_store(
+          b0 | (b1 << 8) | (b2 << 16) | (b3 << 24), &y4[idx[j]]);
+    }
+    c0 += dstep;
+    c0 -= (c0 >= C) ? C : 0;
+  }
+  if (blockIdx.x == 0) {
+    const int64_t e = (nvec << 2) + threadIdx.x;
+    if (e < n) {
+      const uint32_t ce = (uint32_t)(e % C);
+      const float zf = HAS_ZP ? load_zp_f32<SIGNED>(zp, ce) : 0.0f;
+      y[e] = (uint8_t)quant_one<SIGNED, HAS_ZP>(x[e], scale[ce], zf);
+    }
   }
 }
 
@@ -335,6 +420,81 @@ __global__ __launch_bounds__(kThreads) void k_dequant_lastaxis(
   }
 }
 
+// 8-bit input, innermost axis, C % 4 != 0: flat walk, aligned accesses, column
+// carried incrementally (see k_quant_flat_axis).
+template <int KIND, bool HAS_ZP>
+__global__ __launch_bounds__(kThreads) void k_dequant8_flat_axis(
+    const uint8_t *__restrict__ x, float *__restrict__ y, int64_t n, uint32_t C,
+    const float *__restrict__ scale, const void *__restrict__ zp) {
+  const int64_t nvec = n >> 2;
+  const uint32_t *__restrict__ x4 = (const uint32_t *)x;
+  f4a *__restrict__ y4 = (f4a *)y;
+  const int64_t step = (int64_t)gridDim.x * (kThreads * kUnroll);
+  const uint32_t dstep = (uint32_t)((step * 4) % C);
+  const uint32_t dj = (uint32_t)((kThreads * 4) % C);
+  int64_t base = (int64_t)blockIdx.x * (kThreads * kUnroll);
+  uint32_t c0 = (uint32_t)(((base + threadIdx.x) * 4) % C);
+  const uint8_t *__restrict__ zpb = (const uint8_t *)zp;
+  for (; base < nvec; base += step) {
+    uint32_t w[kUnroll];
+    int64_t idx[kUnroll];
+    uint32_t c[kUnroll];
+    uint32_t cj = c0;
+#pragma unroll
+    for (int j = 0; j < kUnroll; ++j) {
+      idx[j] = base + j * kThreads + threadIdx.x;
+      c[j] = cj;
+      cj += dj;
+      cj -= (cj >= C) ? C : 0;
+      if (idx[j] < nvec)
+        w[j] = __builtin_nontemporal_load(&x4[idx[j]]);
+    }
+#pragma unroll
+    for (int j = 0; j < kUnroll; ++j) {
+      if (idx[j] >= nvec)
+        continue;
+      float s[4], z[4];
+      if (c[j] + 4 <= C) {
+        const f4u sv = *(const f4u *)(scale + c[j]);
+        s[0] = sv.x; s[1] = sv.y; s[2] = sv.z; s[3] = sv.w;
+        if (HAS_ZP) {
+          const uint32_t zw = *(const u32_a1 *)(zpb + c[j]);
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            z[e] = q_to_f32<KIND>(zw >> (8 * e));
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          uint32_t ce = c[j] + e;
+          ce -= (ce >= C) ? C : 0;
+          s[e] = scale[ce];
+          if (HAS_ZP)
+            z[e] = load_q_zp_f32<KIND>(zp, ce);
+        }
+      }
+      if (!HAS_ZP)
+        z[0] = z[1] = z[2] = z[3] = 0.0f;
+      f4a o;
+      o.x = dq_one<HAS_ZP>(q_to_f32<KIND>(w[j]), s[0], z[0]);
+      o.y = dq_one<HAS_ZP>(q_to_f32<KIND>(w[j] >> 8), s[1], z[1]);
+      o.z = dq_one<HAS_ZP>(q_to_f32<KIND>(w[j] >> 16), s[2], z[2]);
+      o.w = dq_one<HAS_ZP>(q_to_f32<KIND>(w[j] >> 24), s[3], z[3]);
+      __builtin_nontemporal_store(o, &y4[idx[j]]);
+    }
+    c0 += dstep;
+    c0 -= (c0 >= C) ? C : 0;
+  }
+  if (blockIdx.x == 0) {
+    const int64_t e = (nvec << 2) + threadIdx.x;
+    if (e < n) {
+      const uint32_t ce = (uint32_t)(e % C);
+      const float zf = HAS_ZP ? load_q_zp_f32<KIND>(zp, ce) : 0.0f;
+      y[e] = dq_one<HAS_ZP>(q_to_f32<KIND>(x[e]), scale[ce], zf);
+    }
+  }
+}
+
 // Any element kind, [outer, channels, inner]: one element per lane.
 template <int KIND, bool HAS_ZP>
 __global__ __launch_bounds__(kThreads) void k_dequant_general(
@@ -415,24 +575,28 @@ __global__ __launch_bounds__(kThreads) void k_minmax_params(
     uint8_t *__restrict__ zp_out) {
   float lo = __builtin_inff(), hi = -__builtin_inff();
   const int64_t nvec = n >> 2;
-  const float4 *__restrict__ x4 = (const float4 *)x;
+  const f4a *__restrict__ x4 = (const f4a *)x;
   const bool aligned = (((uintptr_t)x) & 15) == 0;
   if (aligned) {
-    const int64_t step = (int64_t)gridDim.x * (kThreads * kUnroll);
-    for (int64_t base = (int64_t)blockIdx.x * (kThreads * kUnroll);
+    // Read-only pass: eight 16-byte loads in flight per lane, streamed past
+    // the caches (the data is not touched again before the quantize pass has
+    // walked the whole tensor).
+    constexpr int kMU = 8;
+    const int64_t step = (int64_t)gridDim.x * (kThreads * kMU);
+    for (int64_t base = (int64_t)blockIdx.x * (kThreads * kMU);
          base < nvec; base += step) {
-      float4 v[kUnroll];
+      f4a v[kMU];
 #pragma unroll
-      for (int j = 0; j < kUnroll; ++j) {
+      for (int j = 0; j < kMU; ++j) {
         const int64_t idx = base + j * kThreads + threadIdx.x;
         if (idx < nvec)
-          v[j] = x4[idx];
+          v[j] = __builtin_nontemporal_load(&x4[idx]);
         else
-          v[j] = make_float4(__builtin_nanf(""), __builtin_nanf(""),
-              __builtin_nanf(""), __builtin_nanf(""));
+          v[j] = (f4a){__builtin_nanf(""), __builtin_nanf(""),
+              __builtin_nanf(""), __builtin_nanf("")};
       }
 #pragma unroll
-      for (int j = 0; j < kUnroll; ++j) {
+      for (int j = 0; j < kMU; ++j) {
         // The NaN filler above is neutral: minnum / maxnum ignore NaN.
         lo = __builtin_fminf(lo, __builtin_fminf(__builtin_fminf(v[j].x, v[j].y),
                                      __builtin_fminf(v[j].z, v[j].w)));
@@ -586,6 +750,18 @@ hipError_t quantize_dispatch(hipStream_t st, const float *x, int64_t outer,
   }
   if (flip != 0)
     return hipErrorInvalidValue;
+  if (inner == 1 && channels > 1 && channels % 4 != 0 && channels >= 4 &&
+      channels < ((int64_t)1 << 31) && ((((uintptr_t)x) & 15) == 0) &&
+      ((((uintptr_t)y) & 3) == 0)) {
+    const int grid = stream_grid(n >> 2, kThreads * kUnroll);
+    if (has_zp)
+      k_quant_flat_axis<SIGNED, true><<<grid, kThreads, 0, st>>>(
+          x, yo, n, (uint32_t)channels, scale, zp);
+    else
+      k_quant_flat_axis<SIGNED, false><<<grid, kThreads, 0, st>>>(
+          x, yo, n, (uint32_t)channels, scale, zp);
+    return hipGetLastError();
+  }
   if (inner == 1 && channels > 1) {
     const int64_t rows = outer, C = channels;
     const int64_t col_blocks = (C + kThreads * 4 - 1) / (kThreads * 4);
@@ -647,6 +823,20 @@ hipError_t dequantize_dispatch(hipStream_t st, const void *x, int64_t outer,
     else
       k_dequant8_flat<KIND, false>
           <<<grid, kThreads, 0, st>>>(xi, y, n, scale, zp);
+    return hipGetLastError();
+  }
+  if (KIND != kI32 && inner == 1 && channels > 1 && channels % 4 != 0 &&
+      channels >= 4 && channels < ((int64_t)1 << 31) &&
+      ((((uintptr_t)x) & 3) == 0) && ((((uintptr_t)y) & 15) == 0)) {
+    const int grid = stream_grid(n >> 2, kThreads * kUnroll);
+    if (has_zp)
+      k_dequant8_flat_axis<(KIND == kI32 ? kU8 : KIND), true>
+          <<<grid, kThreads, 0, st>>>(
+              (const uint8_t *)x, y, n, (uint32_t)channels, scale, zp);
+    else
+      k_dequant8_flat_axis<(KIND == kI32 ? kU8 : KIND), false>
+          <<<grid, kThreads, 0, st>>>(
+              (const uint8_t *)x, y, n, (uint32_t)channels, scale, zp);
     return hipGetLastError();
   }
   if (inner == 1 && channels > 1) {
@@ -730,9 +920,11 @@ hipError_t launch_dynamic_quantize(hipStream_t s, const DqlScratch &scratch,
         x, n, y, scale, zp, y_shift ? 0x80808080u : 0u);
     return hipGetLastError();
   }
-  int grid = stream_grid(n >> 2, kThreads * kUnroll);
-  if (grid > kDqlMaxBlocks)
-    grid = kDqlMaxBlocks;
+  // Few, long-lived blocks: every block ends with a device-scope release /
+  // acquire pair (cache write-back and invalidate), which is not free.
+  int grid = stream_grid(n >> 2, kThreads * 8);
+  if (grid > 512)
+    grid = 512;
   k_minmax_params<<<grid, kThreads, 0, s>>>(x, n, scratch.partial_min,
       scratch.partial_max, scratch.counter, scale, zp);
   hipError_t e = hipGetLastError();
