@@ -32,6 +32,12 @@ INT8_PEAK_TOPS = 5000.0      # MI355X published dense int8 MFMA rate (no sparsit
 
 METRIC = "int8 MatMulInteger TOPS (% MFMA peak) + Q/DQ GB/s (% HBM), 1 MI355X"
 
+# HBM bytes per launch of the headline kernel, measured with rocprofv3 --pmc
+# (FETCH_SIZE and WRITE_SIZE, one run each, scaled by what the same counters
+# read for a 1 GiB device-to-device copy: FETCH_SIZE x2.0, WRITE_SIZE x1.0);
+# the summary of those runs is profiles/k_gemm_i8_config4_ffn_up.md.
+TRAFFIC_BYTES = {"k_gemm_i8 config4 FFN-up f32": int((7797.4 * 2.0 + 49152.0) * 1024)}
+
 
 def timed(rt, fn, steps, warmup):
     """Returns (host seconds per step, event milliseconds per step)."""
@@ -267,7 +273,12 @@ def main():
                                "output, operands resident in HBM, weights packed once"},
         "roofline": {"bound": "mfma", "achieved": main_res["kernel_tops"], "peak": INT8_PEAK_TOPS,
                      "unit": "TOP/s", "frac": main_res["kernel_tops"] / INT8_PEAK_TOPS,
-                     "traffic": None, "kernel": "k_gemm_i8", "kernel_ms": main_res["kernel_ms"],
+                     "traffic": TRAFFIC_BYTES.get("k_gemm_i8 config4 FFN-up f32") if epi == "f32" else None,
+                     "kernel": "k_gemm_i8<128,128>", "kernel_ms": main_res["kernel_ms"],
+                     "algorithmic_ops": main_res["ops"],
+                     "algorithmic_hbm_bytes": main_res["hbm_bytes_algorithmic"],
+                     "hbm_frac_at_algorithmic_bytes": main_res["hbm_bytes_algorithmic"]
+                     / (main_res["kernel_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS,
                      "hbm_bound_tops": main_res["ops"] / (main_res["hbm_bytes_algorithmic"] / (HBM_PEAK_GBS * 1e9)) / 1e12},
         "cpu_baseline": cpu,
         "device": info,
