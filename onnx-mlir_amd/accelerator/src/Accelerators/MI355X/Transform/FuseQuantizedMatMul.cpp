@@ -1,0 +1,189 @@
+/*
+ * SPDX-License-Identifier: Apache-2.0
+ */
+
+//===---------------------- FuseQuantizedMatMul.cpp -----------------------===//
+//
+// Dynamic quantisation of a linear layer is exported as the chain
+//
+//   %aq, %as, %azp = DynamicQuantizeLinear(%x)
+//   %acc           = MatMulInteger(%aq, %W, %azp, %wzp)
+//   %f             = Cast(%acc) {to = f32}
+//   %s             = Mul(%as, %ws)
+//   %y             = Mul(%f, %s)
+//
+// On the CPU that is five ops and four intermediate tensors.  The MI355X
+// runtime has one entry point for the last four (the int32 accumulator never
+// reaches memory) and one for all five (the 8-bit activation stays on the
+// device).  This pass replaces the chain by an `onnx.Custom` naming that entry
+// point; the ONNX-to-Krnl patterns of the accelerator lower it.
+//
+// Only the association `f32(acc) * (a_scale * b_scale)` is matched.  The other
+// one the reference knows, `(f32(acc) * a_scale) * b_scale`
+// (src/Accelerators/NNPA/Conversion/ONNXToZHigh/ONNXToZHigh.cpp:895-912),
+// rounds differently and is left to the unfused ops so that results stay
+// bit-identical to the CPU's.
+//
+//===----------------------------------------------------------------------===//
+
+#include "mlir/Dialect/Func/IR/FuncOps.h"
+#include "mlir/IR/PatternMatch.h"
+#include "mlir/Pass/Pass.h"
+#include "mlir/Transforms/GreedyPatternRewriteDriver.h"
+
+#include "src/Accelerators/MI355X/Transform/MI355XPasses.hpp"
+#include "src/Dialect/ONNX/ONNXOps.hpp"
+#include "src/Dialect/ONNX/ONNXOps/OpHelper.hpp"
+
+using namespace mlir;
+
+namespace onnx_mlir {
+namespace {
+
+bool isF32Tensor(Value v) {
+  auto type = dyn_cast<RankedTensorType>(v.getType());
+  return type && type.getElementType().isF32();
+}
+
+/// A tensor that statically holds exactly one element.
+bool isSingleElement(Value v) {
+  auto type = dyn_cast<RankedTensorType>(v.getType());
+  return type && type.hasStaticShape() && type.getNumElements() == 1;
+}
+
+/// Scale of the right-hand side: one value, or one per column of `b`.
+bool isColumnScale(Value scale, Value b) {
+  if (isSingleElement(scale))
+    return true;
+  auto scaleType = dyn_cast<RankedTensorType>(scale.getType());
+  auto bType = dyn_cast<RankedTensorType>(b.getType());
+  if (!scaleType || !bType || scaleType.getRank() != 1 || bType.getRank() < 2)
+    return false;
+  int64_t n = bType.getShape().back();
+  return !ShapedType::isDynamic(n) && scaleType.getShape()[0] == n;
+}
+
+struct Chain {
+  ONNXMatMulIntegerOp matmul;
+  ONNXCastOp cast;
+  ONNXMulOp scaleProduct;
+  Value aScale, bScale;
+};
+
+/// Match `Mul(Cast(MatMulInteger), Mul(sa, sb))` in either operand order.  The
+/// intermediate values must have no other user: they disappear.
+bool matchChain(ONNXMulOp mul, Chain &chain) {
+  for (int swap = 0; swap < 2; ++swap) {
+    Value accSide = swap ? mul.getB() : mul.getA();
+    Value scaleSide = swap ? mul.getA() : mul.getB();
+    auto cast = accSide.getDefiningOp<ONNXCastOp>();
+    auto product = scaleSide.getDefiningOp<ONNXMulOp>();
+    if (!cast || !product || !cast->hasOneUse() || !product->hasOneUse())
+      continue;
+    if (!isF32Tensor(cast.getResult()))
+      continue;
+    auto matmul = cast.getInput().getDefiningOp<ONNXMatMulIntegerOp>();
+    if (!matmul || !matmul->hasOneUse())
+      continue;
+    // The accumulator tensor must already have the shape of the result: a
+    // scale that broadcasts the result to more dimensions is not this chain.
+    auto accType = dyn_cast<RankedTensorType>(matmul.getResult().getType());
+    auto outType = dyn_cast<RankedTensorType>(mul.getResult().getType());
+    if (!accType || !outType || accType.getShape() != outType.getShape())
+      continue;
+    // a_scale is per tensor; b_scale per tensor or per column.
+    for (int swapScale = 0; swapScale < 2; ++swapScale) {
+      Value sa = swapScale ? product.getB() : product.getA();
+      Value sb = swapScale ? product.getA() : product.getB();
+      if (!isF32Tensor(sa) || !isF32Tensor(sb) || !isSingleElement(sa) ||
+          !isColumnScale(sb, matmul.getB()))
+        continue;
+      chain = {matmul, cast, product, sa, sb};
+      return true;
+    }
+  }
+  return false;
+}
+
+Value noneIfAbsent(PatternRewriter &rewriter, Location loc, Value v) {
+  if (v && !isNoneValue(v))
+    return v;
+  return ONNXNoneOp::create(rewriter, loc).getResult();
+}
+
+struct FuseScaledMatMulInteger : public OpRewritePattern<ONNXMulOp> {
+  using OpRewritePattern<ONNXMulOp>::OpRewritePattern;
+
+  LogicalResult matchAndRewrite(
+      ONNXMulOp mul, PatternRewriter &rewriter) const final {
+    Chain chain;
+    if (!matchChain(mul, chain))
+      return failure();
+    Location loc = mul.getLoc();
+    ONNXMatMulIntegerOp matmul = chain.matmul;
+
+    // If the left operand comes straight from DynamicQuantizeLinear of which
+    // this chain is the only consumer, take the quantisation along.
+    auto dynQuant = matmul.getA().getDefiningOp<ONNXDynamicQuantizeLinearOp>();
+    bool wholeLayer =
+        dynQuant && matmul.getA() == dynQuant.getY() &&
+        matmul.getAZeroPoint() == dynQuant.getYZeroPoint() &&
+        chain.aScale == dynQuant.getYScale() && dynQuant.getY().hasOneUse() &&
+        dynQuant.getYScale().hasOneUse() && dynQuant.getYZeroPoint().hasOneUse();
+
+    SmallVector<Value, 6> inputs;
+    StringRef callee;
+    if (wholeLayer) {
+      callee = kMI355XDynQuantMatMulDequant;
+      inputs = {dynQuant.getX(), matmul.getB(),
+          noneIfAbsent(rewriter, loc, matmul.getBZeroPoint()), chain.bScale};
+    } else {
+      callee = kMI355XMatMulIntegerDequant;
+      inputs = {matmul.getA(), matmul.getB(),
+          noneIfAbsent(rewriter, loc, matmul.getAZeroPoint()),
+          noneIfAbsent(rewriter, loc, matmul.getBZeroPoint()), chain.aScale,
+          chain.bScale};
+    }
+
+    SmallVector<NamedAttribute, 2> attrs;
+    attrs.emplace_back(
+        rewriter.getNamedAttr("function_name", rewriter.getStringAttr(callee)));
+    if (Attribute nodeName = mul->getAttr("onnx_node_name"))
+      attrs.emplace_back(rewriter.getNamedAttr("onnx_node_name", nodeName));
+    auto fused = ONNXCustomOp::create(rewriter, loc,
+        TypeRange{mul.getResult().getType()}, ValueRange(inputs), attrs);
+    rewriter.replaceOp(mul, fused.getResults());
+    // Cast, MatMulInteger, the scale product and (for the whole layer)
+    // DynamicQuantizeLinear are now dead and pure: the driver erases them.
+    return success();
+  }
+};
+
+struct FuseQuantizedMatMulForMI355XPass
+    : public PassWrapper<FuseQuantizedMatMulForMI355XPass,
+          OperationPass<func::FuncOp>> {
+  MLIR_DEFINE_EXPLICIT_INTERNAL_INLINE_TYPE_ID(FuseQuantizedMatMulForMI355XPass)
+
+  StringRef getArgument() const override {
+    return "fuse-quantized-matmul-for-mi355x";
+  }
+  StringRef getDescription() const override {
+    return "Fuse (DynamicQuantizeLinear ->) MatMulInteger -> Cast -> Mul into "
+           "one call of the MI355X runtime";
+  }
+
+  void runOnOperation() final {
+    RewritePatternSet patterns(&getContext());
+    patterns.insert<FuseScaledMatMulInteger>(&getContext());
+    if (failed(applyPatternsGreedily(getOperation(), std::move(patterns))))
+      signalPassFailure();
+  }
+};
+
+} // namespace
+
+std::unique_ptr<Pass> createFuseQuantizedMatMulForMI355XPass() {
+  return std::make_unique<FuseQuantizedMatMulForMI355XPass>();
+}
+
+} // namespace onnx_mlir

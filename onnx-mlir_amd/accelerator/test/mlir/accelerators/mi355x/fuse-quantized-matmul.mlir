@@ -1,0 +1,58 @@
+// RUN: onnx-mlir-opt --maccel=MI355X --shape-inference --fuse-quantized-matmul-for-mi355x --canonicalize %s -split-input-file | FileCheck %s
+
+// The five-op chain of a dynamically quantised linear layer becomes one op.
+func.func @whole_layer(%x: tensor<128x768xf32>, %w: tensor<768x3072xi8>, %ws: tensor<3072xf32>) -> tensor<*xf32> {
+  %wzp = onnx.Constant dense<0> : tensor<i8>
+  %aq, %as, %azp = "onnx.DynamicQuantizeLinear"(%x) : (tensor<128x768xf32>) -> (tensor<*xui8>, tensor<*xf32>, tensor<*xui8>)
+  %acc = "onnx.MatMulInteger"(%aq, %w, %azp, %wzp) : (tensor<*xui8>, tensor<768x3072xi8>, tensor<*xui8>, tensor<i8>) -> tensor<*xi32>
+  %f = "onnx.Cast"(%acc) {to = f32} : (tensor<*xi32>) -> tensor<*xf32>
+  %s = "onnx.Mul"(%as, %ws) : (tensor<*xf32>, tensor<3072xf32>) -> tensor<*xf32>
+  %y = "onnx.Mul"(%f, %s) : (tensor<*xf32>, tensor<*xf32>) -> tensor<*xf32>
+  return %y : tensor<*xf32>
+// CHECK-LABEL:  func.func @whole_layer
+// CHECK-SAME:   ([[X:%.+]]: tensor<128x768xf32>, [[W:%.+]]: tensor<768x3072xi8>, [[WS:%.+]]: tensor<3072xf32>)
+// CHECK:        [[WZP:%.+]] = onnx.Constant dense<0> : tensor<i8>
+// CHECK:        [[Y:%.+]] = "onnx.Custom"([[X]], [[W]], [[WZP]], [[WS]])
+// CHECK-SAME:   function_name = "om_mi355x_DynQuantMatMulDequant"
+// CHECK-SAME:   -> tensor<128x3072xf32>
+// CHECK-NOT:    onnx.DynamicQuantizeLinear
+// CHECK-NOT:    onnx.MatMulInteger
+// CHECK-NOT:    onnx.Mul
+// CHECK:        return [[Y]]
+}
+
+// -----
+
+// The quantised activation has a second user: it must stay, and only the
+// matmul and its scaling are fused.
+func.func @activation_reused(%x: tensor<128x768xf32>, %w: tensor<768x768xi8>, %ws: tensor<f32>) -> (tensor<*xf32>, tensor<*xui8>) {
+  %none = "onnx.NoValue"() {value} : () -> none
+  %aq, %as, %azp = "onnx.DynamicQuantizeLinear"(%x) : (tensor<128x768xf32>) -> (tensor<*xui8>, tensor<*xf32>, tensor<*xui8>)
+  %acc = "onnx.MatMulInteger"(%aq, %w, %azp, %none) : (tensor<*xui8>, tensor<768x768xi8>, tensor<*xui8>, none) -> tensor<*xi32>
+  %f = "onnx.Cast"(%acc) {to = f32} : (tensor<*xi32>) -> tensor<*xf32>
+  %s = "onnx.Mul"(%as, %ws) : (tensor<*xf32>, tensor<f32>) -> tensor<*xf32>
+  %y = "onnx.Mul"(%s, %f) : (tensor<*xf32>, tensor<*xf32>) -> tensor<*xf32>
+  return %y, %aq : tensor<*xf32>, tensor<*xui8>
+// CHECK-LABEL:  func.func @activation_reused
+// CHECK:        [[AQ:%.+]], [[AS:%.+]], [[AZP:%.+]] = "onnx.DynamicQuantizeLinear"
+// CHECK:        [[Y:%.+]] = "onnx.Custom"([[AQ]], {{%.+}}, [[AZP]], {{%.+}}, [[AS]], {{%.+}})
+// CHECK-SAME:   function_name = "om_mi355x_MatMulIntegerDequant"
+// CHECK-NOT:    onnx.MatMulInteger
+// CHECK:        return [[Y]], [[AQ]]
+}
+
+// -----
+
+// (f32(acc) * a_scale) * b_scale rounds differently from what the fused entry
+// point computes: not fused.
+func.func @other_association(%a: tensor<8x16xui8>, %w: tensor<16x4xi8>, %azp: tensor<ui8>, %as: tensor<f32>, %ws: tensor<f32>) -> tensor<*xf32> {
+  %none = "onnx.NoValue"() {value} : () -> none
+  %acc = "onnx.MatMulInteger"(%a, %w, %azp, %none) : (tensor<8x16xui8>, tensor<16x4xi8>, tensor<ui8>, none) -> tensor<*xi32>
+  %f = "onnx.Cast"(%acc) {to = f32} : (tensor<*xi32>) -> tensor<*xf32>
+  %t = "onnx.Mul"(%f, %as) : (tensor<*xf32>, tensor<f32>) -> tensor<*xf32>
+  %y = "onnx.Mul"(%t, %ws) : (tensor<*xf32>, tensor<f32>) -> tensor<*xf32>
+  return %y : tensor<*xf32>
+// CHECK-LABEL:  func.func @other_association
+// CHECK-NOT:    onnx.Custom
+// CHECK:        onnx.MatMulInteger
+}

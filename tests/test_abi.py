@@ -125,3 +125,59 @@ def test_without_a_gpu_the_ops_fail_loudly(rt):
         rt.QuantizeLinear(np.ones(8, np.float32), np.float32(0.5), np.array(3, np.uint8))
     with pytest.raises(rt.RuntimeError_, match="accelerator unavailable"):
         rt.MatMulInteger(np.ones((2, 2), np.uint8), np.ones((2, 2), np.int8))
+
+
+PLUGIN = os.path.join(ROOT, "onnx-mlir_amd", "accelerator")
+
+
+def _plugin_sources():
+    out = []
+    for base, _, files in os.walk(os.path.join(PLUGIN, "src")):
+        out += [os.path.join(base, f) for f in files if f.endswith((".cpp", ".hpp"))]
+    return out
+
+
+def test_compiler_plugin_calls_only_exported_symbols(rt):
+    """Every callee the onnx-mlir plug-in emits a krnl.call to is a symbol of the
+    runtime, with as many parameters as the plug-in passes."""
+    lib = rt.load()
+    header = open(os.path.join(INCLUDE, "om_mi355x.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    callees = set()
+    for path in _plugin_sources():
+        callees |= set(re.findall(r'"(om_mi355x_\w+)"', open(path).read()))
+    assert {"om_mi355x_QuantizeLinear", "om_mi355x_DequantizeLinear",
+            "om_mi355x_DynamicQuantizeLinear", "om_mi355x_MatMulInteger",
+            "om_mi355x_QLinearMatMul", "om_mi355x_MatMulIntegerDequant",
+            "om_mi355x_DynQuantMatMulDequant", "om_mi355x_MarkConstant"} <= callees
+    for name in callees:
+        assert hasattr(lib, name), f"plug-in calls {name}, which the runtime lacks"
+    # parameter counts: results + operands + integer attributes of each pattern
+    passed = {"om_mi355x_QuantizeLinear": 1 + 3 + 2, "om_mi355x_DequantizeLinear": 1 + 3 + 1,
+              "om_mi355x_DynamicQuantizeLinear": 3 + 1, "om_mi355x_MatMulInteger": 1 + 4,
+              "om_mi355x_QLinearMatMul": 1 + 8 + 1, "om_mi355x_MatMulIntegerDequant": 1 + 6,
+              "om_mi355x_DynQuantMatMulDequant": 1 + 4, "om_mi355x_MarkConstant": 1}
+    for name, count in passed.items():
+        m = re.search(r"\b%s\s*\(([^)]*)\)" % name, header)
+        assert m, name
+        assert len([p for p in m.group(1).split(",") if p.strip()]) == count, name
+
+
+def test_compiler_plugin_version_matches_runtime():
+    header = open(os.path.join(INCLUDE, "om_mi355x.h")).read()
+    runtime = int(re.search(r"#define\s+OM_MI355X_VERSION\s+(0x[0-9a-fA-F]+)", header).group(1), 16)
+    accel = open(os.path.join(PLUGIN, "src", "Accelerators", "MI355X", "MI355XAccelerator.cpp")).read()
+    plugin = int(re.search(r"kRuntimeVersion\s*=\s*(0x[0-9a-fA-F]+)", accel).group(1), 16)
+    assert plugin == runtime
+
+
+def test_compiler_plugin_lit_tests_name_real_entry_points(rt):
+    lib = rt.load()
+    lit = os.path.join(PLUGIN, "test", "mlir", "accelerators", "mi355x")
+    files = [f for f in os.listdir(lit) if f.endswith(".mlir")]
+    assert len(files) >= 4
+    for f in files:
+        text = open(os.path.join(lit, f)).read()
+        assert "// RUN: onnx-mlir-opt --maccel=MI355X" in text
+        for name in set(re.findall(r'"(om_mi355x_\w+)"', text)):
+            assert hasattr(lib, name), (f, name)
