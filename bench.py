@@ -274,7 +274,7 @@ def main():
         "roofline": {"bound": "mfma", "achieved": main_res["kernel_tops"], "peak": INT8_PEAK_TOPS,
                      "unit": "TOP/s", "frac": main_res["kernel_tops"] / INT8_PEAK_TOPS,
                      "traffic": TRAFFIC_BYTES.get("k_gemm_i8 config4 FFN-up f32") if epi == "f32" else None,
-                     "kernel": "k_gemm_i8<128,128>", "kernel_ms": main_res["kernel_ms"],
+                     "kernel": "k_gemm_i8_dma<128,3>", "kernel_ms": main_res["kernel_ms"],
                      "algorithmic_ops": main_res["ops"],
                      "algorithmic_hbm_bytes": main_res["hbm_bytes_algorithmic"],
                      "hbm_frac_at_algorithmic_bytes": main_res["hbm_bytes_algorithmic"]

@@ -17,17 +17,22 @@
 // once into Bt [Npad,Kpad] int8 (K contiguous, zero filled), so both MFMA
 // operands are read as 16 consecutive K bytes per lane.
 //
-// Pipeline: a block owns a BM x BN tile of Y and walks K in steps of 64 bytes.
-// Global loads run two steps ahead of the MFMAs in registers (two register
-// sets), LDS is double buffered, and the block barrier only orders LDS traffic
-// so the global loads stay in flight across it.  LDS rows are 64 bytes; the
-// 16-byte chunk index is XOR-swizzled with bits 2..3 of the row so that both
-// ds_write_b128 (staging) and ds_read_b128 (MFMA operands) are bank-conflict
-// free.
+// Kernels (all walk K in steps of 64 bytes; LDS rows are 64 bytes and the
+// 16-byte chunk index is XOR-swizzled with bits 2..3 of the row, so operand
+// reads and tile writes are bank-conflict free):
+//   k_gemm_i8_dma     tiles copied from global memory straight into a ring of
+//                     three LDS stages (no register staging); the default
+//   k_gemm_i8         tiles staged through registers, LDS double buffered;
+//                     also the byte-wise path for odd K or a misaligned A
+//   k_gemm_i8_stream  A read from a fragment-packed copy straight into MFMA
+//                     operand registers, only Bt through LDS; large problems
+//   k_gemm_i8_skinny  M <= 16: weight streaming, K split over the waves
 
 #include "om_kernels.h"
 
 #include <stdlib.h>
+
+#include <type_traits>
 
 namespace om {
 
@@ -158,16 +163,67 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TM][TN], int mrow0,
     }
   }
 
-  // Wave-uniform: the whole TM x TN grid lies inside the matrix.
-  const bool full = (mrow0 + 32 * TM <= M) && (ncol0 + 32 * TN <= N);
-
   const int32_t az0 = load_zp_i32(azp_ptr, A_OFF, 0);
   const int32_t da0 = oa - (has_azp ? az0 : 0);
   __builtin_amdgcn_sched_barrier(0);
 
   if (!per_row && !has_rs) {
-    // Common case: one zero point for all rows and no offset on B, so no
-    // per-row operand exists and nothing is loaded between the stores.
+    // Common case: one zero point for all rows and no offset on B.  The whole
+    // correction is then one value per column, computed once per lane.
+    uint32_t cj[TN];
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+      cj[j] = (uint32_t)da0 * (uint32_t)cs[j] +
+              (uint32_t)K * (uint32_t)da0 * (uint32_t)db[j];
+
+    // mrow0 and ncol0 are the same for every lane of the wave (callers derive
+    // them from a scalar wave index), so this test and the row addresses below
+    // are scalar work.
+    const bool full = (mrow0 + 32 * TM <= M) && (ncol0 + 32 * TN <= N);
+    if (full) {
+      // Whole grid inside the matrix: no bounds tests, and every address is
+      // (scalar row base) + (one 32-bit lane offset) + constant, so a store
+      // costs the two or three vector instructions that produce its value.
+      constexpr int ES = (EPI == kEpiQ8) ? 1 : 4;
+      char *const base =
+          (char *)ep.out + ((int64_t)mrow0 * N + ncol0) * (int64_t)ES;
+      const uint32_t loff =
+          ((uint32_t)(4 * lh) * (uint32_t)N + (uint32_t)l32) * (uint32_t)ES;
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int64_t rowb =
+              (int64_t)(i * 32 + 8 * (r >> 2) + (r & 3)) * N * (int64_t)ES;
+          char *const rowp = base + rowb;
+#pragma unroll
+          for (int j = 0; j < TN; ++j) {
+            const uint32_t y = (uint32_t)acc[i][j][r] + cj[j];
+            char *const q = rowp + loff + (uint32_t)(j * 32 * ES);
+            // Streaming stores: the result is not read again by this kernel,
+            // and keeping it out of the way in L2 leaves the A and Bt panels
+            // cached for the blocks still in their K loop (measured faster).
+            if (EPI == kEpiI32) {
+              __builtin_nontemporal_store((int32_t)y, (int32_t *)q);
+            } else if (EPI == kEpiF32) {
+              __builtin_nontemporal_store(
+                  (float)(int32_t)y * sj[j], (float *)q);
+            } else {
+              const float f = (float)(int32_t)y * sj[j];
+              int32_t v = (int32_t)((uint32_t)(int32_t)__builtin_rintf(f) +
+                                    (uint32_t)yz);
+              if (ep.narrow == kSaturate) {
+                const int32_t lo = ep.y_unsigned ? 0 : -128;
+                const int32_t hi = ep.y_unsigned ? 255 : 127;
+                v = v < lo ? lo : (v > hi ? hi : v);
+              }
+              *(uint8_t *)q = (uint8_t)(v & 0xFF);
+            }
+          }
+        }
+      }
+      return;
+    }
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
       const int mbase = mrow0 + i * 32 + 4 * lh;
@@ -177,14 +233,9 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TM][TN], int mrow0,
         const int64_t orow = (int64_t)m * N;
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
-          uint32_t y = (uint32_t)acc[i][j][r];
-          y += (uint32_t)da0 * (uint32_t)cs[j];
-          y += (uint32_t)K * (uint32_t)da0 * (uint32_t)db[j];
-          if (full) {
+          const uint32_t y = (uint32_t)acc[i][j][r] + cj[j];
+          if (m < M && n_[j] < N)
             store_one<EPI>(ep, orow + n_[j], y, sj[j], yz);
-          } else if (m < M && n_[j] < N) {
-            store_one<EPI>(ep, orow + n_[j], y, sj[j], yz);
-          }
         }
       }
     }
@@ -226,6 +277,7 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TM][TN], int mrow0,
     }
   }
 }
+
 
 // BM x BN block tile, WGM x WGN waves, each wave a (BM/WGM) x (BN/WGN) tile
 // made of 32x32 MFMA tiles.
@@ -269,8 +321,11 @@ __global__ __launch_bounds__(WGM *WGN * 64, MINB) void k_gemm_i8(
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  // wave index as a scalar: everything derived from it (tile origin, LDS
+  // bases, output rows) then lives in scalar registers
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WGN, wn = wave % WGN;
+
 
   constexpr int kFill = (A_MODE == 1) ? (int)0x80808080 : 0;
 
@@ -400,6 +455,207 @@ __global__ __launch_bounds__(WGM *WGN * 64, MINB) void k_gemm_i8(
     if (++kt >= KT)
       break;
   }
+  gemm_epilogue<TM, TN, A_MODE, EPI>(
+      acc, m0 + wm * WTM, n0 + wn * WTN, M, N, K, ep);
+}
+
+// ---- GEMM, tiles copied from global memory straight into LDS --------------
+// gfx950 can write a 16-byte global load into LDS without passing through
+// vector registers (global_load_lds_dwordx4): LDS address = M0 + lane * 16, so
+// one wave instruction fills 1 KiB of consecutive LDS and the per-lane global
+// address decides what lands where.  That removes the register staging, the
+// ds_write instructions and the wait that tied them to the loads; a wave only
+// issues the copies, waits for its own to land, and meets the others at one
+// barrier per K step.
+//
+// LDS holds a ring of three stages (A tile + Bt tile of one 64-byte K step
+// each, same XOR-swizzled row layout as above).  In step k a wave
+//   waits until its copies for step k have landed (those for k+1 stay in
+//   flight), passes the barrier -- now every wave's step-k data is in LDS and
+//   every wave is done reading stage (k-1)%3 --,
+//   issues its copies for step k+2 into stage (k-1)%3,
+//   reads the operands of stage k%3 and runs the MFMAs.
+// The operand reads are written as inline assembly: the compiler would make
+// every LDS read wait for all outstanding copies into LDS, whichever stage
+// they target.  The counts waited for below are therefore explicit.
+template <int BN, int NSTAGE, int MINB, int A_MODE, int EPI>
+__global__ __launch_bounds__(256, MINB) void k_gemm_i8_dma(
+    const uint8_t *__restrict__ A, const int8_t *__restrict__ Bt, int M, int N,
+    int K, int Kpad, EpiParams ep, int tiles_m, int tiles_n) {
+  // 2 x 2 waves, each a 64 x (BN/2) tile.
+  constexpr int BM = 128, WTM = 64, WTN = BN / 2, TM = 2, TN = WTN / 32;
+  static_assert(BN == 128 || BN == 64, "tile width");
+  constexpr int STAGE = (BM + BN) * BK;
+  constexpr int CB = BN / 64;      // Bt copies per wave and step
+  constexpr int CPW = 2 + CB;      // copies per wave and step
+  __shared__ __attribute__((aligned(1024))) uint8_t sm[NSTAGE * STAGE];
+
+  int pid = blockIdx.x;
+  {
+    const int nb = gridDim.x;
+    const int per = nb >> 3;
+    if (per > 0 && pid < per * 8)
+      pid = (pid & 7) * per + (pid >> 3);
+  }
+  constexpr int GROUP = 8;
+  const int in_group = GROUP * tiles_n;
+  const int group = pid / in_group;
+  const int first_m = group * GROUP;
+  const int gsize = (tiles_m - first_m < GROUP) ? tiles_m - first_m : GROUP;
+  const int tm = first_m + (pid % in_group) % gsize;
+  const int tn = (pid % in_group) / gsize;
+  const int m0 = tm * BM, n0 = tn * BN;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  const int l32 = lane & 31;
+  const int lh = lane >> 5;
+
+  // Copy addressing.  Copy instruction j of a tile fills LDS bytes
+  // [j*1024, (j+1)*1024): lane -> row j*16 + lane/4, chunk position lane%4,
+  // which holds chunk (lane%4) ^ ((row/4)%4) = (lane%4) ^ ((lane/16)%4) of the
+  // row.  A wave issues copies 2*wave, 2*wave+1 of A and CB consecutive copies
+  // of Bt.
+  const int crow = lane >> 2;
+  const int cchunk = (lane & 3) ^ ((lane >> 4) & 3);
+  const uint8_t *ga[2];
+  const int8_t *gb[CB];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int r = (wave * 2 + h) * 16 + crow;
+    const int gm = (m0 + r < M) ? m0 + r : M - 1; // rows past M: never stored
+    ga[h] = A + (int64_t)gm * K + cchunk * 16;
+  }
+#pragma unroll
+  for (int h = 0; h < CB; ++h) {
+    const int r = (wave * CB + h) * 16 + crow;
+    gb[h] = Bt + (int64_t)(n0 + r) * Kpad + cchunk * 16;
+  }
+  typedef __attribute__((address_space(3))) void *lds_ptr;
+  typedef const __attribute__((address_space(1))) void *glb_ptr;
+  auto copy_step = [&](int k0, int stage) {
+    uint8_t *base = sm + stage * STAGE;
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+      __builtin_amdgcn_global_load_lds((glb_ptr)(ga[h] + k0),
+          (lds_ptr)(base + (wave * 2 + h) * 1024), 16, 0, 0);
+#pragma unroll
+    for (int h = 0; h < CB; ++h)
+      __builtin_amdgcn_global_load_lds((glb_ptr)(gb[h] + k0),
+          (lds_ptr)(base + BM * BK + (wave * CB + h) * 1024), 16, 0, 0);
+  };
+
+  // Operand addressing: sub-step s (0,1) of a stage uses chunk 2*s + lane/32 of
+  // row (wave tile row + lane%32); MFMA tile i adds 32 rows = 2048 bytes.
+  const unsigned sm_base = (unsigned)(uintptr_t)(lds_ptr)sm;
+  unsigned ra[2], rb[2];
+#pragma unroll
+  for (int s = 0; s < 2; ++s) {
+    ra[s] = sm_base + lds_off(wm * WTM + l32, s * 2 + lh);
+    rb[s] = sm_base + BM * BK + lds_off(wn * WTN + l32, s * 2 + lh);
+  }
+
+  v16i acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        acc[i][j][r] = 0;
+
+  const int KT = Kpad / BK;
+  const int klast = (KT - 1) * BK;
+  auto kclamp = [&](int step) { return step < KT ? step * BK : klast; };
+#pragma unroll
+  for (int p = 0; p < NSTAGE - 1; ++p)
+    copy_step(kclamp(p), p);
+
+  // One LDS read of an MFMA operand.  Kept opaque to the compiler, see above;
+  // lds_wait<n>() makes the operands it is given valid once at most n reads
+  // are still outstanding (reads complete in order).
+  auto lds_read = [](v4i &f, unsigned addr, auto off) {
+    asm volatile("ds_read_b128 %0, %1 offset:%2"
+                 : "=v"(f)
+                 : "v"(addr), "n"(decltype(off)::value)
+                 : "memory");
+  };
+
+  int stage = 0; // kt % NSTAGE
+  for (int kt = 0; kt < KT; ++kt) {
+    const int prev = (stage == 0) ? NSTAGE - 1 : stage - 1;
+    // Own copies of step kt have landed; those of the NSTAGE-2 steps after it
+    // may still be in flight.
+    __builtin_amdgcn_s_waitcnt(0x0F70 | ((NSTAGE - 2) * CPW));
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    copy_step(kclamp(kt + NSTAGE - 1), prev);
+    __builtin_amdgcn_sched_barrier(0);
+    const unsigned soff = (unsigned)(stage * STAGE);
+    v4i fa0[TM], fb0[TN], fa1[TM], fb1[TN];
+    using O0 = std::integral_constant<int, 0>;
+    using O1 = std::integral_constant<int, 2048>;
+    lds_read(fa0[0], ra[0] + soff, O0{});
+    lds_read(fa0[1], ra[0] + soff, O1{});
+    lds_read(fb0[0], rb[0] + soff, O0{});
+    if (TN == 2)
+      lds_read(fb0[TN - 1], rb[0] + soff, O1{});
+    lds_read(fa1[0], ra[1] + soff, O0{});
+    lds_read(fa1[1], ra[1] + soff, O1{});
+    lds_read(fb1[0], rb[1] + soff, O0{});
+    if (TN == 2)
+      lds_read(fb1[TN - 1], rb[1] + soff, O1{});
+    if (TN == 2)
+      asm volatile("s_waitcnt lgkmcnt(4)"
+                   : "+v"(fa0[0]), "+v"(fa0[1]), "+v"(fb0[0]), "+v"(fb0[TN - 1])
+                   :
+                   : "memory");
+    else
+      asm volatile("s_waitcnt lgkmcnt(3)"
+                   : "+v"(fa0[0]), "+v"(fa0[1]), "+v"(fb0[0])
+                   :
+                   : "memory");
+    if (A_MODE == 1) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        fa0[i] ^= (v4i){(int)0x80808080, (int)0x80808080, (int)0x80808080,
+            (int)0x80808080};
+    }
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
+            fa0[i], fb0[j], acc[i][j], 0, 0, 0);
+    if (TN == 2)
+      asm volatile("s_waitcnt lgkmcnt(0)"
+                   : "+v"(fa1[0]), "+v"(fa1[1]), "+v"(fb1[0]), "+v"(fb1[TN - 1])
+                   :
+                   : "memory");
+    else
+      asm volatile("s_waitcnt lgkmcnt(0)"
+                   : "+v"(fa1[0]), "+v"(fa1[1]), "+v"(fb1[0])
+                   :
+                   : "memory");
+    if (A_MODE == 1) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        fa1[i] ^= (v4i){(int)0x80808080, (int)0x80808080, (int)0x80808080,
+            (int)0x80808080};
+    }
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
+            fa1[i], fb1[j], acc[i][j], 0, 0, 0);
+    stage = (stage == NSTAGE - 1) ? 0 : stage + 1;
+  }
+  // Copies past the last step are still landing in LDS; nothing reads them,
+  // but the block must not release its LDS before they are done.
+  __builtin_amdgcn_s_waitcnt(0x0F70);
 
   gemm_epilogue<TM, TN, A_MODE, EPI>(
       acc, m0 + wm * WTM, n0 + wn * WTN, M, N, K, ep);
@@ -454,7 +710,7 @@ __global__ __launch_bounds__(256, (TM == 1 ? 2 : 1)) void k_gemm_i8_stream(
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31;
   const int lh = lane >> 5;
   const int mrow0 = m0 + wave * 32 * TM;
@@ -897,7 +1153,9 @@ enum TileCfg : int {
   kS256x128 = 3,
   kS128x192 = 4,
   kS128x128 = 5,
-  kNumCfg = 6
+  kD128x128 = 6, // k_gemm_i8_dma (tiles copied straight into LDS)
+  kD128x64 = 7,
+  kNumCfg = 8
 };
 
 bool cfg_is_stream(int c) {
@@ -922,8 +1180,12 @@ int choose_tile(const GemmArgs &g) {
   };
   static const Cand cands[] = {{kS256x192, 256, 192, 1}, {kS256x128, 256, 128, 1},
       {kS128x192, 128, 192, 2}, {kS128x128, 128, 128, 2}};
+  // Measured on MI355X (4096 x 768 x 3072 and its siblings): the kernel that
+  // copies tiles straight into LDS beats the register-staged one on every
+  // shape below the streamed-A threshold, with 128 x 128 tiles even when they
+  // leave some CUs without a block.
   if (!g.a_pack)
-    return kT128x128;
+    return kD128x128;
   int best = kS128x128;
   double best_cost = 1e300;
   for (const Cand &c : cands) {
@@ -989,6 +1251,20 @@ hipError_t gemm_launch_cfg(
         <<<dim3((unsigned)(tiles_m * tiles_n)), 256, 0, st>>>(
             (const uint8_t *)g.A, g.Bt, (int)g.M, (int)g.N, (int)g.K, Kpad, ep,
             tiles_m, tiles_n);
+    return hipGetLastError();
+  }
+  if (cfg == kD128x128 || cfg == kD128x64) {
+    const int bn = (cfg == kD128x128) ? 128 : 64;
+    const int tiles_m = (int)((g.M + 127) / 128);
+    const int tiles_n = (int)((g.N + bn - 1) / bn);
+    const dim3 grid((unsigned)(tiles_m * tiles_n));
+    const uint8_t *A = (const uint8_t *)g.A;
+    if (cfg == kD128x128)
+      k_gemm_i8_dma<128, 3, 3, A_MODE, EPI><<<grid, 256, 0, st>>>(A, g.Bt,
+          (int)g.M, (int)g.N, (int)g.K, Kpad, ep, tiles_m, tiles_n);
+    else
+      k_gemm_i8_dma<64, 3, 4, A_MODE, EPI><<<grid, 256, 0, st>>>(A, g.Bt,
+          (int)g.M, (int)g.N, (int)g.K, Kpad, ep, tiles_m, tiles_n);
     return hipGetLastError();
   }
   if (cfg == kT256x128)
@@ -1092,5 +1368,6 @@ hipError_t launch_gemm(hipStream_t s, const GemmArgs &g) {
     return gemm_launch_epi<2>(s, g, ep, Kpad);
   }
 }
+
 
 } // namespace om

@@ -253,10 +253,11 @@ def test_matmulinteger_shapes(rt, oracle, M, K, N):
     assert np.array_equal(rt.MatMulInteger(A, B, azr, bzc), want)
 
 
-@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 4, 5])
+@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 4, 5, 6, 7])
 def test_every_gemm_kernel_configuration(rt, oracle, cfg, monkeypatch):
     """The tile / kernel choice is a heuristic; force each configuration in turn
-    (0-1 stage A through LDS, 2-5 stream a fragment-packed copy of A) on shapes
+    (0-1 stage A through LDS, 2-5 stream a fragment-packed copy of A, 6-7 copy tiles
+    straight from global memory into LDS) on shapes
     with ragged edges, every operand type and all zero-point forms."""
     monkeypatch.setenv("OM_MI355X_GEMM_TILE", str(cfg))
     rng = np.random.default_rng(100 + cfg)
