@@ -15,17 +15,19 @@
 //
 // Layout: A is used as given ([M,K] row-major, K contiguous).  B is packed
 // once into Bt [Npad,Kpad] int8 (K contiguous, zero filled), so both MFMA
-// operands are read as 16 consecutive K bytes per lane.
+// operands are read as 16 consecutive K bytes per lane; for the kernels that
+// stream it, Bt is additionally kept in MFMA operand order (Bp, k_pack_frag).
 //
 // Kernels (all walk K in steps of 64 bytes; LDS rows are 64 bytes and the
 // 16-byte chunk index is XOR-swizzled with bits 2..3 of the row, so operand
 // reads and tile writes are bank-conflict free):
-//   k_gemm_i8_dma     tiles copied from global memory straight into a ring of
-//                     three LDS stages (no register staging); the default
+//   k_gemm_i8_bs      Bt read from Bp straight into MFMA operand registers,
+//                     only the A tile goes through LDS (copied there without
+//                     passing through registers); more than one tile per CU
+//   k_gemm_i8_dma     A and Bt tiles copied from global memory straight into
+//                     a ring of three LDS stages; up to one tile per CU
 //   k_gemm_i8         tiles staged through registers, LDS double buffered;
-//                     also the byte-wise path for odd K or a misaligned A
-//   k_gemm_i8_stream  A read from a fragment-packed copy straight into MFMA
-//                     operand registers, only Bt through LDS; large problems
+//                     the byte-wise path for odd K or a misaligned A
 //   k_gemm_i8_skinny  M <= 16: weight streaming, K split over the waves
 
 #include "om_kernels.h"
@@ -661,45 +663,41 @@ __global__ __launch_bounds__(256, MINB) void k_gemm_i8_dma(
       acc, m0 + wm * WTM, n0 + wn * WTN, M, N, K, ep);
 }
 
-// ---- GEMM, A streamed to registers ----------------------------------------
-// LDS stores are the scarcest on-chip resource of a CU (about a third of the
-// LDS read rate), so this kernel keeps A out of LDS altogether.  The four
-// waves of a block are stacked along M: a wave owns 32*TM rows that no other
-// wave needs, and reads its A operands straight from global memory in MFMA
-// operand layout (lane = row, 16 K-bytes per lane).  Only the Bt tile, which
-// all four waves share, goes through LDS: a ring of three 64-byte-deep stages.
+// ---- GEMM, Bt streamed to registers from a fragment-ordered copy -----------
+// The right-hand side of a quantised layer is a model constant, so it can be
+// stored once in exactly the order the matrix cores consume it (Bp, the
+// layout written by k_pack_frag): the operand of column tile nt, K step ks,
+// half step sub is one contiguous KiB, 16 bytes per lane.  The four waves of a
+// block sit side by side along N; each owns 32*TN columns that no other wave
+// needs and loads their operands from Bp straight into registers, D steps
+// ahead.  Only the A tile, which all four waves share, goes through LDS, and
+// it gets there without passing through registers (see k_gemm_i8_dma).  Per K
+// step a block therefore moves half as many bytes into LDS as the kernels
+// above, and the copy path into LDS is what bounds those.
 //
-// Global loads run D steps ahead in registers (D register sets, loop unrolled
-// by D so that every set is addressed statically).  Per K step (64 bytes) a
-// wave issues, in this order,
-//   ds_read  B operands of sub-step 1 (this step's stage)
-//   MFMAs of sub-step 0; A registers of sub-step 0 are refilled for step +D
-//   ds_write the staged Bt chunk of step +2 into its stage; refetch step +2+D
-//   ds_read  B operands of sub-step 0 of step +1 (stage published one barrier
-//            ago -- this is what the third stage buys: nothing waits on LDS
-//            right after the barrier)
-//   MFMAs of sub-step 1; A registers of sub-step 1 are refilled for step +D
-//   one LDS-only barrier
-// All loads are unconditional (clamped), so every wait is an exact count.
-template <int TM, int TN, int D, int A_MODE, int EPI>
-__global__ __launch_bounds__(256, (TM == 1 ? 2 : 1)) void k_gemm_i8_stream(
-    const uint8_t *__restrict__ Ap, const int8_t *__restrict__ Bt, int M, int N,
+// Per step, in this order (so that the explicit wait below can count):
+//   wait for own A copies of this step, barrier
+//   LDS reads of the A operands (both half steps), MFMAs of half step 0,
+//   refill its Bp registers for step +D, MFMAs of half step 1, refill,
+//   A copies for step +NST-1 into the stage that was read in the last step.
+template <int TM, int TN, int D, int NST, int MINB, int A_MODE, int EPI>
+__global__ __launch_bounds__(256, MINB) void k_gemm_i8_bs(
+    const uint8_t *__restrict__ A, const int8_t *__restrict__ Bp, int M, int N,
     int K, int Kpad, EpiParams ep, int tiles_m, int tiles_n) {
-  constexpr int BM = 4 * 32 * TM, BN = 32 * TN;
-  constexpr int CH_B = BN * 4 / 256; // 16-byte chunks of Bt per thread, per step
-  static_assert(BN * 4 % 256 == 0, "BN must be a multiple of 64");
-  constexpr int STAGE = BN * BK;
-
-  __shared__ __attribute__((aligned(16))) uint8_t sB[3 * STAGE];
+  constexpr int BM = 32 * TM, BN = 4 * 32 * TN;
+  constexpr int STAGE = BM * BK;
+  constexpr int CA = BM / 64; // A copies (1 KiB each) per wave and step
+  static_assert(BM % 64 == 0, "tile height");
+  __shared__ __attribute__((aligned(1024))) uint8_t sm[NST * STAGE];
 
   int pid = blockIdx.x;
-  if (ep.xcd) {
+  {
     const int nb = gridDim.x;
     const int per = nb >> 3;
     if (per > 0 && pid < per * 8)
       pid = (pid & 7) * per + (pid >> 3);
   }
-  const int GROUP = ep.group;
+  constexpr int GROUP = 8;
   const int in_group = GROUP * tiles_n;
   const int group = pid / in_group;
   const int first_m = group * GROUP;
@@ -713,62 +711,56 @@ __global__ __launch_bounds__(256, (TM == 1 ? 2 : 1)) void k_gemm_i8_stream(
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31;
   const int lh = lane >> 5;
-  const int mrow0 = m0 + wave * 32 * TM;
+  const int ncol0 = n0 + wave * 32 * TN;
 
   const int KT = Kpad / BK;
-  const int klast = (KT - 1) * BK;
-  auto kclamp = [&](int step) { return step < KT ? step * BK : klast; };
+  const int klast = KT - 1;
+  auto sclamp = [&](int step) { return step < KT ? step : klast; };
 
-  // A operand pointers into the fragment-packed copy of A (see k_pack_a): the
-  // operand of MFMA row tile mt, step ks, half step sub is one contiguous KiB,
-  // 16 bytes per lane.  Row tiles past the last one are clamped (they only
-  // feed output rows that are never stored).
-  const uint8_t *__restrict__ arow[TM];
-  {
-    const int mt_max = (M + 31) / 32 - 1;
+  // A copies: copy j of a step fills LDS bytes [j*1024, (j+1)*1024) of the
+  // stage, lane -> row j*16 + lane/4, holding chunk (lane%4) ^ ((lane/16)%4).
+  const int crow = lane >> 2;
+  const int cchunk = (lane & 3) ^ ((lane >> 4) & 3);
+  const uint8_t *ga[CA];
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
-      int mt = (mrow0 >> 5) + i;
-      mt = mt < mt_max ? mt : mt_max;
-      arow[i] = Ap + (int64_t)mt * KT * 2048 + lane * 16;
-    }
+  for (int h = 0; h < CA; ++h) {
+    const int r = (wave * CA + h) * 16 + crow;
+    const int gm = (m0 + r < M) ? m0 + r : M - 1; // rows past M: never stored
+    ga[h] = A + (int64_t)gm * K + cchunk * 16;
   }
-  // Bt staging pointers: chunk q -> row q>>2, 16-byte chunk q&3.
-  const int8_t *__restrict__ brow[CH_B];
-  int bdst[CH_B];
+  typedef __attribute__((address_space(3))) void *lds_ptr;
+  typedef const __attribute__((address_space(1))) void *glb_ptr;
+  auto copy_a = [&](int step, int stage) {
+    uint8_t *base = sm + stage * STAGE + wave * CA * 1024;
 #pragma unroll
-  for (int h = 0; h < CH_B; ++h) {
-    const int q = tid + h * 256;
-    // Bt has round_up(N, kGemmBN) rows; a tile whose width does not divide
-    // that may reach past it: clamp (those columns are never stored).
-    const int npad = (N + kGemmBN - 1) / kGemmBN * kGemmBN;
-    int bn = n0 + (q >> 2);
-    bn = bn < npad ? bn : npad - 1;
-    brow[h] = Bt + (int64_t)bn * Kpad + (q & 3) * 16;
-    bdst[h] = lds_off(q >> 2, q & 3);
-  }
+    for (int h = 0; h < CA; ++h)
+      __builtin_amdgcn_global_load_lds((glb_ptr)(ga[h] + step * BK),
+          (lds_ptr)(base + h * 1024), 16, 0, 0);
+  };
 
-  // k0 is a byte offset along K (64 per step); a step of packed A is 2 KiB.
-  auto load_a = [&](int k0, int sub, v4i(&ra)[TM]) {
+  // Bp operands of this wave's column tiles.
+  const int8_t *gbp[TN];
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
-      ra[i] = *(const v4i *)(arow[i] + k0 * 32 + sub * 1024);
-  };
-  auto load_b = [&](int k0, v4i(&rb)[CH_B]) {
-#pragma unroll
-    for (int h = 0; h < CH_B; ++h)
-      rb[h] = *(const v4i *)(brow[h] + k0);
-  };
-  auto write_b = [&](int stage, const v4i(&rb)[CH_B]) {
-#pragma unroll
-    for (int h = 0; h < CH_B; ++h)
-      *(v4i *)(&sB[stage * STAGE + bdst[h]]) = rb[h];
-  };
-  auto read_frag = [&](int stage, int sub, v4i(&fb)[TN]) {
-    const int c = sub * 2 + lh;
+  for (int j = 0; j < TN; ++j)
+    gbp[j] = Bp + (int64_t)((ncol0 >> 5) + j) * KT * 2048 + lane * 16;
+  auto load_b = [&](int step, int sub, v4i(&fb)[TN]) {
 #pragma unroll
     for (int j = 0; j < TN; ++j)
-      fb[j] = *(const v4i *)(&sB[stage * STAGE + lds_off(j * 32 + l32, c)]);
+      fb[j] = *(const v4i *)(gbp[j] + (int64_t)step * 2048 + sub * 1024);
+  };
+
+  // A operand reads: half step s uses chunk 2*s + lane/32 of row lane%32 of
+  // MFMA row tile i (2048 bytes apart).
+  const unsigned sm_base = (unsigned)(uintptr_t)(lds_ptr)sm;
+  unsigned ra[2];
+#pragma unroll
+  for (int s2 = 0; s2 < 2; ++s2)
+    ra[s2] = sm_base + lds_off(l32, s2 * 2 + lh);
+  auto lds_read = [](v4i &f, unsigned addr, auto off) {
+    asm volatile("ds_read_b128 %0, %1 offset:%2"
+                 : "=v"(f)
+                 : "v"(addr), "n"(decltype(off)::value)
+                 : "memory");
   };
 
   v16i acc[TM][TN];
@@ -780,71 +772,101 @@ __global__ __launch_bounds__(256, (TM == 1 ? 2 : 1)) void k_gemm_i8_stream(
       for (int r = 0; r < 16; ++r)
         acc[i][j][r] = 0;
 
-  auto mfma_sub = [&](const v4i(&ra)[TM], const v4i(&fb)[TN]) {
+  // Prologue: A of steps 0..NST-2 on their way into stages 0..NST-2, then Bp
+  // of steps 0..D-1 into the D register sets.
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
-#pragma unroll
-      for (int j = 0; j < TN; ++j)
-        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
-            ra[i], fb[j], acc[i][j], 0, 0, 0);
-    }
-  };
-
-  // D register sets: as[u][sub] holds A of a step with (step % D) == u;
-  // bs[u] holds the staged Bt chunk of the step two ahead of that.
-  v4i as[D][2][TM];
-  v4i bs[D][CH_B];
-  v4i f0[TN], f1[TN];
-
-  // Prologue.  Bt of steps 0 and 1 goes to stages 0 and 1 through bs[0],
-  // bs[1]; then bs[u] is filled with step 2+u.  as[u] is filled with step u.
-  load_b(0, bs[0]);
-  load_b(kclamp(1), bs[D > 1 ? 1 : 0]);
+  for (int p2 = 0; p2 < NST - 1; ++p2)
+    copy_a(sclamp(p2), p2);
+  v4i bs[D][2][TN];
 #pragma unroll
   for (int u = 0; u < D; ++u) {
-    load_a(kclamp(u), 0, as[u][0]);
-    load_a(kclamp(u), 1, as[u][1]);
+    load_b(sclamp(u), 0, bs[u][0]);
+    load_b(sclamp(u), 1, bs[u][1]);
   }
-  write_b(0, bs[0]);
-  if (D > 1)
-    write_b(1, bs[1]);
-  else {
-    load_b(kclamp(1), bs[0]);
-    write_b(1, bs[0]);
-  }
-#pragma unroll
-  for (int u = 0; u < D; ++u)
-    load_b(kclamp(2 + u), bs[u]);
-  lds_barrier();
-  read_frag(0, 0, f0);
+  __builtin_amdgcn_sched_barrier(0);
+
+  // Memory operations a wave issues per step, and how many of them are
+  // younger than its A copies for the step it is about to start: the Bp loads
+  // of the step those copies were issued in, then NST-2 whole steps.  The
+  // first steps have issued more (the prologue), never fewer.
+  constexpr int PER_STEP = CA + 2 * TN;
+  constexpr int YOUNGER = (NST - 2) * PER_STEP;
+  static_assert(YOUNGER < 64, "wait count");
 
   int kt = 0;
-  int st0 = 0, st1 = 1, st2 = 2; // stages of steps kt, kt+1, kt+2
+  int stage = 0;
   bool done = false;
   while (!done) {
 #pragma unroll
     for (int u = 0; u < D; ++u) {
-      read_frag(st0, 1, f1);
-      mfma_sub(as[u][0], f0);
-      load_a(kclamp(kt + D), 0, as[u][0]);
-      write_b(st2, bs[u]);
-      load_b(kclamp(kt + 2 + D), bs[u]);
-      read_frag(st1, 0, f0);
-      mfma_sub(as[u][1], f1);
-      load_a(kclamp(kt + D), 1, as[u][1]);
-      lds_barrier();
+      __builtin_amdgcn_s_waitcnt(
+          0x0F70 | (YOUNGER & 15) | ((YOUNGER >> 4) << 14));
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+      const unsigned soff = (unsigned)(stage * STAGE);
+      v4i fa0[TM], fa1[TM];
+      using O = std::integral_constant<int, 0>;
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        lds_read(fa0[i], ra[0] + soff + i * 2048, O{});
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        lds_read(fa1[i], ra[1] + soff + i * 2048, O{});
+      // first half landed (reads complete in order); the empty statements
+      // make the registers count as written here, after the wait
+      asm volatile("s_waitcnt lgkmcnt(%0)" : : "n"(TM) : "memory");
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        asm volatile("" : "+v"(fa0[i]));
+      if (A_MODE == 1) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+          fa0[i] ^= (v4i){(int)0x80808080, (int)0x80808080, (int)0x80808080,
+              (int)0x80808080};
+      }
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
+              fa0[i], bs[u][0][j], acc[i][j], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      load_b(sclamp(kt + D), 0, bs[u][0]);
+      __builtin_amdgcn_sched_barrier(0);
+      asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        asm volatile("" : "+v"(fa1[i]));
+      if (A_MODE == 1) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+          fa1[i] ^= (v4i){(int)0x80808080, (int)0x80808080, (int)0x80808080,
+              (int)0x80808080};
+      }
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
+              fa1[i], bs[u][1][j], acc[i][j], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      load_b(sclamp(kt + D), 1, bs[u][1]);
+      __builtin_amdgcn_sched_barrier(0);
+      // The stage read in the previous step is free: every wave passed this
+      // step's barrier after finishing those reads.
+      copy_a(sclamp(kt + NST - 1), stage == 0 ? NST - 1 : stage - 1);
+      __builtin_amdgcn_sched_barrier(0);
+      stage = (stage == NST - 1) ? 0 : stage + 1;
       if (++kt >= KT) {
         done = true;
         break;
       }
-      const int t = st0;
-      st0 = st1;
-      st1 = st2;
-      st2 = t;
     }
   }
+  // A copies past the last step are still landing in LDS.
+  __builtin_amdgcn_s_waitcnt(0x0F70);
 
-  gemm_epilogue<TM, TN, A_MODE, EPI>(acc, mrow0, n0, M, N, K, ep);
+  gemm_epilogue<TM, TN, A_MODE, EPI>(acc, m0, ncol0, M, N, K, ep);
 }
 
 // ---- skinny GEMM (M <= 16): weight streaming -------------------------------
@@ -1017,58 +1039,34 @@ __global__ __launch_bounds__(256) void k_pack_b(const uint8_t *__restrict__ B,
   }
 }
 
-// ---- pack A ---------------------------------------------------------------
-// Rewrites A [M,K] (row-major) in MFMA operand order for k_gemm_i8_stream:
-//   Ap[mt][ks][sub][lane][16 bytes],  lane = half*32 + row,
-//   bytes = A[mt*32 + row][ks*64 + (sub*2 + half)*16 .. +16]
-// so that a wave fetches one operand (32 rows x 32 K-bytes... x 2 halves) as a
-// single contiguous KiB.  uint8 is moved to int8 (minus 128) on the way and
-// everything outside [M,K] is zero in that domain, which also makes K that is
-// not a multiple of 64 (or 16) legal for the fast kernel.
-// A block handles one 32-row tile and four K steps (256 bytes of each row):
-// eight consecutive threads read 128 contiguous bytes of a row.
-template <bool A_UNSIGNED, bool ALIGNED>
-__global__ __launch_bounds__(256) void k_pack_a(const uint8_t *__restrict__ A,
-    int64_t M, int64_t K, int KT, uint8_t *__restrict__ Ap) {
-  const int mt = blockIdx.y;
+// ---- fragment order ----------------------------------------------------------
+// Rewrites a row-major int8 matrix X [R, Kpad] (R a multiple of 32, Kpad of
+// 64; here: the packed Bt) into the order in which the matrix cores consume
+// it, so that a wave can load an MFMA operand with one fully coalesced
+// instruction:
+//   Xp[rt][ks][sub][lane][16 bytes],  rt = row / 32, ks = K step of 64 bytes,
+//   lane = (chunk & 1) * 32 + row % 32, sub = chunk >> 1 for the 16-byte chunk
+//   `chunk` (0..3) of the step.
+// One block handles one row tile and four K steps.
+__global__ __launch_bounds__(256) void k_pack_frag(
+    const int8_t *__restrict__ X, int64_t Kpad, int KT, int8_t *__restrict__ Xp) {
+  const int rt = blockIdx.y;
   const int ks0 = blockIdx.x * 4;
-  const int tid = threadIdx.x;
 #pragma unroll
   for (int h = 0; h < 2; ++h) {
-    const int row = tid >> 3;
-    const int c16 = (tid & 7) + 8 * h; // 16-byte chunk within the 256 bytes
+    const int q = threadIdx.x + h * 256; // 512 chunks: 32 rows x 16 chunks
+    const int row = q >> 4;
+    const int c16 = q & 15;
     const int ks = ks0 + (c16 >> 2);
     if (ks >= KT)
       continue;
     const int c = c16 & 3;
-    const int64_t m = (int64_t)mt * 32 + row;
-    const int64_t k = (int64_t)ks * 64 + c * 16;
-    v4i v = {0, 0, 0, 0};
-    if (ALIGNED) {
-      if (m < M && k < K) {
-        v = *(const v4i *)(A + m * K + k);
-        if (A_UNSIGNED)
-          v ^= (v4i){(int)0x80808080, (int)0x80808080, (int)0x80808080,
-              (int)0x80808080};
-      }
-    } else {
-      uint32_t w[4] = {0, 0, 0, 0};
-#pragma unroll
-      for (int b = 0; b < 16; ++b) {
-        uint32_t byte = 0;
-        if (m < M && k + b < K) {
-          byte = A[m * K + k + b];
-          if (A_UNSIGNED)
-            byte ^= 0x80u;
-        }
-        w[b >> 2] |= byte << ((b & 3) * 8);
-      }
-      v = (v4i){(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
-    }
+    const v4i v = *(const v4i *)(X + ((int64_t)rt * 32 + row) * Kpad +
+                                 (int64_t)ks * 64 + c * 16);
     const int sub = c >> 1, half = c & 1;
     const int64_t o =
-        ((((int64_t)mt * KT + ks) * 2 + sub) * 64 + half * 32 + row) * 16;
-    *(v4i *)(Ap + o) = v;
+        ((((int64_t)rt * KT + ks) * 2 + sub) * 64 + half * 32 + row) * 16;
+    *(v4i *)(Xp + o) = v;
   }
 }
 
@@ -1096,119 +1094,54 @@ __global__ __launch_bounds__(256) void k_rowsum_a(
 
 // ---- launch ---------------------------------------------------------------
 
-template <int BM, int BN, int WGM, int WGN, int MINB, int A_MODE, int EPI>
-hipError_t gemm_launch_tile(
-    hipStream_t st, const GemmArgs &g, const EpiParams &ep, int Kpad) {
-  const int tiles_m = (int)((g.M + BM - 1) / BM);
-  const int tiles_n = (int)((g.N + BN - 1) / BN);
-  const dim3 grid((unsigned)(tiles_m * tiles_n));
-  constexpr int threads = WGM * WGN * 64;
-  k_gemm_i8<BM, BN, WGM, WGN, MINB, A_MODE, EPI, true>
-      <<<grid, threads, 0, st>>>((const uint8_t *)g.A, g.Bt, (int)g.M,
-          (int)g.N, (int)g.K, Kpad, ep, tiles_m, tiles_n);
-  return hipGetLastError();
-}
-
-hipError_t launch_pack_a(hipStream_t st, const void *A, bool a_unsigned,
-    int64_t M, int64_t K, uint8_t *Ap) {
-  const int KT = (int)(round_up(K > 0 ? K : 1, kGemmBK) / kGemmBK);
-  const int MT = (int)((M + 31) / 32);
-  const bool aligned = (K % 16 == 0) && ((((uintptr_t)A) & 15) == 0);
-  dim3 grid((unsigned)((KT + 3) / 4), (unsigned)MT);
-  if (a_unsigned) {
-    if (aligned)
-      k_pack_a<true, true><<<grid, 256, 0, st>>>(
-          (const uint8_t *)A, M, K, KT, Ap);
-    else
-      k_pack_a<true, false><<<grid, 256, 0, st>>>(
-          (const uint8_t *)A, M, K, KT, Ap);
-  } else {
-    if (aligned)
-      k_pack_a<false, true><<<grid, 256, 0, st>>>(
-          (const uint8_t *)A, M, K, KT, Ap);
-    else
-      k_pack_a<false, false><<<grid, 256, 0, st>>>(
-          (const uint8_t *)A, M, K, KT, Ap);
-  }
-  return hipGetLastError();
-}
-
-template <int TM, int TN, int D, int A_MODE, int EPI>
-hipError_t gemm_launch_stream(
-    hipStream_t st, const GemmArgs &g, const EpiParams &ep, int Kpad) {
-  constexpr int BM = 4 * 32 * TM, BN = 32 * TN;
-  const int tiles_m = (int)((g.M + BM - 1) / BM);
-  const int tiles_n = (int)((g.N + BN - 1) / BN);
-  k_gemm_i8_stream<TM, TN, D, A_MODE, EPI>
-      <<<dim3((unsigned)(tiles_m * tiles_n)), 256, 0, st>>>(g.a_pack, g.Bt,
-          (int)g.M, (int)g.N, (int)g.K, Kpad, ep, tiles_m, tiles_n);
-  return hipGetLastError();
-}
-
 // Kernel / tile configurations.
 enum TileCfg : int {
-  kT128x128 = 0, // k_gemm_i8, BM x BN
-  kT256x128 = 1,
-  kS256x192 = 2, // k_gemm_i8_stream (needs the packed copy of A)
-  kS256x128 = 3,
-  kS128x192 = 4,
-  kS128x128 = 5,
-  kD128x128 = 6, // k_gemm_i8_dma (tiles copied straight into LDS)
-  kD128x64 = 7,
-  kNumCfg = 8
+  kT128x128 = 0, // k_gemm_i8: register-staged tiles (and the byte-wise path)
+  kD128x128 = 1, // k_gemm_i8_dma: tiles copied straight into LDS
+  kB128x128 = 2, // k_gemm_i8_bs: Bt from its fragment-ordered copy
+  kB128x256 = 3,
+  kNumCfg = 4
 };
 
-bool cfg_is_stream(int c) {
-  return c == kS256x192 || c == kS256x128 || c == kS128x192 || c == kS128x128;
-}
+bool cfg_needs_bp(int c) { return c == kB128x128 || c == kB128x256; }
 
-// Tile choice.  Each configuration is costed as (rounds of tiles over the 256
-// CUs) x (tile area), i.e. matrix-core time including the idle tail of the
-// last round; among near-equal costs the larger tile wins (fewer LDS and L2
-// bytes per MFMA).  The streamed-A kernels are only eligible when the caller
-// provided the buffer for the packed copy of A.
-int choose_tile(const GemmArgs &g) {
-  // Override for tests and tuning: OM_MI355X_GEMM_TILE=<TileCfg value>.
+// Kernel choice for problems with more than 16 rows, K % 64 == 0 and a
+// 16-byte aligned A (anything else takes the byte-wise path of k_gemm_i8).
+// Measured on MI355X over the BERT-base and Llama-7B layer shapes and square
+// problems up to 8192:
+//  * at most one 128 x 128 tile per CU: k_gemm_i8_dma is fastest (a lone
+//    block per CU gains nothing from the lighter LDS traffic of the others);
+//  * otherwise the kernels that stream Bt from its fragment-ordered copy win,
+//    with 128 x 256 tiles unless those would leave most CUs idle in a second,
+//    nearly empty round (between 1 and 1.4 tiles per CU).
+// Override for tests and tuning: OM_MI355X_GEMM_TILE=<TileCfg value>.
+int choose_tile(int64_t M, int64_t N) {
   const char *force = getenv("OM_MI355X_GEMM_TILE");
   if (force && force[0]) {
     const int c = atoi(force);
-    if (c >= 0 && c < kNumCfg && (!cfg_is_stream(c) || g.a_pack))
+    if (c >= 0 && c < kNumCfg)
       return c;
   }
-  struct Cand {
-    int cfg, bm, bn, per_cu;
-  };
-  static const Cand cands[] = {{kS256x192, 256, 192, 1}, {kS256x128, 256, 128, 1},
-      {kS128x192, 128, 192, 2}, {kS128x128, 128, 128, 2}};
-  // Measured on MI355X (4096 x 768 x 3072 and its siblings): the kernel that
-  // copies tiles straight into LDS beats the register-staged one on every
-  // shape below the streamed-A threshold, with 128 x 128 tiles even when they
-  // leave some CUs without a block.
-  if (!g.a_pack)
+  const int64_t tm = (M + 127) / 128;
+  const int64_t t128 = tm * ((N + 127) / 128);
+  if (t128 <= 256)
     return kD128x128;
-  int best = kS128x128;
-  double best_cost = 1e300;
-  for (const Cand &c : cands) {
-    const int64_t tiles =
-        ((g.M + c.bm - 1) / c.bm) * ((g.N + c.bn - 1) / c.bn);
-    const int64_t slots = 256 * c.per_cu;
-    const int64_t rounds = (tiles + slots - 1) / slots;
-    // two co-resident tiles share a CU's matrix cores
-    double cost = (double)rounds * c.per_cu * c.bm * c.bn;
-    // small tiles pay more LDS / L2 traffic per MFMA
-    cost *= 1.0 + 24.0 / c.bm + 24.0 / c.bn;
-    if (cost < best_cost) {
-      best_cost = cost;
-      best = c.cfg;
-    }
-  }
-  return best;
+  const int64_t t256 = tm * ((N + 255) / 256);
+  if (t256 <= 256 || t256 * 10 >= 256 * 14)
+    return kB128x256;
+  return kB128x128;
+}
+
+bool gemm_fast_path(int64_t M, int64_t K, const void *A) {
+  return M > 16 && K % 64 == 0 && ((((uintptr_t)A) & 15) == 0);
 }
 
 template <int A_MODE, int EPI>
 hipError_t gemm_launch_cfg(
     hipStream_t st, const GemmArgs &g, const EpiParams &ep, int Kpad) {
   const char *force = getenv("OM_MI355X_GEMM_TILE");
+  const uint8_t *A = (const uint8_t *)g.A;
+  const int M = (int)g.M, N = (int)g.N, K = (int)g.K;
   if (g.M <= 16 && g.K % 16 == 0 && ((((uintptr_t)g.A) & 15) == 0) &&
       !(force && force[0])) {
     // 32 columns per block halves the reads of A (measured faster whenever
@@ -1216,60 +1149,51 @@ hipError_t gemm_launch_cfg(
     if ((g.N + 31) / 32 >= 256)
       k_gemm_i8_skinny<2, A_MODE, EPI>
           <<<dim3((unsigned)((g.N + 31) / 32)), 512, 0, st>>>(
-              (const uint8_t *)g.A, g.Bt, (int)g.M, (int)g.N, (int)g.K, Kpad,
-              ep);
+              A, g.Bt, M, N, K, Kpad, ep);
     else
       k_gemm_i8_skinny<1, A_MODE, EPI>
           <<<dim3((unsigned)((g.N + 15) / 16)), 512, 0, st>>>(
-              (const uint8_t *)g.A, g.Bt, (int)g.M, (int)g.N, (int)g.K, Kpad,
-              ep);
+              A, g.Bt, M, N, K, Kpad, ep);
     return hipGetLastError();
   }
-  const int cfg = choose_tile(g);
-  if (cfg_is_stream(cfg)) {
-    // A_MODE 1 (raw uint8) is shifted to int8 by the pack; 0 and 2 are copied.
-    hipError_t e = launch_pack_a(st, g.A, A_MODE == 1, g.M, g.K, g.a_pack);
-    if (e != hipSuccess)
-      return e;
-    switch (cfg) {
-    case kS256x192:
-      return gemm_launch_stream<2, 6, 3, A_MODE, EPI>(st, g, ep, Kpad);
-    case kS256x128:
-      return gemm_launch_stream<2, 4, 3, A_MODE, EPI>(st, g, ep, Kpad);
-    case kS128x192:
-      return gemm_launch_stream<1, 6, 4, A_MODE, EPI>(st, g, ep, Kpad);
-    default:
-      return gemm_launch_stream<1, 4, 4, A_MODE, EPI>(st, g, ep, Kpad);
-    }
-  }
-  const bool aligned = (g.K % 64 == 0) && ((((uintptr_t)g.A) & 15) == 0);
-  if (!aligned) {
-    // Byte-wise staging of A for odd K or a misaligned A.
-    const int tiles_m = (int)((g.M + 127) / 128);
-    const int tiles_n = (int)((g.N + 127) / 128);
+  const int tiles_m = (int)((g.M + 127) / 128);
+  const int tiles_n128 = (int)((g.N + 127) / 128);
+  if (!gemm_fast_path(g.M, g.K, g.A)) {
+    // Byte-wise staging of A for odd K or a misaligned A (and the forced
+    // configurations of the tests when M <= 16).
     k_gemm_i8<128, 128, 2, 2, 2, A_MODE, EPI, false>
+        <<<dim3((unsigned)(tiles_m * tiles_n128)), 256, 0, st>>>(
+            A, g.Bt, M, N, K, Kpad, ep, tiles_m, tiles_n128);
+    return hipGetLastError();
+  }
+  int cfg = choose_tile(g.M, g.N);
+  if (cfg_needs_bp(cfg) && !g.Bp)
+    cfg = kD128x128;
+  switch (cfg) {
+  case kB128x256: {
+    const int tiles_n = (int)((g.N + 255) / 256);
+    k_gemm_i8_bs<4, 2, 4, 4, 2, A_MODE, EPI>
         <<<dim3((unsigned)(tiles_m * tiles_n)), 256, 0, st>>>(
-            (const uint8_t *)g.A, g.Bt, (int)g.M, (int)g.N, (int)g.K, Kpad, ep,
-            tiles_m, tiles_n);
-    return hipGetLastError();
+            A, g.Bp, M, N, K, Kpad, ep, tiles_m, tiles_n);
+    break;
   }
-  if (cfg == kD128x128 || cfg == kD128x64) {
-    const int bn = (cfg == kD128x128) ? 128 : 64;
-    const int tiles_m = (int)((g.M + 127) / 128);
-    const int tiles_n = (int)((g.N + bn - 1) / bn);
-    const dim3 grid((unsigned)(tiles_m * tiles_n));
-    const uint8_t *A = (const uint8_t *)g.A;
-    if (cfg == kD128x128)
-      k_gemm_i8_dma<128, 3, 3, A_MODE, EPI><<<grid, 256, 0, st>>>(A, g.Bt,
-          (int)g.M, (int)g.N, (int)g.K, Kpad, ep, tiles_m, tiles_n);
-    else
-      k_gemm_i8_dma<64, 3, 4, A_MODE, EPI><<<grid, 256, 0, st>>>(A, g.Bt,
-          (int)g.M, (int)g.N, (int)g.K, Kpad, ep, tiles_m, tiles_n);
-    return hipGetLastError();
+  case kB128x128:
+    k_gemm_i8_bs<4, 1, 4, 3, 3, A_MODE, EPI>
+        <<<dim3((unsigned)(tiles_m * tiles_n128)), 256, 0, st>>>(
+            A, g.Bp, M, N, K, Kpad, ep, tiles_m, tiles_n128);
+    break;
+  case kD128x128:
+    k_gemm_i8_dma<128, 3, 3, A_MODE, EPI>
+        <<<dim3((unsigned)(tiles_m * tiles_n128)), 256, 0, st>>>(
+            A, g.Bt, M, N, K, Kpad, ep, tiles_m, tiles_n128);
+    break;
+  default:
+    k_gemm_i8<128, 128, 2, 2, 3, A_MODE, EPI, true>
+        <<<dim3((unsigned)(tiles_m * tiles_n128)), 256, 0, st>>>(
+            A, g.Bt, M, N, K, Kpad, ep, tiles_m, tiles_n128);
+    break;
   }
-  if (cfg == kT256x128)
-    return gemm_launch_tile<256, 128, 2, 2, 2, A_MODE, EPI>(st, g, ep, Kpad);
-  return gemm_launch_tile<128, 128, 2, 2, 3, A_MODE, EPI>(st, g, ep, Kpad);
+  return hipGetLastError();
 }
 
 template <int A_MODE>
@@ -1306,19 +1230,20 @@ hipError_t launch_pack_b(hipStream_t s, const void *B, bool b_unsigned,
   return hipGetLastError();
 }
 
-size_t gemm_a_pack_bytes(int64_t M, int64_t K, int64_t N) {
-  // The packed copy pays off once there are enough rows and columns for the
-  // large tiles; below that the kernels that stage A through LDS are used.
-  if (M < 128 || N < 128 || K < 64)
-    return 0;
-  // Measured on MI355X: below ~3e10 multiply-accumulates the extra pass over A
-  // and the single round of large tiles cost more than they save.
-  const char *force = getenv("OM_MI355X_GEMM_TILE");
-  if (!(force && force[0]) && (double)M * (double)N * (double)K < 3e10)
-    return 0;
-  const int64_t KT = round_up(K, kGemmBK) / kGemmBK;
-  const int64_t MT = (M + 31) / 32;
-  return (size_t)(MT * KT * 2048);
+bool gemm_wants_bp(int64_t M, int64_t K, int64_t N, const void *A) {
+  (void)K;
+  return gemm_fast_path(M, K, A) && cfg_needs_bp(choose_tile(M, N));
+}
+
+hipError_t launch_pack_bp(
+    hipStream_t s, const int8_t *Bt, int64_t K, int64_t N, int8_t *Bp) {
+  // Bt is [Npad, Kpad] and fully written (padding is zero).
+  const int64_t Kpad = round_up(K > 0 ? K : 1, kGemmBK);
+  const int64_t Npad = round_up(N, kGemmBN);
+  const int KT = (int)(Kpad / kGemmBK);
+  dim3 grid((unsigned)((KT + 3) / 4), (unsigned)(Npad / 32));
+  k_pack_frag<<<grid, 256, 0, s>>>(Bt, Kpad, KT, Bp);
+  return hipGetLastError();
 }
 
 hipError_t launch_rowsum_a(hipStream_t s, const void *A, bool a_unsigned,

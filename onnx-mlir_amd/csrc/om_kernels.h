@@ -58,8 +58,8 @@ struct GemmArgs {
   const void *A;       // [M,K] row-major, u8 or i8
   bool a_unsigned;     // A holds u8
   bool a_preshifted;   // A already holds (u8 - 128) as int8; offsets as for u8
-  uint8_t *a_pack;     // scratch of gemm_a_pack_bytes() bytes, or null
   const int8_t *Bt;    // packed [Npad,Kpad]
+  const int8_t *Bp;    // fragment-ordered copy of Bt (launch_pack_bp), or null
   bool b_unsigned;     // original B was u8 (packed values are B - 128)
   int64_t M, K, N;
   const void *a_zp;    // element type follows A; may be null
@@ -84,11 +84,12 @@ struct GemmArgs {
 
 hipError_t launch_gemm(hipStream_t s, const GemmArgs &g);
 
-// Bytes of scratch the GEMM wants for a fragment-ordered copy of A (0 when
-// the shape is too small for that path).  With GemmArgs::a_pack set to such a
-// buffer launch_gemm may repack A and stream it to the matrix cores without
-// staging it in LDS.
-size_t gemm_a_pack_bytes(int64_t M, int64_t K, int64_t N);
+// True when launch_gemm would use the fragment-ordered copy of Bt for this
+// problem (GemmArgs::Bp); the caller then builds it with launch_pack_bp, into
+// a buffer of round_up(N, kGemmBN) * round_up(K, kGemmBK) bytes.
+bool gemm_wants_bp(int64_t M, int64_t K, int64_t N, const void *A);
+hipError_t launch_pack_bp(
+    hipStream_t s, const int8_t *Bt, int64_t K, int64_t N, int8_t *Bp);
 
 // Fill n 32-bit words with v.
 hipError_t launch_fill_u32(hipStream_t s, uint32_t *p, int64_t n, uint32_t v);
