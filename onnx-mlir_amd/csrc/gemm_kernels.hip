@@ -675,12 +675,17 @@ __global__ __launch_bounds__(256, MINB) void k_gemm_i8_dma(
 // step a block therefore moves half as many bytes into LDS as the kernels
 // above, and the copy path into LDS is what bounds those.
 //
+// PIPE (needs NST >= 4) reads the operands of each half step one half step
+// early, see the loop.  It pays for the 128 x 256 tile and not for the
+// 128 x 128 one (measured).
+//
 // Per step, in this order (so that the explicit wait below can count):
 //   wait for own A copies of this step, barrier
 //   LDS reads of the A operands (both half steps), MFMAs of half step 0,
 //   refill its Bp registers for step +D, MFMAs of half step 1, refill,
 //   A copies for step +NST-1 into the stage that was read in the last step.
-template <int TM, int TN, int D, int NST, int MINB, int A_MODE, int EPI>
+template <int TM, int TN, int D, int NST, int MINB, bool PIPE, int A_MODE,
+    int EPI>
 __global__ __launch_bounds__(256, MINB) void k_gemm_i8_bs(
     const uint8_t *__restrict__ A, const int8_t *__restrict__ Bp, int M, int N,
     int K, int Kpad, EpiParams ep, int tiles_m, int tiles_n) {
@@ -786,82 +791,172 @@ __global__ __launch_bounds__(256, MINB) void k_gemm_i8_bs(
   __builtin_amdgcn_sched_barrier(0);
 
   // Memory operations a wave issues per step, and how many of them are
-  // younger than its A copies for the step it is about to start: the Bp loads
-  // of the step those copies were issued in, then NST-2 whole steps.  The
-  // first steps have issued more (the prologue), never fewer.
+  // younger than the A copies it has to wait for at the top of a step.  The A
+  // copies are the last operations of a step, so those of step k were
+  // followed by NST-2 whole steps when step k starts.  The first steps have
+  // issued more (the prologue), never fewer.
   constexpr int PER_STEP = CA + 2 * TN;
-  constexpr int YOUNGER = (NST - 2) * PER_STEP;
-  static_assert(YOUNGER < 64, "wait count");
+  constexpr int AHEAD = PIPE ? 1 : 0; // PIPE waits for the copies of step k+1
+  constexpr int YOUNGER = (NST - 2 - AHEAD) * PER_STEP;
+  static_assert(YOUNGER < 64 && NST - 2 - AHEAD >= 0 && D >= NST - 2,
+      "wait count");
+  const v4i flip = {(int)0x80808080, (int)0x80808080, (int)0x80808080,
+      (int)0x80808080};
+  using O = std::integral_constant<int, 0>;
 
   int kt = 0;
   int stage = 0;
   bool done = false;
-  while (!done) {
+  if constexpr (!PIPE) {
+    while (!done) {
 #pragma unroll
-    for (int u = 0; u < D; ++u) {
-      __builtin_amdgcn_s_waitcnt(
-          0x0F70 | (YOUNGER & 15) | ((YOUNGER >> 4) << 14));
-      __builtin_amdgcn_s_barrier();
-      __builtin_amdgcn_sched_barrier(0);
-      const unsigned soff = (unsigned)(stage * STAGE);
-      v4i fa0[TM], fa1[TM];
-      using O = std::integral_constant<int, 0>;
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-        lds_read(fa0[i], ra[0] + soff + i * 2048, O{});
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-        lds_read(fa1[i], ra[1] + soff + i * 2048, O{});
-      // first half landed (reads complete in order); the empty statements
-      // make the registers count as written here, after the wait
-      asm volatile("s_waitcnt lgkmcnt(%0)" : : "n"(TM) : "memory");
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-        asm volatile("" : "+v"(fa0[i]));
-      if (A_MODE == 1) {
+      for (int u = 0; u < D; ++u) {
+        __builtin_amdgcn_s_waitcnt(
+            0x0F70 | (YOUNGER & 15) | ((YOUNGER >> 4) << 14));
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        const unsigned soff = (unsigned)(stage * STAGE);
+        v4i fa0[TM], fa1[TM];
 #pragma unroll
         for (int i = 0; i < TM; ++i)
-          fa0[i] ^= (v4i){(int)0x80808080, (int)0x80808080, (int)0x80808080,
-              (int)0x80808080};
-      }
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
-              fa0[i], bs[u][0][j], acc[i][j], 0, 0, 0);
-      __builtin_amdgcn_sched_barrier(0);
-      load_b(sclamp(kt + D), 0, bs[u][0]);
-      __builtin_amdgcn_sched_barrier(0);
-      asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-        asm volatile("" : "+v"(fa1[i]));
-      if (A_MODE == 1) {
+          lds_read(fa0[i], ra[0] + soff + i * 2048, O{});
 #pragma unroll
         for (int i = 0; i < TM; ++i)
-          fa1[i] ^= (v4i){(int)0x80808080, (int)0x80808080, (int)0x80808080,
-              (int)0x80808080};
-      }
+          lds_read(fa1[i], ra[1] + soff + i * 2048, O{});
+        // first half landed (reads complete in order); the empty statements
+        // make the registers count as written here, after the wait
+        asm volatile("s_waitcnt lgkmcnt(%0)" : : "n"(TM) : "memory");
 #pragma unroll
-      for (int i = 0; i < TM; ++i)
+        for (int i = 0; i < TM; ++i)
+          asm volatile("" : "+v"(fa0[i]));
+        if (A_MODE == 1) {
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
-              fa1[i], bs[u][1][j], acc[i][j], 0, 0, 0);
-      __builtin_amdgcn_sched_barrier(0);
-      load_b(sclamp(kt + D), 1, bs[u][1]);
-      __builtin_amdgcn_sched_barrier(0);
-      // The stage read in the previous step is free: every wave passed this
-      // step's barrier after finishing those reads.
-      copy_a(sclamp(kt + NST - 1), stage == 0 ? NST - 1 : stage - 1);
-      __builtin_amdgcn_sched_barrier(0);
-      stage = (stage == NST - 1) ? 0 : stage + 1;
-      if (++kt >= KT) {
-        done = true;
-        break;
+          for (int i = 0; i < TM; ++i)
+            fa0[i] ^= flip;
+        }
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
+                fa0[i], bs[u][0][j], acc[i][j], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        load_b(sclamp(kt + D), 0, bs[u][0]);
+        __builtin_amdgcn_sched_barrier(0);
+        asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+          asm volatile("" : "+v"(fa1[i]));
+        if (A_MODE == 1) {
+#pragma unroll
+          for (int i = 0; i < TM; ++i)
+            fa1[i] ^= flip;
+        }
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
+                fa1[i], bs[u][1][j], acc[i][j], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        load_b(sclamp(kt + D), 1, bs[u][1]);
+        __builtin_amdgcn_sched_barrier(0);
+        // The stage read in the previous step is free: every wave passed this
+        // step's barrier after finishing those reads.
+        copy_a(sclamp(kt + NST - 1), stage == 0 ? NST - 1 : stage - 1);
+        __builtin_amdgcn_sched_barrier(0);
+        stage = (stage == NST - 1) ? 0 : stage + 1;
+        if (++kt >= KT) {
+          done = true;
+          break;
+        }
       }
     }
+  } else {
+    // Software-pipelined operand reads: the barrier at the top of step k
+    // publishes stage k+1, so the first-half operands of step k+1 can be read
+    // while the second-half MFMAs of step k run, and the second-half operands
+    // of step k while its first-half MFMAs run.  No MFMA waits on an LDS read
+    // issued just before it.
+    {
+      constexpr int P0 = (NST - 2) * CA + 2 * D * TN; // younger than step 0's
+      static_assert(P0 < 64, "wait count");
+      __builtin_amdgcn_s_waitcnt(0x0F70 | (P0 & 15) | ((P0 >> 4) << 14));
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    v4i fa0[TM];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+      lds_read(fa0[i], ra[0] + i * 2048, O{});
+    while (!done) {
+#pragma unroll
+      for (int u = 0; u < D; ++u) {
+        __builtin_amdgcn_s_waitcnt(
+            0x0F70 | (YOUNGER & 15) | ((YOUNGER >> 4) << 14));
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        const unsigned soff = (unsigned)(stage * STAGE);
+        const int nstage = (stage == NST - 1) ? 0 : stage + 1;
+        const unsigned noff = (unsigned)(nstage * STAGE);
+        v4i fa1[TM], fn0[TM];
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+          lds_read(fa1[i], ra[1] + soff + i * 2048, O{});
+        // the first-half operands were requested a step ago
+        asm volatile("s_waitcnt lgkmcnt(%0)" : : "n"(TM) : "memory");
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+          asm volatile("" : "+v"(fa0[i]));
+        if (A_MODE == 1) {
+#pragma unroll
+          for (int i = 0; i < TM; ++i)
+            fa0[i] ^= flip;
+        }
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
+                fa0[i], bs[u][0][j], acc[i][j], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        load_b(sclamp(kt + D), 0, bs[u][0]);
+        __builtin_amdgcn_sched_barrier(0);
+        asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+          asm volatile("" : "+v"(fa1[i]));
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+          lds_read(fn0[i], ra[0] + noff + i * 2048, O{});
+        if (A_MODE == 1) {
+#pragma unroll
+          for (int i = 0; i < TM; ++i)
+            fa1[i] ^= flip;
+        }
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
+                fa1[i], bs[u][1][j], acc[i][j], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        load_b(sclamp(kt + D), 1, bs[u][1]);
+        __builtin_amdgcn_sched_barrier(0);
+        copy_a(sclamp(kt + NST - 1), stage == 0 ? NST - 1 : stage - 1);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+          fa0[i] = fn0[i];
+        stage = nstage;
+        if (++kt >= KT) {
+          done = true;
+          break;
+        }
+      }
+    }
+    // the operands requested for the step after the last one
+    asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");
   }
   // A copies past the last step are still landing in LDS.
   __builtin_amdgcn_s_waitcnt(0x0F70);
@@ -1172,13 +1267,13 @@ hipError_t gemm_launch_cfg(
   switch (cfg) {
   case kB128x256: {
     const int tiles_n = (int)((g.N + 255) / 256);
-    k_gemm_i8_bs<4, 2, 4, 4, 2, A_MODE, EPI>
+    k_gemm_i8_bs<4, 2, 4, 4, 2, true, A_MODE, EPI>
         <<<dim3((unsigned)(tiles_m * tiles_n)), 256, 0, st>>>(
             A, g.Bp, M, N, K, Kpad, ep, tiles_m, tiles_n);
     break;
   }
   case kB128x128:
-    k_gemm_i8_bs<4, 1, 4, 3, 3, A_MODE, EPI>
+    k_gemm_i8_bs<4, 1, 4, 3, 3, false, A_MODE, EPI>
         <<<dim3((unsigned)(tiles_m * tiles_n128)), 256, 0, st>>>(
             A, g.Bp, M, N, K, Kpad, ep, tiles_m, tiles_n128);
     break;
