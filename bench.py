@@ -35,8 +35,8 @@ METRIC = "int8 MatMulInteger TOPS (% MFMA peak) + Q/DQ GB/s (% HBM), 1 MI355X"
 # HBM bytes per launch of the headline kernel, measured with rocprofv3 --pmc
 # (FETCH_SIZE and WRITE_SIZE, one run each, scaled by what the same counters
 # read for a 1 GiB device-to-device copy: FETCH_SIZE x2.0, WRITE_SIZE x1.0);
-# the summary of those runs is profiles/k_gemm_i8_config4_ffn_up.md.
-TRAFFIC_BYTES = {"k_gemm_i8 config4 FFN-up f32": int((7797.4 * 2.0 + 49152.0) * 1024)}
+# the summary of those runs is profiles/k_gemm_i8_bs_config4_ffn_up.md.
+TRAFFIC_BYTES = {"config4 FFN-up f32": int((7817.0 * 2.0 + 49180.0) * 1024)}
 
 
 def timed(rt, fn, steps, warmup):
@@ -197,8 +197,8 @@ def cpu_baseline_gemm(oracle, wl, M, K, N, budget_s=20.0):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=1000)
+    ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--workload", default="config4_ffn_up",
                     choices=["config4_ffn_up", "config4_ffn_up_i32"])
     ap.add_argument("--no-extras", action="store_true", help="skip the Q/DQ and other-shape measurements")
@@ -273,8 +273,8 @@ def main():
                                "output, operands resident in HBM, weights packed once"},
         "roofline": {"bound": "mfma", "achieved": main_res["kernel_tops"], "peak": INT8_PEAK_TOPS,
                      "unit": "TOP/s", "frac": main_res["kernel_tops"] / INT8_PEAK_TOPS,
-                     "traffic": TRAFFIC_BYTES.get("k_gemm_i8 config4 FFN-up f32") if epi == "f32" else None,
-                     "kernel": "k_gemm_i8_dma<128,3>", "kernel_ms": main_res["kernel_ms"],
+                     "traffic": TRAFFIC_BYTES.get("config4 FFN-up f32") if epi == "f32" else None,
+                     "kernel": "k_gemm_i8_bs<4,2,4,4,2,true> (128x256 tiles)", "kernel_ms": main_res["kernel_ms"],
                      "algorithmic_ops": main_res["ops"],
                      "algorithmic_hbm_bytes": main_res["hbm_bytes_algorithmic"],
                      "hbm_frac_at_algorithmic_bytes": main_res["hbm_bytes_algorithmic"]
