@@ -14,21 +14,26 @@
 // which is exact because int32 addition and multiplication wrap.
 //
 // Layout: A is used as given ([M,K] row-major, K contiguous).  B is packed
-// once into Bt [Npad,Kpad] int8 (K contiguous, zero filled), so both MFMA
-// operands are read as 16 consecutive K bytes per lane; for the kernels that
-// stream it, Bt is additionally kept in MFMA operand order (Bp, k_pack_frag).
+// once into Bp, the order in which the matrix cores consume it (k_pack_b):
+//   Bp[nt][ks][sub][lane][16 bytes], nt = column / 32, ks = K step of 64
+//   bytes, sub = half step; lane l holds, for column nt*32 + l%32, the 16 K
+//   bytes starting at ks*64 + (sub*2 + l/32)*16
+// int8 (u8 shifted by -128), zero filled up to [Npad, Kpad].  The operand of
+// one MFMA is one contiguous KiB, 16 bytes per lane, whether it is loaded
+// into registers or copied into LDS.
 //
-// Kernels (all walk K in steps of 64 bytes; LDS rows are 64 bytes and the
-// 16-byte chunk index is XOR-swizzled with bits 2..3 of the row, so operand
-// reads and tile writes are bank-conflict free):
-//   k_gemm_i8_bs      Bt read from Bp straight into MFMA operand registers,
-//                     only the A tile goes through LDS (copied there without
-//                     passing through registers); more than one tile per CU
-//   k_gemm_i8_dma     A and Bt tiles copied from global memory straight into
-//                     a ring of three LDS stages; up to one tile per CU
-//   k_gemm_i8         tiles staged through registers, LDS double buffered;
-//                     the byte-wise path for odd K or a misaligned A
-//   k_gemm_i8_skinny  M <= 16: weight streaming, K split over the waves
+// Kernels (all walk K in steps of 64 bytes):
+//   k_gemm_i8_bs         Bp read straight into MFMA operand registers, only
+//                        the A tile goes through LDS (copied there without
+//                        passing through registers); more than one tile per CU
+//   k_gemm_i8_dma        A and Bp tiles copied from global memory straight
+//                        into a ring of three LDS stages; up to one tile per CU
+//   k_gemm_i8            tiles staged through registers, LDS double buffered;
+//                        the byte-wise path for odd K or a misaligned A
+//   k_gemm_i8_skinny_bp  M <= 32: weight streaming, K split over the waves
+// A tiles in LDS have 64-byte rows whose 16-byte chunk index is XOR-swizzled
+// with bits 2..3 of the row (bank-conflict free writes and operand reads); Bp
+// tiles in LDS keep their global order.
 
 #include "om_kernels.h"
 
@@ -203,7 +208,7 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TM][TN], int mrow0,
             const uint32_t y = (uint32_t)acc[i][j][r] + cj[j];
             char *const q = rowp + loff + (uint32_t)(j * 32 * ES);
             // Streaming stores: the result is not read again by this kernel,
-            // and keeping it out of the way in L2 leaves the A and Bt panels
+            // and keeping it out of the way in L2 leaves the A and Bp panels
             // cached for the blocks still in their K loop (measured faster).
             if (EPI == kEpiI32) {
               __builtin_nontemporal_store((int32_t)y, (int32_t *)q);
@@ -289,7 +294,7 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TM][TN], int mrow0,
 template <int BM, int BN, int WGM, int WGN, int MINB, int A_MODE, int EPI,
     bool ALIGNED>
 __global__ __launch_bounds__(WGM *WGN * 64, MINB) void k_gemm_i8(
-    const uint8_t *__restrict__ A, const int8_t *__restrict__ Bt, int M, int N,
+    const uint8_t *__restrict__ A, const int8_t *__restrict__ Bp, int M, int N,
     int K, int Kpad, EpiParams ep, int tiles_m, int tiles_n) {
   constexpr int THREADS = WGM * WGN * 64;
   constexpr int WTM = BM / WGM, WTN = BN / WGN; // wave tile
@@ -304,7 +309,7 @@ __global__ __launch_bounds__(WGM *WGN * 64, MINB) void k_gemm_i8(
   // Tile order.  Consecutive workgroup ids are dealt round-robin to the 8
   // XCDs, each with its own L2; renumber so that one XCD gets a contiguous
   // range, then walk that range in groups of 8 tile rows so the tiles resident
-  // on an XCD share a few A panels and Bt panels.
+  // on an XCD share a few A panels and Bp panels.
   int pid = blockIdx.x;
   {
     const int nb = gridDim.x;
@@ -330,6 +335,7 @@ __global__ __launch_bounds__(WGM *WGN * 64, MINB) void k_gemm_i8(
 
 
   constexpr int kFill = (A_MODE == 1) ? (int)0x80808080 : 0;
+  const int KTs = Kpad / BK; // K steps: stride between column tiles of Bp
 
   // Global loads only fetch; uint8 data is shifted to int8 after it is read
   // back from LDS.  In the byte-wise path chunks outside [M,K] are filled with
@@ -366,10 +372,15 @@ __global__ __launch_bounds__(WGM *WGN * 64, MINB) void k_gemm_i8(
     }
 #pragma unroll
     for (int h = 0; h < CH_B; ++h) {
+      // Chunk q of the stage's Bp tile: KiB q/64 is (column tile (q/64)/2,
+      // half step (q/64)%2), 16 bytes per lane.  Bp is padded to
+      // [Npad, Kpad]: always in bounds and aligned.
       const int q = tid + h * THREADS;
-      const int r = q >> 2, c = q & 3;
-      // Bt is padded to [Npad, Kpad]: always in bounds and aligned.
-      rb[h] = *(const v4i *)(Bt + (int64_t)(n0 + r) * Kpad + k0 + c * 16);
+      const int ci = q >> 6;
+      rb[h] = *(const v4i *)(Bp +
+                             ((int64_t)((n0 >> 5) + (ci >> 1)) * KTs +
+                                 (k0 >> 6)) * 2048 +
+                             (ci & 1) * 1024 + (q & 63) * 16);
     }
   };
   auto store_lds = [&](int buf, const v4i(&ra)[CH_A], const v4i(&rb)[CH_B]) {
@@ -381,7 +392,7 @@ __global__ __launch_bounds__(WGM *WGN * 64, MINB) void k_gemm_i8(
 #pragma unroll
     for (int h = 0; h < CH_B; ++h) {
       const int q = tid + h * THREADS;
-      *(v4i *)(&sB[buf][lds_off(q >> 2, q & 3)]) = rb[h];
+      *(v4i *)(&sB[buf][q * 16]) = rb[h];
     }
   };
 
@@ -414,7 +425,8 @@ __global__ __launch_bounds__(WGM *WGN * 64, MINB) void k_gemm_i8(
       }
 #pragma unroll
       for (int j = 0; j < TN; ++j)
-        fb[j] = *(const v4i *)(&sB[buf][lds_off(wn * WTN + j * 32 + l32, c)]);
+        fb[j] = *(const v4i *)(&sB[buf][(((wn * TN + j) * 2 + s) * 64 + lane) *
+                                        16]);
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -470,8 +482,9 @@ __global__ __launch_bounds__(WGM *WGN * 64, MINB) void k_gemm_i8(
 // issues the copies, waits for its own to land, and meets the others at one
 // barrier per K step.
 //
-// LDS holds a ring of three stages (A tile + Bt tile of one 64-byte K step
-// each, same XOR-swizzled row layout as above).  In step k a wave
+// LDS holds a ring of three stages (A tile + Bp tile of one 64-byte K step
+// each; the A tile in the XOR-swizzled row layout, the Bp tile as it is in
+// global memory).  In step k a wave
 //   waits until its copies for step k have landed (those for k+1 stay in
 //   flight), passes the barrier -- now every wave's step-k data is in LDS and
 //   every wave is done reading stage (k-1)%3 --,
@@ -482,13 +495,13 @@ __global__ __launch_bounds__(WGM *WGN * 64, MINB) void k_gemm_i8(
 // they target.  The counts waited for below are therefore explicit.
 template <int BN, int NSTAGE, int MINB, int A_MODE, int EPI>
 __global__ __launch_bounds__(256, MINB) void k_gemm_i8_dma(
-    const uint8_t *__restrict__ A, const int8_t *__restrict__ Bt, int M, int N,
+    const uint8_t *__restrict__ A, const int8_t *__restrict__ Bp, int M, int N,
     int K, int Kpad, EpiParams ep, int tiles_m, int tiles_n) {
   // 2 x 2 waves, each a 64 x (BN/2) tile.
   constexpr int BM = 128, WTM = 64, WTN = BN / 2, TM = 2, TN = WTN / 32;
   static_assert(BN == 128 || BN == 64, "tile width");
   constexpr int STAGE = (BM + BN) * BK;
-  constexpr int CB = BN / 64;      // Bt copies per wave and step
+  constexpr int CB = BN / 64;      // Bp copies per wave and step
   constexpr int CPW = 2 + CB;      // copies per wave and step
   __shared__ __attribute__((aligned(1024))) uint8_t sm[NSTAGE * STAGE];
 
@@ -515,11 +528,13 @@ __global__ __launch_bounds__(256, MINB) void k_gemm_i8_dma(
   const int l32 = lane & 31;
   const int lh = lane >> 5;
 
-  // Copy addressing.  Copy instruction j of a tile fills LDS bytes
+  // Copy addressing.  Copy instruction j of the A tile fills LDS bytes
   // [j*1024, (j+1)*1024): lane -> row j*16 + lane/4, chunk position lane%4,
   // which holds chunk (lane%4) ^ ((row/4)%4) = (lane%4) ^ ((lane/16)%4) of the
-  // row.  A wave issues copies 2*wave, 2*wave+1 of A and CB consecutive copies
-  // of Bt.
+  // row.  Copy instruction c of the Bp tile moves KiB c of the stage, which
+  // is (column tile c/2, half step c%2), unchanged.  A wave issues copies
+  // 2*wave, 2*wave+1 of A and CB consecutive copies of Bp.
+  const int KT = Kpad / BK;
   const int crow = lane >> 2;
   const int cchunk = (lane & 3) ^ ((lane >> 4) & 3);
   const uint8_t *ga[2];
@@ -532,8 +547,9 @@ __global__ __launch_bounds__(256, MINB) void k_gemm_i8_dma(
   }
 #pragma unroll
   for (int h = 0; h < CB; ++h) {
-    const int r = (wave * CB + h) * 16 + crow;
-    gb[h] = Bt + (int64_t)(n0 + r) * Kpad + cchunk * 16;
+    const int c = wave * CB + h;
+    gb[h] = Bp + (int64_t)((n0 >> 5) + (c >> 1)) * KT * 2048 + (c & 1) * 1024 +
+            lane * 16;
   }
   typedef __attribute__((address_space(3))) void *lds_ptr;
   typedef const __attribute__((address_space(1))) void *glb_ptr;
@@ -545,7 +561,7 @@ __global__ __launch_bounds__(256, MINB) void k_gemm_i8_dma(
           (lds_ptr)(base + (wave * 2 + h) * 1024), 16, 0, 0);
 #pragma unroll
     for (int h = 0; h < CB; ++h)
-      __builtin_amdgcn_global_load_lds((glb_ptr)(gb[h] + k0),
+      __builtin_amdgcn_global_load_lds((glb_ptr)(gb[h] + k0 * 32),
           (lds_ptr)(base + BM * BK + (wave * CB + h) * 1024), 16, 0, 0);
   };
 
@@ -556,7 +572,7 @@ __global__ __launch_bounds__(256, MINB) void k_gemm_i8_dma(
 #pragma unroll
   for (int s = 0; s < 2; ++s) {
     ra[s] = sm_base + lds_off(wm * WTM + l32, s * 2 + lh);
-    rb[s] = sm_base + BM * BK + lds_off(wn * WTN + l32, s * 2 + lh);
+    rb[s] = sm_base + BM * BK + ((wn * TN * 2 + s) * 64 + lane) * 16;
   }
 
   v16i acc[TM][TN];
@@ -568,7 +584,6 @@ __global__ __launch_bounds__(256, MINB) void k_gemm_i8_dma(
       for (int r = 0; r < 16; ++r)
         acc[i][j][r] = 0;
 
-  const int KT = Kpad / BK;
   const int klast = (KT - 1) * BK;
   auto kclamp = [&](int step) { return step < KT ? step * BK : klast; };
 #pragma unroll
@@ -663,21 +678,19 @@ __global__ __launch_bounds__(256, MINB) void k_gemm_i8_dma(
       acc, m0 + wm * WTM, n0 + wn * WTN, M, N, K, ep);
 }
 
-// ---- GEMM, Bt streamed to registers from a fragment-ordered copy -----------
-// The right-hand side of a quantised layer is a model constant, so it can be
-// stored once in exactly the order the matrix cores consume it (Bp, the
-// layout written by k_pack_frag): the operand of column tile nt, K step ks,
-// half step sub is one contiguous KiB, 16 bytes per lane.  The four waves of a
-// block sit side by side along N; each owns 32*TN columns that no other wave
-// needs and loads their operands from Bp straight into registers, D steps
-// ahead.  Only the A tile, which all four waves share, goes through LDS, and
-// it gets there without passing through registers (see k_gemm_i8_dma).  Per K
-// step a block therefore moves half as many bytes into LDS as the kernels
-// above, and the copy path into LDS is what bounds those.
+// ---- GEMM, Bp streamed to registers -----------------------------------------
+// The right-hand side is stored in exactly the order the matrix cores consume
+// it: the operand of column tile nt, K step ks, half step sub is one
+// contiguous KiB, 16 bytes per lane.  The four waves of a block sit side by
+// side along N; each owns 32*TN columns that no other wave needs and loads
+// their operands from Bp straight into registers, D steps ahead.  Only the A
+// tile, which all four waves share, goes through LDS, and it gets there
+// without passing through registers (see k_gemm_i8_dma).  Per K step a block
+// therefore moves half as many bytes into LDS as that kernel, and the copy
+// path into LDS is what bounds it.
 //
 // PIPE (needs NST >= 4) reads the operands of each half step one half step
-// early, see the loop.  It pays for the 128 x 256 tile and not for the
-// 128 x 128 one (measured).
+// early, see the loop.
 //
 // Per step, in this order (so that the explicit wait below can count):
 //   wait for own A copies of this step, barrier
@@ -964,109 +977,92 @@ __global__ __launch_bounds__(256, MINB) void k_gemm_i8_bs(
   gemm_epilogue<TM, TN, A_MODE, EPI>(acc, m0, ncol0, M, N, K, ep);
 }
 
-// ---- skinny GEMM (M <= 16): weight streaming -------------------------------
-// With at most 16 rows the product is bound by reading the weights once, so
-// the kernel is organised around keeping many KiB of Bt in flight per CU and
-// nothing else: a block owns 32 output columns, its 8 waves split K between
-// them, and each wave streams its slice of the 32 Bt rows straight from
-// global memory into v_mfma_i32_16x16x64_i8 operands (lane = column, 16
-// K-bytes per lane; a wave instruction reads 16 rows x 64 contiguous bytes).
-// The tiny A operand (rows padded to 16 with zeros) comes from L2.  The eight
-// partial 16x32 results are summed through LDS and the usual epilogue runs on
-// the sum.  No LDS staging, no barrier in the K loop.
-template <int NG, int A_MODE, int EPI>
-__global__ __launch_bounds__(512) void k_gemm_i8_skinny(
-    const uint8_t *__restrict__ A, const int8_t *__restrict__ Bt, int M, int N,
+// ---- skinny GEMM (M <= 32): weight streaming -------------------------------
+// With at most 32 rows the product is bound by reading the weights once, so
+// the kernel is organised around keeping many KiB of Bp in flight per CU and
+// nothing else: a block owns one 32-column tile, whose operands for all of K
+// are one contiguous run of Bp (2 KiB per K step); its 8 waves take
+// contiguous slices of K, and every Bp load is a fully coalesced KiB.  A (at
+// most 32 rows, zero rows above M) is read from L2 in operand layout.  The
+// eight partial 32x32 results are summed through LDS.  No LDS staging, no
+// barrier in the K loop.
+template <int A_MODE, int EPI>
+__global__ __launch_bounds__(512) void k_gemm_i8_skinny_bp(
+    const uint8_t *__restrict__ A, const int8_t *__restrict__ Bp, int M, int N,
     int K, int Kpad, EpiParams ep) {
-  constexpr int WAVES = 8, U = 8;
-  __shared__ int32_t part[WAVES][NG][4][64];
+  constexpr int WAVES = 8, U = 4;
+  __shared__ int32_t part[WAVES][16][64];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int l16 = lane & 15;
-  const int lq = lane >> 4; // K quarter of the 64-byte step
-  const int n0 = blockIdx.x * 16 * NG;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l32 = lane & 31;
+  const int lh = lane >> 5;
+  const int nt = blockIdx.x;
 
   const int KT = Kpad / BK;
   const int per = (KT + WAVES - 1) / WAVES;
   const int kt_begin = wave * per;
   const int kt_end = (kt_begin + per < KT) ? kt_begin + per : KT;
 
-  // Row l16 of A (clamped; rows >= M are zeroed after the load).
-  const bool row_ok = l16 < M;
-  const uint8_t *__restrict__ ap =
-      A + (int64_t)(row_ok ? l16 : 0) * K + (lq * 16 < K ? lq * 16 : 0);
-  const int8_t *__restrict__ bp0 = Bt + (int64_t)(n0 + l16) * Kpad + lq * 16;
-  const int8_t *__restrict__ bp1 = bp0 + (int64_t)(NG > 1 ? 16 : 0) * Kpad;
-  const int klim = K - lq * 16; // chunks starting at or past this are absent
-
-  v4i acc0 = {0, 0, 0, 0}, acc1 = {0, 0, 0, 0};
+  const bool row_ok = l32 < M;
+  const uint8_t *__restrict__ ap = A + (int64_t)(row_ok ? l32 : 0) * K;
+  const int8_t *__restrict__ bp = Bp + (int64_t)nt * KT * 2048 + lane * 16;
   constexpr int kFill = (A_MODE == 1) ? (int)0x80808080 : 0;
+
+  v16i acc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r)
+    acc[r] = 0;
   for (int kt = kt_begin; kt < kt_end; kt += U) {
-    v4i a[U], b0[U], b1[U];
+    v4i a[U][2], b[U][2];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       // steps past this wave's slice reload its last step and are discarded
       const int s = (kt + u < kt_end) ? kt + u : kt_end - 1;
-      const int k0 = s * BK;
-      const int ka = (k0 < klim) ? k0 : 0; // in bounds whatever K is
-      a[u] = *(const v4i *)(ap + ka);
-      if (!(row_ok && k0 < klim))
-        a[u] = (v4i){kFill, kFill, kFill, kFill};
-      b0[u] = *(const v4i *)(bp0 + k0);
-      if (NG > 1)
-        b1[u] = *(const v4i *)(bp1 + k0);
+#pragma unroll
+      for (int sub = 0; sub < 2; ++sub) {
+        const int k0 = s * BK + (sub * 2 + lh) * 16;
+        const bool in = row_ok && k0 < K; // K % 16 == 0: a chunk is in or out
+        a[u][sub] = *(const v4i *)(ap + (in ? k0 : 0));
+        if (!in)
+          a[u][sub] = (v4i){kFill, kFill, kFill, kFill};
+        b[u][sub] = *(const v4i *)(bp + (int64_t)s * 2048 + sub * 1024);
+      }
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       if (kt + u < kt_end) {
-        v4i av = a[u];
-        if (A_MODE == 1)
-          av ^= (v4i){(int)0x80808080, (int)0x80808080, (int)0x80808080,
-              (int)0x80808080};
-        acc0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, b0[u], acc0, 0, 0, 0);
-        if (NG > 1)
-          acc1 =
-              __builtin_amdgcn_mfma_i32_16x16x64_i8(av, b1[u], acc1, 0, 0, 0);
+#pragma unroll
+        for (int sub = 0; sub < 2; ++sub) {
+          v4i av = a[u][sub];
+          if (A_MODE == 1)
+            av ^= (v4i){(int)0x80808080, (int)0x80808080, (int)0x80808080,
+                (int)0x80808080};
+          acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(
+              av, b[u][sub], acc, 0, 0, 0);
+        }
       }
     }
   }
 #pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    part[wave][0][r][lane] = acc0[r];
-    if (NG > 1)
-      part[wave][1][r][lane] = acc1[r];
-  }
+  for (int r = 0; r < 16; ++r)
+    part[wave][r][lane] = acc[r];
   __syncthreads();
 
-  // 16x16 accumulator layout: lane holds column (lane & 15); register r holds
-  // row 4*(lane/16) + r.  Thread t finishes element (g, r, lane) = t.
-  const int g = tid >> 8, r = (tid >> 6) & 3;
-  if (g >= NG)
-    return;
-  uint32_t y = 0;
-#pragma unroll
-  for (int w = 0; w < WAVES; ++w)
-    y += (uint32_t)part[w][g][r][lane];
-  const int m = 4 * lq + r;
-  const int n = n0 + g * 16 + l16;
-  if (m >= M || n >= N)
-    return;
-
+  // 32x32 accumulator layout: lane holds column (lane & 31); register r holds
+  // row 8*(r/4) + 4*(lane/32) + r%4.  Thread t finishes elements (r, lane)
+  // with r = t / 64 and r + 8.
   constexpr bool A_OFF = (A_MODE != 0);
   const int32_t oa = A_OFF ? 128 : 0;
   const int32_t ob = ep.b_unsigned ? 128 : 0;
-  int32_t da = oa, db = ob, rs = 0;
-  if (ep.a_zp_len > 0)
-    da = oa - load_zp_i32(ep.a_zp, A_OFF, ep.a_zp_len > 1 ? m : 0);
+  const int n = nt * 32 + l32;
+  if (n >= N)
+    return;
+  int32_t db = ob;
   if (ep.b_zp_len > 0)
     db = ob - load_zp_i32(ep.b_zp, ep.b_unsigned, ep.b_zp_len > 1 ? n : 0);
-  if (ep.rowsum)
-    rs = ep.rowsum[m];
-  y += (uint32_t)da * (uint32_t)ep.colsum[n];
-  y += (uint32_t)db * (uint32_t)rs;
-  y += (uint32_t)K * (uint32_t)da * (uint32_t)db;
+  const int32_t cs = ep.colsum[n];
   float sj = 0.0f;
   int32_t yz = 0;
   if (EPI != kEpiI32) {
@@ -1076,21 +1072,42 @@ __global__ __launch_bounds__(512) void k_gemm_i8_skinny(
       yz = load_zp_i32(ep.y_zp, ep.y_unsigned, 0);
     }
   }
-  store_one<EPI>(ep, (int64_t)m * N + n, y, sj, yz);
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int r = (tid >> 6) + h * 8;
+    const int m = 8 * (r >> 2) + 4 * lh + (r & 3);
+    if (m >= M)
+      continue;
+    uint32_t y = 0;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w)
+      y += (uint32_t)part[w][r][lane];
+    int32_t da = oa, rs = 0;
+    if (ep.a_zp_len > 0)
+      da = oa - load_zp_i32(ep.a_zp, A_OFF, ep.a_zp_len > 1 ? m : 0);
+    if (ep.rowsum)
+      rs = ep.rowsum[m];
+    y += (uint32_t)da * (uint32_t)cs;
+    y += (uint32_t)db * (uint32_t)rs;
+    y += (uint32_t)K * (uint32_t)da * (uint32_t)db;
+    store_one<EPI>(ep, (int64_t)m * N + n, y, sj, yz);
+  }
 }
 
 // ---- pack B ---------------------------------------------------------------
-// One block transposes a 64(k) x 64(n) tile through LDS and adds the tile's
-// column sums into colsum with int32 atomics (integer adds commute, so the
-// result does not depend on arrival order).
+// One block transposes a 64(k) x 64(n) tile of B [K,N] through LDS, writes it
+// in MFMA operand order (see the top of the file) and adds the tile's column
+// sums into colsum with int32 atomics (integer adds commute, so the result
+// does not depend on arrival order).
 constexpr int PT = 64;
 
 template <bool B_UNSIGNED>
 __global__ __launch_bounds__(256) void k_pack_b(const uint8_t *__restrict__ B,
-    int64_t K, int64_t N, int64_t Kpad, int8_t *__restrict__ Bt,
+    int64_t K, int64_t N, int KT, int8_t *__restrict__ Bp,
     int32_t *__restrict__ colsum) {
   __shared__ uint8_t tile[PT][PT + 4];
-  const int64_t k0 = (int64_t)blockIdx.y * PT;
+  const int ks = blockIdx.y; // K step of 64
+  const int64_t k0 = (int64_t)ks * PT;
   const int64_t n0 = (int64_t)blockIdx.x * PT;
   const int tid = threadIdx.x;
   // Read: thread -> row k = tid/4, 16 columns starting at (tid%4)*16.
@@ -1110,58 +1127,29 @@ __global__ __launch_bounds__(256) void k_pack_b(const uint8_t *__restrict__ B,
     }
   }
   __syncthreads();
-  // Write: thread -> column n = tid/4, 16 k values starting at (tid%4)*16.
+  // Write: thread -> column n = tid/4, 16-byte chunk c = tid%4 of the step.
   {
     const int nr = tid >> 2;
-    const int kc = (tid & 3) * 16;
+    const int c = tid & 3;
     uint32_t w[4] = {0, 0, 0, 0};
     int32_t sum = 0;
 #pragma unroll
     for (int b = 0; b < 16; ++b) {
-      const uint8_t v = tile[kc + b][nr];
+      const uint8_t v = tile[c * 16 + b][nr];
       sum += (int32_t)(int8_t)v;
       w[b >> 2] |= (uint32_t)v << ((b & 3) * 8);
     }
     const int64_t n = n0 + nr;
-    // Bt has Npad >= gridDim.x*64 rows and Kpad >= gridDim.y*64 columns.
-    *(v4i *)(Bt + n * Kpad + k0 + kc) =
-        (v4i){(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+    // The grid covers [Npad, Kpad] exactly: every byte of Bp is written.
+    const int64_t o =
+        ((((n >> 5) * KT + ks) * 2 + (c >> 1)) * 64 + (c & 1) * 32 + (n & 31)) *
+        16;
+    *(v4i *)(Bp + o) = (v4i){(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
     // Fold the four k-chunks of this column (lanes 4n..4n+3) before the atomic.
     sum += __shfl_xor(sum, 1, 64);
     sum += __shfl_xor(sum, 2, 64);
     if ((tid & 3) == 0 && sum != 0)
       atomicAdd(&colsum[n], sum);
-  }
-}
-
-// ---- fragment order ----------------------------------------------------------
-// Rewrites a row-major int8 matrix X [R, Kpad] (R a multiple of 32, Kpad of
-// 64; here: the packed Bt) into the order in which the matrix cores consume
-// it, so that a wave can load an MFMA operand with one fully coalesced
-// instruction:
-//   Xp[rt][ks][sub][lane][16 bytes],  rt = row / 32, ks = K step of 64 bytes,
-//   lane = (chunk & 1) * 32 + row % 32, sub = chunk >> 1 for the 16-byte chunk
-//   `chunk` (0..3) of the step.
-// One block handles one row tile and four K steps.
-__global__ __launch_bounds__(256) void k_pack_frag(
-    const int8_t *__restrict__ X, int64_t Kpad, int KT, int8_t *__restrict__ Xp) {
-  const int rt = blockIdx.y;
-  const int ks0 = blockIdx.x * 4;
-#pragma unroll
-  for (int h = 0; h < 2; ++h) {
-    const int q = threadIdx.x + h * 256; // 512 chunks: 32 rows x 16 chunks
-    const int row = q >> 4;
-    const int c16 = q & 15;
-    const int ks = ks0 + (c16 >> 2);
-    if (ks >= KT)
-      continue;
-    const int c = c16 & 3;
-    const v4i v = *(const v4i *)(X + ((int64_t)rt * 32 + row) * Kpad +
-                                 (int64_t)ks * 64 + c * 16);
-    const int sub = c >> 1, half = c & 1;
-    const int64_t o =
-        ((((int64_t)rt * KT + ks) * 2 + sub) * 64 + half * 32 + row) * 16;
-    *(v4i *)(Xp + o) = v;
   }
 }
 
@@ -1193,22 +1181,16 @@ __global__ __launch_bounds__(256) void k_rowsum_a(
 enum TileCfg : int {
   kT128x128 = 0, // k_gemm_i8: register-staged tiles (and the byte-wise path)
   kD128x128 = 1, // k_gemm_i8_dma: tiles copied straight into LDS
-  kB128x128 = 2, // k_gemm_i8_bs: Bt from its fragment-ordered copy
-  kB128x256 = 3,
-  kNumCfg = 4
+  kB128x256 = 2, // k_gemm_i8_bs: Bp straight into registers
+  kNumCfg = 3
 };
 
-bool cfg_needs_bp(int c) { return c == kB128x128 || c == kB128x256; }
-
-// Kernel choice for problems with more than 16 rows, K % 64 == 0 and a
+// Kernel choice for problems with more than 32 rows, K % 64 == 0 and a
 // 16-byte aligned A (anything else takes the byte-wise path of k_gemm_i8).
 // Measured on MI355X over the BERT-base and Llama-7B layer shapes and square
-// problems up to 8192:
-//  * at most one 128 x 128 tile per CU: k_gemm_i8_dma is fastest (a lone
-//    block per CU gains nothing from the lighter LDS traffic of the others);
-//  * otherwise the kernels that stream Bt from its fragment-ordered copy win,
-//    with 128 x 256 tiles unless those would leave most CUs idle in a second,
-//    nearly empty round (between 1 and 1.4 tiles per CU).
+// problems up to 8192: a 128 x 256 tile of k_gemm_i8_bs costs about 1.7 times
+// a 128 x 128 tile of k_gemm_i8_dma, so it wins when it needs at most half as
+// many rounds over the 256 CUs and fills at least one round.
 // Override for tests and tuning: OM_MI355X_GEMM_TILE=<TileCfg value>.
 int choose_tile(int64_t M, int64_t N) {
   const char *force = getenv("OM_MI355X_GEMM_TILE");
@@ -1219,12 +1201,11 @@ int choose_tile(int64_t M, int64_t N) {
   }
   const int64_t tm = (M + 127) / 128;
   const int64_t t128 = tm * ((N + 127) / 128);
-  if (t128 <= 256)
-    return kD128x128;
   const int64_t t256 = tm * ((N + 255) / 256);
-  if (t256 <= 256 || t256 * 10 >= 256 * 14)
+  const int64_t r128 = (t128 + 255) / 256, r256 = (t256 + 255) / 256;
+  if (t256 >= 256 && r256 * 17 < r128 * 10)
     return kB128x256;
-  return kB128x128;
+  return kD128x128;
 }
 
 bool gemm_fast_path(int64_t M, int64_t K, const void *A) {
@@ -1237,18 +1218,11 @@ hipError_t gemm_launch_cfg(
   const char *force = getenv("OM_MI355X_GEMM_TILE");
   const uint8_t *A = (const uint8_t *)g.A;
   const int M = (int)g.M, N = (int)g.N, K = (int)g.K;
-  if (g.M <= 16 && g.K % 16 == 0 && ((((uintptr_t)g.A) & 15) == 0) &&
+  if (g.M <= 32 && g.K % 16 == 0 && ((((uintptr_t)g.A) & 15) == 0) &&
       !(force && force[0])) {
-    // 32 columns per block halves the reads of A (measured faster whenever
-    // that still gives every CU a block); 16 columns for narrower outputs.
-    if ((g.N + 31) / 32 >= 256)
-      k_gemm_i8_skinny<2, A_MODE, EPI>
-          <<<dim3((unsigned)((g.N + 31) / 32)), 512, 0, st>>>(
-              A, g.Bt, M, N, K, Kpad, ep);
-    else
-      k_gemm_i8_skinny<1, A_MODE, EPI>
-          <<<dim3((unsigned)((g.N + 15) / 16)), 512, 0, st>>>(
-              A, g.Bt, M, N, K, Kpad, ep);
+    k_gemm_i8_skinny_bp<A_MODE, EPI>
+        <<<dim3((unsigned)((g.N + 31) / 32)), 512, 0, st>>>(
+            A, g.Bp, M, N, K, Kpad, ep);
     return hipGetLastError();
   }
   const int tiles_m = (int)((g.M + 127) / 128);
@@ -1258,13 +1232,10 @@ hipError_t gemm_launch_cfg(
     // configurations of the tests when M <= 16).
     k_gemm_i8<128, 128, 2, 2, 2, A_MODE, EPI, false>
         <<<dim3((unsigned)(tiles_m * tiles_n128)), 256, 0, st>>>(
-            A, g.Bt, M, N, K, Kpad, ep, tiles_m, tiles_n128);
+            A, g.Bp, M, N, K, Kpad, ep, tiles_m, tiles_n128);
     return hipGetLastError();
   }
-  int cfg = choose_tile(g.M, g.N);
-  if (cfg_needs_bp(cfg) && !g.Bp)
-    cfg = kD128x128;
-  switch (cfg) {
+  switch (choose_tile(g.M, g.N)) {
   case kB128x256: {
     const int tiles_n = (int)((g.N + 255) / 256);
     k_gemm_i8_bs<4, 2, 4, 4, 2, true, A_MODE, EPI>
@@ -1272,20 +1243,15 @@ hipError_t gemm_launch_cfg(
             A, g.Bp, M, N, K, Kpad, ep, tiles_m, tiles_n);
     break;
   }
-  case kB128x128:
-    k_gemm_i8_bs<4, 1, 4, 3, 3, false, A_MODE, EPI>
-        <<<dim3((unsigned)(tiles_m * tiles_n128)), 256, 0, st>>>(
-            A, g.Bp, M, N, K, Kpad, ep, tiles_m, tiles_n128);
-    break;
   case kD128x128:
     k_gemm_i8_dma<128, 3, 3, A_MODE, EPI>
         <<<dim3((unsigned)(tiles_m * tiles_n128)), 256, 0, st>>>(
-            A, g.Bt, M, N, K, Kpad, ep, tiles_m, tiles_n128);
+            A, g.Bp, M, N, K, Kpad, ep, tiles_m, tiles_n128);
     break;
   default:
     k_gemm_i8<128, 128, 2, 2, 3, A_MODE, EPI, true>
         <<<dim3((unsigned)(tiles_m * tiles_n128)), 256, 0, st>>>(
-            A, g.Bt, M, N, K, Kpad, ep, tiles_m, tiles_n128);
+            A, g.Bp, M, N, K, Kpad, ep, tiles_m, tiles_n128);
     break;
   }
   return hipGetLastError();
@@ -1307,37 +1273,22 @@ hipError_t gemm_launch_epi(
 } // namespace
 
 hipError_t launch_pack_b(hipStream_t s, const void *B, bool b_unsigned,
-    int64_t K, int64_t N, int8_t *Bt, int32_t *colsum) {
-  const int64_t Kpad = round_up(K, kGemmBK);
+    int64_t K, int64_t N, int8_t *Bp, int32_t *colsum) {
+  const int64_t Kpad = round_up(K > 0 ? K : 1, kGemmBK);
   const int64_t Npad = round_up(N, kGemmBN);
   hipError_t e = launch_fill_u32(s, (uint32_t *)colsum, Npad, 0u);
   if (e != hipSuccess)
     return e;
   // kGemmBK and kGemmBN are multiples of the 64 x 64 pack tile, so the grid
-  // covers [Npad, Kpad] exactly and every byte of Bt is written.
+  // covers [Npad, Kpad] exactly and every byte of Bp is written.
+  const int KT = (int)(Kpad / kGemmBK);
   dim3 grid((unsigned)(Npad / PT), (unsigned)(Kpad / PT));
   if (b_unsigned)
     k_pack_b<true><<<grid, 256, 0, s>>>(
-        (const uint8_t *)B, K, N, Kpad, Bt, colsum);
+        (const uint8_t *)B, K, N, KT, Bp, colsum);
   else
     k_pack_b<false><<<grid, 256, 0, s>>>(
-        (const uint8_t *)B, K, N, Kpad, Bt, colsum);
-  return hipGetLastError();
-}
-
-bool gemm_wants_bp(int64_t M, int64_t K, int64_t N, const void *A) {
-  (void)K;
-  return gemm_fast_path(M, K, A) && cfg_needs_bp(choose_tile(M, N));
-}
-
-hipError_t launch_pack_bp(
-    hipStream_t s, const int8_t *Bt, int64_t K, int64_t N, int8_t *Bp) {
-  // Bt is [Npad, Kpad] and fully written (padding is zero).
-  const int64_t Kpad = round_up(K > 0 ? K : 1, kGemmBK);
-  const int64_t Npad = round_up(N, kGemmBN);
-  const int KT = (int)(Kpad / kGemmBK);
-  dim3 grid((unsigned)((KT + 3) / 4), (unsigned)(Npad / 32));
-  k_pack_frag<<<grid, 256, 0, s>>>(Bt, Kpad, KT, Bp);
+        (const uint8_t *)B, K, N, KT, Bp, colsum);
   return hipGetLastError();
 }
 

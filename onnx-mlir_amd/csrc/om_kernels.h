@@ -40,15 +40,16 @@ hipError_t launch_dynamic_quantize(hipStream_t s, const DqlScratch &scratch,
     bool y_shift);
 
 // ---- int8 GEMM ------------------------------------------------------------
-// B [K,N] row-major (u8 or i8) -> Bt [Npad, Kpad] int8, K-contiguous, with
-// u8 shifted to int8 by -128, zero filled outside [N,K]; colsum[n] = sum_k of
-// the int8 values written (int32), colsum has Npad entries.
+// B [K,N] row-major (u8 or i8) -> Bp, Npad * Kpad bytes of int8 in MFMA
+// operand order: Bp[n/32][k/64][half step][lane][16 B], u8 shifted to int8
+// by -128, zero filled outside [N,K]; colsum[n] = sum_k of the int8 values
+// written (int32), colsum has Npad entries.
 constexpr int kGemmBK = 64;    // K granularity of the packed operand
 constexpr int kGemmBN = 256;   // N granularity of the packed operand (largest tile)
 inline int64_t round_up(int64_t v, int64_t m) { return (v + m - 1) / m * m; }
 
 hipError_t launch_pack_b(hipStream_t s, const void *B, bool b_unsigned,
-    int64_t K, int64_t N, int8_t *Bt, int32_t *colsum);
+    int64_t K, int64_t N, int8_t *Bp, int32_t *colsum);
 
 // rowsum[m] = sum_k (A[m,k] - (a_unsigned ? 128 : 0)).
 hipError_t launch_rowsum_a(hipStream_t s, const void *A, bool a_unsigned,
@@ -58,8 +59,7 @@ struct GemmArgs {
   const void *A;       // [M,K] row-major, u8 or i8
   bool a_unsigned;     // A holds u8
   bool a_preshifted;   // A already holds (u8 - 128) as int8; offsets as for u8
-  const int8_t *Bt;    // packed [Npad,Kpad]
-  const int8_t *Bp;    // fragment-ordered copy of Bt (launch_pack_bp), or null
+  const int8_t *Bp;    // B in MFMA operand order (launch_pack_b)
   bool b_unsigned;     // original B was u8 (packed values are B - 128)
   int64_t M, K, N;
   const void *a_zp;    // element type follows A; may be null
@@ -83,13 +83,6 @@ struct GemmArgs {
 };
 
 hipError_t launch_gemm(hipStream_t s, const GemmArgs &g);
-
-// True when launch_gemm would use the fragment-ordered copy of Bt for this
-// problem (GemmArgs::Bp); the caller then builds it with launch_pack_bp, into
-// a buffer of round_up(N, kGemmBN) * round_up(K, kGemmBK) bytes.
-bool gemm_wants_bp(int64_t M, int64_t K, int64_t N, const void *A);
-hipError_t launch_pack_bp(
-    hipStream_t s, const int8_t *Bt, int64_t K, int64_t N, int8_t *Bp);
 
 // Fill n 32-bit words with v.
 hipError_t launch_fill_u32(hipStream_t s, uint32_t *p, int64_t n, uint32_t v);

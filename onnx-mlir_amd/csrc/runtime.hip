@@ -79,11 +79,10 @@ struct DevCopy {
 std::unordered_map<const void *, DevCopy> g_const_copies;
 // Packed right-hand sides of constant B, keyed by B's data pointer.
 struct PackedB {
-  int8_t *bt;
+  int8_t *bp;
   int32_t *colsum;
   int64_t K, N;
   bool is_unsigned;
-  int8_t *bp; // fragment-ordered copy of bt, made on first use
 };
 std::unordered_map<const void *, PackedB> g_packed;
 
@@ -457,17 +456,13 @@ bool matmul_dims(const View &a, const View &b, const char *op, int64_t &M,
 }
 
 // Packed form of B: from the cache when B was declared constant, otherwise
-// packed into pool buffers for this call only.  With want_bp the
-// fragment-ordered copy of the packed matrix is produced as well (for a
-// constant: on the first call that asks for it).
-bool packed_b(Call &call, const View &b, int64_t K, int64_t N, bool want_bp,
-    const int8_t *&bt, const int32_t *&colsum, const int8_t *&bp) {
+// packed into pool buffers for this call only.
+bool packed_b(Call &call, const View &b, int64_t K, int64_t N,
+    const int8_t *&bp, const int32_t *&colsum) {
   const bool uns = b.dtype == OM_MI355X_TYPE_UINT8;
   const int64_t Kpad = round_up(K > 0 ? K : 1, kGemmBK);
   const int64_t Npad = round_up(N, kGemmBN);
-  const size_t bt_bytes = (size_t)Kpad * Npad;
-  bp = nullptr;
-  bool constant, cached = false;
+  bool constant;
   {
     std::lock_guard<std::mutex> lk(g_mem_mutex);
     constant = g_constants.count(b.data) != 0;
@@ -475,94 +470,49 @@ bool packed_b(Call &call, const View &b, int64_t K, int64_t N, bool want_bp,
       auto it = g_packed.find(b.data);
       if (it != g_packed.end() && it->second.K == K && it->second.N == N &&
           it->second.is_unsigned == uns) {
-        bt = it->second.bt;
-        colsum = it->second.colsum;
         bp = it->second.bp;
-        cached = true;
+        colsum = it->second.colsum;
+        return true;
       }
     }
   }
-  if (cached && (!want_bp || bp))
-    return true;
-
-  if (!cached) {
-    const void *db = call.in(b);
-    if (!call.ok)
+  const void *db = call.in(b);
+  if (!call.ok)
+    return false;
+  int8_t *pbp;
+  int32_t *pcs;
+  if (constant) {
+    void *p = nullptr, *q = nullptr;
+    if (hipMalloc(&p, (size_t)Kpad * Npad) != hipSuccess ||
+        hipMalloc(&q, (size_t)Npad * 4) != hipSuccess) {
+      fail(EIO, "hipMalloc for a packed constant failed");
+      call.ok = false;
       return false;
-    int8_t *pbt;
-    int32_t *pcs;
-    if (constant) {
-      void *p = nullptr, *q = nullptr;
-      if (hipMalloc(&p, bt_bytes) != hipSuccess ||
-          hipMalloc(&q, (size_t)Npad * 4) != hipSuccess) {
-        fail(EIO, "hipMalloc for a packed constant failed");
-        call.ok = false;
-        return false;
-      }
-      pbt = (int8_t *)p;
-      pcs = (int32_t *)q;
-    } else {
-      pbt = (int8_t *)call.temp(bt_bytes);
-      pcs = (int32_t *)call.temp((size_t)Npad * 4);
-      if (!call.ok)
-        return false;
     }
-    call.check(launch_pack_b(call.c.stream, db, uns, K, N, pbt, pcs), "pack B");
+    pbp = (int8_t *)p;
+    pcs = (int32_t *)q;
+  } else {
+    pbp = (int8_t *)call.temp((size_t)Kpad * Npad);
+    pcs = (int32_t *)call.temp((size_t)Npad * 4);
     if (!call.ok)
       return false;
-    bt = pbt;
-    colsum = pcs;
   }
-
-  int8_t *pbp = nullptr;
-  if (want_bp) {
-    if (constant) {
-      void *p = nullptr;
-      if (hipMalloc(&p, bt_bytes) != hipSuccess) {
-        fail(EIO, "hipMalloc for a packed constant failed");
-        call.ok = false;
-        return false;
-      }
-      pbp = (int8_t *)p;
-    } else {
-      pbp = (int8_t *)call.temp(bt_bytes);
-      if (!call.ok)
-        return false;
-    }
-    call.check(launch_pack_bp(call.c.stream, bt, K, N, pbp), "reorder B");
-    if (!call.ok)
-      return false;
-    bp = pbp;
-  }
-
+  call.check(launch_pack_b(call.c.stream, db, uns, K, N, pbp, pcs), "pack B");
+  if (!call.ok)
+    return false;
   if (constant) {
     // Other threads use their own streams: make the packed data final first.
     call.check(hipStreamSynchronize(call.c.stream), "pack B synchronise");
     std::lock_guard<std::mutex> lk(g_mem_mutex);
-    auto it = g_packed.find(b.data);
-    if (!cached) {
-      if (it != g_packed.end()) {
-        (void)hipFree(it->second.bt);
-        (void)hipFree(it->second.colsum);
-        if (it->second.bp)
-          (void)hipFree(it->second.bp);
-        g_packed.erase(it);
-      }
-      g_packed.emplace(b.data,
-          PackedB{const_cast<int8_t *>(bt), const_cast<int32_t *>(colsum), K,
-              N, uns, pbp});
-    } else if (pbp) {
-      if (it != g_packed.end() && it->second.bt == bt) {
-        if (it->second.bp) {
-          // another thread got there first: use its copy
-          (void)hipFree(pbp);
-          bp = it->second.bp;
-        } else {
-          it->second.bp = pbp;
-        }
-      }
+    auto ins = g_packed.emplace(b.data, PackedB{pbp, pcs, K, N, uns});
+    if (!ins.second) {
+      (void)hipFree(ins.first->second.bp);
+      (void)hipFree(ins.first->second.colsum);
+      ins.first->second = PackedB{pbp, pcs, K, N, uns};
     }
   }
+  bp = pbp;
+  colsum = pcs;
   return true;
 }
 
@@ -669,8 +619,7 @@ void run_matmul(const MatmulSpec &sp) {
   g.K = K;
   g.N = N;
   const int32_t *colsum = nullptr;
-  if (!packed_b(call, b, K, N, gemm_wants_bp(M, K, N, g.A), g.Bt, colsum,
-          g.Bp)) {
+  if (!packed_b(call, b, K, N, g.Bp, colsum)) {
     call.finish();
     return;
   }
@@ -946,8 +895,7 @@ void om_mi355x_DynQuantMatMulDequant(OMTensor *y_t, const OMTensor *x_t,
   g.K = K;
   g.N = N;
   const int32_t *colsum = nullptr;
-  if (!call.ok || !packed_b(call, b, K, N, gemm_wants_bp(M, K, N, g.A), g.Bt,
-                      colsum, g.Bp)) {
+  if (!call.ok || !packed_b(call, b, K, N, g.Bp, colsum)) {
     call.finish();
     return;
   }
@@ -994,10 +942,8 @@ void om_mi355x_ClearCache(void) {
     (void)hipFree(kv.second.dev);
   g_const_copies.clear();
   for (auto &kv : g_packed) {
-    (void)hipFree(kv.second.bt);
+    (void)hipFree(kv.second.bp);
     (void)hipFree(kv.second.colsum);
-    if (kv.second.bp)
-      (void)hipFree(kv.second.bp);
   }
   g_packed.clear();
   g_constants.clear();
@@ -1029,10 +975,8 @@ void om_mi355x_free(void *p) {
     g_constants.erase(p);
     auto it = g_packed.find(p);
     if (it != g_packed.end()) {
-      (void)hipFree(it->second.bt);
+      (void)hipFree(it->second.bp);
       (void)hipFree(it->second.colsum);
-      if (it->second.bp)
-        (void)hipFree(it->second.bp);
       g_packed.erase(it);
     }
   }
