@@ -28,8 +28,15 @@ hipError_t launch_dequantize(hipStream_t s, const void *x, QKind xkind,
 struct DqlScratch {
   float *partial_min; // [kDqlMaxBlocks]
   float *partial_max; // [kDqlMaxBlocks]
-  unsigned *counter;  // [1]
+  unsigned *counter;  // [16], zeroed once: [0] two-pass arrivals, [4] barrier
+                      // of the one-launch kernel, [8] set if that barrier ever
+                      // timed out
+  int grid_blocks;    // dql_grid_blocks(), or 0 to disable the one-launch path
+  unsigned spin_limit; // polls a block waits at the barrier before giving up
 };
+// Blocks of the one-launch DynamicQuantizeLinear kernel that fit the current
+// device at once (0 if it cannot run here).
+int dql_grid_blocks();
 constexpr int kDqlMaxBlocks = 4096;
 
 // y u8[n], scale f32[1], zp u8[1].  If y_shift is true the stored bytes are

@@ -121,7 +121,7 @@ bool probe_device() {
 struct Ctx {
   bool ready = false;
   hipStream_t stream = nullptr;
-  DqlScratch dql = {nullptr, nullptr, nullptr};
+  DqlScratch dql = {nullptr, nullptr, nullptr, 0, 0};
   float *dql_scale = nullptr; // scale / zero point of the fused path
   uint8_t *dql_zp = nullptr;
   std::multimap<size_t, void *> pool;
@@ -145,10 +145,33 @@ struct Ctx {
     dql_scale = (float *)(dql.counter + 16);
     dql_zp = (uint8_t *)(dql.counter + 32);
     HIP_OK(hipMemset(dql.counter, 0, 256));
+    dql.grid_blocks = dql_grid_blocks();
+    dql.spin_limit = 1u << 20; // about a second of polling
+    if (const char *v = getenv("OM_MI355X_DQL_SPIN_LIMIT"))
+      dql.spin_limit = (unsigned)strtoul(v, nullptr, 10);
     HIP_OK(hipEventCreate(&ev0));
     HIP_OK(hipEventCreate(&ev1));
     ready = true;
     return true;
+  }
+
+  // Call after the stream has been synchronised.  The one-launch
+  // DynamicQuantizeLinear kernel raises a flag if its grid barrier ever timed
+  // out (its output is then missing); report that and stop using the kernel.
+  bool dql_barrier_ok() {
+    if (!ready || dql.grid_blocks == 0)
+      return true;
+    unsigned flag = 0;
+    if (hipMemcpy(&flag, dql.counter + 8, sizeof(flag),
+            hipMemcpyDeviceToHost) != hipSuccess)
+      return true;
+    if (!flag)
+      return true;
+    (void)hipMemset(dql.counter, 0, 256);
+    dql.grid_blocks = 0;
+    fail(EIO, "DynamicQuantizeLinear: the grid barrier of the one-launch "
+              "kernel timed out; its output was not written");
+    return false;
   }
 
   void *take(size_t bytes) {
@@ -280,6 +303,7 @@ struct Call {
   Ctx &c;
   bool ok = true;
   bool touched_host = false;
+  bool used_dql = false; // launched DynamicQuantizeLinear (see dql_barrier_ok)
   struct Back {
     void *host;
     void *dev;
@@ -391,6 +415,8 @@ struct Call {
       hipError_t e = hipStreamSynchronize(c.stream);
       if (e != hipSuccess && ok)
         fail(EIO, "stream synchronisation failed: %s", hipGetErrorString(e));
+      else if (used_dql && !c.dql_barrier_ok())
+        ok = false;
     }
     for (void *p : temps)
       c.give(p);
@@ -809,6 +835,7 @@ void om_mi355x_DynamicQuantizeLinear(OMTensor *y_t, OMTensor *scale_t,
   uint8_t *dy = (uint8_t *)call.out(y);
   float *ds = (float *)call.out(sc);
   uint8_t *dz = (uint8_t *)call.out(zp);
+  call.used_dql = true;
   if (call.ok)
     call.check(launch_dynamic_quantize(
                    call.c.stream, call.c.dql, dx, x.numel, dy, ds, dz, false),
@@ -882,6 +909,7 @@ void om_mi355x_DynQuantMatMulDequant(OMTensor *y_t, const OMTensor *x_t,
   // Quantized activations stay on the GPU, stored as (u8 - 128) so the GEMM
   // stages them without a per-byte fix-up.
   uint8_t *aq = (uint8_t *)call.temp((size_t)M * K);
+  call.used_dql = true;
   if (call.ok)
     call.check(launch_dynamic_quantize(call.c.stream, call.c.dql, dx, M * K,
                    aq, call.c.dql_scale, call.c.dql_zp, true),
@@ -1019,7 +1047,7 @@ int om_mi355x_synchronize(void) {
     fail(EIO, "stream synchronisation failed: %s", hipGetErrorString(e));
     return -1;
   }
-  return 0;
+  return t_ctx.dql_barrier_ok() ? 0 : -1;
 }
 
 int om_mi355x_timer_start(void) {

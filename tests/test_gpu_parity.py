@@ -183,7 +183,10 @@ def test_misaligned_device_views_are_handled(rt, oracle):
 # --------------------------------------------------------------------------
 # DynamicQuantizeLinear
 # --------------------------------------------------------------------------
-@pytest.mark.parametrize("shape", [(1,), (6,), (3, 4), (1023,), (128, 768), (257, 1031), (4096, 768)])
+# (4096, 768) and (2051, 1031) take the one-launch kernel with 4 float4 per thread,
+# (4096, 3072) and (3001, 4099) the one with 16; the last three have 1-3 tail elements.
+@pytest.mark.parametrize("shape", [(1,), (6,), (3, 4), (1023,), (128, 768), (257, 1031), (4096, 768),
+                                   (2051, 1031), (4096, 3072), (3001, 4099)])
 def test_dynamic_quantize(rt, oracle, shape):
     rng = np.random.default_rng(int(np.prod(shape)))
     x = rng.normal(0, 1, shape).astype(np.float32)
@@ -206,6 +209,45 @@ def test_dynamic_quantize_edge_inputs(rt, oracle):
         gy, gs, gz = rt.DynamicQuantizeLinear(x)
         assert same_f32(np.float32(gs), np.float32(ws)), x[:4]
         assert int(gz) == int(wz) and np.array_equal(gy, wy), x[:4]
+
+
+def test_dynamic_quantize_mid_size_with_nan_and_inf(rt, oracle):
+    # the one-launch kernel: NaN ignored by min / max and quantized to 0, +inf saturates
+    rng = np.random.default_rng(5)
+    x = rng.normal(0, 3, 2_200_003).astype(np.float32)
+    x[rng.integers(0, x.size, 1000)] = np.nan
+    for extra in (None, np.inf):
+        if extra is not None:
+            x[12345] = extra
+        wy, ws, wz = oracle.dynamic_quantize_linear(x)
+        gy, gs, gz = rt.DynamicQuantizeLinear(x)
+        assert same_f32(np.float32(gs), np.float32(ws))
+        assert int(gz) == int(wz) and np.array_equal(gy, wy)
+
+
+def test_dynamic_quantize_barrier_timeout_is_reported():
+    """The one-launch kernel waits at a grid barrier for a bounded number of polls.
+    With the bound forced to zero from the host every block gives up at once (and
+    exits normally); the runtime must report that instead of returning garbage,
+    and must keep working (two-launch path) afterwards."""
+    import subprocess, sys, textwrap
+    code = textwrap.dedent("""
+        import sys, numpy as np
+        sys.path.insert(0, %r)
+        import om_mi355x as rt
+        x = np.random.default_rng(0).normal(0, 1, (4096, 768)).astype(np.float32)
+        try:
+            rt.DynamicQuantizeLinear(x)
+            print("NO-ERROR")
+        except rt.RuntimeError_ as e:
+            print("ERROR-OK" if "barrier" in str(e) else "WRONG-ERROR %%s" %% e)
+        y, s, z = rt.DynamicQuantizeLinear(x)
+        lo, hi = np.float32(min(x.min(), 0)), np.float32(max(x.max(), 0))
+        print("RECOVERED" if np.float32(s) == (hi - lo) / np.float32(255) else "BAD")
+    """ % os.path.join(os.path.dirname(HERE), "onnx-mlir_amd"))
+    env = dict(os.environ, OM_MI355X_DQL_SPIN_LIMIT="0")
+    out = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=110)
+    assert "ERROR-OK" in out.stdout and "RECOVERED" in out.stdout, out.stdout + out.stderr
 
 
 def test_dynamic_quantize_invariants_large(rt):
