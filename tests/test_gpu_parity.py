@@ -392,6 +392,44 @@ def test_constant_weight_shared_by_every_kernel_family(rt, oracle):
         rt.clear_cache()
 
 
+def test_concurrent_host_threads(rt, oracle):
+    """Entry points are re-entrant: four host threads (each gets its own stream)
+    run DynamicQuantizeLinear on a tensor that takes the one-launch kernel,
+    MatMulInteger on a shared constant weight and QuantizeLinear at the same time."""
+    import threading
+    rng = np.random.default_rng(99)
+    B = _rand_q(rng, np.int8, (256, 1024))
+    rt.mark_constant(B)
+    xs = [rng.normal(0, 1 + t, (2100, 1001)).astype(np.float32) for t in range(4)]
+    As = [_rand_q(rng, np.uint8, (300 + 64 * t, 256)) for t in range(4)]
+    want_dql = [oracle.dynamic_quantize_linear(x) for x in xs]
+    want_mm = [oracle.matmul_integer(A, B, np.array(3, np.uint8), None) for A in As]
+    sc, zp = np.float32(0.05), np.array(7, np.uint8)
+    want_q = [oracle.quantize_linear(x, sc, zp) for x in xs]
+    errors = []
+
+    def work(t):
+        try:
+            for _ in range(3):
+                y, s, z = rt.DynamicQuantizeLinear(xs[t])
+                assert np.array_equal(y, want_dql[t][0]) and int(z) == int(want_dql[t][2])
+                assert np.array_equal(rt.MatMulInteger(As[t], B, np.array(3, np.uint8), None), want_mm[t])
+                assert np.array_equal(rt.QuantizeLinear(xs[t], sc, zp), want_q[t])
+        except BaseException as e:  # noqa: BLE001 - reported below
+            errors.append((t, repr(e)))
+
+    try:
+        threads = [threading.Thread(target=work, args=(t,)) for t in range(4)]
+        for th in threads:
+            th.start()
+        for th in threads:
+            th.join(100)
+        assert not errors, errors
+        assert not any(th.is_alive() for th in threads)
+    finally:
+        rt.clear_cache()
+
+
 # --------------------------------------------------------------------------
 # QLinearMatMul and the fused layers at the benchmark configurations
 # --------------------------------------------------------------------------
