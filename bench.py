@@ -35,8 +35,8 @@ METRIC = "int8 MatMulInteger TOPS (% MFMA peak) + Q/DQ GB/s (% HBM), 1 MI355X"
 # HBM bytes per launch of the headline kernel, measured with rocprofv3 --pmc
 # (FETCH_SIZE and WRITE_SIZE, one run each, scaled by what the same counters
 # read for a 1 GiB device-to-device copy: FETCH_SIZE x2.0, WRITE_SIZE x1.0);
-# the summary of those runs is profiles/k_gemm_i8_bs_config4_ffn_up.md.
-TRAFFIC_BYTES = {"config4 FFN-up f32": int((7817.0 * 2.0 + 49180.0) * 1024)}
+# the summary of those runs is profiles/k_gemm_i8_dma_config4_ffn_up.md.
+TRAFFIC_BYTES = {"config4 FFN-up f32": int((7779.0 * 2.0 + 49190.0) * 1024)}
 
 
 def timed(rt, fn, steps, warmup):
@@ -103,6 +103,30 @@ def decode_case(rt, wl, M, steps, warmup):
     return res
 
 
+def fused_case(rt, wl, name, M, K, N, w_i8, w_scale, steps, warmup):
+    """DynamicQuantizeLinear -> MatMulInteger -> Cast -> Mul as one call: fp32
+    activations in, fp32 out (the chain the quantized models contain)."""
+    rng = np.random.default_rng(0xF00D + M + K + N)
+    X = rng.normal(0, 1, (M, K)).astype(np.float32)
+    dX = rt.DeviceArray.from_numpy(X)
+    dW = rt.DeviceArray.from_numpy(w_i8)
+    dS = rt.DeviceArray.from_numpy(w_scale)
+    dY = rt.DeviceArray((M, N), np.float32)
+    rt.mark_constant(dW)
+    fn = rt.PreparedCall("om_mi355x_DynQuantMatMulDequant", dY, dX, dW, None, dS)
+    host_s, ev_ms = timed(rt, fn, steps, warmup)
+    fn.check()
+    fn.close()
+    ops = 2.0 * M * N * K
+    nbytes = 4 * M * K + K * N + 4 * M * N
+    res = {"name": name, "M": M, "K": K, "N": N, "ms_per_step": host_s * 1e3, "kernel_ms": ev_ms,
+           "tops": ops / (ev_ms * 1e-3) / 1e12, "hbm_bytes_algorithmic": nbytes,
+           "hbm_frac_at_algorithmic_bytes": nbytes / (ev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+    for d in (dX, dW, dS, dY):
+        d.free()
+    return res
+
+
 def qdq_cases(rt, wl, rows, cols, steps, warmup, only=None):
     c = wl.config2(rows, cols)
     n = rows * cols
@@ -159,6 +183,12 @@ def only_mode(rt, wl, what, steps, warmup):
         c = wl.config4("ffn_up", M=8)
         r = gemm_case(rt, wl, "config4 FFN-up", 4096, 768, 3072, c["W"], c["w_scale"], steps, warmup, "f32")
         return {"only": what, **r}
+    if what == "fused_ffn_up":
+        c = wl.config4("ffn_up", M=8)
+        r = fused_case(rt, wl, "config4 ffn_up fused layer", 4096, 768, 3072, c["W"], c["w_scale"], steps, warmup)
+        return {"only": what, **r}
+    if what == "decode":
+        return {"only": what, **decode_case(rt, wl, 1, steps, warmup)}
     if what == "gemm_prefill_up":
         c = wl.config5("up", M=8)
         r = gemm_case(rt, wl, "config5 prefill up", 2048, 4096, 11008, c["W"], c["w_scale"], steps, warmup, "f32")
@@ -202,10 +232,11 @@ def main():
     ap.add_argument("--workload", default="config4_ffn_up",
                     choices=["config4_ffn_up", "config4_ffn_up_i32"])
     ap.add_argument("--no-extras", action="store_true", help="skip the Q/DQ and other-shape measurements")
-    ap.add_argument("--extras", default="gemm,decode,qdq", help="which extra groups to measure")
+    ap.add_argument("--extras", default="gemm,fused,decode,qdq", help="which extra groups to measure")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--only", default=None,
-                    choices=["copy", "gemm_ffn_up", "gemm_prefill_up", "quantize_per_axis", "dequantize_per_axis",
+                    choices=["copy", "gemm_ffn_up", "gemm_prefill_up", "fused_ffn_up", "decode",
+                             "quantize_per_axis", "dequantize_per_axis",
                              "quantize_per_tensor", "dequantize_per_tensor", "dynamic_quantize"],
                     help="launch just this kernel --steps times (for rocprofv3 counter runs)")
     args = ap.parse_args()
@@ -243,6 +274,14 @@ def main():
             gemms.append(gemm_case(rt, wl, f"config5 prefill {name}", 2048, k, n, cc["W"], cc["w_scale"],
                                    max(10, args.steps // 10), max(2, args.warmup // 10), "f32"))
         extras["gemm"] = gemms
+    if "fused" in groups:
+        fused = []
+        for name, (k, n) in wl.CONFIG4_SHAPES.items():
+            if name in ("ffn_up", "ffn_down"):
+                cc = wl.config4(name, M=8)
+                fused.append(fused_case(rt, wl, f"config4 {name} fused layer", 4096, k, n, cc["W"],
+                                        cc["w_scale"], args.steps, args.warmup))
+        extras["fused"] = fused
     if "decode" in groups:
         extras["decode"] = [decode_case(rt, wl, m, args.steps, args.warmup) for m in (1, 4, 16)]
     if "qdq" in groups:
@@ -274,7 +313,7 @@ def main():
         "roofline": {"bound": "mfma", "achieved": main_res["kernel_tops"], "peak": INT8_PEAK_TOPS,
                      "unit": "TOP/s", "frac": main_res["kernel_tops"] / INT8_PEAK_TOPS,
                      "traffic": TRAFFIC_BYTES.get("config4 FFN-up f32") if epi == "f32" else None,
-                     "kernel": "k_gemm_i8_bs<4,2,4,4,2,true> (128x256 tiles)", "kernel_ms": main_res["kernel_ms"],
+                     "kernel": "k_gemm_i8_dma<128,3,3> (128x128 tiles)", "kernel_ms": main_res["kernel_ms"],
                      "algorithmic_ops": main_res["ops"],
                      "algorithmic_hbm_bytes": main_res["hbm_bytes_algorithmic"],
                      "hbm_frac_at_algorithmic_bytes": main_res["hbm_bytes_algorithmic"]
