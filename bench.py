@@ -103,6 +103,30 @@ def decode_case(rt, wl, M, steps, warmup):
     return res
 
 
+def qlinear_case(rt, wl, steps, warmup):
+    """Config 3: QLinearMatMul, uint8 x uint8 -> uint8 with both zero points
+    non-zero (row sums of A and the per-row correction are part of the step)."""
+    c = wl.config3()
+    M, K = c["A"].shape
+    N = c["B"].shape[1]
+    d = {k: rt.DeviceArray.from_numpy(np.asarray(c[k])) for k in
+         ("A", "a_scale", "a_zp", "B", "b_scale", "b_zp", "y_scale", "y_zp")}
+    dY = rt.DeviceArray((M, N), np.uint8)
+    rt.mark_constant(d["B"])
+    fn = rt.PreparedCall("om_mi355x_QLinearMatMul", dY, d["A"], d["a_scale"], d["a_zp"], d["B"],
+                         d["b_scale"], d["b_zp"], d["y_scale"], d["y_zp"], rt.WRAP)
+    host_s, ev_ms = timed(rt, fn, steps, warmup)
+    fn.check()
+    fn.close()
+    ops = 2.0 * M * N * K
+    res = {"name": "config3 QLinearMatMul u8 x u8 -> u8", "M": M, "K": K, "N": N,
+           "ms_per_step": host_s * 1e3, "kernel_ms": ev_ms, "tops": ops / (ev_ms * 1e-3) / 1e12,
+           "hbm_bytes_algorithmic": M * K + K * N + M * N}
+    for a in list(d.values()) + [dY]:
+        a.free()
+    return res
+
+
 def fused_case(rt, wl, name, M, K, N, w_i8, w_scale, steps, warmup):
     """DynamicQuantizeLinear -> MatMulInteger -> Cast -> Mul as one call: fp32
     activations in, fp32 out (the chain the quantized models contain)."""
@@ -273,6 +297,7 @@ def main():
             cc = wl.config5(name, M=8)
             gemms.append(gemm_case(rt, wl, f"config5 prefill {name}", 2048, k, n, cc["W"], cc["w_scale"],
                                    max(10, args.steps // 10), max(2, args.warmup // 10), "f32"))
+        gemms.append(qlinear_case(rt, wl, args.steps, args.warmup))
         extras["gemm"] = gemms
     if "fused" in groups:
         fused = []

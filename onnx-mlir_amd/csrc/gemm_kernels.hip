@@ -68,7 +68,7 @@ struct EpiParams {
   int64_t a_zp_len;
   const void *b_zp;
   int64_t b_zp_len;
-  const int32_t *rowsum;
+  bool need_rowsum;      // B carries an offset: row sums of A' are needed
   const int32_t *colsum;
   const float *a_scale;
   const float *b_scale;
@@ -87,6 +87,16 @@ __device__ __forceinline__ int32_t load_zp_i32(
     const void *p, bool is_unsigned, int64_t i) {
   return is_unsigned ? (int32_t)((const uint8_t *)p)[i]
                      : (int32_t)((const int8_t *)p)[i];
+}
+
+// Sum of the 16 int8 values of an MFMA A operand register group (one lane:
+// one row, 16 consecutive K bytes).  Kernels add these up over K when the
+// epilogue needs rowsum(A'), i.e. when B carries an offset.
+__device__ __forceinline__ int32_t frag_rowsum(v4i f) {
+  int32_t s = __builtin_amdgcn_sdot4(f.x, 0x01010101, 0, false);
+  s = __builtin_amdgcn_sdot4(f.y, 0x01010101, s, false);
+  s = __builtin_amdgcn_sdot4(f.z, 0x01010101, s, false);
+  return __builtin_amdgcn_sdot4(f.w, 0x01010101, s, false);
 }
 
 // Epilogue shared by the GEMM kernels: applies the zero-point correction and
@@ -120,8 +130,9 @@ __device__ __forceinline__ void store_one(const EpiParams &ep, int64_t o,
 }
 
 template <int TM, int TN, int A_MODE, int EPI>
-__device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TM][TN], int mrow0,
-    int ncol0, int M, int N, int K, const EpiParams &ep) {
+__device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TM][TN],
+    const int32_t (&rsp)[TM], int mrow0, int ncol0, int M, int N, int K,
+    const EpiParams &ep) {
   const int lane = threadIdx.x & 63;
   const int l32 = lane & 31;
   const int lh = lane >> 5;
@@ -145,8 +156,14 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TM][TN], int mrow0,
   const bool has_azp = ep.a_zp_len > 0;
   const void *azp_ptr = has_azp ? ep.a_zp : (const void *)ep.colsum;
   const bool per_row = ep.a_zp_len > 1;
-  const bool has_rs = ep.rowsum != nullptr;
-  const int32_t *rs_ptr = has_rs ? ep.rowsum : ep.colsum;
+  const bool has_rs = ep.need_rowsum;
+  // rsp[i]: this lane's share of rowsum(A') for row (lane % 32) of row tile i
+  // (the two lanes of a row each saw every other 16-byte chunk of K).  After
+  // the fold, lane l and lane l+32 both hold the whole sum of row l % 32.
+  int32_t rsf[TM];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+    rsf[i] = has_rs ? rsp[i] + __shfl_xor(rsp[i], 32, 64) : 0;
 
   int n_[TN];
   int32_t db[TN], cs[TN];
@@ -174,9 +191,10 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TM][TN], int mrow0,
   const int32_t da0 = oa - (has_azp ? az0 : 0);
   __builtin_amdgcn_sched_barrier(0);
 
-  if (!per_row && !has_rs) {
-    // Common case: one zero point for all rows and no offset on B.  The whole
-    // correction is then one value per column, computed once per lane.
+  if (!per_row) {
+    // Common case: one zero point for all rows.  The correction is one value
+    // per column, computed once per lane, plus db[j] * rowsum(row) when B
+    // carries an offset.
     uint32_t cj[TN];
 #pragma unroll
     for (int j = 0; j < TN; ++j)
@@ -187,48 +205,62 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TM][TN], int mrow0,
     // them from a scalar wave index), so this test and the row addresses below
     // are scalar work.
     const bool full = (mrow0 + 32 * TM <= M) && (ncol0 + 32 * TN <= N);
-    if (full) {
+    constexpr int ES = (EPI == kEpiQ8) ? 1 : 4;
+    char *const base =
+        (char *)ep.out + ((int64_t)mrow0 * N + ncol0) * (int64_t)ES;
+    const uint32_t loff =
+        ((uint32_t)(4 * lh) * (uint32_t)N + (uint32_t)l32) * (uint32_t)ES;
+    // One element: row tile i, register r (row 8*(r/4) + 4*lh + r%4 of the
+    // tile), column tile j.  RS: add the row-sum term.
+    auto emit = [&](auto rs_c, int i, int r, int j, int32_t rs_row,
+                    char *rowp) {
+      uint32_t y = (uint32_t)acc[i][j][r] + cj[j];
+      if (decltype(rs_c)::value)
+        y += (uint32_t)db[j] * (uint32_t)rs_row;
+      char *const q = rowp + loff + (uint32_t)(j * 32 * ES);
+      // Streaming stores: the result is not read again by this kernel, and
+      // keeping it out of the way in L2 leaves the A and Bp panels cached for
+      // the blocks still in their K loop (measured faster).
+      if (EPI == kEpiI32) {
+        __builtin_nontemporal_store((int32_t)y, (int32_t *)q);
+      } else if (EPI == kEpiF32) {
+        __builtin_nontemporal_store((float)(int32_t)y * sj[j], (float *)q);
+      } else {
+        const float f = (float)(int32_t)y * sj[j];
+        int32_t v =
+            (int32_t)((uint32_t)(int32_t)__builtin_rintf(f) + (uint32_t)yz);
+        if (ep.narrow == kSaturate) {
+          const int32_t lo = ep.y_unsigned ? 0 : -128;
+          const int32_t hi = ep.y_unsigned ? 255 : 127;
+          v = v < lo ? lo : (v > hi ? hi : v);
+        }
+        *(uint8_t *)q = (uint8_t)(v & 0xFF);
+      }
+    };
+    auto whole = [&](auto rs_c) {
       // Whole grid inside the matrix: no bounds tests, and every address is
       // (scalar row base) + (one 32-bit lane offset) + constant, so a store
-      // costs the two or three vector instructions that produce its value.
-      constexpr int ES = (EPI == kEpiQ8) ? 1 : 4;
-      char *const base =
-          (char *)ep.out + ((int64_t)mrow0 * N + ncol0) * (int64_t)ES;
-      const uint32_t loff =
-          ((uint32_t)(4 * lh) * (uint32_t)N + (uint32_t)l32) * (uint32_t)ES;
+      // costs the few vector instructions that produce its value.
 #pragma unroll
       for (int i = 0; i < TM; ++i) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
+          const int rr = 8 * (r >> 2) + 4 * lh + (r & 3);
+          const int32_t rs_row =
+              decltype(rs_c)::value ? __shfl(rsf[i], rr, 64) : 0;
           const int64_t rowb =
               (int64_t)(i * 32 + 8 * (r >> 2) + (r & 3)) * N * (int64_t)ES;
-          char *const rowp = base + rowb;
 #pragma unroll
-          for (int j = 0; j < TN; ++j) {
-            const uint32_t y = (uint32_t)acc[i][j][r] + cj[j];
-            char *const q = rowp + loff + (uint32_t)(j * 32 * ES);
-            // Streaming stores: the result is not read again by this kernel,
-            // and keeping it out of the way in L2 leaves the A and Bp panels
-            // cached for the blocks still in their K loop (measured faster).
-            if (EPI == kEpiI32) {
-              __builtin_nontemporal_store((int32_t)y, (int32_t *)q);
-            } else if (EPI == kEpiF32) {
-              __builtin_nontemporal_store(
-                  (float)(int32_t)y * sj[j], (float *)q);
-            } else {
-              const float f = (float)(int32_t)y * sj[j];
-              int32_t v = (int32_t)((uint32_t)(int32_t)__builtin_rintf(f) +
-                                    (uint32_t)yz);
-              if (ep.narrow == kSaturate) {
-                const int32_t lo = ep.y_unsigned ? 0 : -128;
-                const int32_t hi = ep.y_unsigned ? 255 : 127;
-                v = v < lo ? lo : (v > hi ? hi : v);
-              }
-              *(uint8_t *)q = (uint8_t)(v & 0xFF);
-            }
-          }
+          for (int j = 0; j < TN; ++j)
+            emit(rs_c, i, r, j, rs_row, base + rowb);
         }
       }
+    };
+    if (full) {
+      if (has_rs)
+        whole(std::true_type{});
+      else
+        whole(std::false_type{});
       return;
     }
 #pragma unroll
@@ -236,11 +268,14 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TM][TN], int mrow0,
       const int mbase = mrow0 + i * 32 + 4 * lh;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
+        const int rr = 8 * (r >> 2) + 4 * lh + (r & 3);
         const int m = mbase + 8 * (r >> 2) + (r & 3);
+        const int32_t rs_row = __shfl(rsf[i], rr, 64);
         const int64_t orow = (int64_t)m * N;
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
-          const uint32_t y = (uint32_t)acc[i][j][r] + cj[j];
+          const uint32_t y = (uint32_t)acc[i][j][r] + cj[j] +
+                             (uint32_t)db[j] * (uint32_t)rs_row;
           if (m < M && n_[j] < N)
             store_one<EPI>(ep, orow + n_[j], y, sj[j], yz);
         }
@@ -249,8 +284,8 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TM][TN], int mrow0,
     return;
   }
 
-  // Per-row zero points and / or row sums: four rows at a time, to keep the
-  // register footprint of this rarely taken path small.
+  // Per-row zero points: four rows at a time, to keep the register footprint
+  // of this rarely taken path small.
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
     const int mbase = mrow0 + i * 32 + 4 * lh;
@@ -263,8 +298,7 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TM][TN], int mrow0,
         const int mc = m < M ? m : M - 1;
         const int32_t az = load_zp_i32(azp_ptr, A_OFF, per_row ? mc : 0);
         da[rr] = oa - (has_azp ? az : 0);
-        const int32_t rv = rs_ptr[has_rs ? mc : 0];
-        rs[rr] = has_rs ? rv : 0;
+        rs[rr] = __shfl(rsf[i], 8 * rg + 4 * lh + rr, 64);
       }
 #pragma unroll
       for (int rr = 0; rr < 4; ++rr) {
@@ -407,6 +441,11 @@ __global__ __launch_bounds__(WGM *WGN * 64, MINB) void k_gemm_i8(
 
   const int l32 = lane & 31;
   const int lh = lane >> 5;
+  const bool need_rs = ep.need_rowsum;
+  int32_t rsp[TM];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+    rsp[i] = 0;
 
   auto compute = [&](int buf) {
 #pragma unroll
@@ -422,6 +461,8 @@ __global__ __launch_bounds__(WGM *WGN * 64, MINB) void k_gemm_i8(
         if (A_MODE == 1)
           fa[i] ^= (v4i){(int)0x80808080, (int)0x80808080, (int)0x80808080,
               (int)0x80808080};
+        if (need_rs)
+          rsp[i] += frag_rowsum(fa[i]);
       }
 #pragma unroll
       for (int j = 0; j < TN; ++j)
@@ -470,7 +511,7 @@ __global__ __launch_bounds__(WGM *WGN * 64, MINB) void k_gemm_i8(
       break;
   }
   gemm_epilogue<TM, TN, A_MODE, EPI>(
-      acc, m0 + wm * WTM, n0 + wn * WTN, M, N, K, ep);
+      acc, rsp, m0 + wm * WTM, n0 + wn * WTN, M, N, K, ep);
 }
 
 // ---- GEMM, tiles copied from global memory straight into LDS --------------
@@ -600,6 +641,12 @@ __global__ __launch_bounds__(256, MINB) void k_gemm_i8_dma(
                  : "memory");
   };
 
+  const bool need_rs = ep.need_rowsum;
+  int32_t rsp[TM];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+    rsp[i] = 0;
+
   int stage = 0; // kt % NSTAGE
   for (int kt = 0; kt < KT; ++kt) {
     const int prev = (stage == 0) ? NSTAGE - 1 : stage - 1;
@@ -640,6 +687,11 @@ __global__ __launch_bounds__(256, MINB) void k_gemm_i8_dma(
         fa0[i] ^= (v4i){(int)0x80808080, (int)0x80808080, (int)0x80808080,
             (int)0x80808080};
     }
+    if (need_rs) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        rsp[i] += frag_rowsum(fa0[i]);
+    }
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -662,6 +714,11 @@ __global__ __launch_bounds__(256, MINB) void k_gemm_i8_dma(
         fa1[i] ^= (v4i){(int)0x80808080, (int)0x80808080, (int)0x80808080,
             (int)0x80808080};
     }
+    if (need_rs) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        rsp[i] += frag_rowsum(fa1[i]);
+    }
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -675,7 +732,7 @@ __global__ __launch_bounds__(256, MINB) void k_gemm_i8_dma(
   __builtin_amdgcn_s_waitcnt(0x0F70);
 
   gemm_epilogue<TM, TN, A_MODE, EPI>(
-      acc, m0 + wm * WTM, n0 + wn * WTN, M, N, K, ep);
+      acc, rsp, m0 + wm * WTM, n0 + wn * WTN, M, N, K, ep);
 }
 
 // ---- GEMM, Bp streamed to registers -----------------------------------------
@@ -817,6 +874,12 @@ __global__ __launch_bounds__(256, MINB) void k_gemm_i8_bs(
       (int)0x80808080};
   using O = std::integral_constant<int, 0>;
 
+  const bool need_rs = ep.need_rowsum;
+  int32_t rsp[TM];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+    rsp[i] = 0;
+
   int kt = 0;
   int stage = 0;
   bool done = false;
@@ -847,6 +910,11 @@ __global__ __launch_bounds__(256, MINB) void k_gemm_i8_bs(
           for (int i = 0; i < TM; ++i)
             fa0[i] ^= flip;
         }
+        if (need_rs) {
+#pragma unroll
+          for (int i = 0; i < TM; ++i)
+            rsp[i] += frag_rowsum(fa0[i]);
+        }
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -864,6 +932,11 @@ __global__ __launch_bounds__(256, MINB) void k_gemm_i8_bs(
 #pragma unroll
           for (int i = 0; i < TM; ++i)
             fa1[i] ^= flip;
+        }
+        if (need_rs) {
+#pragma unroll
+          for (int i = 0; i < TM; ++i)
+            rsp[i] += frag_rowsum(fa1[i]);
         }
 #pragma unroll
         for (int i = 0; i < TM; ++i)
@@ -926,6 +999,11 @@ __global__ __launch_bounds__(256, MINB) void k_gemm_i8_bs(
           for (int i = 0; i < TM; ++i)
             fa0[i] ^= flip;
         }
+        if (need_rs) {
+#pragma unroll
+          for (int i = 0; i < TM; ++i)
+            rsp[i] += frag_rowsum(fa0[i]);
+        }
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -946,6 +1024,11 @@ __global__ __launch_bounds__(256, MINB) void k_gemm_i8_bs(
 #pragma unroll
           for (int i = 0; i < TM; ++i)
             fa1[i] ^= flip;
+        }
+        if (need_rs) {
+#pragma unroll
+          for (int i = 0; i < TM; ++i)
+            rsp[i] += frag_rowsum(fa1[i]);
         }
 #pragma unroll
         for (int i = 0; i < TM; ++i)
@@ -974,7 +1057,7 @@ __global__ __launch_bounds__(256, MINB) void k_gemm_i8_bs(
   // A copies past the last step are still landing in LDS.
   __builtin_amdgcn_s_waitcnt(0x0F70);
 
-  gemm_epilogue<TM, TN, A_MODE, EPI>(acc, m0, ncol0, M, N, K, ep);
+  gemm_epilogue<TM, TN, A_MODE, EPI>(acc, rsp, m0, ncol0, M, N, K, ep);
 }
 
 // ---- skinny GEMM (M <= 32): weight streaming -------------------------------
@@ -992,6 +1075,7 @@ __global__ __launch_bounds__(512) void k_gemm_i8_skinny_bp(
     int K, int Kpad, EpiParams ep) {
   constexpr int WAVES = 8, U = 4;
   __shared__ int32_t part[WAVES][16][64];
+  __shared__ int32_t part_rs[WAVES][64];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -1014,6 +1098,8 @@ __global__ __launch_bounds__(512) void k_gemm_i8_skinny_bp(
 #pragma unroll
   for (int r = 0; r < 16; ++r)
     acc[r] = 0;
+  const bool need_rs = ep.need_rowsum;
+  int32_t rsp = 0; // this lane's share of rowsum(A') of row lane % 32
   for (int kt = kt_begin; kt < kt_end; kt += U) {
     v4i a[U][2], b[U][2];
 #pragma unroll
@@ -1039,6 +1125,8 @@ __global__ __launch_bounds__(512) void k_gemm_i8_skinny_bp(
           if (A_MODE == 1)
             av ^= (v4i){(int)0x80808080, (int)0x80808080, (int)0x80808080,
                 (int)0x80808080};
+          if (need_rs)
+            rsp += frag_rowsum(av);
           acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(
               av, b[u][sub], acc, 0, 0, 0);
         }
@@ -1048,6 +1136,7 @@ __global__ __launch_bounds__(512) void k_gemm_i8_skinny_bp(
 #pragma unroll
   for (int r = 0; r < 16; ++r)
     part[wave][r][lane] = acc[r];
+  part_rs[wave][lane] = rsp;
   __syncthreads();
 
   // 32x32 accumulator layout: lane holds column (lane & 31); register r holds
@@ -1085,8 +1174,11 @@ __global__ __launch_bounds__(512) void k_gemm_i8_skinny_bp(
     int32_t da = oa, rs = 0;
     if (ep.a_zp_len > 0)
       da = oa - load_zp_i32(ep.a_zp, A_OFF, ep.a_zp_len > 1 ? m : 0);
-    if (ep.rowsum)
-      rs = ep.rowsum[m];
+    if (need_rs) {
+#pragma unroll
+      for (int w = 0; w < WAVES; ++w)
+        rs += part_rs[w][m] + part_rs[w][m + 32];
+    }
     y += (uint32_t)da * (uint32_t)cs;
     y += (uint32_t)db * (uint32_t)rs;
     y += (uint32_t)K * (uint32_t)da * (uint32_t)db;
@@ -1151,28 +1243,6 @@ __global__ __launch_bounds__(256) void k_pack_b(const uint8_t *__restrict__ B,
     if ((tid & 3) == 0 && sum != 0)
       atomicAdd(&colsum[n], sum);
   }
-}
-
-// rowsum[m] = sum_k A'[m,k]; one wave per row.
-template <bool A_UNSIGNED>
-__global__ __launch_bounds__(256) void k_rowsum_a(
-    const uint8_t *__restrict__ A, int64_t M, int64_t K,
-    int32_t *__restrict__ rowsum) {
-  const int64_t m = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (m >= M)
-    return;
-  const int lane = threadIdx.x & 63;
-  const uint8_t *__restrict__ row = A + m * K;
-  int32_t sum = 0;
-  for (int64_t k = lane; k < K; k += 64) {
-    const uint8_t v = row[k];
-    sum += A_UNSIGNED ? ((int32_t)v - 128) : (int32_t)(int8_t)v;
-  }
-#pragma unroll
-  for (int off = 32; off >= 1; off >>= 1)
-    sum += __shfl_xor(sum, off, 64);
-  if (lane == 0)
-    rowsum[m] = sum;
 }
 
 // ---- launch ---------------------------------------------------------------
@@ -1292,18 +1362,6 @@ hipError_t launch_pack_b(hipStream_t s, const void *B, bool b_unsigned,
   return hipGetLastError();
 }
 
-hipError_t launch_rowsum_a(hipStream_t s, const void *A, bool a_unsigned,
-    int64_t M, int64_t K, int32_t *rowsum) {
-  if (M == 0)
-    return hipSuccess;
-  const unsigned grid = (unsigned)((M + 3) / 4);
-  if (a_unsigned)
-    k_rowsum_a<true><<<grid, 256, 0, s>>>((const uint8_t *)A, M, K, rowsum);
-  else
-    k_rowsum_a<false><<<grid, 256, 0, s>>>((const uint8_t *)A, M, K, rowsum);
-  return hipGetLastError();
-}
-
 hipError_t launch_gemm(hipStream_t s, const GemmArgs &g) {
   if (g.M == 0 || g.N == 0)
     return hipSuccess;
@@ -1316,7 +1374,7 @@ hipError_t launch_gemm(hipStream_t s, const GemmArgs &g) {
   ep.a_zp_len = g.a_zp ? g.a_zp_len : 0;
   ep.b_zp = g.b_zp;
   ep.b_zp_len = g.b_zp ? g.b_zp_len : 0;
-  ep.rowsum = g.rowsum;
+  ep.need_rowsum = g.b_unsigned || (g.b_zp != nullptr && g.b_zp_len > 0);
   ep.colsum = g.colsum;
   ep.a_scale = g.a_scale;
   ep.b_scale = g.b_scale;

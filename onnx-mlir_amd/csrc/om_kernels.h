@@ -58,10 +58,6 @@ inline int64_t round_up(int64_t v, int64_t m) { return (v + m - 1) / m * m; }
 hipError_t launch_pack_b(hipStream_t s, const void *B, bool b_unsigned,
     int64_t K, int64_t N, int8_t *Bp, int32_t *colsum);
 
-// rowsum[m] = sum_k (A[m,k] - (a_unsigned ? 128 : 0)).
-hipError_t launch_rowsum_a(hipStream_t s, const void *A, bool a_unsigned,
-    int64_t M, int64_t K, int32_t *rowsum);
-
 struct GemmArgs {
   const void *A;       // [M,K] row-major, u8 or i8
   bool a_unsigned;     // A holds u8
@@ -73,7 +69,6 @@ struct GemmArgs {
   int64_t a_zp_len;    // 0, 1 or M
   const void *b_zp;    // element type follows B; may be null
   int64_t b_zp_len;    // 0, 1 or N
-  const int32_t *rowsum; // sum_k A' per row; may be null when B offset is 0
   const int32_t *colsum; // sum_k B' per column (Npad entries)
   Epilogue epi;
   // kEpiF32: out = f32(acc) * (a_scale[0] * b_scale[j or 0])

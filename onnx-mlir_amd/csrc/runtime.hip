@@ -654,15 +654,6 @@ void run_matmul(const MatmulSpec &sp) {
   g.a_zp_len = azl;
   g.b_zp = sp.b_zp ? call.in(bzp) : nullptr;
   g.b_zp_len = bzl;
-  // Row sums of A are only needed when B carries an offset.
-  g.rowsum = nullptr;
-  if (b_uns || sp.b_zp) {
-    int32_t *rs = (int32_t *)call.temp((size_t)M * 4);
-    if (call.ok)
-      call.check(
-          launch_rowsum_a(call.c.stream, g.A, a_uns, M, K, rs), "row sums");
-    g.rowsum = rs;
-  }
   g.epi = sp.epi;
   if (sp.epi != kEpiI32) {
     g.a_scale = (const float *)call.in(as);
@@ -932,15 +923,6 @@ void om_mi355x_DynQuantMatMulDequant(OMTensor *y_t, const OMTensor *x_t,
   g.a_zp_len = 1;
   g.b_zp = bzp_t ? call.in(bzp) : nullptr;
   g.b_zp_len = bzl;
-  g.rowsum = nullptr;
-  if (g.b_unsigned || bzp_t) {
-    int32_t *rs = (int32_t *)call.temp((size_t)M * 4);
-    // Row sums of the shifted bytes are the int8 sums.
-    if (call.ok)
-      call.check(
-          launch_rowsum_a(call.c.stream, aq, false, M, K, rs), "row sums");
-    g.rowsum = rs;
-  }
   g.epi = kEpiF32;
   g.a_scale = call.c.dql_scale;
   g.b_scale = (const float *)call.in(bs);
