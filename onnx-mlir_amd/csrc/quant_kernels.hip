@@ -72,6 +72,7 @@ __device__ __forceinline__ uint32_t quant_four(
 // kThreads*UNROLL float4 per step; `flip` is 0, or 0x80808080 to store the
 // result minus 128 as int8.
 constexpr int kUnroll = 4;
+constexpr int kRowUnroll = 8; // rows in flight per thread in the row-walking per-axis kernels
 
 template <bool SIGNED, bool HAS_ZP>
 __global__ __launch_bounds__(kThreads) void k_quant_flat(
@@ -135,13 +136,13 @@ __global__ __launch_bounds__(kThreads) void k_quant_lastaxis(
       (r_begin + rows_per_block < rows) ? r_begin + rows_per_block : rows;
   if (ncol == 4) {
     int64_t r = r_begin;
-    for (; r + kUnroll <= r_end; r += kUnroll) {
-      f4u v[kUnroll];
+    for (; r + kRowUnroll <= r_end; r += kRowUnroll) {
+      f4u v[kRowUnroll];
 #pragma unroll
-      for (int j = 0; j < kUnroll; ++j)
+      for (int j = 0; j < kRowUnroll; ++j)
         v[j] = __builtin_nontemporal_load((const f4u *)(x + (r + j) * C + c0));
 #pragma unroll
-      for (int j = 0; j < kUnroll; ++j) {
+      for (int j = 0; j < kRowUnroll; ++j) {
         uint32_t b0 = quant_one<SIGNED, HAS_ZP>(v[j].x, s[0], z[0]);
         uint32_t b1 = quant_one<SIGNED, HAS_ZP>(v[j].y, s[1], z[1]);
         uint32_t b2 = quant_one<SIGNED, HAS_ZP>(v[j].z, s[2], z[2]);
@@ -389,19 +390,21 @@ __global__ __launch_bounds__(kThreads) void k_dequant_lastaxis(
       (r_begin + rows_per_block < rows) ? r_begin + rows_per_block : rows;
   if (ncol == 4) {
     int64_t r = r_begin;
-    for (; r + kUnroll <= r_end; r += kUnroll) {
-      uint32_t q[kUnroll][4];
+    for (; r + kRowUnroll <= r_end; r += kRowUnroll) {
+      uint32_t q[kRowUnroll][4];
 #pragma unroll
-      for (int j = 0; j < kUnroll; ++j)
+      for (int j = 0; j < kRowUnroll; ++j)
         load_four_q<KIND>(x, (r + j) * C + c0, q[j]);
 #pragma unroll
-      for (int j = 0; j < kUnroll; ++j) {
+      for (int j = 0; j < kRowUnroll; ++j) {
         f4u o;
         o.x = dq_one<HAS_ZP>(q_to_f32<KIND>(q[j][0]), s[0], z[0]);
         o.y = dq_one<HAS_ZP>(q_to_f32<KIND>(q[j][1]), s[1], z[1]);
         o.z = dq_one<HAS_ZP>(q_to_f32<KIND>(q[j][2]), s[2], z[2]);
         o.w = dq_one<HAS_ZP>(q_to_f32<KIND>(q[j][3]), s[3], z[3]);
-        *(f4u *)(y + (r + j) * C + c0) = o;
+        // streaming store: measured 3 % faster here (and 14 % slower for
+        // the 4-byte stores of the quantize kernel, which keeps plain ones)
+        __builtin_nontemporal_store(o, (f4u *)(y + (r + j) * C + c0));
       }
     }
     for (; r < r_end; ++r) {
