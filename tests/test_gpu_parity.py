@@ -455,6 +455,25 @@ def test_qlinearmatmul_int8_and_per_row_column_zero_points(rt, oracle):
         assert got.dtype == np.int8 and np.array_equal(got, want)
 
 
+def test_qlinearmatmul_per_column_b_scale(rt, oracle):
+    """Per-channel weight scales in QLinearMatMul have no counterpart in the
+    reference (its tests and lowering use scalar scales), so this is parity
+    unpinned: the expected value composes the oracle's integer matmul with the
+    reference's requantize op order, s_j = (a_scale * b_scale[j]) / y_scale."""
+    rng = np.random.default_rng(52)
+    M, K, N = 200, 192, 384
+    a, b = _rand_q(rng, np.uint8, (M, K)), _rand_q(rng, np.uint8, (K, N))
+    az, bz = np.array(121, np.uint8), _rand_q(rng, np.uint8, (N,))
+    a_s, y_s, yz = np.float32(0.013), np.float32(0.41), np.array(17, np.uint8)
+    b_s = rng.uniform(1e-3, 2e-2, N).astype(np.float32)
+    acc = oracle.matmul_integer(a, b, az, bz).astype(np.int32)
+    sj = ((a_s * b_s).astype(np.float32) / y_s).astype(np.float32)
+    q = np.rint(acc.astype(np.float32) * sj[None, :]).astype(np.int64) + int(yz)
+    for mode, want in ((rt.WRAP, (q & 0xFF).astype(np.uint8)), (rt.SATURATE, np.clip(q, 0, 255).astype(np.uint8))):
+        got = rt.QLinearMatMul(a, a_s, az, b, b_s, bz, y_s, yz, mode)
+        assert got.dtype == np.uint8 and np.array_equal(got, want)
+
+
 def test_config1_graph_separate_ops_and_fused(rt, oracle):
     c = wl.config1()
     aq, a_s, a_zp = oracle.dynamic_quantize_linear(c["A"])
