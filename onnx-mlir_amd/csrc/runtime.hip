@@ -18,6 +18,7 @@
 #include <stdarg.h>
 #include <stdio.h>
 #include <string.h>
+#include <time.h>
 
 #include <map>
 #include <mutex>
@@ -299,6 +300,56 @@ bool view_of(const OMTensor *t, const char *name, View &v) {
 
 // One entry-point invocation: resolves tensors to GPU pointers, remembers
 // which host outputs need copying back and which pool buffers to return.
+// ---------------------------------------------------------------------------
+// Timing support.  Entry points normally return as soon as their kernels are
+// queued when all tensors live on the GPU.  Two environment variables change
+// that, for measurements:
+//   OM_MI355X_SYNC=1         every entry point waits for its kernels, so that
+//                            the before / after instrumentation points the
+//                            compiler puts around each ONNX op
+//                            (src/Runtime/OMInstrument.c:156-170) bracket the
+//                            op's real duration;
+//   OM_MI355X_PERF_REPORT=1  the same, and the runtime prints its own lines in
+//                            that format, "==PERF-REPORT==, <op>, <entry
+//                            point>, before|after, <seconds since the last
+//                            line>, <seconds since the first line>", to the
+//                            file named by ONNX_MLIR_INSTRUMENT_FILE or to
+//                            stdout (as OMInstrument.c:290-300 does).
+bool env_flag(const char *name) {
+  const char *v = getenv(name);
+  return v && v[0] && v[0] != '0';
+}
+bool sync_every_call() {
+  static const bool on = env_flag("OM_MI355X_SYNC");
+  return on;
+}
+bool report_enabled() {
+  static const bool on = env_flag("OM_MI355X_PERF_REPORT");
+  return on;
+}
+double now_seconds() {
+  struct timespec ts;
+  clock_gettime(CLOCK_MONOTONIC, &ts);
+  return (double)ts.tv_sec + 1e-9 * (double)ts.tv_nsec;
+}
+void report_line(const char *op, const char *when, double t) {
+  static std::mutex m;
+  static FILE *out = nullptr;
+  static double t_first = 0.0, t_last = 0.0;
+  std::lock_guard<std::mutex> lk(m);
+  if (!out) {
+    const char *name = getenv("ONNX_MLIR_INSTRUMENT_FILE");
+    out = (name && name[0]) ? fopen(name, "w") : nullptr;
+    if (!out)
+      out = stdout;
+    t_first = t_last = t;
+  }
+  fprintf(out, "==PERF-REPORT==, onnx.%s, om_mi355x_%s, %s, %.6f, %.6f\n", op, op,
+      when, t - t_last, t - t_first);
+  fflush(out);
+  t_last = t;
+}
+
 struct Call {
   Ctx &c;
   bool ok = true;
@@ -312,7 +363,16 @@ struct Call {
   std::vector<Back> backs;
   std::vector<void *> temps;
 
-  explicit Call(Ctx &ctx) : c(ctx) { ok = c.init(); }
+  const char *op;
+  double t_begin = 0.0;
+
+  Call(Ctx &ctx, const char *op_name) : c(ctx), op(op_name) {
+    ok = c.init();
+    if (ok && report_enabled()) {
+      t_begin = now_seconds();
+      report_line(op, "before", t_begin);
+    }
+  }
 
   void *temp(size_t bytes) {
     void *p = c.take(bytes);
@@ -411,7 +471,7 @@ struct Call {
         }
       }
     }
-    if (touched_host && c.ready) {
+    if ((touched_host || sync_every_call() || report_enabled()) && c.ready) {
       hipError_t e = hipStreamSynchronize(c.stream);
       if (e != hipSuccess && ok)
         fail(EIO, "stream synchronisation failed: %s", hipGetErrorString(e));
@@ -421,6 +481,8 @@ struct Call {
     for (void *p : temps)
       c.give(p);
     temps.clear();
+    if (report_enabled() && c.ready)
+      report_line(op, "after", now_seconds());
   }
 };
 
@@ -631,7 +693,7 @@ void run_matmul(const MatmulSpec &sp) {
   if (M == 0 || N == 0)
     return;
 
-  Call call(t_ctx);
+  Call call(t_ctx, sp.op);
   if (!call.ok)
     return;
   const bool a_uns = a.dtype == OM_MI355X_TYPE_UINT8;
@@ -751,7 +813,7 @@ void om_mi355x_QuantizeLinear(OMTensor *y_t, const OMTensor *x_t,
     return;
   if (x.numel == 0)
     return;
-  Call call(t_ctx);
+  Call call(t_ctx, "QuantizeLinear");
   if (!call.ok)
     return;
   const float *dx = (const float *)call.in(x);
@@ -787,7 +849,7 @@ void om_mi355x_DequantizeLinear(OMTensor *y_t, const OMTensor *x_t,
     return;
   if (x.numel == 0)
     return;
-  Call call(t_ctx);
+  Call call(t_ctx, "DequantizeLinear");
   if (!call.ok)
     return;
   const void *dx = call.in(x);
@@ -819,7 +881,7 @@ void om_mi355x_DynamicQuantizeLinear(OMTensor *y_t, OMTensor *scale_t,
   }
   if (x.numel == 0)
     return;
-  Call call(t_ctx);
+  Call call(t_ctx, "DynamicQuantizeLinear");
   if (!call.ok)
     return;
   const float *dx = (const float *)call.in(x);
@@ -893,7 +955,7 @@ void om_mi355x_DynQuantMatMulDequant(OMTensor *y_t, const OMTensor *x_t,
   }
   if (M == 0 || N == 0)
     return;
-  Call call(t_ctx);
+  Call call(t_ctx, "DynQuantMatMulDequant");
   if (!call.ok)
     return;
   const float *dx = (const float *)call.in(x);

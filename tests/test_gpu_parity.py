@@ -250,6 +250,32 @@ def test_dynamic_quantize_barrier_timeout_is_reported():
     assert "ERROR-OK" in out.stdout and "RECOVERED" in out.stdout, out.stdout + out.stderr
 
 
+def test_perf_report_lines_have_the_reference_format(tmp_path):
+    """OM_MI355X_PERF_REPORT=1 makes every entry point synchronous and prints a
+    before / after pair per call in the format of src/Runtime/OMInstrument.c:164
+    ("==PERF-REPORT==, op, node, before|after, since last, since start")."""
+    import re, subprocess, sys, textwrap
+    report = tmp_path / "perf.txt"
+    code = textwrap.dedent("""
+        import sys, numpy as np
+        sys.path.insert(0, %r)
+        import om_mi355x as rt
+        x = np.random.default_rng(0).normal(0, 1, (64, 128)).astype(np.float32)
+        y, s, z = rt.DynamicQuantizeLinear(x)
+        b = np.random.default_rng(1).integers(-127, 128, (128, 96)).astype(np.int8)
+        rt.MatMulInteger(y, b, z, None)
+    """ % os.path.join(os.path.dirname(HERE), "onnx-mlir_amd"))
+    env = dict(os.environ, OM_MI355X_PERF_REPORT="1", ONNX_MLIR_INSTRUMENT_FILE=str(report))
+    out = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=110)
+    assert out.returncode == 0, out.stderr
+    lines = report.read_text().strip().splitlines()
+    pat = re.compile(r"^==PERF-REPORT==, (onnx\.\w+), (\w+), (before|after), (\d+\.\d{6}), (\d+\.\d{6})$")
+    got = [pat.match(l).groups() for l in lines]
+    assert [(g[0], g[2]) for g in got] == [("onnx.DynamicQuantizeLinear", "before"), ("onnx.DynamicQuantizeLinear", "after"),
+                                           ("onnx.MatMulInteger", "before"), ("onnx.MatMulInteger", "after")]
+    assert all(float(g[3]) >= 0 for g in got) and float(got[-1][4]) >= float(got[0][4])
+
+
 def test_dynamic_quantize_invariants_large(rt):
     # properties that hold at any size: zp in range, the extremes map to 0 / 255
     x = wl.normal_f32(2, 0, (2048, 4099), 2.0)
