@@ -37,6 +37,7 @@ enum class MI355XNarrowMode : int64_t {
 extern MI355XNarrowMode mi355xNarrowMode;
 extern bool mi355xDisableFusion;
 extern bool mi355xDisableMarkConstant;
+extern bool mi355xDisableKeepOnDevice;
 extern std::string mi355xOps;
 
 } // namespace onnx_mlir

@@ -49,8 +49,13 @@ void addPassesMI355X(OwningOpRef<ModuleOp> &module, PassManager &pm,
     if (inputLevel <= ONNXLevel)
       addONNXToKrnlPasses(
           pm, OptimizationLevel, /*enableCSE=*/true, ONNXOpStats);
-    if (inputLevel <= MLIRLevel)
+    if (inputLevel <= MLIRLevel) {
       addKrnlToAffinePasses(pm);
+      // Needs the final set of users of each buffer (after write-only allocs
+      // are gone) and has to come before deallocations are inserted.
+      if (!mi355xDisableKeepOnDevice)
+        pm.addNestedPass<func::FuncOp>(createKeepBuffersOnMI355XPass());
+    }
   }
 
   if (emissionTarget >= EmitLLVMIR && inputLevel <= LLVMLevel)

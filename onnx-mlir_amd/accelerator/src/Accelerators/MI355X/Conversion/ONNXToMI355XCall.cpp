@@ -105,14 +105,17 @@ void emitCall(ConversionPatternRewriter &rewriter, Location loc,
 /// keeps its address for the life of the model
 /// (src/Conversion/KrnlToLLVM/KrnlGlobal.cpp:74-200).  Registering an address
 /// twice is a no-op in the runtime, so the call may sit in front of every use.
+/// The constant is passed as an output: a call with no results and only read
+/// effects (src/Dialect/Krnl/KrnlOps.cpp:168-180) counts as trivially dead and
+/// would not survive canonicalisation.
 void markIfConstant(
     ConversionPatternRewriter &rewriter, Location loc, Value v) {
   if (mi355xDisableMarkConstant || isAbsent(v))
     return;
   if (!v.getDefiningOp<KrnlGlobalOp>())
     return;
-  KrnlCallOp::create(rewriter, loc, std::string("om_mi355x_MarkConstant"),
-      /*numOfOutput=*/static_cast<int64_t>(0), ValueRange{v});
+  KrnlCallOp::create(rewriter, loc, std::string(kMI355XMarkConstant),
+      /*numOfOutput=*/static_cast<int64_t>(1), ValueRange{v});
 }
 
 /// Allocate the results of `op` with the op's own shape helper.

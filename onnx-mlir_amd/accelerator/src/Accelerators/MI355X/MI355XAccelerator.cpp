@@ -76,6 +76,9 @@ void MI355XAccelerator::registerPasses(int /*optLevel*/) const {
   mlir::registerPass([]() -> std::unique_ptr<mlir::Pass> {
     return onnx_mlir::createFuseQuantizedMatMulForMI355XPass();
   });
+  mlir::registerPass([]() -> std::unique_ptr<mlir::Pass> {
+    return onnx_mlir::createKeepBuffersOnMI355XPass();
+  });
 }
 
 void MI355XAccelerator::configurePasses() const { configurePassesMI355X(); }

@@ -20,11 +20,22 @@ constexpr const char *kMI355XMatMulIntegerDequant =
 constexpr const char *kMI355XDynQuantMatMulDequant =
     "om_mi355x_DynQuantMatMulDequant";
 
+/// Bookkeeping entry points of the runtime (no computation).
+constexpr const char *kMI355XMarkConstant = "om_mi355x_MarkConstant";
+constexpr const char *kMI355XKeepOnDevice = "om_mi355x_KeepOnDevice";
+constexpr const char *kMI355XRelease = "om_mi355x_Release";
+
 /// --fuse-quantized-matmul-for-mi355x
 ///   MatMulInteger -> Cast(f32) -> Mul(a_scale * b_scale)
 ///   DynamicQuantizeLinear -> MatMulInteger -> Cast(f32) -> Mul(...)
 /// become one `onnx.Custom` each.
 std::unique_ptr<mlir::Pass> createFuseQuantizedMatMulForMI355XPass();
+
+/// --keep-buffers-on-mi355x
+/// Runs on Krnl/MemRef IR.  A `memref.alloc` that only MI355X calls touch gets
+/// `om_mi355x_KeepOnDevice` after the allocation and `om_mi355x_Release`
+/// after its last user, so that it never travels to the host and back.
+std::unique_ptr<mlir::Pass> createKeepBuffersOnMI355XPass();
 
 } // namespace onnx_mlir
 #endif

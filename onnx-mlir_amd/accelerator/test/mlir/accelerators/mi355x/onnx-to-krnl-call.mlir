@@ -68,7 +68,7 @@ func.func @matmul_integer_constant_weight(%a: tensor<128x4xui8>, %azp: tensor<ui
 // CHECK-LABEL:  func.func @matmul_integer_constant_weight
 // CHECK:        [[B:%.+]] = "krnl.global"()
 // CHECK:        "krnl.call"([[B]])
-// CHECK-SAME:   funcName = "om_mi355x_MarkConstant", numOfOutput = 0 : si64
+// CHECK-SAME:   funcName = "om_mi355x_MarkConstant", numOfOutput = 1 : si64
 // CHECK:        [[Y:%.+]] = memref.alloc() {{.*}}: memref<128x2xi32>
 // CHECK:        "krnl.call"([[Y]], {{%.+}}, [[B]], {{%.+}}, {{%.+}})
 // CHECK-SAME:   funcName = "om_mi355x_MatMulInteger", numOfOutput = 1 : si64

@@ -87,6 +87,16 @@ struct PackedB {
 };
 std::unordered_map<const void *, PackedB> g_packed;
 
+// Host buffers backed by GPU memory (om_mi355x_KeepOnDevice): start address ->
+// (GPU copy, bytes).  Guarded by g_mem_mutex.
+struct Backing {
+  void *dev;
+  size_t bytes;    // size of the host buffer
+  size_t capacity; // size of the GPU block (what the pool files it under)
+  hipStream_t stream; // stream of the thread that declared it
+};
+std::map<uintptr_t, Backing> g_backed;
+
 bool probe_device() {
   int count = 0;
   hipError_t e = hipGetDeviceCount(&count);
@@ -209,6 +219,18 @@ struct Ctx {
     pool.emplace(it->second, p);
     taken.erase(it);
   }
+  // A pool block whose ownership leaves the pool (a backing that outlives the
+  // call); adopt() files such a block back.
+  void *take_owned(size_t bytes, size_t *capacity) {
+    void *p = take(bytes);
+    if (!p)
+      return nullptr;
+    auto it = taken.find(p);
+    *capacity = it->second;
+    taken.erase(it);
+    return p;
+  }
+  void adopt(void *p, size_t capacity) { pool.emplace(capacity, p); }
   void drop_pool() {
     for (auto &kv : pool)
       (void)hipFree(kv.second);
@@ -218,6 +240,22 @@ struct Ctx {
 };
 
 thread_local Ctx t_ctx;
+
+// GPU address that stands for host address p, if p lies in a buffer declared
+// with om_mi355x_KeepOnDevice; null otherwise.
+void *backed_lookup(const void *p) {
+  std::lock_guard<std::mutex> lk(g_mem_mutex);
+  if (g_backed.empty())
+    return nullptr;
+  auto it = g_backed.upper_bound((uintptr_t)p);
+  if (it == g_backed.begin())
+    return nullptr;
+  --it;
+  const uintptr_t off = (uintptr_t)p - it->first;
+  if (off >= it->second.bytes)
+    return nullptr;
+  return (char *)it->second.dev + off;
+}
 
 bool is_device_ptr(const void *p) {
   {
@@ -386,6 +424,8 @@ struct Call {
   const void *in(const View &v) {
     if (!ok || v.numel == 0)
       return v.data;
+    if (void *d = backed_lookup(v.data))
+      return d;
     if (is_device_ptr(v.data))
       return v.data;
     {
@@ -442,6 +482,8 @@ struct Call {
   void *out(const View &v) {
     if (!ok || v.numel == 0)
       return v.data;
+    if (void *d = backed_lookup(v.data))
+      return d;
     if (is_device_ptr(v.data))
       return v.data;
     void *d = temp(v.bytes);
@@ -1006,6 +1048,65 @@ void om_mi355x_MarkConstant(const OMTensor *t) {
   g_constants.insert(p);
 }
 
+// The GPU blocks come from the calling thread's pool and go back to it, so a
+// model that declares and releases the same buffers on every inference
+// allocates only during the first one.  Work that uses a block is queued on
+// the declaring thread's stream; a release from that thread needs no wait
+// (the next user of the block is ordered behind it on the same stream), a
+// release from another thread waits for that stream first.
+void om_mi355x_KeepOnDevice(const OMTensor *t) {
+  View v;
+  if (!t || !view_of(t, "tensor", v) || v.bytes == 0)
+    return;
+  if (!t_ctx.init())
+    return;
+  if (is_device_ptr(v.data))
+    return; // already GPU memory: nothing to back
+  Backing old = {nullptr, 0, 0, nullptr};
+  {
+    std::lock_guard<std::mutex> lk(g_mem_mutex);
+    auto it = g_backed.find((uintptr_t)v.data);
+    if (it != g_backed.end()) {
+      if (it->second.bytes == v.bytes)
+        return;
+      old = it->second; // same address, other size: a buffer that was freed
+      g_backed.erase(it); // and allocated again without a release
+    }
+  }
+  if (old.dev) {
+    if (old.stream != t_ctx.stream)
+      (void)hipStreamSynchronize(old.stream);
+    t_ctx.adopt(old.dev, old.capacity);
+  }
+  size_t capacity = 0;
+  void *d = t_ctx.take_owned(v.bytes, &capacity);
+  if (!d)
+    return;
+  std::lock_guard<std::mutex> lk(g_mem_mutex);
+  g_backed[(uintptr_t)v.data] = Backing{d, v.bytes, capacity, t_ctx.stream};
+}
+
+void om_mi355x_Release(const OMTensor *t) {
+  if (!t)
+    return;
+  const void *p = omTensorGetDataPtr(t);
+  Backing b;
+  {
+    std::lock_guard<std::mutex> lk(g_mem_mutex);
+    auto it = g_backed.find((uintptr_t)p);
+    if (it == g_backed.end())
+      return;
+    b = it->second;
+    g_backed.erase(it);
+  }
+  if (t_ctx.ready && b.stream == t_ctx.stream) {
+    t_ctx.adopt(b.dev, b.capacity);
+    return;
+  }
+  (void)hipStreamSynchronize(b.stream);
+  (void)hipFree(b.dev);
+}
+
 void om_mi355x_ClearCache(void) {
   if (t_ctx.ready)
     (void)hipStreamSynchronize(t_ctx.stream);
@@ -1019,6 +1120,9 @@ void om_mi355x_ClearCache(void) {
   }
   g_packed.clear();
   g_constants.clear();
+  for (auto &kv : g_backed)
+    (void)hipFree(kv.second.dev);
+  g_backed.clear();
   t_ctx.drop_pool();
 }
 

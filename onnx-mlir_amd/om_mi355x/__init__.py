@@ -85,6 +85,8 @@ def _declare(lib, shim):
         "om_mi355x_QLinearMatMul": [P, P, P, P, P, P, P, P, P, I64],
         "om_mi355x_DynQuantMatMulDequant": [P, P, P, P, P],
         "om_mi355x_MarkConstant": [P],
+        "om_mi355x_KeepOnDevice": [P],
+        "om_mi355x_Release": [P],
         "om_mi355x_ClearCache": [],
         "OMInitAccelMI355X": [],
         "OMShutdownAccelMI355X": [],
@@ -249,6 +251,24 @@ def mark_constant(t: Tensor):
 def clear_cache():
     load()
     _lib.om_mi355x_ClearCache()
+
+
+def keep_on_device(t: np.ndarray):
+    """Back the host buffer of ``t`` with GPU memory: until ``release`` the ops
+    use that memory whenever they are handed ``t`` and never touch the host
+    buffer (what a compiled model does for results that only feed other
+    offloaded ops)."""
+    load()
+    with _OMT(t) as h:
+        _lib.om_mi355x_KeepOnDevice(h)
+    _check()
+
+
+def release(t: np.ndarray):
+    load()
+    with _OMT(t) as h:
+        _lib.om_mi355x_Release(h)
+    _check()
 
 
 def synchronize():

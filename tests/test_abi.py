@@ -149,14 +149,16 @@ def test_compiler_plugin_calls_only_exported_symbols(rt):
     assert {"om_mi355x_QuantizeLinear", "om_mi355x_DequantizeLinear",
             "om_mi355x_DynamicQuantizeLinear", "om_mi355x_MatMulInteger",
             "om_mi355x_QLinearMatMul", "om_mi355x_MatMulIntegerDequant",
-            "om_mi355x_DynQuantMatMulDequant", "om_mi355x_MarkConstant"} <= callees
+            "om_mi355x_DynQuantMatMulDequant", "om_mi355x_MarkConstant",
+            "om_mi355x_KeepOnDevice", "om_mi355x_Release"} <= callees
     for name in callees:
         assert hasattr(lib, name), f"plug-in calls {name}, which the runtime lacks"
     # parameter counts: results + operands + integer attributes of each pattern
     passed = {"om_mi355x_QuantizeLinear": 1 + 3 + 2, "om_mi355x_DequantizeLinear": 1 + 3 + 1,
               "om_mi355x_DynamicQuantizeLinear": 3 + 1, "om_mi355x_MatMulInteger": 1 + 4,
               "om_mi355x_QLinearMatMul": 1 + 8 + 1, "om_mi355x_MatMulIntegerDequant": 1 + 6,
-              "om_mi355x_DynQuantMatMulDequant": 1 + 4, "om_mi355x_MarkConstant": 1}
+              "om_mi355x_DynQuantMatMulDequant": 1 + 4, "om_mi355x_MarkConstant": 1,
+              "om_mi355x_KeepOnDevice": 1, "om_mi355x_Release": 1}
     for name, count in passed.items():
         m = re.search(r"\b%s\s*\(([^)]*)\)" % name, header)
         assert m, name
@@ -175,7 +177,7 @@ def test_compiler_plugin_lit_tests_name_real_entry_points(rt):
     lib = rt.load()
     lit = os.path.join(PLUGIN, "test", "mlir", "accelerators", "mi355x")
     files = [f for f in os.listdir(lit) if f.endswith(".mlir")]
-    assert len(files) >= 4
+    assert len(files) >= 5
     for f in files:
         text = open(os.path.join(lit, f)).read()
         assert "// RUN: onnx-mlir-opt --maccel=MI355X" in text

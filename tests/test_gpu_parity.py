@@ -418,6 +418,57 @@ def test_constant_weight_shared_by_every_kernel_family(rt, oracle):
         rt.clear_cache()
 
 
+def test_host_buffers_kept_on_device_between_ops(rt, oracle):
+    """The compiled-model flow: intermediates are plain host allocations that the
+    accelerator pass declares device-backed.  The chain DynamicQuantizeLinear ->
+    MatMulInteger -> QuantizeLinear then runs without touching them (they keep
+    their sentinel bytes), and the final host output is exact."""
+    rng = np.random.default_rng(61)
+    M, K, N = 300, 256, 384
+    x = rng.normal(0, 1, (M, K)).astype(np.float32)
+    W = _rand_q(rng, np.int8, (K, N))
+    aq = np.full((M, K), 0xAB, np.uint8)
+    a_s = np.full((), -777.0, np.float32)
+    a_z = np.full((), 0xCD, np.uint8)
+    acc = np.full((M, N), 0x5A5A5A5A, np.int32)
+    for t in (aq, a_s, a_z, acc):
+        rt.keep_on_device(t)
+    try:
+        calls = [rt.PreparedCall("om_mi355x_DynamicQuantizeLinear", aq, a_s, a_z, x),
+                 rt.PreparedCall("om_mi355x_MatMulInteger", acc, aq, W, a_z, None)]
+        for c in calls:
+            c()
+            c.check()
+        got = rt.DequantizeLinear(acc, np.float32(0.5), None)     # host output: staged and copied back
+        waq, ws, wz = oracle.dynamic_quantize_linear(x)
+        want = oracle.matmul_integer(waq, W, wz, None).astype(np.float32) * np.float32(0.5)
+        assert np.array_equal(got, want)
+        assert (aq == 0xAB).all() and a_s == np.float32(-777.0) and a_z == 0xCD and (acc == 0x5A5A5A5A).all()
+        for c in calls:
+            c.close()
+    finally:
+        for t in (aq, a_s, a_z, acc):
+            rt.release(t)
+    # after the release the same buffers are ordinary host tensors again
+    y, s, z = rt.DynamicQuantizeLinear(x)
+    assert np.array_equal(y, waq)
+    # a second inference reuses the released GPU blocks; this time another
+    # host thread releases, which has to wait for the work queued here
+    import threading
+    for t in (aq, acc):
+        rt.keep_on_device(t)
+    rt.QuantizeLinear(x, s, z, out=aq)
+    rt.MatMulInteger(aq, W, z, None, out=acc)
+    got = rt.DequantizeLinear(acc, np.float32(0.25), None)
+    assert np.array_equal(got, oracle.matmul_integer(waq, W, wz, None).astype(np.float32) * np.float32(0.25))
+    assert (aq == 0xAB).all() and (acc == 0x5A5A5A5A).all()
+    th = threading.Thread(target=lambda: [rt.release(t) for t in (aq, acc)])
+    th.start()
+    th.join()
+    rt.MatMulInteger(waq, W, wz, None, out=acc)
+    assert np.array_equal(acc, oracle.matmul_integer(waq, W, wz, None))
+
+
 def test_concurrent_host_threads(rt, oracle):
     """Entry points are re-entrant: four host threads (each gets its own stream)
     run DynamicQuantizeLinear on a tensor that takes the one-launch kernel,
