@@ -170,83 +170,66 @@ __global__ __launch_bounds__(kThreads) void k_quant_lastaxis(
 // ---- per-axis quantize, innermost axis, rows not 16-byte aligned -----------
 // When C % 4 != 0 the rows of a [rows, C] tensor start at odd alignments and
 // the row-walking kernel above would issue misaligned 16-byte loads and
-// misaligned 4-byte stores.  This kernel walks the flat array instead, so
-// every data access is aligned, and carries the column of each float4 along
-// incrementally (one modulo per thread at the start, then add-and-wrap).
-// Scale and zero point are fetched per float4 from L1 / L2 (they are tiny);
-// the rare float4 that straddles the end of a row takes a scalar path.
+// misaligned 4-byte stores.  This kernel works on the flat array cut into
+// aligned vectors of four elements.  Vector i covers columns (4 i + e) mod C,
+// which repeats every C / gcd(C, 4) vectors (every four rows when C is odd).
+// `period` is a multiple of that, so a thread that takes vectors v, v +
+// period, v + 2 period, ... meets the same four columns each time: it loads
+// their scales and zero points once, like the row-walking kernel, and every
+// data access is aligned and coalesced.
 template <bool SIGNED, bool HAS_ZP>
-__global__ __launch_bounds__(kThreads) void k_quant_flat_axis(
+__global__ __launch_bounds__(kThreads) void k_quant_periodic(
     const float *__restrict__ x, uint8_t *__restrict__ y, int64_t n, uint32_t C,
-    const float *__restrict__ scale, const void *__restrict__ zp) {
+    int64_t period, const float *__restrict__ scale,
+    const void *__restrict__ zp, int periods_per_block) {
+  const int64_t v = (int64_t)blockIdx.x * kThreads + threadIdx.x;
   const int64_t nvec = n >> 2;
-  const f4a *__restrict__ x4 = (const f4a *)x;
-  uint32_t *__restrict__ y4 = (uint32_t *)y;
-  const int64_t step = (int64_t)gridDim.x * (kThreads * kUnroll);
-  const uint32_t dstep = (uint32_t)((step * 4) % C);
-  const uint32_t dj = (uint32_t)((kThreads * 4) % C);
-  int64_t base = (int64_t)blockIdx.x * (kThreads * kUnroll);
-  uint32_t c0 = (uint32_t)(((base + threadIdx.x) * 4) % C);
-  const uint8_t *__restrict__ zpb = (const uint8_t *)zp;
-  for (; base < nvec; base += step) {
-    f4a v[kUnroll];
-    int64_t idx[kUnroll];
-    uint32_t c[kUnroll];
-    uint32_t cj = c0;
-#pragma unroll
-    for (int j = 0; j < kUnroll; ++j) {
-      idx[j] = base + j * kThreads + threadIdx.x;
-      c[j] = cj;
-      cj += dj;
-      cj -= (cj >= C) ? C : 0;
-      if (idx[j] < nvec)
-        v[j] = __builtin_nontemporal_load(&x4[idx[j]]);
-    }
-#pragma unroll
-    for (int j = 0; j < kUnroll; ++j) {
-      if (idx[j] >= nvec)
-        continue;
-      float s[4], z[4];
-      if (c[j] + 4 <= C) {
-        const f4u sv = *(const f4u *)(scale + c[j]);
-        s[0] = sv.x; s[1] = sv.y; s[2] = sv.z; s[3] = sv.w;
-        if (HAS_ZP) {
-          const uint32_t zw = *(const u32_a1 *)(zpb + c[j]);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const uint32_t b = (zw >> (8 * e)) & 0xFFu;
-            z[e] = SIGNED ? (float)(int32_t)(int8_t)b : (float)b;
-          }
-        }
-      } else {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          uint32_t ce = c[j] + e;
-          ce -= (ce >= C) ? C : 0;
-          s[e] = scale[ce];
-          if (HAS_ZP)
-            z[e] = load_zp_f32<SIGNED>(zp, ce);
-        }
-      }
-      if (!HAS_ZP)
-        z[0] = z[1] = z[2] = z[3] = 0.0f;
-      const uint32_t b0 = quant_one<SIGNED, HAS_ZP>(v[j].x, s[0], z[0]);
-      const uint32_t b1 = quant_one<SIGNED, HAS_ZP>(v[j].y, s[1], z[1]);
-      const uint32_t b2 = quant_one<SIGNED, HAS_ZP>(v[j].z, s[2], z[2]);
-      const uint32_t b3 = quant_one<SIGNED, HAS_ZP>(v[j].w, s[3], z[3]);
-      __builtin_nontemporal_store(
-          b0 | (b1 << 8) | (b2 << 16) | (b3 << 24), &y4[idx[j]]);
-    }
-    c0 += dstep;
-    c0 -= (c0 >= C) ? C : 0;
-  }
-  if (blockIdx.x == 0) {
+  if (blockIdx.x == 0 && blockIdx.y == 0) {
     const int64_t e = (nvec << 2) + threadIdx.x;
     if (e < n) {
       const uint32_t ce = (uint32_t)(e % C);
       const float zf = HAS_ZP ? load_zp_f32<SIGNED>(zp, ce) : 0.0f;
       y[e] = (uint8_t)quant_one<SIGNED, HAS_ZP>(x[e], scale[ce], zf);
     }
+  }
+  if (v >= period)
+    return;
+  float s[4], z[4];
+  {
+    uint32_t c = (uint32_t)(((uint64_t)v * 4) % C);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      s[e] = scale[c];
+      z[e] = HAS_ZP ? load_zp_f32<SIGNED>(zp, c) : 0.0f;
+      c = (c + 1 == C) ? 0 : c + 1;
+    }
+  }
+  const f4a *__restrict__ x4 = (const f4a *)x;
+  uint32_t *__restrict__ y4 = (uint32_t *)y;
+  int64_t idx = (int64_t)blockIdx.y * periods_per_block * period + v;
+  const int64_t end = idx + (int64_t)periods_per_block * period;
+  const int64_t stop = end < nvec ? end : nvec;
+  for (; idx + (kRowUnroll - 1) * period < stop; idx += kRowUnroll * period) {
+    f4a q[kRowUnroll];
+#pragma unroll
+    for (int j = 0; j < kRowUnroll; ++j)
+      q[j] = __builtin_nontemporal_load(&x4[idx + j * period]);
+#pragma unroll
+    for (int j = 0; j < kRowUnroll; ++j) {
+      const uint32_t b0 = quant_one<SIGNED, HAS_ZP>(q[j].x, s[0], z[0]);
+      const uint32_t b1 = quant_one<SIGNED, HAS_ZP>(q[j].y, s[1], z[1]);
+      const uint32_t b2 = quant_one<SIGNED, HAS_ZP>(q[j].z, s[2], z[2]);
+      const uint32_t b3 = quant_one<SIGNED, HAS_ZP>(q[j].w, s[3], z[3]);
+      y4[idx + j * period] = b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
+    }
+  }
+  for (; idx < stop; idx += period) {
+    const f4a q = x4[idx];
+    const uint32_t b0 = quant_one<SIGNED, HAS_ZP>(q.x, s[0], z[0]);
+    const uint32_t b1 = quant_one<SIGNED, HAS_ZP>(q.y, s[1], z[1]);
+    const uint32_t b2 = quant_one<SIGNED, HAS_ZP>(q.z, s[2], z[2]);
+    const uint32_t b3 = quant_one<SIGNED, HAS_ZP>(q.w, s[3], z[3]);
+    y4[idx] = b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
   }
 }
 
@@ -425,78 +408,63 @@ __global__ __launch_bounds__(kThreads) void k_dequant_lastaxis(
   }
 }
 
-// 8-bit input, innermost axis, C % 4 != 0: flat walk, aligned accesses, column
-// carried incrementally (see k_quant_flat_axis).
+// 8-bit input, innermost axis, C % 4 != 0: aligned vectors of the flat array,
+// each thread on a fixed set of four columns (see k_quant_periodic).
 template <int KIND, bool HAS_ZP>
-__global__ __launch_bounds__(kThreads) void k_dequant8_flat_axis(
+__global__ __launch_bounds__(kThreads) void k_dequant8_periodic(
     const uint8_t *__restrict__ x, float *__restrict__ y, int64_t n, uint32_t C,
-    const float *__restrict__ scale, const void *__restrict__ zp) {
+    int64_t period, const float *__restrict__ scale,
+    const void *__restrict__ zp, int periods_per_block) {
+  const int64_t v = (int64_t)blockIdx.x * kThreads + threadIdx.x;
   const int64_t nvec = n >> 2;
-  const uint32_t *__restrict__ x4 = (const uint32_t *)x;
-  f4a *__restrict__ y4 = (f4a *)y;
-  const int64_t step = (int64_t)gridDim.x * (kThreads * kUnroll);
-  const uint32_t dstep = (uint32_t)((step * 4) % C);
-  const uint32_t dj = (uint32_t)((kThreads * 4) % C);
-  int64_t base = (int64_t)blockIdx.x * (kThreads * kUnroll);
-  uint32_t c0 = (uint32_t)(((base + threadIdx.x) * 4) % C);
-  const uint8_t *__restrict__ zpb = (const uint8_t *)zp;
-  for (; base < nvec; base += step) {
-    uint32_t w[kUnroll];
-    int64_t idx[kUnroll];
-    uint32_t c[kUnroll];
-    uint32_t cj = c0;
-#pragma unroll
-    for (int j = 0; j < kUnroll; ++j) {
-      idx[j] = base + j * kThreads + threadIdx.x;
-      c[j] = cj;
-      cj += dj;
-      cj -= (cj >= C) ? C : 0;
-      if (idx[j] < nvec)
-        w[j] = __builtin_nontemporal_load(&x4[idx[j]]);
-    }
-#pragma unroll
-    for (int j = 0; j < kUnroll; ++j) {
-      if (idx[j] >= nvec)
-        continue;
-      float s[4], z[4];
-      if (c[j] + 4 <= C) {
-        const f4u sv = *(const f4u *)(scale + c[j]);
-        s[0] = sv.x; s[1] = sv.y; s[2] = sv.z; s[3] = sv.w;
-        if (HAS_ZP) {
-          const uint32_t zw = *(const u32_a1 *)(zpb + c[j]);
-#pragma unroll
-          for (int e = 0; e < 4; ++e)
-            z[e] = q_to_f32<KIND>(zw >> (8 * e));
-        }
-      } else {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          uint32_t ce = c[j] + e;
-          ce -= (ce >= C) ? C : 0;
-          s[e] = scale[ce];
-          if (HAS_ZP)
-            z[e] = load_q_zp_f32<KIND>(zp, ce);
-        }
-      }
-      if (!HAS_ZP)
-        z[0] = z[1] = z[2] = z[3] = 0.0f;
-      f4a o;
-      o.x = dq_one<HAS_ZP>(q_to_f32<KIND>(w[j]), s[0], z[0]);
-      o.y = dq_one<HAS_ZP>(q_to_f32<KIND>(w[j] >> 8), s[1], z[1]);
-      o.z = dq_one<HAS_ZP>(q_to_f32<KIND>(w[j] >> 16), s[2], z[2]);
-      o.w = dq_one<HAS_ZP>(q_to_f32<KIND>(w[j] >> 24), s[3], z[3]);
-      __builtin_nontemporal_store(o, &y4[idx[j]]);
-    }
-    c0 += dstep;
-    c0 -= (c0 >= C) ? C : 0;
-  }
-  if (blockIdx.x == 0) {
+  if (blockIdx.x == 0 && blockIdx.y == 0) {
     const int64_t e = (nvec << 2) + threadIdx.x;
     if (e < n) {
       const uint32_t ce = (uint32_t)(e % C);
       const float zf = HAS_ZP ? load_q_zp_f32<KIND>(zp, ce) : 0.0f;
       y[e] = dq_one<HAS_ZP>(q_to_f32<KIND>(x[e]), scale[ce], zf);
     }
+  }
+  if (v >= period)
+    return;
+  float s[4], z[4];
+  {
+    uint32_t c = (uint32_t)(((uint64_t)v * 4) % C);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      s[e] = scale[c];
+      z[e] = HAS_ZP ? load_q_zp_f32<KIND>(zp, c) : 0.0f;
+      c = (c + 1 == C) ? 0 : c + 1;
+    }
+  }
+  const uint32_t *__restrict__ x4 = (const uint32_t *)x;
+  f4a *__restrict__ y4 = (f4a *)y;
+  int64_t idx = (int64_t)blockIdx.y * periods_per_block * period + v;
+  const int64_t end = idx + (int64_t)periods_per_block * period;
+  const int64_t stop = end < nvec ? end : nvec;
+  for (; idx + (kRowUnroll - 1) * period < stop; idx += kRowUnroll * period) {
+    uint32_t w[kRowUnroll];
+#pragma unroll
+    for (int j = 0; j < kRowUnroll; ++j)
+      w[j] = __builtin_nontemporal_load(&x4[idx + j * period]);
+#pragma unroll
+    for (int j = 0; j < kRowUnroll; ++j) {
+      f4a o;
+      o.x = dq_one<HAS_ZP>(q_to_f32<KIND>(w[j]), s[0], z[0]);
+      o.y = dq_one<HAS_ZP>(q_to_f32<KIND>(w[j] >> 8), s[1], z[1]);
+      o.z = dq_one<HAS_ZP>(q_to_f32<KIND>(w[j] >> 16), s[2], z[2]);
+      o.w = dq_one<HAS_ZP>(q_to_f32<KIND>(w[j] >> 24), s[3], z[3]);
+      __builtin_nontemporal_store(o, &y4[idx + j * period]);
+    }
+  }
+  for (; idx < stop; idx += period) {
+    const uint32_t w = x4[idx];
+    f4a o;
+    o.x = dq_one<HAS_ZP>(q_to_f32<KIND>(w), s[0], z[0]);
+    o.y = dq_one<HAS_ZP>(q_to_f32<KIND>(w >> 8), s[1], z[1]);
+    o.z = dq_one<HAS_ZP>(q_to_f32<KIND>(w >> 16), s[2], z[2]);
+    o.w = dq_one<HAS_ZP>(q_to_f32<KIND>(w >> 24), s[3], z[3]);
+    y4[idx] = o;
   }
 }
 
@@ -868,6 +836,46 @@ inline int stream_grid(int64_t work_items, int64_t per_block) {
   return (int)(need < cap ? need : cap);
 }
 
+// Launch shape of the periodic kernels: `period` is the column period of the
+// 4-element vectors (C / gcd(C, 4)), repeated until it is a multiple of 8 and
+// spans at least four blocks' worth of threads; grid.x covers one period, grid.y splits the
+// periods, about 4096 blocks in total and at least 16 periods per block.
+struct PeriodicGrid {
+  dim3 grid;
+  int64_t period;
+  int per_block;
+};
+PeriodicGrid periodic_grid(int64_t nvec, int64_t C) {
+  const int64_t g = (C % 2 == 0) ? 2 : 1; // C % 4 != 0 here
+  int64_t period = C / g;
+  // A multiple of 8 vectors, so that a thread's accesses keep their position
+  // within a 128-byte line from one period to the next and every wave writes
+  // whole lines.
+  while (period % 8 != 0)
+    period *= 2;
+  const int64_t want = 4 * kThreads;
+  if (period < want)
+    period *= (want + period - 1) / period;
+  const int64_t gx = (period + kThreads - 1) / kThreads;
+  const int64_t periods = (nvec + period - 1) / period;
+  int64_t gy = 4096 / gx;
+  if (gy < 1)
+    gy = 1;
+  int64_t per_block = (periods + gy - 1) / gy;
+  if (per_block < 16)
+    per_block = 16;
+  gy = (periods + per_block - 1) / per_block;
+  if (gy > 65535) {
+    per_block = (periods + 65534) / 65535;
+    gy = (periods + per_block - 1) / per_block;
+  }
+  PeriodicGrid pg;
+  pg.grid = dim3((unsigned)gx, (unsigned)gy);
+  pg.period = period;
+  pg.per_block = (int)per_block;
+  return pg;
+}
+
 template <bool SIGNED>
 hipError_t quantize_dispatch(hipStream_t st, const float *x, int64_t outer,
     int64_t channels, int64_t inner, const float *scale, const void *zp,
@@ -898,16 +906,16 @@ hipError_t quantize_dispatch(hipStream_t st, const float *x, int64_t outer,
   }
   if (flip != 0)
     return hipErrorInvalidValue;
-  if (inner == 1 && channels > 1 && channels % 4 != 0 && channels >= 4 &&
+  if (inner == 1 && channels > 1 && channels % 4 != 0 &&
       channels < ((int64_t)1 << 31) && ((((uintptr_t)x) & 15) == 0) &&
-      ((((uintptr_t)y) & 3) == 0)) {
-    const int grid = stream_grid(n >> 2, kThreads * kUnroll);
+      ((((uintptr_t)y) & 3) == 0) && (n >> 2) > 0) {
+    const PeriodicGrid pg = periodic_grid(n >> 2, channels);
     if (has_zp)
-      k_quant_flat_axis<SIGNED, true><<<grid, kThreads, 0, st>>>(
-          x, yo, n, (uint32_t)channels, scale, zp);
+      k_quant_periodic<SIGNED, true><<<pg.grid, kThreads, 0, st>>>(
+          x, yo, n, (uint32_t)channels, pg.period, scale, zp, pg.per_block);
     else
-      k_quant_flat_axis<SIGNED, false><<<grid, kThreads, 0, st>>>(
-          x, yo, n, (uint32_t)channels, scale, zp);
+      k_quant_periodic<SIGNED, false><<<pg.grid, kThreads, 0, st>>>(
+          x, yo, n, (uint32_t)channels, pg.period, scale, zp, pg.per_block);
     return hipGetLastError();
   }
   if (inner == 1 && channels > 1) {
@@ -974,17 +982,17 @@ hipError_t dequantize_dispatch(hipStream_t st, const void *x, int64_t outer,
     return hipGetLastError();
   }
   if (KIND != kI32 && inner == 1 && channels > 1 && channels % 4 != 0 &&
-      channels >= 4 && channels < ((int64_t)1 << 31) &&
-      ((((uintptr_t)x) & 3) == 0) && ((((uintptr_t)y) & 15) == 0)) {
-    const int grid = stream_grid(n >> 2, kThreads * kUnroll);
+      channels < ((int64_t)1 << 31) && ((((uintptr_t)x) & 3) == 0) &&
+      ((((uintptr_t)y) & 15) == 0) && (n >> 2) > 0) {
+    const PeriodicGrid pg = periodic_grid(n >> 2, channels);
     if (has_zp)
-      k_dequant8_flat_axis<(KIND == kI32 ? kU8 : KIND), true>
-          <<<grid, kThreads, 0, st>>>(
-              (const uint8_t *)x, y, n, (uint32_t)channels, scale, zp);
+      k_dequant8_periodic<(KIND == kI32 ? kU8 : KIND), true>
+          <<<pg.grid, kThreads, 0, st>>>((const uint8_t *)x, y, n,
+              (uint32_t)channels, pg.period, scale, zp, pg.per_block);
     else
-      k_dequant8_flat_axis<(KIND == kI32 ? kU8 : KIND), false>
-          <<<grid, kThreads, 0, st>>>(
-              (const uint8_t *)x, y, n, (uint32_t)channels, scale, zp);
+      k_dequant8_periodic<(KIND == kI32 ? kU8 : KIND), false>
+          <<<pg.grid, kThreads, 0, st>>>((const uint8_t *)x, y, n,
+              (uint32_t)channels, pg.period, scale, zp, pg.per_block);
     return hipGetLastError();
   }
   if (inner == 1 && channels > 1) {
