@@ -82,6 +82,49 @@ def gemm_case(rt, wl, name, M, K, N, w_i8, w_scale, steps, warmup, epilogue="f32
     return res
 
 
+def spread_case(rt, wl, M, K, N, w_i8, w_scale, steps, warmup, sets=6, chunks=20):
+    """The headline GEMM timed two more ways.  (1) In `chunks` separate event
+    brackets, to show the run-to-run spread (p10 / median / p90 of the bracket
+    averages).  (2) Rotating over `sets` activation/output buffer pairs, 320 MB
+    in all for M=4096, N=3072, so that no launch finds its output or its
+    activations in the 256 MB last-level cache from the launch before."""
+    rng = np.random.default_rng(0xC0FFEE00 + M + K + N)
+    dW = rt.DeviceArray.from_numpy(w_i8)
+    dS = rt.DeviceArray.from_numpy(w_scale)
+    dAs = rt.DeviceArray.from_numpy(np.array(0.0173, np.float32))
+    dAz = rt.DeviceArray.from_numpy(np.array(131, np.uint8))
+    rt.mark_constant(dW)
+    bufs, calls = [], []
+    for _ in range(sets):
+        dA = rt.DeviceArray.from_numpy(rng.integers(0, 256, (M, K), dtype=np.uint8))
+        dY = rt.DeviceArray((M, N), np.float32)
+        bufs += [dA, dY]
+        calls.append(rt.PreparedCall("om_mi355x_MatMulIntegerDequant", dY, dA, dW, dAz, None, dAs, dS))
+    per = max(1, steps // chunks)
+    times = []
+    for i in range(chunks + 2):
+        _, ev_ms = timed(rt, calls[0], per, warmup if i == 0 else 0)
+        if i >= 2:
+            times.append(ev_ms)
+    state = {"i": 0}
+
+    def rotate():
+        calls[state["i"] % sets]()
+        state["i"] += 1
+
+    _, rot_ms = timed(rt, rotate, steps, warmup)
+    for c in calls:
+        c.check()
+        c.close()
+    for d in bufs + [dW, dS, dAs, dAz]:
+        d.free()
+    q = np.percentile(np.array(times), [10, 50, 90])
+    return {"launches_per_bracket": per, "brackets": chunks,
+            "kernel_ms_p10": float(q[0]), "kernel_ms_median": float(q[1]), "kernel_ms_p90": float(q[2]),
+            "buffer_sets": sets, "rotated_kernel_ms": rot_ms,
+            "rotated_tops": 2.0 * M * N * K / (rot_ms * 1e-3) / 1e12}
+
+
 def decode_case(rt, wl, M, steps, warmup):
     c = wl.config5("up", M=M)
     K, N = c["W"].shape
@@ -299,6 +342,8 @@ def main():
                                    max(10, args.steps // 10), max(2, args.warmup // 10), "f32"))
         gemms.append(qlinear_case(rt, wl, args.steps, args.warmup))
         extras["gemm"] = gemms
+        extras["headline_spread"] = spread_case(rt, wl, M, K, N, c["W"], c["w_scale"],
+                                                args.steps, args.warmup)
     if "fused" in groups:
         fused = []
         for name, (k, n) in wl.CONFIG4_SHAPES.items():
