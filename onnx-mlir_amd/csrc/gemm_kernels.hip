@@ -1279,7 +1279,9 @@ int choose_tile(int64_t M, int64_t N) {
 }
 
 bool gemm_fast_path(int64_t M, int64_t K, const void *A) {
-  return M > 16 && K % 64 == 0 && ((((uintptr_t)A) & 15) == 0);
+  // K == 0 (an empty sum) has no bytes of A to read: only the byte-wise path
+  // checks every address against K.
+  return M > 16 && K > 0 && K % 64 == 0 && ((((uintptr_t)A) & 15) == 0);
 }
 
 template <int A_MODE, int EPI>
@@ -1288,7 +1290,7 @@ hipError_t gemm_launch_cfg(
   const char *force = getenv("OM_MI355X_GEMM_TILE");
   const uint8_t *A = (const uint8_t *)g.A;
   const int M = (int)g.M, N = (int)g.N, K = (int)g.K;
-  if (g.M <= 32 && g.K % 16 == 0 && ((((uintptr_t)g.A) & 15) == 0) &&
+  if (g.M <= 32 && g.K > 0 && g.K % 16 == 0 && ((((uintptr_t)g.A) & 15) == 0) &&
       !(force && force[0])) {
     k_gemm_i8_skinny_bp<A_MODE, EPI>
         <<<dim3((unsigned)((g.N + 31) / 32)), 512, 0, st>>>(

@@ -1074,9 +1074,7 @@ hipStream_t g_grid_stream = nullptr; // stream of the last such launch
 hipError_t launch_dynamic_quantize(hipStream_t s, const DqlScratch &scratch,
     const float *x, int64_t n, uint8_t *y, float *scale, uint8_t *zp,
     bool y_shift) {
-  if (n == 0)
-    return hipSuccess;
-  if (n <= kSmallMax) {
+  if (n <= kSmallMax) { // n == 0 included: scale and zero point are written
     k_dql_small<<<1, kSmallThreads, 0, s>>>(
         x, n, y, scale, zp, y_shift ? 0x80808080u : 0u);
     return hipGetLastError();

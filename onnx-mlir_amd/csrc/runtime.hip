@@ -921,8 +921,8 @@ void om_mi355x_DynamicQuantizeLinear(OMTensor *y_t, OMTensor *scale_t,
                  "scalar f32 scale and scalar ui8 zero point");
     return;
   }
-  if (x.numel == 0)
-    return;
+  // No elements: scale and zero point are still results (0 and 0: the range
+  // is widened to include 0, DynamicQuantizeLinear.cpp:64-83).
   Call call(t_ctx, "DynamicQuantizeLinear");
   if (!call.ok)
     return;

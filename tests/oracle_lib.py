@@ -130,7 +130,7 @@ class Oracle:
     def qlinear_matmul(self, a, a_scale, a_zp, b, b_scale, b_zp, y_scale, y_zp, mode=WRAP):
         a, b = np.ascontiguousarray(a), np.ascontiguousarray(b)
         K, N = b.shape
-        M = a.size // K
+        M = a.size // K if K else int(np.prod(a.shape[:-1]))
         az = np.ascontiguousarray(a_zp, a.dtype).reshape(-1)
         bz = np.ascontiguousarray(b_zp, b.dtype).reshape(-1)
         yz = np.ascontiguousarray(y_zp).reshape(-1)

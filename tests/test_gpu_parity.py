@@ -309,6 +309,49 @@ def test_matmulinteger_small_exhaustive_shapes(rt, oracle, adt, bdt):
                     assert np.array_equal(got, want), (M, K, N, adt, bdt)
 
 
+def test_empty_tensors(rt, oracle):
+    """A dynamic dimension can be 0 at run time: every op then returns an empty
+    result (or, for K = 0, the value of an empty sum) without launching on
+    nothing.  DynamicQuantizeLinear of no elements: min = max = 0 after the
+    widening to include 0, so scale 0 and zero point 0."""
+    rng = np.random.default_rng(5)
+    sc, zp = np.float32(0.1), np.array(3, np.uint8)
+    for shape in ((0,), (0, 7), (5, 0)):
+        x = np.zeros(shape, np.float32)
+        assert rt.QuantizeLinear(x, sc, zp).shape == shape
+        assert rt.DequantizeLinear(np.zeros(shape, np.uint8), sc, zp).shape == shape
+        y, s, z = rt.DynamicQuantizeLinear(x)
+        wy, ws, wz = oracle.dynamic_quantize_linear(x)
+        assert y.shape == shape and same_f32(np.float32(s), np.float32(ws)) and int(z) == int(wz)
+    if True:
+        C = 5
+        scv = rng.uniform(0.01, 0.1, C).astype(np.float32)
+        zpv = rng.integers(0, 256, C).astype(np.uint8)
+        assert rt.QuantizeLinear(np.zeros((0, C), np.float32), scv, zpv, axis=1).shape == (0, C)
+        assert rt.DequantizeLinear(np.zeros((0, C), np.uint8), scv, zpv, axis=1).shape == (0, C)
+    for M, K, N in ((0, 16, 8), (4, 16, 0), (4, 0, 8), (0, 0, 0), (40, 0, 300)):
+        A, B = _rand_q(rng, np.uint8, (M, K)), _rand_q(rng, np.int8, (K, N))
+        az = np.array(9, np.uint8)
+        got = rt.MatMulInteger(A, B, az, None)
+        assert got.shape == (M, N) and got.dtype == np.int32
+        assert np.array_equal(got, oracle.matmul_integer(A, B, az, None)), (M, K, N)
+        bs = rng.uniform(0.001, 0.01, N).astype(np.float32)
+        gf = rt.MatMulIntegerDequant(A, B, az, None, np.float32(0.02), bs)
+        assert gf.shape == (M, N) and not gf.any()
+        Bu = _rand_q(rng, np.uint8, (K, N))
+        gq = rt.QLinearMatMul(A, np.float32(0.01), az, Bu, np.float32(0.005), np.array(120, np.uint8),
+                              np.float32(0.5), np.array(7, np.uint8))
+        wq = oracle.qlinear_matmul(A, np.float32(0.01), az, Bu, np.float32(0.005), np.array(120, np.uint8),
+                                   np.float32(0.5), np.array(7, np.uint8))
+        assert gq.shape == (M, N) and np.array_equal(gq, wq), (M, K, N)
+    x = np.zeros((0, 16), np.float32)
+    B = _rand_q(rng, np.int8, (16, 8))
+    assert rt.DynQuantMatMulDequant(x, B, None, np.float32(0.02)).shape == (0, 8)
+    got = rt.DynQuantMatMulDequant(np.zeros((4, 0), np.float32), _rand_q(rng, np.int8, (0, 8)), None,
+                                   np.float32(0.02))
+    assert got.shape == (4, 8) and not got.any()
+
+
 @pytest.mark.parametrize("M,K,N", [(128, 768, 768), (130, 200, 260), (257, 1000, 129), (64, 4096, 192),
                                    (1, 4096, 1000), (4, 640, 11008), (16, 333, 77), (500, 48, 500)])
 def test_matmulinteger_shapes(rt, oracle, M, K, N):
