@@ -447,34 +447,16 @@ __global__ __launch_bounds__(WGM *WGN * 64, MINB) void k_gemm_i8(
   for (int i = 0; i < TM; ++i)
     rsp[i] = 0;
 
-  auto compute = [&](int buf) {
+  // Operands of half step s (32 of the stage's 64 K bytes) of this wave's tile.
+  auto read_frags = [&](int buf, int s2, v4i(&fa)[TM], v4i(&fb)[TN]) {
+    const int c = s2 * 2 + lh;
 #pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      const int c = s * 2 + lh;
-      v4i fa[TM], fb[TN];
+    for (int i = 0; i < TM; ++i)
+      fa[i] = *(const v4i *)(&sA[buf][lds_off(wm * WTM + i * 32 + l32, c)]);
 #pragma unroll
-      for (int i = 0; i < TM; ++i) {
-        fa[i] = *(const v4i *)(&sA[buf][lds_off(wm * WTM + i * 32 + l32, c)]);
-        // uint8 -> int8 (minus 128) on the operand registers: VALU work that
-        // runs beside the MFMAs and keeps the staging path free of any use
-        // of freshly loaded data.
-        if (A_MODE == 1)
-          fa[i] ^= (v4i){(int)0x80808080, (int)0x80808080, (int)0x80808080,
-              (int)0x80808080};
-        if (need_rs)
-          rsp[i] += frag_rowsum(fa[i]);
-      }
-#pragma unroll
-      for (int j = 0; j < TN; ++j)
-        fb[j] = *(const v4i *)(&sB[buf][(((wn * TN + j) * 2 + s) * 64 + lane) *
-                                        16]);
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
-              fa[i], fb[j], acc[i][j], 0, 0, 0);
-    }
+    for (int j = 0; j < TN; ++j)
+      fb[j] = *(const v4i *)(&sB[buf][(((wn * TN + j) * 2 + s2) * 64 + lane) *
+                                      16]);
   };
 
   // Every load and LDS store below is unconditional (steps past the end are
@@ -491,25 +473,69 @@ __global__ __launch_bounds__(WGM *WGN * 64, MINB) void k_gemm_i8(
   load_global(kclamp(2), ra0, rb0);
   lds_barrier();
 
-  int kt = 0;
-  while (true) {
-    // even step: MFMAs on buffer 0; step kt+1 goes to buffer 1 from set 1,
-    // then set 1 fetches step kt+3.
-    compute(0);
+  // One K step on LDS buffer `buf`: request all operands of the step, put the
+  // next step's tile (already in registers) into the other buffer -- every
+  // wave finished reading that one before the last barrier --, refill those
+  // registers two steps ahead, then run the MFMAs of both half steps.  RS is
+  // whether row sums of A are needed, fixed outside the loop so that the loop
+  // body has no branch.
+  auto k_step = [&](int buf, v4i(&ra)[CH_A], v4i(&rb)[CH_B], int knext,
+                    auto RS) {
+    v4i fa0[TM], fb0[TN], fa1[TM], fb1[TN];
+    read_frags(buf, 0, fa0, fb0);
+    read_frags(buf, 1, fa1, fb1);
     __builtin_amdgcn_sched_barrier(0);
-    store_lds(1, ra1, rb1);
-    load_global(kclamp(kt + 3), ra1, rb1);
-    lds_barrier();
-    if (++kt >= KT)
-      break;
-    compute(1);
+    store_lds(buf ^ 1, ra, rb);
+    load_global(knext, ra, rb);
     __builtin_amdgcn_sched_barrier(0);
-    store_lds(0, ra0, rb0);
-    load_global(kclamp(kt + 3), ra0, rb0);
+    const v4i flip = {(int)0x80808080, (int)0x80808080, (int)0x80808080,
+        (int)0x80808080};
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      // uint8 -> int8 (minus 128) on the operand registers: VALU work that
+      // runs beside the MFMAs
+      if (A_MODE == 1)
+        fa0[i] ^= flip;
+      if (decltype(RS)::value)
+        rsp[i] += frag_rowsum(fa0[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
+            fa0[i], fb0[j], acc[i][j], 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      if (A_MODE == 1)
+        fa1[i] ^= flip;
+      if (decltype(RS)::value)
+        rsp[i] += frag_rowsum(fa1[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
+            fa1[i], fb1[j], acc[i][j], 0, 0, 0);
     lds_barrier();
-    if (++kt >= KT)
-      break;
-  }
+  };
+  auto k_loop = [&](auto RS) {
+    int kt = 0;
+    while (true) {
+      k_step(0, ra1, rb1, kclamp(kt + 3), RS);
+      if (++kt >= KT)
+        break;
+      k_step(1, ra0, rb0, kclamp(kt + 3), RS);
+      if (++kt >= KT)
+        break;
+    }
+  };
+  if (need_rs)
+    k_loop(std::true_type{});
+  else
+    k_loop(std::false_type{});
   gemm_epilogue<TM, TN, A_MODE, EPI>(
       acc, rsp, m0 + wm * WTM, n0 + wn * WTN, M, N, K, ep);
 }
