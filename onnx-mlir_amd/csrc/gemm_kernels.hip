@@ -29,7 +29,7 @@
 //   k_gemm_i8_dma        A and Bp tiles copied from global memory straight
 //                        into a ring of three LDS stages; up to one tile per CU
 //   k_gemm_i8            tiles staged through registers, LDS double buffered;
-//                        the byte-wise path for odd K or a misaligned A
+//                        also the general path: any K, any alignment of A
 //   k_gemm_i8_skinny_bp  M <= 32: weight streaming, K split over the waves
 // A tiles in LDS have 64-byte rows whose 16-byte chunk index is XOR-swizzled
 // with bits 2..3 of the row (bank-conflict free writes and operand reads); Bp
@@ -46,6 +46,8 @@ namespace om {
 namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v4i_any __attribute__((ext_vector_type(4), aligned(1)));
+enum : int { kLoadBytes = 0, kLoadAligned = 1, kLoadAny = 2 };
 typedef int v16i __attribute__((ext_vector_type(16)));
 
 constexpr int BK = kGemmBK;
@@ -324,9 +326,12 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TM][TN],
 // made of 32x32 MFMA tiles.
 // A_MODE: 0 = int8 as is, 1 = uint8 (XOR 0x80 while staging), 2 = already
 // shifted (stored as u8-128) -- offsets as for uint8, no XOR.
-// ALIGNED: K % 64 == 0 and A 16-byte aligned (vector loads), else byte loads.
+// A_LOAD: kLoadAligned = K % 64 == 0 and A 16-byte aligned (plain vector
+// loads); kLoadAny = any K and alignment, at least 16 bytes of A (16-byte
+// loads at byte addresses, the bytes past the end of a row replaced); kLoadBytes
+// = byte loads (an A of fewer than 16 bytes, K = 0).
 template <int BM, int BN, int WGM, int WGN, int MINB, int A_MODE, int EPI,
-    bool ALIGNED>
+    int A_LOAD>
 __global__ __launch_bounds__(WGM *WGN * 64, MINB) void k_gemm_i8(
     const uint8_t *__restrict__ A, const int8_t *__restrict__ Bp, int M, int N,
     int K, int Kpad, EpiParams ep, int tiles_m, int tiles_n) {
@@ -372,7 +377,7 @@ __global__ __launch_bounds__(WGM *WGN * 64, MINB) void k_gemm_i8(
   const int KTs = Kpad / BK; // K steps: stride between column tiles of Bp
 
   // Global loads only fetch; uint8 data is shifted to int8 after it is read
-  // back from LDS.  In the byte-wise path chunks outside [M,K] are filled with
+  // back from LDS.  In the general paths bytes outside [M,K] are replaced by
   // the byte that the shift maps to 0.
   auto load_global = [&](int k0, v4i(&ra)[CH_A], v4i(&rb)[CH_B]) {
 #pragma unroll
@@ -382,7 +387,7 @@ __global__ __launch_bounds__(WGM *WGN * 64, MINB) void k_gemm_i8(
       const int gm = m0 + r;
       const int gk = k0 + c * 16;
       v4i v = {kFill, kFill, kFill, kFill};
-      if (ALIGNED) {
+      if (A_LOAD == kLoadAligned) {
         // K % 64 == 0, so every chunk lies inside its row.  Rows past M are
         // clamped to the last row: they only feed output rows that are never
         // stored, and an unconditional load lets the hardware counter of
@@ -390,6 +395,41 @@ __global__ __launch_bounds__(WGM *WGN * 64, MINB) void k_gemm_i8(
         // would force a full drain).
         const int gmc = gm < M ? gm : M - 1;
         v = *(const v4i *)(A + (int64_t)gmc * K + gk);
+      } else if (A_LOAD == kLoadAny) {
+        // One 16-byte load per chunk at whatever address the chunk has.  The
+        // chunk at the end of a row holds K - gk < 16 of its bytes; the rest
+        // (the next row's, or nothing: the load is moved back to end with the
+        // buffer and its bytes shifted down) become the fill byte.  Chunks
+        // outside [M, K] load the first 16 bytes and keep none of them.
+        const bool valid = gm < M && gk < K;
+        const int64_t total = (int64_t)M * K;
+        const int64_t off = valid ? (int64_t)gm * K + gk : 0;
+        const int len = valid ? (K - gk < 16 ? K - gk : 16) : 0;
+        const int64_t off2 = off + 16 <= total ? off : total - 16;
+        const int sh = (int)(off - off2) * 8; // bits to shift down, < 128
+        const v4i_any raw = *(const v4i_any *)(A + off2);
+        uint64_t lo = (uint32_t)raw.x | ((uint64_t)(uint32_t)raw.y << 32);
+        uint64_t hi = (uint32_t)raw.z | ((uint64_t)(uint32_t)raw.w << 32);
+        if (sh >= 64) {
+          lo = hi;
+          hi = 0;
+        }
+        const int s1 = sh & 63;
+        if (s1) {
+          lo = (lo >> s1) | (hi << (64 - s1));
+          hi >>= s1;
+        }
+        const uint64_t fill64 =
+            (uint32_t)kFill | ((uint64_t)(uint32_t)kFill << 32);
+        const uint64_t mlo =
+            len >= 8 ? ~(uint64_t)0 : (((uint64_t)1 << (8 * len)) - 1);
+        const uint64_t mhi =
+            len >= 16 ? ~(uint64_t)0
+                      : (len > 8 ? (((uint64_t)1 << (8 * (len - 8))) - 1) : 0);
+        lo = (lo & mlo) | (fill64 & ~mlo);
+        hi = (hi & mhi) | (fill64 & ~mhi);
+        v = (v4i){(int)(uint32_t)lo, (int)(uint32_t)(lo >> 32),
+            (int)(uint32_t)hi, (int)(uint32_t)(hi >> 32)};
       } else {
         uint32_t w[4] = {0, 0, 0, 0};
 #pragma unroll
@@ -1275,14 +1315,14 @@ __global__ __launch_bounds__(256) void k_pack_b(const uint8_t *__restrict__ B,
 
 // Kernel / tile configurations.
 enum TileCfg : int {
-  kT128x128 = 0, // k_gemm_i8: register-staged tiles (and the byte-wise path)
+  kT128x128 = 0, // k_gemm_i8: register-staged tiles (and the general path)
   kD128x128 = 1, // k_gemm_i8_dma: tiles copied straight into LDS
   kB128x256 = 2, // k_gemm_i8_bs: Bp straight into registers
   kNumCfg = 3
 };
 
 // Kernel choice for problems with more than 32 rows, K % 64 == 0 and a
-// 16-byte aligned A (anything else takes the byte-wise path of k_gemm_i8).
+// 16-byte aligned A (anything else takes the general path of k_gemm_i8).
 // Measured on MI355X over the BERT-base and Llama-7B layer shapes and square
 // problems up to 8192: a 128 x 256 tile of k_gemm_i8_bs costs about 1.7 times
 // a 128 x 128 tile of k_gemm_i8_dma, so it wins when it needs at most half as
@@ -1305,7 +1345,7 @@ int choose_tile(int64_t M, int64_t N) {
 }
 
 bool gemm_fast_path(int64_t M, int64_t K, const void *A) {
-  // K == 0 (an empty sum) has no bytes of A to read: only the byte-wise path
+  // K == 0 (an empty sum) has no bytes of A to read: only the general path
   // checks every address against K.
   return M > 16 && K > 0 && K % 64 == 0 && ((((uintptr_t)A) & 15) == 0);
 }
@@ -1326,11 +1366,16 @@ hipError_t gemm_launch_cfg(
   const int tiles_m = (int)((g.M + 127) / 128);
   const int tiles_n128 = (int)((g.N + 127) / 128);
   if (!gemm_fast_path(g.M, g.K, g.A)) {
-    // Byte-wise staging of A for odd K or a misaligned A (and the forced
-    // configurations of the tests when M <= 16).
-    k_gemm_i8<128, 128, 2, 2, 2, A_MODE, EPI, false>
-        <<<dim3((unsigned)(tiles_m * tiles_n128)), 256, 0, st>>>(
-            A, g.Bp, M, N, K, Kpad, ep, tiles_m, tiles_n128);
+    // Any K, any alignment of A (and the forced configurations of the tests
+    // when M <= 16); byte loads only for an A of fewer than 16 bytes.
+    if (g.M * g.K >= 16)
+      k_gemm_i8<128, 128, 2, 2, 2, A_MODE, EPI, kLoadAny>
+          <<<dim3((unsigned)(tiles_m * tiles_n128)), 256, 0, st>>>(
+              A, g.Bp, M, N, K, Kpad, ep, tiles_m, tiles_n128);
+    else
+      k_gemm_i8<128, 128, 2, 2, 2, A_MODE, EPI, kLoadBytes>
+          <<<dim3((unsigned)(tiles_m * tiles_n128)), 256, 0, st>>>(
+              A, g.Bp, M, N, K, Kpad, ep, tiles_m, tiles_n128);
     return hipGetLastError();
   }
   switch (choose_tile(g.M, g.N)) {
@@ -1347,7 +1392,7 @@ hipError_t gemm_launch_cfg(
             A, g.Bp, M, N, K, Kpad, ep, tiles_m, tiles_n128);
     break;
   default:
-    k_gemm_i8<128, 128, 2, 2, 3, A_MODE, EPI, true>
+    k_gemm_i8<128, 128, 2, 2, 3, A_MODE, EPI, kLoadAligned>
         <<<dim3((unsigned)(tiles_m * tiles_n128)), 256, 0, st>>>(
             A, g.Bp, M, N, K, Kpad, ep, tiles_m, tiles_n128);
     break;
