@@ -65,7 +65,7 @@ def gemm_case(rt, wl, name, M, K, N, w_i8, w_scale, steps, warmup, epilogue="f32
     rt.mark_constant(dW)             # weights: packed once, like any model constant
     if epilogue == "f32":
         dY = rt.DeviceArray((M, N), np.float32)
-        fn = rt.PreparedCall("om_mi355x_MatMulIntegerDequant", dY, dA, dW, dAz, None, dAs, dS)
+        fn = rt.PreparedCall("om_mi355x_MatMulIntegerDequant", dY, dA, dW, dAz, None, dAs, dS, None)
     else:
         dY = rt.DeviceArray((M, N), np.int32)
         fn = rt.PreparedCall("om_mi355x_MatMulInteger", dY, dA, dW, dAz, None)
@@ -99,7 +99,7 @@ def spread_case(rt, wl, M, K, N, w_i8, w_scale, steps, warmup, sets=6, chunks=20
         dA = rt.DeviceArray.from_numpy(rng.integers(0, 256, (M, K), dtype=np.uint8))
         dY = rt.DeviceArray((M, N), np.float32)
         bufs += [dA, dY]
-        calls.append(rt.PreparedCall("om_mi355x_MatMulIntegerDequant", dY, dA, dW, dAz, None, dAs, dS))
+        calls.append(rt.PreparedCall("om_mi355x_MatMulIntegerDequant", dY, dA, dW, dAz, None, dAs, dS, None))
     per = max(1, steps // chunks)
     times = []
     for i in range(chunks + 2):
@@ -133,7 +133,7 @@ def decode_case(rt, wl, M, steps, warmup):
     dS = rt.DeviceArray.from_numpy(c["w_scale"])
     dY = rt.DeviceArray((M, N), np.float32)
     rt.mark_constant(dW)
-    fn = rt.PreparedCall("om_mi355x_DynQuantMatMulDequant", dY, dX, dW, None, dS)
+    fn = rt.PreparedCall("om_mi355x_DynQuantMatMulDequant", dY, dX, dW, None, dS, None)
     host_s, ev_ms = timed(rt, fn, steps, warmup)
     fn.check()
     fn.close()
@@ -180,7 +180,7 @@ def fused_case(rt, wl, name, M, K, N, w_i8, w_scale, steps, warmup):
     dS = rt.DeviceArray.from_numpy(w_scale)
     dY = rt.DeviceArray((M, N), np.float32)
     rt.mark_constant(dW)
-    fn = rt.PreparedCall("om_mi355x_DynQuantMatMulDequant", dY, dX, dW, None, dS)
+    fn = rt.PreparedCall("om_mi355x_DynQuantMatMulDequant", dY, dX, dW, None, dS, None)
     host_s, ev_ms = timed(rt, fn, steps, warmup)
     fn.check()
     fn.close()

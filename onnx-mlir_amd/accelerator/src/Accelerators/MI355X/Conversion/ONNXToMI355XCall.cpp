@@ -267,8 +267,9 @@ struct QLinearMatMulToMI355X
 //===----------------------------------------------------------------------===//
 // onnx.Custom created by the fusion pass.
 //   void om_mi355x_MatMulIntegerDequant(y, a, b, a_zp|NULL, b_zp|NULL,
-//                                       a_scale, b_scale)
-//   void om_mi355x_DynQuantMatMulDequant(y, x, b, b_zp|NULL, b_scale)
+//                                       a_scale, b_scale, bias|NULL)
+//   void om_mi355x_DynQuantMatMulDequant(y, x, b, b_zp|NULL, b_scale,
+//                                        bias|NULL)
 // In both, input 0 is [.., M, K] and input 1 is [K, N]; the result is
 // [.., M, N].  onnx.Custom has no shape rule for that, so the dimensions are
 // taken from the operands here.
@@ -303,7 +304,10 @@ struct FusedMatMulToMI355X : public OpConversionPattern<ONNXCustomOp> {
     dims.back() = create.krnlIE.getShapeAsDim(inputs[1], 1);
     Value y = create.mem.alignedAlloc(yType, dims);
 
-    markIfConstant(rewriter, loc, inputs[1]);
+    // Weights, and whichever of zero point, scales and bias are constants:
+    // uploaded once instead of with every call.
+    for (size_t i = 1; i < inputs.size(); ++i)
+      markIfConstant(rewriter, loc, inputs[i]);
     emitCall(rewriter, loc, callee, {y}, inputs);
     rewriter.replaceOp(op, y);
     return success();

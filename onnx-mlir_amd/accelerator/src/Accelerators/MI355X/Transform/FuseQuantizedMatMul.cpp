@@ -11,11 +11,14 @@
 //   %f             = Cast(%acc) {to = f32}
 //   %s             = Mul(%as, %ws)
 //   %y             = Mul(%f, %s)
+//   %z             = Add(%y, %bias)          (optional)
 //
-// On the CPU that is five ops and four intermediate tensors.  The MI355X
-// runtime has one entry point for the last four (the int32 accumulator never
-// reaches memory) and one for all five (the 8-bit activation stays on the
-// device).  This pass replaces the chain by an `onnx.Custom` naming that entry
+// On the CPU that is five or six ops and as many intermediate tensors.  The
+// MI355X runtime has one entry point for everything after the quantisation
+// (the int32 accumulator never reaches memory) and one for the whole chain
+// (the 8-bit activation stays on the device).  A bias that is added to the
+// scaled result -- one value, or one per column -- goes along: the kernel
+// rounds the product to f32 and then adds, as Mul followed by Add does.  This pass replaces the chain by an `onnx.Custom` naming that entry
 // point; the ONNX-to-Krnl patterns of the accelerator lower it.
 //
 // Only the association `f32(acc) * (a_scale * b_scale)` is matched.  The other
@@ -131,18 +134,37 @@ struct FuseScaledMatMulInteger : public OpRewritePattern<ONNXMulOp> {
         chain.aScale == dynQuant.getYScale() && dynQuant.getY().hasOneUse() &&
         dynQuant.getYScale().hasOneUse() && dynQuant.getYZeroPoint().hasOneUse();
 
-    SmallVector<Value, 6> inputs;
+    // A bias added to the scaled result (its only user) is taken along.
+    Operation *root = mul;
+    Value bias;
+    if (mul->hasOneUse()) {
+      if (auto add = dyn_cast<ONNXAddOp>(*mul->user_begin())) {
+        Value other = add.getA() == mul.getResult() ? add.getB() : add.getA();
+        bool shaped =
+            isF32Tensor(other) &&
+            (isSingleElement(other) || isColumnScale(other, matmul.getB())) &&
+            add.getResult().getType() == mul.getResult().getType();
+        if (shaped && other != mul.getResult()) {
+          root = add;
+          bias = other;
+        }
+      }
+    }
+    rewriter.setInsertionPoint(root);
+
+    SmallVector<Value, 8> inputs;
     StringRef callee;
     if (wholeLayer) {
       callee = kMI355XDynQuantMatMulDequant;
       inputs = {dynQuant.getX(), matmul.getB(),
-          noneIfAbsent(rewriter, loc, matmul.getBZeroPoint()), chain.bScale};
+          noneIfAbsent(rewriter, loc, matmul.getBZeroPoint()), chain.bScale,
+          noneIfAbsent(rewriter, loc, bias)};
     } else {
       callee = kMI355XMatMulIntegerDequant;
       inputs = {matmul.getA(), matmul.getB(),
           noneIfAbsent(rewriter, loc, matmul.getAZeroPoint()),
           noneIfAbsent(rewriter, loc, matmul.getBZeroPoint()), chain.aScale,
-          chain.bScale};
+          chain.bScale, noneIfAbsent(rewriter, loc, bias)};
     }
 
     SmallVector<NamedAttribute, 2> attrs;
@@ -151,10 +173,11 @@ struct FuseScaledMatMulInteger : public OpRewritePattern<ONNXMulOp> {
     if (Attribute nodeName = mul->getAttr("onnx_node_name"))
       attrs.emplace_back(rewriter.getNamedAttr("onnx_node_name", nodeName));
     auto fused = ONNXCustomOp::create(rewriter, loc,
-        TypeRange{mul.getResult().getType()}, ValueRange(inputs), attrs);
-    rewriter.replaceOp(mul, fused.getResults());
-    // Cast, MatMulInteger, the scale product and (for the whole layer)
-    // DynamicQuantizeLinear are now dead and pure: the driver erases them.
+        TypeRange{root->getResult(0).getType()}, ValueRange(inputs), attrs);
+    rewriter.replaceOp(root, fused.getResults());
+    // Mul (when the Add was the root), Cast, MatMulInteger, the scale product
+    // and (for the whole layer) DynamicQuantizeLinear are now dead and pure:
+    // the driver erases them.
     return success();
   }
 };

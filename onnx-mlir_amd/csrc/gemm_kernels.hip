@@ -77,6 +77,8 @@ struct EpiParams {
   int64_t b_scale_len;
   const float *y_scale;
   const void *y_zp;
+  const float *bias;     // kEpiF32: added after the scaling; null = none
+  int64_t bias_len;      // 1 or N
   void *out;
   bool b_unsigned;
   bool y_unsigned;
@@ -111,13 +113,15 @@ __device__ __forceinline__ int32_t frag_rowsum(v4i f) {
 // unconditional (indices clamped, absent operands redirected to valid memory
 // and masked afterwards) and all loads precede the stores, so the stores can
 // be issued back to back without waiting on one another.
+// bj: the bias of the column, or -0.0f, which leaves every value (both zeros
+// included) as it is.
 template <int EPI>
 __device__ __forceinline__ void store_one(const EpiParams &ep, int64_t o,
-    uint32_t y, float sj, int32_t yz) {
+    uint32_t y, float sj, int32_t yz, float bj) {
   if (EPI == kEpiI32) {
     ((int32_t *)ep.out)[o] = (int32_t)y;
   } else if (EPI == kEpiF32) {
-    ((float *)ep.out)[o] = (float)(int32_t)y * sj;
+    ((float *)ep.out)[o] = (float)(int32_t)y * sj + bj;
   } else {
     const float f = (float)(int32_t)y * sj;
     const int32_t q = (int32_t)__builtin_rintf(f);
@@ -169,11 +173,16 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TM][TN],
 
   int n_[TN];
   int32_t db[TN], cs[TN];
-  float sj[TN];
+  float sj[TN], bj[TN];
+  const bool has_bias = EPI == kEpiF32 && ep.bias != nullptr;
+  const float *bias_ptr = has_bias ? ep.bias : (const float *)ep.colsum;
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
     n_[j] = ncol0 + j * 32 + l32;
     const int nc = n_[j] < N ? n_[j] : N - 1;
+    // the product is rounded before the bias is added, as Mul then Add are
+    const float bv = bias_ptr[has_bias && ep.bias_len > 1 ? nc : 0];
+    bj[j] = has_bias ? bv : -0.0f;
     const int32_t bz =
         load_zp_i32(bzp_ptr, B_UNSIGNED, ep.b_zp_len > 1 ? nc : 0);
     db[j] = ob - (has_bzp ? bz : 0);
@@ -226,7 +235,8 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TM][TN],
       if (EPI == kEpiI32) {
         __builtin_nontemporal_store((int32_t)y, (int32_t *)q);
       } else if (EPI == kEpiF32) {
-        __builtin_nontemporal_store((float)(int32_t)y * sj[j], (float *)q);
+        __builtin_nontemporal_store(
+            (float)(int32_t)y * sj[j] + bj[j], (float *)q);
       } else {
         const float f = (float)(int32_t)y * sj[j];
         int32_t v =
@@ -279,7 +289,7 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TM][TN],
           const uint32_t y = (uint32_t)acc[i][j][r] + cj[j] +
                              (uint32_t)db[j] * (uint32_t)rs_row;
           if (m < M && n_[j] < N)
-            store_one<EPI>(ep, orow + n_[j], y, sj[j], yz);
+            store_one<EPI>(ep, orow + n_[j], y, sj[j], yz, bj[j]);
         }
       }
     }
@@ -314,7 +324,7 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TM][TN],
           y += (uint32_t)db[j] * (uint32_t)rs[rr];
           y += (uint32_t)K * (uint32_t)da[rr] * (uint32_t)db[j];
           if (m < M && n_[j] < N)
-            store_one<EPI>(ep, orow + n_[j], y, sj[j], yz);
+            store_one<EPI>(ep, orow + n_[j], y, sj[j], yz, bj[j]);
         }
       }
     }
@@ -1218,8 +1228,10 @@ __global__ __launch_bounds__(512) void k_gemm_i8_skinny_bp(
   if (ep.b_zp_len > 0)
     db = ob - load_zp_i32(ep.b_zp, ep.b_unsigned, ep.b_zp_len > 1 ? n : 0);
   const int32_t cs = ep.colsum[n];
-  float sj = 0.0f;
+  float sj = 0.0f, bj = -0.0f;
   int32_t yz = 0;
+  if (EPI == kEpiF32 && ep.bias != nullptr)
+    bj = ep.bias[ep.bias_len > 1 ? n : 0];
   if (EPI != kEpiI32) {
     sj = ep.a_scale[0] * ep.b_scale[ep.b_scale_len == 1 ? 0 : n];
     if (EPI == kEpiQ8) {
@@ -1248,7 +1260,7 @@ __global__ __launch_bounds__(512) void k_gemm_i8_skinny_bp(
     y += (uint32_t)da * (uint32_t)cs;
     y += (uint32_t)db * (uint32_t)rs;
     y += (uint32_t)K * (uint32_t)da * (uint32_t)db;
-    store_one<EPI>(ep, (int64_t)m * N + n, y, sj, yz);
+    store_one<EPI>(ep, (int64_t)m * N + n, y, sj, yz, bj);
   }
 }
 
@@ -1454,6 +1466,8 @@ hipError_t launch_gemm(hipStream_t s, const GemmArgs &g) {
   ep.b_scale_len = g.b_scale_len;
   ep.y_scale = g.y_scale;
   ep.y_zp = g.y_zp;
+  ep.bias = g.epi == kEpiF32 ? g.bias : nullptr;
+  ep.bias_len = g.bias_len;
   ep.out = g.out;
   ep.b_unsigned = g.b_unsigned;
   ep.y_unsigned = g.y_unsigned;

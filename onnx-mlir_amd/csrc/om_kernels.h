@@ -71,7 +71,7 @@ struct GemmArgs {
   int64_t b_zp_len;    // 0, 1 or N
   const int32_t *colsum; // sum_k B' per column (Npad entries)
   Epilogue epi;
-  // kEpiF32: out = f32(acc) * (a_scale[0] * b_scale[j or 0])
+  // kEpiF32: out = f32(acc) * (a_scale[0] * b_scale[j or 0]) [+ bias[j or 0]]
   // kEpiQ8 : s = (a_scale[0]*b_scale[0]) / y_scale[0];
   //          out = narrow(i32(rne(f32(acc) * s)) + y_zp)
   const float *a_scale;
@@ -79,6 +79,8 @@ struct GemmArgs {
   int64_t b_scale_len; // 1 or N
   const float *y_scale;
   const void *y_zp;
+  const float *bias;   // kEpiF32 only; may be null
+  int64_t bias_len;    // 1 or N
   bool y_unsigned;
   NarrowMode narrow;
   void *out;           // i32 / f32 / u8|i8 [M,N]

@@ -739,12 +739,25 @@ struct MatmulSpec {
   Epilogue epi;
   const OMTensor *y, *a, *b, *a_zp, *b_zp;
   const OMTensor *a_scale = nullptr, *b_scale = nullptr, *y_scale = nullptr,
-                 *y_zp = nullptr;
+                 *y_zp = nullptr, *bias = nullptr;
   NarrowMode narrow = kWrap;
 };
 
+// Optional bias of the f32 epilogue: f32, one value or one per column.
+bool bias_ok(const OMTensor *bias_t, int64_t N, const char *op, View &bias) {
+  if (!bias_t)
+    return true;
+  if (!view_of(bias_t, "bias", bias))
+    return false;
+  if (bias.dtype != OM_MI355X_TYPE_FLOAT || (bias.numel != 1 && bias.numel != N)) {
+    fail(EINVAL, "%s: bias must be f32, scalar or [N]", op);
+    return false;
+  }
+  return true;
+}
+
 void run_matmul(const MatmulSpec &sp) {
-  View y, a, b, azp, bzp, as, bs, ys, yzp;
+  View y, a, b, azp, bzp, as, bs, ys, yzp, bias;
   if (!view_of(sp.y, "y", y) || !view_of(sp.a, "a", a) ||
       !view_of(sp.b, "b", b))
     return;
@@ -790,6 +803,8 @@ void run_matmul(const MatmulSpec &sp) {
       return;
     }
   }
+  if (!bias_ok(sp.bias, N, sp.op, bias))
+    return;
   if (sp.epi == kEpiQ8) {
     if (!view_of(sp.y_scale, "y_scale", ys) ||
         !view_of(sp.y_zp, "y_zero_point", yzp))
@@ -832,6 +847,10 @@ void run_matmul(const MatmulSpec &sp) {
     g.a_scale = (const float *)call.in(as);
     g.b_scale = (const float *)call.in(bs);
     g.b_scale_len = bs.numel;
+  }
+  if (sp.bias) {
+    g.bias = (const float *)call.in(bias);
+    g.bias_len = bias.numel;
   }
   if (sp.epi == kEpiQ8) {
     g.y_scale = (const float *)call.in(ys);
@@ -1015,10 +1034,11 @@ void om_mi355x_MatMulInteger(OMTensor *y, const OMTensor *a,
 
 void om_mi355x_MatMulIntegerDequant(OMTensor *y, const OMTensor *a,
     const OMTensor *b, const OMTensor *a_zp, const OMTensor *b_zp,
-    const OMTensor *a_scale, const OMTensor *b_scale) {
+    const OMTensor *a_scale, const OMTensor *b_scale, const OMTensor *bias) {
   MatmulSpec sp = {"MatMulIntegerDequant", kEpiF32, y, a, b, a_zp, b_zp};
   sp.a_scale = a_scale;
   sp.b_scale = b_scale;
+  sp.bias = bias;
   run_matmul(sp);
 }
 
@@ -1040,9 +1060,10 @@ void om_mi355x_QLinearMatMul(OMTensor *y, const OMTensor *a,
 }
 
 void om_mi355x_DynQuantMatMulDequant(OMTensor *y_t, const OMTensor *x_t,
-    const OMTensor *b_t, const OMTensor *bzp_t, const OMTensor *bscale_t) {
+    const OMTensor *b_t, const OMTensor *bzp_t, const OMTensor *bscale_t,
+    const OMTensor *bias_t) {
   const char *op = "DynQuantMatMulDequant";
-  View y, x, b, bzp, bs;
+  View y, x, b, bzp, bs, bias;
   if (!view_of(y_t, "y", y) || !view_of(x_t, "x", x) ||
       !view_of(b_t, "b", b) || !view_of(bscale_t, "b_scale", bs))
     return;
@@ -1064,6 +1085,8 @@ void om_mi355x_DynQuantMatMulDequant(OMTensor *y_t, const OMTensor *x_t,
     fail(EINVAL, "%s: output or b_scale shape is wrong", op);
     return;
   }
+  if (!bias_ok(bias_t, N, op, bias))
+    return;
   if (M == 0 || N == 0)
     return;
   Call call(t_ctx, "DynQuantMatMulDequant");
@@ -1100,6 +1123,10 @@ void om_mi355x_DynQuantMatMulDequant(OMTensor *y_t, const OMTensor *x_t,
   g.a_scale = call.c.dql_scale;
   g.b_scale = (const float *)call.in(bs);
   g.b_scale_len = bs.numel;
+  if (bias_t) {
+    g.bias = (const float *)call.in(bias);
+    g.bias_len = bias.numel;
+  }
   g.out = call.out(y);
   if (call.ok)
     call.check(launch_gemm(call.c.stream, g), op);

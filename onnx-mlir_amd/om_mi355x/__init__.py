@@ -81,9 +81,9 @@ def _declare(lib, shim):
         "om_mi355x_DequantizeLinear": [P, P, P, P, I64],
         "om_mi355x_DynamicQuantizeLinear": [P, P, P, P],
         "om_mi355x_MatMulInteger": [P, P, P, P, P],
-        "om_mi355x_MatMulIntegerDequant": [P, P, P, P, P, P, P],
+        "om_mi355x_MatMulIntegerDequant": [P, P, P, P, P, P, P, P],
         "om_mi355x_QLinearMatMul": [P, P, P, P, P, P, P, P, P, I64],
-        "om_mi355x_DynQuantMatMulDequant": [P, P, P, P, P],
+        "om_mi355x_DynQuantMatMulDequant": [P, P, P, P, P, P],
         "om_mi355x_MarkConstant": [P],
         "om_mi355x_KeepOnDevice": [P],
         "om_mi355x_Release": [P],
@@ -351,16 +351,17 @@ def MatMulInteger(a: Tensor, b: Tensor, a_zero_point: Optional[Tensor] = None,
 
 def MatMulIntegerDequant(a: Tensor, b: Tensor, a_zero_point: Optional[Tensor],
                          b_zero_point: Optional[Tensor], a_scale: Tensor, b_scale: Tensor,
-                         out: Optional[Tensor] = None) -> Tensor:
+                         bias: Optional[Tensor] = None, out: Optional[Tensor] = None) -> Tensor:
     load()
     a, b = _host(a), _host(b)
     a_scale, b_scale = _host(a_scale, np.float32), _host(b_scale, np.float32)
     az = None if a_zero_point is None else _host(a_zero_point)
     bz = None if b_zero_point is None else _host(b_zero_point)
+    bias = None if bias is None else _host(bias, np.float32)
     y = out if out is not None else _like(a, _mm_shape(a, b), np.float32)
     with _OMT(y) as hy, _OMT(a) as ha, _OMT(b) as hb, _OMT(az) as haz, _OMT(bz) as hbz, \
-            _OMT(a_scale) as has, _OMT(b_scale) as hbs:
-        _lib.om_mi355x_MatMulIntegerDequant(hy, ha, hb, haz, hbz, has, hbs)
+            _OMT(a_scale) as has, _OMT(b_scale) as hbs, _OMT(bias) as hbias:
+        _lib.om_mi355x_MatMulIntegerDequant(hy, ha, hb, haz, hbz, has, hbs, hbias)
     _check()
     return y
 
@@ -384,13 +385,16 @@ def QLinearMatMul(a: Tensor, a_scale: Tensor, a_zero_point: Tensor, b: Tensor,
 
 
 def DynQuantMatMulDequant(x: Tensor, b: Tensor, b_zero_point: Optional[Tensor],
-                          b_scale: Tensor, out: Optional[Tensor] = None) -> Tensor:
+                          b_scale: Tensor, bias: Optional[Tensor] = None,
+                          out: Optional[Tensor] = None) -> Tensor:
     load()
     x, b, b_scale = _host(x), _host(b), _host(b_scale, np.float32)
     bz = None if b_zero_point is None else _host(b_zero_point)
+    bias = None if bias is None else _host(bias, np.float32)
     y = out if out is not None else _like(x, _mm_shape(x, b), np.float32)
-    with _OMT(y) as hy, _OMT(x) as hx, _OMT(b) as hb, _OMT(bz) as hbz, _OMT(b_scale) as hbs:
-        _lib.om_mi355x_DynQuantMatMulDequant(hy, hx, hb, hbz, hbs)
+    with _OMT(y) as hy, _OMT(x) as hx, _OMT(b) as hb, _OMT(bz) as hbz, _OMT(b_scale) as hbs, \
+            _OMT(bias) as hbias:
+        _lib.om_mi355x_DynQuantMatMulDequant(hy, hx, hb, hbz, hbs, hbias)
     _check()
     return y
 

@@ -156,8 +156,8 @@ def test_compiler_plugin_calls_only_exported_symbols(rt):
     # parameter counts: results + operands + integer attributes of each pattern
     passed = {"om_mi355x_QuantizeLinear": 1 + 3 + 2, "om_mi355x_DequantizeLinear": 1 + 3 + 1,
               "om_mi355x_DynamicQuantizeLinear": 3 + 1, "om_mi355x_MatMulInteger": 1 + 4,
-              "om_mi355x_QLinearMatMul": 1 + 8 + 1, "om_mi355x_MatMulIntegerDequant": 1 + 6,
-              "om_mi355x_DynQuantMatMulDequant": 1 + 4, "om_mi355x_MarkConstant": 1,
+              "om_mi355x_QLinearMatMul": 1 + 8 + 1, "om_mi355x_MatMulIntegerDequant": 1 + 7,
+              "om_mi355x_DynQuantMatMulDequant": 1 + 5, "om_mi355x_MarkConstant": 1,
               "om_mi355x_KeepOnDevice": 1, "om_mi355x_Release": 1}
     for name, count in passed.items():
         m = re.search(r"\b%s\s*\(([^)]*)\)" % name, header)

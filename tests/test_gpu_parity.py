@@ -309,6 +309,35 @@ def test_matmulinteger_small_exhaustive_shapes(rt, oracle, adt, bdt):
                     assert np.array_equal(got, want), (M, K, N, adt, bdt)
 
 
+@pytest.mark.parametrize("M,K,N", [(4, 256, 200), (40, 100, 33), (300, 128, 260), (2048, 1024, 512)])
+def test_fused_epilogue_with_bias(rt, oracle, M, K, N):
+    """Linear layers carry a bias: MatMulInteger -> Cast -> Mul(a_scale * b_scale) -> Add(bias).
+    The product is rounded to f32 first and the bias added to it, as the two
+    ONNX ops would; a bias of one element is broadcast; -0.0 results survive a
+    missing bias and a +0.0 bias alike as IEEE addition says."""
+    rng = np.random.default_rng(M + 3 * N)
+    A, B = _rand_q(rng, np.uint8, (M, K)), _rand_q(rng, np.int8, (K, N))
+    az = _rand_q(rng, np.uint8, ())
+    a_s = np.float32(0.0173)
+    bs = rng.uniform(1e-3, 1e-2, N).astype(np.float32)
+    bs[::7] *= np.float32(-1.0)          # negative scales: products of accumulator 0 are -0.0
+    acc = oracle.matmul_integer(A, B, az, None)
+    prod = oracle.dequant_epilogue(acc, a_s, bs)
+    for bias in (rng.normal(0, 3, N).astype(np.float32), np.array([1.5], np.float32),
+                 np.zeros(N, np.float32)):
+        got = rt.MatMulIntegerDequant(A, B, az, None, a_s, bs, bias)
+        assert same_f32(got, prod + bias), bias.shape
+    assert same_f32(rt.MatMulIntegerDequant(A, B, az, None, a_s, bs), prod)
+    # whole layer
+    x = rng.normal(0, 1, (M, K)).astype(np.float32)
+    xq, xs, xz = oracle.dynamic_quantize_linear(x)
+    want = oracle.dequant_epilogue(oracle.matmul_integer(xq, B, xz, None), xs, bs)
+    bias = rng.normal(0, 3, N).astype(np.float32)
+    assert same_f32(rt.DynQuantMatMulDequant(x, B, None, bs, bias), want + bias)
+    with pytest.raises(rt.RuntimeError_):
+        rt.MatMulIntegerDequant(A, B, az, None, a_s, bs, np.zeros(N + 1, np.float32))
+
+
 def test_empty_tensors(rt, oracle):
     """A dynamic dimension can be 0 at run time: every op then returns an empty
     result (or, for K = 0, the value of an empty sum) without launching on
