@@ -83,8 +83,6 @@ struct EpiParams {
   bool b_unsigned;
   bool y_unsigned;
   int narrow;
-  int group;   // tile rows per scheduling group
-  int xcd;     // renumber workgroups per XCD
 };
 
 __device__ __forceinline__ int32_t load_zp_i32(
@@ -1472,8 +1470,6 @@ hipError_t launch_gemm(hipStream_t s, const GemmArgs &g) {
   ep.b_unsigned = g.b_unsigned;
   ep.y_unsigned = g.y_unsigned;
   ep.narrow = (int)g.narrow;
-  ep.group = 8;
-  ep.xcd = 1;
   const int a_mode = g.a_preshifted ? 2 : (g.a_unsigned ? 1 : 0);
   switch (a_mode) {
   case 0:

@@ -377,8 +377,20 @@ bool view_of(const OMTensor *t, const char *name, View &v) {
   v.shape = omTensorGetShape(t);
   const int64_t *strides = omTensorGetStrides(t);
   v.numel = 1;
-  for (int64_t i = 0; i < v.rank; ++i)
+  if (v.rank < 0 || (v.rank > 0 && (!v.shape || !strides))) {
+    fail(EINVAL, "%s: tensor has no shape", name);
+    return false;
+  }
+  for (int64_t i = 0; i < v.rank; ++i) {
+    // a dimension that was never resolved (-1) or a product beyond 2^62
+    if (v.shape[i] < 0 ||
+        (v.shape[i] > 0 && v.numel > ((int64_t)1 << 62) / v.shape[i])) {
+      fail(EINVAL, "%s: dimension %lld is %lld", name, (long long)i,
+          (long long)v.shape[i]);
+      return false;
+    }
     v.numel *= v.shape[i];
+  }
   // Row-major contiguous is what memref.alloc and the entry-point wrapper
   // produce (src/Runtime/OMTensor.inc:185-192); anything else is refused.
   int64_t expect = 1;

@@ -108,6 +108,19 @@ def test_argument_validation_sets_einval(rt):
                          None, np.zeros(2, np.int8))
     with pytest.raises(rt.RuntimeError_, match="expected f32 x"):
         rt.DynamicQuantizeLinear(np.zeros(4, np.int32))
+    with pytest.raises(rt.RuntimeError_, match="bias must be f32, scalar or"):
+        rt.MatMulIntegerDequant(np.zeros((4, 6), np.uint8), np.zeros((6, 3), np.int8), None, None,
+                                np.float32(1), np.float32(1), np.zeros(2, np.float32))
+    # a dimension that was never resolved
+    buf = np.zeros(16, np.float32)
+    shape = (ctypes.c_int64 * 2)(-1, 4)
+    h = rt._shim.omTensorCreate(buf.ctypes.data, shape, 2, 1)
+    try:
+        rt._lib.om_mi355x_DynamicQuantizeLinear(h, h, h, h)
+        with pytest.raises(rt.RuntimeError_, match="dimension 0 is -1"):
+            rt._check()
+    finally:
+        rt._shim.omTensorDestroy(h)
 
 
 def test_incompatible_version_is_refused(rt):
