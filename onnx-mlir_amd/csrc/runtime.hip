@@ -258,6 +258,7 @@ struct Ctx {
     if (it != pool.end() && it->first <= bytes * 2) {
       void *p = it->second;
       taken[p] = it->first;
+      pool_bytes -= it->first;
       pool.erase(it);
       return p;
     }
@@ -268,6 +269,7 @@ struct Ctx {
       for (auto &kv : pool)
         (void)hipFree(kv.second);
       pool.clear();
+      pool_bytes = 0;
       e = hipMalloc(&p, bytes);
     }
     if (e != hipSuccess) {
@@ -281,7 +283,7 @@ struct Ctx {
     auto it = taken.find(p);
     if (it == taken.end())
       return;
-    pool.emplace(it->second, p);
+    adopt(p, it->second);
     taken.erase(it);
   }
   // A pool block whose ownership leaves the pool (a backing that outlives the
@@ -295,11 +297,25 @@ struct Ctx {
     taken.erase(it);
     return p;
   }
-  void adopt(void *p, size_t capacity) { pool.emplace(capacity, p); }
+  // Idle blocks are kept for reuse up to kPoolCap bytes per host thread; past
+  // that (shapes that keep changing) a block goes back to the driver, after
+  // the work that may still use it.
+  static constexpr size_t kPoolCap = (size_t)16 << 30;
+  size_t pool_bytes = 0;
+  void adopt(void *p, size_t capacity) {
+    if (pool_bytes + capacity > kPoolCap) {
+      (void)hipStreamSynchronize(stream);
+      (void)hipFree(p);
+      return;
+    }
+    pool.emplace(capacity, p);
+    pool_bytes += capacity;
+  }
   void drop_pool() {
     for (auto &kv : pool)
       (void)hipFree(kv.second);
     pool.clear();
+    pool_bytes = 0;
   }
   std::unordered_map<void *, size_t> taken;
 };
