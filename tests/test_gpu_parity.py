@@ -649,6 +649,49 @@ def test_config4_layers_reduced_m(rt, oracle, name):
     assert same_f32(rt.DynQuantMatMulDequant(c["X"], c["W"], None, c["w_scale"]), want)
 
 
+def _check_full_size_layer(rt, oracle, c, sample_rows):
+    """A layer at its benchmark size.  The oracle is too slow for the whole
+    matrix, so: (1) exact comparison of sampled rows (first, last, both sides of
+    tile edges, random ones) of the fused result; (2) two checksums over the
+    whole int32 accumulator, which every element enters: its column sums must
+    equal (sum of the rows of A - zp) x W and its row sums (A - zp) x (sum of
+    the columns of W), in arithmetic modulo 2^32."""
+    X, W, ws = c["X"], c["W"], c["w_scale"]
+    M, K = X.shape
+    N = W.shape[1]
+    aq, a_s, a_zp = oracle.dynamic_quantize_linear(X)
+    got = rt.DynQuantMatMulDequant(X, W, None, ws)
+    rng = np.random.default_rng(M + N)
+    rows = sorted(set([0, 1, 31, 32, 127, 128, 255, 256, M - 129, M - 128, M - 2, M - 1]
+                      + list(rng.integers(0, M, sample_rows))))
+    rows = [r for r in rows if 0 <= r < M]
+    want = oracle.dequant_epilogue(oracle.matmul_integer(aq[rows], W, a_zp, None), a_s, ws)
+    assert same_f32(got[rows], want)
+    acc = rt.MatMulInteger(aq, W, a_zp, None)
+    # all partial sums stay below 2^53: float64 arithmetic is exact here
+    a_colsum = aq.sum(axis=0, dtype=np.int64) - M * int(a_zp)          # [K]
+    w_rowsum = W.sum(axis=1, dtype=np.int64)                           # [K]
+    want_cols = np.zeros(N, np.float64)
+    for k0 in range(0, K, 1024):
+        want_cols += a_colsum[k0:k0 + 1024].astype(np.float64) @ W[k0:k0 + 1024].astype(np.float64)
+    want_rows = (aq.astype(np.float64) - float(a_zp)) @ w_rowsum.astype(np.float64)
+    mod = 1 << 32
+    assert np.array_equal(acc.sum(axis=0, dtype=np.int64) % mod, want_cols.astype(np.int64) % mod)
+    assert np.array_equal(acc.sum(axis=1, dtype=np.int64) % mod, want_rows.astype(np.int64) % mod)
+    # and the fused result is that accumulator, scaled
+    assert same_f32(got, oracle.dequant_epilogue(acc, a_s, ws))
+
+
+@pytest.mark.parametrize("name", list(wl.CONFIG4_SHAPES))
+def test_config4_layers_full_size(rt, oracle, name):
+    _check_full_size_layer(rt, oracle, wl.config4(name), 48)
+
+
+@pytest.mark.parametrize("name", list(wl.CONFIG5_SHAPES))
+def test_config5_prefill_full_size(rt, oracle, name):
+    _check_full_size_layer(rt, oracle, wl.config5(name), 12)
+
+
 @pytest.mark.parametrize("M", [1, 4, 16])
 def test_config5_decode_shapes(rt, oracle, M):
     c = wl.config5("up", M=M)
