@@ -57,6 +57,26 @@ __device__ __forceinline__ int lds_off(int r, int c) {
   return r * BK + ((c ^ ((r >> 2) & 3)) << 4);
 }
 
+// A pointer that is the same in every lane, pinned to scalar registers: the
+// compiler then addresses memory as (scalar base + 32-bit lane offset) and
+// cannot turn base + offset into a per-lane pointer that it advances with
+// vector adds.
+// A 32-bit lane offset whose widening to 64 bits stays next to its use: hoisted
+// out of a loop it would arrive as a 64-bit register pair, and the load would
+// then take the per-lane 64-bit address form.
+__device__ __forceinline__ uint32_t lane_offset(uint32_t o) {
+  asm volatile("" : "+v"(o));
+  return o;
+}
+
+template <typename T>
+__device__ __forceinline__ T *scalar_ptr(T *p) {
+  const uint64_t a = (uint64_t)p;
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
+  return (T *)(((uint64_t)hi << 32) | lo);
+}
+
 // Barrier that orders LDS accesses only; global loads already issued keep
 // flying across it.
 __device__ __forceinline__ void lds_barrier() {
@@ -870,20 +890,24 @@ __global__ __launch_bounds__(256, MINB) void k_gemm_i8_bs(
   // stage, lane -> row j*16 + lane/4, holding chunk (lane%4) ^ ((lane/16)%4).
   const int crow = lane >> 2;
   const int cchunk = (lane & 3) ^ ((lane >> 4) & 3);
-  const uint8_t *ga[CA];
+  // Scalar base (tile origin + K step) plus a 32-bit lane offset that does not
+  // change from step to step: no vector address arithmetic in the loop.
+  const uint8_t *const abase = A + (int64_t)m0 * K;
+  uint32_t ga[CA];
 #pragma unroll
   for (int h = 0; h < CA; ++h) {
     const int r = (wave * CA + h) * 16 + crow;
-    const int gm = (m0 + r < M) ? m0 + r : M - 1; // rows past M: never stored
-    ga[h] = A + (int64_t)gm * K + cchunk * 16;
+    const int rc = (m0 + r < M) ? r : M - 1 - m0; // rows past M: never stored
+    ga[h] = (uint32_t)rc * (uint32_t)K + (uint32_t)cchunk * 16u;
   }
   typedef __attribute__((address_space(3))) void *lds_ptr;
   typedef const __attribute__((address_space(1))) void *glb_ptr;
   auto copy_a = [&](int step, int stage) {
     uint8_t *base = sm + stage * STAGE + wave * CA * 1024;
+    const uint8_t *const src = scalar_ptr(abase + step * BK);
 #pragma unroll
     for (int h = 0; h < CA; ++h)
-      __builtin_amdgcn_global_load_lds((glb_ptr)(ga[h] + step * BK),
+      __builtin_amdgcn_global_load_lds((glb_ptr)(src + lane_offset(ga[h])),
           (lds_ptr)(base + h * 1024), 16, 0, 0);
   };
 
@@ -892,10 +916,20 @@ __global__ __launch_bounds__(256, MINB) void k_gemm_i8_bs(
 #pragma unroll
   for (int j = 0; j < TN; ++j)
     gbp[j] = Bp + (int64_t)((ncol0 >> 5) + j) * KT * 2048 + lane * 16;
+  // Buffer addressing: one descriptor in scalar registers for this wave's
+  // column tiles, a 32-bit lane offset, and the step as a scalar offset.
+  const __amdgpu_buffer_rsrc_t brsrc = __builtin_amdgcn_make_buffer_rsrc(
+      (void *)(Bp + (int64_t)(ncol0 >> 5) * KT * 2048), 0, TN * KT * 2048,
+      0x00020000);
+  int boff[TN];
+#pragma unroll
+  for (int j = 0; j < TN; ++j)
+    boff[j] = j * KT * 2048 + lane * 16;
   auto load_b = [&](int step, int sub, v4i(&fb)[TN]) {
 #pragma unroll
     for (int j = 0; j < TN; ++j)
-      fb[j] = *(const v4i *)(gbp[j] + (int64_t)step * 2048 + sub * 1024);
+      fb[j] = __builtin_amdgcn_raw_buffer_load_b128(
+          brsrc, boff[j], step * 2048 + sub * 1024, 0);
   };
 
   // A operand reads: half step s uses chunk 2*s + lane/32 of row lane%32 of
