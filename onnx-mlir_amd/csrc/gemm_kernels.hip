@@ -742,85 +742,93 @@ __global__ __launch_bounds__(256, MINB) void k_gemm_i8_dma(
     rsp[i] = 0;
 
   int stage = 0; // kt % NSTAGE
-  for (int kt = 0; kt < KT; ++kt) {
-    const int prev = (stage == 0) ? NSTAGE - 1 : stage - 1;
-    // Own copies of step kt have landed; those of the NSTAGE-2 steps after it
-    // may still be in flight.
-    __builtin_amdgcn_s_waitcnt(0x0F70 | ((NSTAGE - 2) * CPW));
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_sched_barrier(0);
-    copy_step(kclamp(kt + NSTAGE - 1), prev);
-    __builtin_amdgcn_sched_barrier(0);
-    const unsigned soff = (unsigned)(stage * STAGE);
-    v4i fa0[TM], fb0[TN], fa1[TM], fb1[TN];
-    using O0 = std::integral_constant<int, 0>;
-    using O1 = std::integral_constant<int, 2048>;
-    lds_read(fa0[0], ra[0] + soff, O0{});
-    lds_read(fa0[1], ra[0] + soff, O1{});
-    lds_read(fb0[0], rb[0] + soff, O0{});
-    if (TN == 2)
-      lds_read(fb0[TN - 1], rb[0] + soff, O1{});
-    lds_read(fa1[0], ra[1] + soff, O0{});
-    lds_read(fa1[1], ra[1] + soff, O1{});
-    lds_read(fb1[0], rb[1] + soff, O0{});
-    if (TN == 2)
-      lds_read(fb1[TN - 1], rb[1] + soff, O1{});
-    if (TN == 2)
-      asm volatile("s_waitcnt lgkmcnt(4)"
-                   : "+v"(fa0[0]), "+v"(fa0[1]), "+v"(fb0[0]), "+v"(fb0[TN - 1])
-                   :
-                   : "memory");
-    else
-      asm volatile("s_waitcnt lgkmcnt(3)"
-                   : "+v"(fa0[0]), "+v"(fa0[1]), "+v"(fb0[0])
-                   :
-                   : "memory");
-    if (A_MODE == 1) {
-#pragma unroll
+  // Whether row sums of A are needed is fixed here, outside the loop, so that
+  // the loop body has no branch.
+  auto k_loop = [&](auto RS) {
+    for (int kt = 0; kt < KT; ++kt) {
+      const int prev = (stage == 0) ? NSTAGE - 1 : stage - 1;
+      // Own copies of step kt have landed; those of the NSTAGE-2 steps after it
+      // may still be in flight.
+      __builtin_amdgcn_s_waitcnt(0x0F70 | ((NSTAGE - 2) * CPW));
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+      copy_step(kclamp(kt + NSTAGE - 1), prev);
+      __builtin_amdgcn_sched_barrier(0);
+      const unsigned soff = (unsigned)(stage * STAGE);
+      v4i fa0[TM], fb0[TN], fa1[TM], fb1[TN];
+      using O0 = std::integral_constant<int, 0>;
+      using O1 = std::integral_constant<int, 2048>;
+      lds_read(fa0[0], ra[0] + soff, O0{});
+      lds_read(fa0[1], ra[0] + soff, O1{});
+      lds_read(fb0[0], rb[0] + soff, O0{});
+      if (TN == 2)
+        lds_read(fb0[TN - 1], rb[0] + soff, O1{});
+      lds_read(fa1[0], ra[1] + soff, O0{});
+      lds_read(fa1[1], ra[1] + soff, O1{});
+      lds_read(fb1[0], rb[1] + soff, O0{});
+      if (TN == 2)
+        lds_read(fb1[TN - 1], rb[1] + soff, O1{});
+      if (TN == 2)
+        asm volatile("s_waitcnt lgkmcnt(4)"
+                     : "+v"(fa0[0]), "+v"(fa0[1]), "+v"(fb0[0]), "+v"(fb0[TN - 1])
+                     :
+                     : "memory");
+      else
+        asm volatile("s_waitcnt lgkmcnt(3)"
+                     : "+v"(fa0[0]), "+v"(fa0[1]), "+v"(fb0[0])
+                     :
+                     : "memory");
+      if (A_MODE == 1) {
+  #pragma unroll
+        for (int i = 0; i < TM; ++i)
+          fa0[i] ^= (v4i){(int)0x80808080, (int)0x80808080, (int)0x80808080,
+              (int)0x80808080};
+      }
+      if (decltype(RS)::value) {
+  #pragma unroll
+        for (int i = 0; i < TM; ++i)
+          rsp[i] += frag_rowsum(fa0[i]);
+      }
+  #pragma unroll
       for (int i = 0; i < TM; ++i)
-        fa0[i] ^= (v4i){(int)0x80808080, (int)0x80808080, (int)0x80808080,
-            (int)0x80808080};
-    }
-    if (need_rs) {
-#pragma unroll
+  #pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
+              fa0[i], fb0[j], acc[i][j], 0, 0, 0);
+      if (TN == 2)
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(fa1[0]), "+v"(fa1[1]), "+v"(fb1[0]), "+v"(fb1[TN - 1])
+                     :
+                     : "memory");
+      else
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(fa1[0]), "+v"(fa1[1]), "+v"(fb1[0])
+                     :
+                     : "memory");
+      if (A_MODE == 1) {
+  #pragma unroll
+        for (int i = 0; i < TM; ++i)
+          fa1[i] ^= (v4i){(int)0x80808080, (int)0x80808080, (int)0x80808080,
+              (int)0x80808080};
+      }
+      if (decltype(RS)::value) {
+  #pragma unroll
+        for (int i = 0; i < TM; ++i)
+          rsp[i] += frag_rowsum(fa1[i]);
+      }
+  #pragma unroll
       for (int i = 0; i < TM; ++i)
-        rsp[i] += frag_rowsum(fa0[i]);
+  #pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
+              fa1[i], fb1[j], acc[i][j], 0, 0, 0);
+      stage = (stage == NSTAGE - 1) ? 0 : stage + 1;
     }
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-      for (int j = 0; j < TN; ++j)
-        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
-            fa0[i], fb0[j], acc[i][j], 0, 0, 0);
-    if (TN == 2)
-      asm volatile("s_waitcnt lgkmcnt(0)"
-                   : "+v"(fa1[0]), "+v"(fa1[1]), "+v"(fb1[0]), "+v"(fb1[TN - 1])
-                   :
-                   : "memory");
-    else
-      asm volatile("s_waitcnt lgkmcnt(0)"
-                   : "+v"(fa1[0]), "+v"(fa1[1]), "+v"(fb1[0])
-                   :
-                   : "memory");
-    if (A_MODE == 1) {
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-        fa1[i] ^= (v4i){(int)0x80808080, (int)0x80808080, (int)0x80808080,
-            (int)0x80808080};
-    }
-    if (need_rs) {
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-        rsp[i] += frag_rowsum(fa1[i]);
-    }
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-      for (int j = 0; j < TN; ++j)
-        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
-            fa1[i], fb1[j], acc[i][j], 0, 0, 0);
-    stage = (stage == NSTAGE - 1) ? 0 : stage + 1;
-  }
+  };
+  if (need_rs)
+    k_loop(std::true_type{});
+  else
+    k_loop(std::false_type{});
   // Copies past the last step are still landing in LDS; nothing reads them,
   // but the block must not release its LDS before they are done.
   __builtin_amdgcn_s_waitcnt(0x0F70);
