@@ -857,7 +857,7 @@ __global__ __launch_bounds__(256, MINB) void k_gemm_i8_dma(
 //   refill its Bp registers for step +D, MFMAs of half step 1, refill,
 //   A copies for step +NST-1 into the stage that was read in the last step.
 template <int TM, int TN, int D, int NST, int MINB, bool PIPE, int A_MODE,
-    int EPI>
+    int EPI, bool RS>
 __global__ __launch_bounds__(256, MINB) void k_gemm_i8_bs(
     const uint8_t *__restrict__ A, const int8_t *__restrict__ Bp, int M, int N,
     int K, int Kpad, EpiParams ep, int tiles_m, int tiles_n) {
@@ -990,7 +990,9 @@ __global__ __launch_bounds__(256, MINB) void k_gemm_i8_bs(
       (int)0x80808080};
   using O = std::integral_constant<int, 0>;
 
-  const bool need_rs = ep.need_rowsum;
+  // RS: row sums of A are needed (B carries an offset); a template argument
+  // so that the loop body has no branch.
+  constexpr bool need_rs = RS;
   int32_t rsp[TM];
 #pragma unroll
   for (int i = 0; i < TM; ++i)
@@ -1433,9 +1435,14 @@ hipError_t gemm_launch_cfg(
   switch (choose_tile(g.M, g.N)) {
   case kB128x256: {
     const int tiles_n = (int)((g.N + 255) / 256);
-    k_gemm_i8_bs<4, 2, 4, 4, 2, true, A_MODE, EPI>
-        <<<dim3((unsigned)(tiles_m * tiles_n)), 256, 0, st>>>(
-            A, g.Bp, M, N, K, Kpad, ep, tiles_m, tiles_n);
+    if (ep.need_rowsum)
+      k_gemm_i8_bs<4, 2, 4, 4, 2, true, A_MODE, EPI, true>
+          <<<dim3((unsigned)(tiles_m * tiles_n)), 256, 0, st>>>(
+              A, g.Bp, M, N, K, Kpad, ep, tiles_m, tiles_n);
+    else
+      k_gemm_i8_bs<4, 2, 4, 4, 2, true, A_MODE, EPI, false>
+          <<<dim3((unsigned)(tiles_m * tiles_n)), 256, 0, st>>>(
+              A, g.Bp, M, N, K, Kpad, ep, tiles_m, tiles_n);
     break;
   }
   case kD128x128:
