@@ -919,25 +919,35 @@ __global__ __launch_bounds__(256, MINB) void k_gemm_i8_bs(
           (lds_ptr)(base + h * 1024), 16, 0, 0);
   };
 
-  // Bp operands of this wave's column tiles.
-  const int8_t *gbp[TN];
-#pragma unroll
-  for (int j = 0; j < TN; ++j)
-    gbp[j] = Bp + (int64_t)((ncol0 >> 5) + j) * KT * 2048 + lane * 16;
-  // Buffer addressing: one descriptor in scalar registers for this wave's
-  // column tiles, a 32-bit lane offset, and the step as a scalar offset.
-  const __amdgpu_buffer_rsrc_t brsrc = __builtin_amdgcn_make_buffer_rsrc(
-      (void *)(Bp + (int64_t)(ncol0 >> 5) * KT * 2048), 0, TN * KT * 2048,
-      0x00020000);
+  // Bp operands of this wave's column tiles, by buffer addressing: one
+  // descriptor in scalar registers, a 32-bit lane offset, and the step as a
+  // scalar offset.  The loads are written as inline assembly because the
+  // compiler, which cannot count memory operations across the loop's back
+  // edge, would otherwise wait for every outstanding one (vmcnt(0)) before
+  // the first use of these registers in each trip, draining the prefetch.  No
+  // wait of their own is needed: a step's operands were requested D >= 2 steps
+  // earlier, and the wait for the A copies at the top of each step covers
+  // everything issued up to two steps before it.
+  v4i brsrc;
+  {
+    const uint64_t a = (uint64_t)(Bp + (int64_t)(ncol0 >> 5) * KT * 2048);
+    brsrc.x = __builtin_amdgcn_readfirstlane((int)(uint32_t)a);
+    brsrc.y = __builtin_amdgcn_readfirstlane((int)((uint32_t)(a >> 32) & 0xFFFFu));
+    brsrc.z = __builtin_amdgcn_readfirstlane(TN * KT * 2048); // bytes covered
+    brsrc.w = 0x00020000; // raw buffer, 32-bit elements
+  }
   int boff[TN];
 #pragma unroll
   for (int j = 0; j < TN; ++j)
     boff[j] = j * KT * 2048 + lane * 16;
   auto load_b = [&](int step, int sub, v4i(&fb)[TN]) {
+    const int soff = step * 2048 + sub * 1024;
 #pragma unroll
     for (int j = 0; j < TN; ++j)
-      fb[j] = __builtin_amdgcn_raw_buffer_load_b128(
-          brsrc, boff[j], step * 2048 + sub * 1024, 0);
+      asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen"
+                   : "=v"(fb[j])
+                   : "v"(boff[j]), "s"(brsrc), "s"(soff)
+                   : "memory");
   };
 
   // A operand reads: half step s uses chunk 2*s + lane/32 of row lane%32 of
