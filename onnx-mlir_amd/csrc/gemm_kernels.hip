@@ -1382,7 +1382,8 @@ enum TileCfg : int {
   kT128x128 = 0, // k_gemm_i8: register-staged tiles (and the general path)
   kD128x128 = 1, // k_gemm_i8_dma: tiles copied straight into LDS
   kB128x256 = 2, // k_gemm_i8_bs: Bp straight into registers
-  kNumCfg = 3
+  kD128x64 = 3,  // k_gemm_i8_dma with 128 x 64 tiles
+  kNumCfg = 4
 };
 
 // Kernel choice for problems with more than 32 rows, K % 64 == 0 and a
@@ -1390,9 +1391,13 @@ enum TileCfg : int {
 // Measured on MI355X over the BERT-base and Llama-7B layer shapes and square
 // problems up to 8192: a 128 x 256 tile of k_gemm_i8_bs costs about 1.7 times
 // a 128 x 128 tile of k_gemm_i8_dma, so it wins when it needs at most half as
-// many rounds over the 256 CUs and fills at least one round.
+// many rounds over the 256 CUs and fills at least one round.  When 128 x 128
+// tiles cover at most half the CUs, 128 x 64 tiles spread the work over twice
+// as many (512x1024x4096: 10.1 -> 8.8 us); with 192 tiles for 256 CUs the
+// half-width tiles lose (4096x768x768 7.2 -> 7.6 us, 4096x3072x768 18.6 ->
+// 19.4 us).
 // Override for tests and tuning: OM_MI355X_GEMM_TILE=<TileCfg value>.
-int choose_tile(int64_t M, int64_t N) {
+int choose_tile(int64_t M, int64_t N, int64_t K) {
   const char *force = getenv("OM_MI355X_GEMM_TILE");
   if (force && force[0]) {
     const int c = atoi(force);
@@ -1405,6 +1410,9 @@ int choose_tile(int64_t M, int64_t N) {
   const int64_t r128 = (t128 + 255) / 256, r256 = (t256 + 255) / 256;
   if (t256 >= 256 && r256 * 17 < r128 * 10)
     return kB128x256;
+  (void)K;
+  if (N > 64 && t128 <= 128)
+    return kD128x64;
   return kD128x128;
 }
 
@@ -1442,7 +1450,7 @@ hipError_t gemm_launch_cfg(
               A, g.Bp, M, N, K, Kpad, ep, tiles_m, tiles_n128);
     return hipGetLastError();
   }
-  switch (choose_tile(g.M, g.N)) {
+  switch (choose_tile(g.M, g.N, g.K)) {
   case kB128x256: {
     const int tiles_n = (int)((g.N + 255) / 256);
     if (ep.need_rowsum)
@@ -1453,6 +1461,13 @@ hipError_t gemm_launch_cfg(
       k_gemm_i8_bs<4, 2, 4, 4, 2, true, A_MODE, EPI, false>
           <<<dim3((unsigned)(tiles_m * tiles_n)), 256, 0, st>>>(
               A, g.Bp, M, N, K, Kpad, ep, tiles_m, tiles_n);
+    break;
+  }
+  case kD128x64: {
+    const int tiles_n64 = (int)((g.N + 63) / 64);
+    k_gemm_i8_dma<64, 3, 3, A_MODE, EPI>
+        <<<dim3((unsigned)(tiles_m * tiles_n64)), 256, 0, st>>>(
+            A, g.Bp, M, N, K, Kpad, ep, tiles_m, tiles_n64);
     break;
   }
   case kD128x128:

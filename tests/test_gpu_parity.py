@@ -394,12 +394,12 @@ def test_matmulinteger_shapes(rt, oracle, M, K, N):
     assert np.array_equal(rt.MatMulInteger(A, B, azr, bzc), want)
 
 
-@pytest.mark.parametrize("cfg", [0, 1, 2])
+@pytest.mark.parametrize("cfg", [0, 1, 2, 3])
 def test_every_gemm_kernel_configuration(rt, oracle, cfg, monkeypatch):
     """The kernel choice is a heuristic; force each configuration in turn (0 stages
     tiles through registers, 1 copies them straight into LDS, 2 streams B
-    straight into registers) on shapes with ragged edges, every operand type
-    and all zero-point forms."""
+    straight into registers, 3 is 1 with 128 x 64 tiles) on shapes with ragged
+    edges, every operand type and all zero-point forms."""
     monkeypatch.setenv("OM_MI355X_GEMM_TILE", str(cfg))
     rng = np.random.default_rng(100 + cfg)
     for (M, K, N), adt, bdt in (((300, 200, 500), np.uint8, np.int8), ((129, 64, 193), np.int8, np.uint8),
@@ -419,6 +419,82 @@ def test_every_gemm_kernel_configuration(rt, oracle, cfg, monkeypatch):
     aq, a_s, a_zp = oracle.dynamic_quantize_linear(x)
     wantf = oracle.dequant_epilogue(oracle.matmul_integer(aq, W, a_zp, None), a_s, ws)
     assert same_f32(rt.DynQuantMatMulDequant(x, W, None, ws), wantf)
+
+
+def test_matmul_random_shapes_around_dispatch_boundaries(rt, oracle):
+    """Seeded sweep over shapes that sit on both sides of every dispatch
+    condition (M 16/17, 32/33, 128/129; K a multiple of 64, of 16, of neither;
+    N around 32, 64, 128, 256), all operand types and zero-point forms, the
+    three epilogues."""
+    rng = np.random.default_rng(2024)
+    Ms = [1, 2, 15, 16, 17, 31, 32, 33, 64, 127, 128, 129, 200, 257]
+    Ks = [1, 3, 16, 17, 48, 63, 64, 65, 80, 128, 130, 192, 200, 256, 1000]
+    Ns = [1, 5, 31, 32, 33, 63, 64, 65, 127, 128, 129, 255, 256, 257, 300]
+    for case in range(400):
+        M, K, N = (int(rng.choice(v)) for v in (Ms, Ks, Ns))
+        adt, bdt = (rng.choice([np.uint8, np.int8]) for _ in range(2))
+        A, B = _rand_q(rng, adt, (M, K)), _rand_q(rng, bdt, (K, N))
+        az = [None, _rand_q(rng, adt, ()), _rand_q(rng, adt, (M,))][int(rng.integers(0, 3))]
+        bz = [None, _rand_q(rng, bdt, ()), _rand_q(rng, bdt, (N,))][int(rng.integers(0, 3))]
+        tag = (case, M, K, N, adt.__name__, bdt.__name__, None if az is None else az.shape,
+               None if bz is None else bz.shape)
+        acc = oracle.matmul_integer(A, B, az, bz)
+        kind = case % 3
+        if kind == 0:
+            assert np.array_equal(rt.MatMulInteger(A, B, az, bz), acc), tag
+        elif kind == 1:
+            a_s = np.float32(rng.uniform(0.001, 0.1))
+            bs = rng.uniform(1e-3, 1e-2, N if case % 2 else 1).astype(np.float32)
+            bias = [None, rng.normal(0, 2, N).astype(np.float32)][case % 4 // 2]
+            want = oracle.dequant_epilogue(acc, a_s, bs)
+            if bias is not None:
+                want = want + bias
+            assert same_f32(rt.MatMulIntegerDequant(A, B, az, bz, a_s, bs, bias), want), tag
+        else:
+            ydt = rng.choice([np.uint8, np.int8])
+            azq = _rand_q(rng, adt, ()) if az is None else az
+            bzq = _rand_q(rng, bdt, ()) if bz is None else bz
+            yz = _rand_q(rng, ydt, ())
+            a_s, b_s, y_s = (np.float32(v) for v in (0.02, 0.01, rng.uniform(0.05, 2.0)))
+            for mode in (rt.WRAP, rt.SATURATE):
+                want = oracle.qlinear_matmul(A, a_s, azq, B, b_s, bzq, y_s, yz, mode)
+                got = rt.QLinearMatMul(A, a_s, azq, B, b_s, bzq, y_s, yz, mode)
+                assert np.array_equal(got, want), tag + (mode,)
+
+
+def test_quantize_random_shapes_and_axes(rt, oracle):
+    """Seeded sweep over ranks 1-4, every axis, per-tensor and per-axis
+    parameters, both output types, for QuantizeLinear, DequantizeLinear (8-bit
+    and int32 input) and DynamicQuantizeLinear."""
+    rng = np.random.default_rng(4048)
+    dims = [1, 2, 3, 4, 5, 7, 8, 16, 31, 33, 64, 100, 257]
+    for case in range(300):
+        rank = int(rng.integers(1, 5))
+        shape = tuple(int(rng.choice(dims)) for _ in range(rank))
+        axis = int(rng.integers(-rank, rank))
+        x = rng.normal(0, 3, shape).astype(np.float32)
+        qdt = rng.choice([np.uint8, np.int8])
+        info = np.iinfo(qdt)
+        C = shape[axis] if case % 3 else 1
+        sc = rng.uniform(0.005, 0.5, C).astype(np.float32)
+        zp = rng.integers(info.min, info.max + 1, C).astype(qdt) if case % 4 else None
+        if C == 1:
+            sc = sc.reshape(())
+            zp = None if zp is None else zp.reshape(())
+        tag = (case, shape, axis, qdt.__name__, C, zp is None)
+        wq = oracle.quantize_linear(x, sc, zp, axis=axis, out_dtype=qdt)
+        gq = rt.QuantizeLinear(x, sc, zp, axis=axis) if zp is not None or qdt == np.uint8 else None
+        if gq is not None:
+            assert np.array_equal(gq, wq), tag
+        assert same_f32(rt.DequantizeLinear(wq, sc, zp, axis=axis),
+                        oracle.dequantize_linear(wq, sc, zp, axis=axis)), tag
+        xi = rng.integers(-70000, 70000, shape).astype(np.int32)
+        zi = None if zp is None else zp.astype(np.int32)
+        assert same_f32(rt.DequantizeLinear(xi, sc, zi, axis=axis),
+                        oracle.dequantize_linear(xi, sc, zi, axis=axis)), tag
+        wy, ws, wz = oracle.dynamic_quantize_linear(x)
+        gy, gs, gz = rt.DynamicQuantizeLinear(x)
+        assert np.array_equal(gy, wy) and same_f32(np.float32(gs), ws) and int(gz) == int(wz), tag
 
 
 def test_large_gemm_takes_the_wide_tile_path(rt, oracle):
