@@ -23,16 +23,21 @@ hipError_t launch_dequantize(hipStream_t s, const void *x, QKind xkind,
     const void *zp, float *y);
 
 // Scratch a DynamicQuantizeLinear launch needs: per-block partial min / max
-// and an arrival counter that must be zero before the first launch (the
-// kernel leaves it zero).
+// and an arrival counter of the two-launch path, which must be zero before the
+// first launch (the kernel leaves it zero), and the per-block slots of the
+// one-launch kernel.
 struct DqlScratch {
   float *partial_min; // [kDqlMaxBlocks]
   float *partial_max; // [kDqlMaxBlocks]
-  unsigned *counter;  // [16], zeroed once: [0] two-pass arrivals, [4] barrier
-                      // of the one-launch kernel, [8] set if that barrier ever
-                      // timed out
+  unsigned *counter;  // [16], zeroed once: [0] two-pass arrivals, [8] set if
+                      // the exchange of the one-launch kernel ever timed out
   int grid_blocks;    // dql_grid_blocks(), or 0 to disable the one-launch path
-  unsigned spin_limit; // polls a block waits at the barrier before giving up
+  unsigned spin_limit; // polls a thread of the one-launch kernel waits for
+                       // another block's result before giving up
+  unsigned long long *grid_slots; // [2 * kDqlMaxBlocks], zeroed once: per
+                      // block (launch number << 32 | float bits) of its min,
+                      // then of its max
+  unsigned epoch;     // launch number of the one-launch kernel (host side)
 };
 // Blocks of the one-launch DynamicQuantizeLinear kernel that fit the current
 // device at once (0 if it cannot run here).
@@ -42,7 +47,7 @@ constexpr int kDqlMaxBlocks = 4096;
 // y u8[n], scale f32[1], zp u8[1].  If y_shift is true the stored bytes are
 // y ^ 0x80 (the value minus 128 as int8), the form the GEMM consumes, and
 // row sums are not needed because they are not produced here.
-hipError_t launch_dynamic_quantize(hipStream_t s, const DqlScratch &scratch,
+hipError_t launch_dynamic_quantize(hipStream_t s, DqlScratch &scratch,
     const float *x, int64_t n, uint8_t *y, float *scale, uint8_t *zp,
     bool y_shift);
 

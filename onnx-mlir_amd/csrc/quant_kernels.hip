@@ -676,30 +676,25 @@ __global__ __launch_bounds__(kSmallThreads) void k_dql_small(
   }
 }
 
-// Mid-sized tensors (up to kGridMaxPerThread float4 per thread of a grid that
-// fills the device once): the whole op in one cooperative launch.  Every
-// thread keeps its elements in registers across a grid-wide barrier, so x is
+// Mid-sized tensors (up to 16 float4 per thread of a grid that fills the
+// device once): the whole op in one launch.  Every thread keeps its elements
+// in registers while the blocks exchange their minima and maxima, so x is
 // read once, nothing but the result is written, and there is one launch
 // instead of two.  The grid is one block per CU, each of which needs a whole
 // CU's registers, and the launcher keeps at most one such kernel in flight,
 // so its blocks become resident together as soon as older work has drained
 // (a cooperative launch would guarantee that, but costs about 30 us per
-// launch on this platform).  The wait at the barrier is bounded all the same:
-// a block that gives up raises `failed` and writes nothing.
-//
-// Barrier: `arrive` counts block arrivals, then departures.  A block waits
-// until it reads >= gridDim.x; departures only add to it, so a slow block
-// still passes; the last block to depart (ticket 2*gridDim.x - 1) resets it.
+// launch on this platform).  The wait for the other blocks is bounded all the
+// same: a block that gives up raises `failed` and writes nothing.
 constexpr int kGridThreads = 1024;
 
 template <int NV>
 __global__ __launch_bounds__(kGridThreads) void k_dql_grid(
     const float *__restrict__ x, int64_t n, uint8_t *__restrict__ y,
     float *__restrict__ scale_out, uint8_t *__restrict__ zp_out, uint32_t flip,
-    float *partial_min, float *partial_max, unsigned *arrive, unsigned *failed,
-    unsigned spin_limit) {
+    unsigned long long *slot_lo, unsigned long long *slot_hi, unsigned epoch,
+    unsigned *failed, unsigned spin_limit) {
   __shared__ float s_lo[kGridThreads / 64], s_hi[kGridThreads / 64];
-  __shared__ bool s_ok;
   const int64_t nvec = n >> 2;
   const int64_t total = (int64_t)gridDim.x * kGridThreads;
   const int64_t gtid = (int64_t)blockIdx.x * kGridThreads + threadIdx.x;
@@ -746,61 +741,52 @@ __global__ __launch_bounds__(kGridThreads) void k_dql_grid(
   };
   block_reduce(lo, hi);
 
+  // Grid-wide exchange of the block results in two memory round trips.  Block
+  // b publishes (tag, min) and (tag, max) as two 64-bit device-scope atomic
+  // stores into its own slots, where tag is this launch's number: value and
+  // "it is there" travel in one word, so no fence and no arrival counter are
+  // needed, and nothing has to be reset between launches.  Every block then
+  // reads all slots with device-scope atomic loads (served where every XCD
+  // sees them, no cache to invalidate), each thread polling one slot until it
+  // carries the tag, and folds them itself: same values, same order of
+  // operations up to the commutative min / max, so all blocks agree.  The wait
+  // is bounded: a thread that gives up makes its block raise `failed` and
+  // write nothing.
   if (threadIdx.x == 0) {
-    __hip_atomic_store(&partial_min[blockIdx.x], lo, __ATOMIC_RELAXED,
-        __HIP_MEMORY_SCOPE_AGENT);
-    __hip_atomic_store(&partial_max[blockIdx.x], hi, __ATOMIC_RELAXED,
-        __HIP_MEMORY_SCOPE_AGENT);
-    // The partials above and below are device-scope atomics, performed where
-    // every XCD sees them; nothing else is published, so the arrival needs
-    // no cache write-back -- only to be issued after the two stores have
-    // completed, which the workgroup-scope fence waits for.
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __hip_atomic_fetch_add(
-        arrive, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    // Poll with relaxed loads (an acquire per poll would invalidate the L2 of
-    // this XCD every time); the partials are read with device-scope atomic
-    // loads afterwards, so no cache has to be invalidated at all.
-    bool ok = false;
+    const unsigned long long tag = (unsigned long long)epoch << 32;
+    __hip_atomic_store(&slot_lo[blockIdx.x], tag | __float_as_uint(lo),
+        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(&slot_hi[blockIdx.x], tag | __float_as_uint(hi),
+        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  bool ok = true;
+  lo = __builtin_inff();
+  hi = -__builtin_inff();
+  for (unsigned i = threadIdx.x; i < gridDim.x; i += kGridThreads) {
+    unsigned long long a = 0, b = 0;
+    bool got = false;
     for (unsigned spin = 0; spin < spin_limit; ++spin) {
-      if (__hip_atomic_load(arrive, __ATOMIC_RELAXED,
-              __HIP_MEMORY_SCOPE_AGENT) >= gridDim.x) {
-        ok = true;
+      a = __hip_atomic_load(
+          &slot_lo[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      b = __hip_atomic_load(
+          &slot_hi[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if ((unsigned)(a >> 32) == epoch && (unsigned)(b >> 32) == epoch) {
+        got = true;
         break;
       }
       __builtin_amdgcn_s_sleep(8);
     }
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-    if (!ok)
+    ok = ok && got;
+    lo = __builtin_fminf(lo, __uint_as_float((unsigned)a));
+    hi = __builtin_fmaxf(hi, __uint_as_float((unsigned)b));
+  }
+  if (!__syncthreads_and(ok)) {
+    if (threadIdx.x == 0)
       __hip_atomic_store(
           failed, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    s_ok = ok;
-  }
-  __syncthreads();
-  const bool ok = s_ok;
-
-  // Every block folds all partials itself (same values, same order of
-  // operations up to the commutative min / max): no second barrier.
-  lo = __builtin_inff();
-  hi = -__builtin_inff();
-  if (ok) {
-    for (unsigned i = threadIdx.x; i < gridDim.x; i += kGridThreads) {
-      lo = __builtin_fminf(lo, __hip_atomic_load(&partial_min[i],
-                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-      hi = __builtin_fmaxf(hi, __hip_atomic_load(&partial_max[i],
-                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-    }
+    return;
   }
   block_reduce(lo, hi);
-  if (threadIdx.x == 0) {
-    const unsigned ticket = __hip_atomic_fetch_add(
-        arrive, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (ticket == 2 * gridDim.x - 1)
-      __hip_atomic_store(
-          arrive, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
-  if (!ok)
-    return;
 
   float scale, zpf;
   dynamic_params(lo, hi, scale, zpf);
@@ -1071,7 +1057,7 @@ std::mutex g_grid_mutex;
 hipStream_t g_grid_stream = nullptr; // stream of the last such launch
 } // namespace
 
-hipError_t launch_dynamic_quantize(hipStream_t s, const DqlScratch &scratch,
+hipError_t launch_dynamic_quantize(hipStream_t s, DqlScratch &scratch,
     const float *x, int64_t n, uint8_t *y, float *scale, uint8_t *zp,
     bool y_shift) {
   if (n <= kSmallMax) { // n == 0 included: scale and zero point are written
@@ -1086,10 +1072,12 @@ hipError_t launch_dynamic_quantize(hipStream_t s, const DqlScratch &scratch,
     const int64_t total = (int64_t)scratch.grid_blocks * kGridThreads;
     const int64_t nvec = n >> 2;
     void (*fn_launch)(const float *, int64_t, uint8_t *, float *, uint8_t *,
-        uint32_t, float *, float *, unsigned *, unsigned *, unsigned) = nullptr;
-    // Below about two million elements the barrier costs more than the
-    // second launch and the second read (measured: 10.7 us against 8.3 us).
-    if (nvec < (int64_t)1 << 19)
+        uint32_t, unsigned long long *, unsigned long long *, unsigned,
+        unsigned *, unsigned) = nullptr;
+    // Below about half a million elements the exchange between the blocks
+    // costs as much as the second launch and the second read (measured at
+    // 512 Ki elements: 7.9 us against 8.1 us; at 32 Ki: 7.8 against 7.1).
+    if (nvec < (int64_t)1 << 17)
       fn_launch = nullptr;
     else if (nvec <= 4 * total)
       fn_launch = k_dql_grid<4>;
@@ -1098,8 +1086,9 @@ hipError_t launch_dynamic_quantize(hipStream_t s, const DqlScratch &scratch,
     if (fn_launch) {
       const uint32_t flip = y_shift ? 0x80808080u : 0u;
       const unsigned spin_limit = scratch.spin_limit;
-      float *pmin = scratch.partial_min, *pmax = scratch.partial_max;
-      unsigned *arrive = scratch.counter + 4, *failed = scratch.counter + 8;
+      unsigned long long *slot_lo = scratch.grid_slots;
+      unsigned long long *slot_hi = scratch.grid_slots + kDqlMaxBlocks;
+      unsigned *failed = scratch.counter + 8;
       // At most one of these kernels is in flight per process: two of them
       // dispatched at the same time from different streams could each hold
       // part of the device and wait for the rest.  If the previous one was
@@ -1112,9 +1101,11 @@ hipError_t launch_dynamic_quantize(hipStream_t s, const DqlScratch &scratch,
         // (same stream: the previous one finishes before this one starts)
         if (!g_grid_stream || g_grid_stream == s ||
             hipStreamQuery(g_grid_stream) == hipSuccess) {
+          if (++scratch.epoch == 0) // 0 is what untouched slots hold
+            scratch.epoch = 1;
           hipLaunchKernelGGL(fn_launch, dim3((unsigned)scratch.grid_blocks),
-              dim3(kGridThreads), 0, s, x, n, y, scale, zp, flip, pmin, pmax,
-              arrive, failed, spin_limit);
+              dim3(kGridThreads), 0, s, x, n, y, scale, zp, flip, slot_lo,
+              slot_hi, scratch.epoch, failed, spin_limit);
           hipError_t e = hipGetLastError();
           if (e != hipSuccess)
             return e;

@@ -132,7 +132,7 @@ bool probe_device() {
 struct Ctx {
   bool ready = false;
   hipStream_t stream = nullptr;
-  DqlScratch dql = {nullptr, nullptr, nullptr, 0, 0};
+  DqlScratch dql = {nullptr, nullptr, nullptr, 0, 0, nullptr, 0};
   float *dql_scale = nullptr; // scale / zero point of the fused path
   uint8_t *dql_zp = nullptr;
   std::multimap<size_t, void *> pool;
@@ -154,13 +154,16 @@ struct Ctx {
     HIP_OK(hipSetDevice(0));
     HIP_OK(hipStreamCreateWithFlags(&stream, hipStreamNonBlocking));
     void *p = nullptr;
-    HIP_OK(hipMalloc(&p, sizeof(float) * 2 * kDqlMaxBlocks + 256));
+    HIP_OK(hipMalloc(&p, sizeof(float) * 2 * kDqlMaxBlocks + 256 +
+                             sizeof(unsigned long long) * 2 * kDqlMaxBlocks));
     dql.partial_min = (float *)p;
     dql.partial_max = dql.partial_min + kDqlMaxBlocks;
     dql.counter = (unsigned *)(dql.partial_max + kDqlMaxBlocks);
     dql_scale = (float *)(dql.counter + 16);
     dql_zp = (uint8_t *)(dql.counter + 32);
-    HIP_OK(hipMemset(dql.counter, 0, 256));
+    dql.grid_slots = (unsigned long long *)((char *)dql.counter + 256);
+    HIP_OK(hipMemset(dql.counter, 0,
+        256 + sizeof(unsigned long long) * 2 * kDqlMaxBlocks));
     dql.grid_blocks = dql_grid_blocks();
     dql.spin_limit = 1u << 20; // about a second of polling
     if (const char *v = getenv("OM_MI355X_DQL_SPIN_LIMIT"))
@@ -185,8 +188,9 @@ struct Ctx {
       return true;
     (void)hipMemset(dql.counter, 0, 256);
     dql.grid_blocks = 0;
-    fail(EIO, "DynamicQuantizeLinear: the grid barrier of the one-launch "
-              "kernel timed out; its output was not written");
+    fail(EIO, "DynamicQuantizeLinear: the blocks of the one-launch kernel "
+              "timed out waiting for one another (grid barrier); its output "
+              "was not written");
     return false;
   }
 
