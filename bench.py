@@ -264,6 +264,24 @@ def only_mode(rt, wl, what, steps, warmup):
     return {"only": what, **r[what]}
 
 
+def host_cpu():
+    """Model name and logical CPU counts of the host (as the OS reports them)."""
+    name = ""
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    name = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    try:
+        usable = len(os.sched_getaffinity(0))
+    except AttributeError:
+        usable = os.cpu_count()
+    return {"model": name, "logical_cpus": os.cpu_count(), "usable_cpus": usable}
+
+
 def cpu_baseline_gemm(oracle, wl, M, K, N, budget_s=20.0):
     """The oracle's restatement of the reference's CPU pass structure for the
     same MatMulInteger + Cast + Mul, timed on this host's cores."""
@@ -284,7 +302,7 @@ def cpu_baseline_gemm(oracle, wl, M, K, N, budget_s=20.0):
         times.append(time.perf_counter() - t0)
     best = float(np.median(times))
     return {"value": 2.0 * M * N * K / best / 1e12, "unit": "TOPS", "cores": oracle.num_threads(),
-            "kind": "port",
+            "kind": "port", "host": host_cpu(),
             "sample": f"full M={M} K={K} N={N} MatMulInteger+Cast+Mul, median of {len(times)} runs of the "
                       "oracle's restatement of the reference's CPU passes (int32 copies, zero-point "
                       "passes, 4x8x8-blocked int32 GEMM, OpenMP over row tiles); not onnx-mlir codegen",
