@@ -20,9 +20,13 @@
 #include <string.h>
 #include <time.h>
 
+#include <algorithm>
+#include <condition_variable>
+#include <functional>
 #include <map>
 #include <mutex>
 #include <string>
+#include <thread>
 #include <unordered_map>
 #include <unordered_set>
 #include <vector>
@@ -124,6 +128,195 @@ bool probe_device() {
   return true;
 }
 
+// ---------------------------------------------------------------------------
+// Large copies between pageable host memory and the GPU
+// ---------------------------------------------------------------------------
+// A direct hipMemcpy on pageable memory reaches a third of the link rate.  A
+// lane moves every step-th piece of a buffer through page-locked slots of its
+// own: the DMA of one piece runs while the CPU copies the neighbouring piece
+// between its slot and the host buffer.  One core copies about 34 GB/s and the
+// link carries 56 GB/s, so the calling thread's lane is joined by lanes run by
+// helper threads (OM_MI355X_COPY_THREADS, default 2, 0 = none).
+struct CopyLane {
+  static constexpr int kSlots = 3;
+  static constexpr size_t kSlotBytes = (size_t)4 << 20;
+  hipStream_t stream = nullptr;
+  void *slot[kSlots] = {nullptr, nullptr, nullptr};
+  hipEvent_t ev[kSlots] = {nullptr, nullptr, nullptr};
+  hipEvent_t done = nullptr; // end of this lane's last to_device()
+  bool ready = false;
+
+  // `borrowed`: the stream to issue on; null = a stream of the lane's own.
+  bool init(hipStream_t borrowed) {
+    if (ready)
+      return true;
+    void *p = nullptr;
+    if (hipHostMalloc(&p, kSlots * kSlotBytes, hipHostMallocDefault) !=
+        hipSuccess) {
+      (void)hipGetLastError();
+      return false;
+    }
+    bool good = true;
+    for (int i = 0; i < kSlots && good; ++i)
+      good = hipEventCreateWithFlags(&ev[i], hipEventDisableTiming) ==
+             hipSuccess;
+    good = good && hipEventCreateWithFlags(&done, hipEventDisableTiming) ==
+                       hipSuccess;
+    if (good && !borrowed)
+      good = hipStreamCreateWithFlags(&stream, hipStreamNonBlocking) ==
+             hipSuccess;
+    else
+      stream = borrowed;
+    if (!good) {
+      (void)hipGetLastError();
+      for (int i = 0; i < kSlots; ++i)
+        if (ev[i]) {
+          (void)hipEventDestroy(ev[i]);
+          ev[i] = nullptr;
+        }
+      if (done) {
+        (void)hipEventDestroy(done);
+        done = nullptr;
+      }
+      (void)hipHostFree(p);
+      return false;
+    }
+    for (int i = 0; i < kSlots; ++i)
+      slot[i] = (char *)p + (size_t)i * kSlotBytes;
+    ready = true;
+    return true;
+  }
+
+  // Pieces first, first+step, ... of `bytes` (piece <= kSlotBytes each), from
+  // GPU memory into host memory.  Queued on the lane's stream; returns when
+  // this lane's share of the host buffer is complete.
+  hipError_t to_host(char *host, const char *dev, size_t bytes, size_t piece,
+      size_t first, size_t step) {
+    const size_t n = (bytes + piece - 1) / piece;
+    const size_t mine = first < n ? (n - first + step - 1) / step : 0;
+    auto offset = [&](size_t k) { return (first + k * step) * piece; };
+    auto length = [&](size_t k) {
+      return offset(k) + piece <= bytes ? piece : bytes - offset(k);
+    };
+    auto drain = [&](size_t k) -> hipError_t {
+      hipError_t e = hipEventSynchronize(ev[k % kSlots]);
+      if (e == hipSuccess)
+        memcpy(host + offset(k), slot[k % kSlots], length(k));
+      return e;
+    };
+    for (size_t k = 0; k < mine; ++k) {
+      const int sl = (int)(k % kSlots);
+      hipError_t e = hipMemcpyAsync(slot[sl], dev + offset(k), length(k),
+          hipMemcpyDeviceToHost, stream);
+      if (e == hipSuccess)
+        e = hipEventRecord(ev[sl], stream);
+      if (e == hipSuccess && k + 1 >= (size_t)kSlots)
+        e = drain(k + 1 - kSlots);
+      if (e != hipSuccess)
+        return e;
+    }
+    for (size_t k = (mine >= (size_t)kSlots ? mine - kSlots + 1 : 0); k < mine;
+         ++k) {
+      hipError_t e = drain(k);
+      if (e != hipSuccess)
+        return e;
+    }
+    return hipSuccess;
+  }
+
+  // The same pieces from host memory into GPU memory.  Returns when the host
+  // buffer has been read; the DMAs are queued on the lane's stream and `done`
+  // is recorded behind the last of them.
+  hipError_t to_device(char *dev, const char *host, size_t bytes, size_t piece,
+      size_t first, size_t step) {
+    const size_t n = (bytes + piece - 1) / piece;
+    for (size_t k = 0, i = first; i < n; ++k, i += step) {
+      const int sl = (int)(k % kSlots);
+      const size_t off = i * piece;
+      const size_t len = off + piece <= bytes ? piece : bytes - off;
+      // The slot may still feed an earlier DMA (an event that was never
+      // recorded counts as complete).
+      hipError_t e = hipEventSynchronize(ev[sl]);
+      if (e != hipSuccess)
+        return e;
+      memcpy(slot[sl], host + off, len);
+      e = hipMemcpyAsync(dev + off, slot[sl], len, hipMemcpyHostToDevice,
+          stream);
+      if (e == hipSuccess)
+        e = hipEventRecord(ev[sl], stream);
+      if (e != hipSuccess)
+        return e;
+    }
+    return hipEventRecord(done, stream);
+  }
+};
+
+// A helper thread with a lane of its own.  Helpers are created once, never
+// destroyed (they sleep on their condition variable until the process ends)
+// and serve one calling thread at a time.
+struct CopyHelper {
+  std::mutex m;
+  std::condition_variable cv;
+  std::function<hipError_t(CopyLane &)> job;
+  bool pending = false, finished = true;
+  hipError_t result = hipSuccess;
+  CopyLane lane;
+
+  void loop() {
+    (void)hipSetDevice(0);
+    std::unique_lock<std::mutex> lk(m);
+    for (;;) {
+      cv.wait(lk, [&] { return pending; });
+      pending = false;
+      std::function<hipError_t(CopyLane &)> j = std::move(job);
+      lk.unlock();
+      hipError_t e = lane.init(nullptr) ? j(lane) : hipErrorOutOfMemory;
+      lk.lock();
+      result = e;
+      finished = true;
+      cv.notify_all();
+    }
+  }
+  void start(std::function<hipError_t(CopyLane &)> j) {
+    std::lock_guard<std::mutex> lk(m);
+    job = std::move(j);
+    pending = true;
+    finished = false;
+    cv.notify_all();
+  }
+  hipError_t wait() {
+    std::unique_lock<std::mutex> lk(m);
+    cv.wait(lk, [&] { return finished; });
+    return result;
+  }
+};
+
+struct CopyHelpers {
+  std::mutex in_use; // held by the calling thread that employs the helpers
+  std::vector<CopyHelper *> list;
+};
+
+CopyHelpers *copy_helpers() {
+  static CopyHelpers *set = [] {
+    CopyHelpers *s = new CopyHelpers; // lives until the process ends
+    long want = 2;
+    if (const char *v = getenv("OM_MI355X_COPY_THREADS"))
+      want = strtol(v, nullptr, 10);
+    for (long i = 0; i < want && i < 4; ++i) {
+      CopyHelper *h = new CopyHelper;
+      try {
+        std::thread(&CopyHelper::loop, h).detach();
+      } catch (...) {
+        delete h;
+        break;
+      }
+      s->list.push_back(h);
+    }
+    return s;
+  }();
+  return set;
+}
+
 // Per-thread execution context: one stream (default priority), the scratch of
 // DynamicQuantizeLinear, a pool of reusable GPU buffers and timer events.
 // Buffers of the pool are only ever used by work on this stream, so handing a
@@ -137,11 +330,10 @@ struct Ctx {
   uint8_t *dql_zp = nullptr;
   std::multimap<size_t, void *> pool;
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
-  // Page-locked staging for large copies back to pageable host memory.
-  static constexpr int kStageSlots = 3;
-  static constexpr size_t kStageBytes = (size_t)4 << 20;
-  void *stage[kStageSlots] = {nullptr, nullptr, nullptr};
-  hipEvent_t stage_ev[kStageSlots] = {nullptr, nullptr, nullptr};
+  // Large copies from and to pageable host memory (see CopyLane).
+  static constexpr size_t kStagedFrom = (size_t)8 << 20;
+  CopyLane lane;             // the calling thread's lane, on `stream`
+  hipEvent_t fork_ev = nullptr; // where the helpers' streams join `stream`
 
   bool init() {
     if (ready)
@@ -195,63 +387,58 @@ struct Ctx {
   }
 
   bool stage_ready() {
-    if (stage[0])
-      return true;
-    void *p = nullptr;
-    if (hipHostMalloc(&p, kStageSlots * kStageBytes, hipHostMallocDefault) !=
-        hipSuccess) {
+    if (!fork_ev && hipEventCreateWithFlags(&fork_ev, hipEventDisableTiming) !=
+                        hipSuccess) {
       (void)hipGetLastError();
+      fork_ev = nullptr;
       return false;
     }
-    for (int i = 0; i < kStageSlots; ++i) {
-      if (hipEventCreateWithFlags(&stage_ev[i], hipEventDisableTiming) !=
-          hipSuccess) {
-        (void)hipGetLastError();
-        (void)hipHostFree(p);
-        return false;
-      }
-    }
-    for (int i = 0; i < kStageSlots; ++i)
-      stage[i] = (char *)p + (size_t)i * kStageBytes;
-    return true;
+    return lane.init(stream);
   }
 
-  // Device memory to pageable host memory through the page-locked slots: the
-  // DMA of one piece runs while the CPU copies the piece before it out of its
-  // slot (a direct copy to pageable memory reaches a third of the link rate).
-  // Queued on `stream` behind the work that produces the data; returns when
-  // the host buffer is complete.
-  hipError_t copy_back_staged(void *host, const void *dev, size_t bytes) {
-    const size_t n = (bytes + kStageBytes - 1) / kStageBytes;
-    auto piece = [&](size_t i) {
-      return (i + 1 < n) ? kStageBytes : bytes - i * kStageBytes;
-    };
-    auto drain = [&](size_t j) -> hipError_t {
-      hipError_t e = hipEventSynchronize(stage_ev[j % kStageSlots]);
+  // One buffer of at least kStagedFrom bytes between pageable host memory and
+  // GPU memory, split into pieces that go round-robin to this thread's lane
+  // and to the helpers (if no other thread employs them).  In stream order
+  // with the work queued on `stream` before and after; returns when the host
+  // buffer is complete (to_host) or has been read (to_device).
+  hipError_t copy_staged(void *host, void *dev, size_t bytes, bool to_host) {
+    const size_t piece =
+        bytes >= ((size_t)32 << 20) ? CopyLane::kSlotBytes : (size_t)2 << 20;
+    const size_t n = (bytes + piece - 1) / piece;
+    CopyHelpers *hs = copy_helpers();
+    std::unique_lock<std::mutex> use(hs->in_use, std::try_to_lock);
+    size_t nh = 0;
+    if (use.owns_lock() && n >= 2)
+      nh = std::min(hs->list.size(), n - 1);
+    const size_t lanes = 1 + nh;
+    hipError_t e = hipSuccess;
+    if (nh) {
+      e = hipEventRecord(fork_ev, stream);
       if (e != hipSuccess)
         return e;
-      memcpy((char *)host + j * kStageBytes, stage[j % kStageSlots], piece(j));
-      return hipSuccess;
-    };
-    for (size_t i = 0; i < n; ++i) {
-      const int slot = (int)(i % kStageSlots);
-      hipError_t e = hipMemcpyAsync(stage[slot],
-          (const char *)dev + i * kStageBytes, piece(i), hipMemcpyDeviceToHost,
-          stream);
+    }
+    char *h = (char *)host, *d = (char *)dev;
+    hipEvent_t fork = fork_ev;
+    for (size_t i = 0; i < nh; ++i)
+      hs->list[i]->start([=](CopyLane &l) -> hipError_t {
+        // Behind everything the calling thread has queued so far (the
+        // kernels that write the data, or the last use of the GPU buffer).
+        hipError_t r = hipStreamWaitEvent(l.stream, fork, 0);
+        if (r != hipSuccess)
+          return r;
+        return to_host ? l.to_host(h, d, bytes, piece, i + 1, lanes)
+                       : l.to_device(d, h, bytes, piece, i + 1, lanes);
+      });
+    e = to_host ? lane.to_host(h, d, bytes, piece, 0, lanes)
+                : lane.to_device(d, h, bytes, piece, 0, lanes);
+    for (size_t i = 0; i < nh; ++i) {
+      hipError_t r = hs->list[i]->wait();
+      if (r == hipSuccess && !to_host)
+        r = hipStreamWaitEvent(stream, hs->list[i]->lane.done, 0);
       if (e == hipSuccess)
-        e = hipEventRecord(stage_ev[slot], stream);
-      if (e == hipSuccess && i + 1 >= (size_t)kStageSlots)
-        e = drain(i + 1 - kStageSlots);
-      if (e != hipSuccess)
-        return e;
+        e = r;
     }
-    for (size_t j = (n >= (size_t)kStageSlots ? n - kStageSlots + 1 : 0); j < n;
-         ++j) {
-      hipError_t e = drain(j);
-      if (e != hipSuccess)
-        return e;
-    }
-    return hipSuccess;
+    return e;
   }
 
   void *take(size_t bytes) {
@@ -565,8 +752,11 @@ struct Call {
     d = temp(v.bytes);
     if (!d)
       return nullptr;
-    hipError_t e =
-        hipMemcpyAsync(d, v.data, v.bytes, hipMemcpyHostToDevice, c.stream);
+    hipError_t e;
+    if (v.bytes >= Ctx::kStagedFrom && c.stage_ready())
+      e = c.copy_staged(v.data, d, v.bytes, false);
+    else
+      e = hipMemcpyAsync(d, v.data, v.bytes, hipMemcpyHostToDevice, c.stream);
     if (e != hipSuccess) {
       fail(EIO, "host-to-device copy failed: %s", hipGetErrorString(e));
       ok = false;
@@ -602,8 +792,8 @@ struct Call {
     if (ok) {
       for (const Back &b : backs) {
         hipError_t e;
-        if (b.bytes >= 2 * Ctx::kStageBytes && c.stage_ready())
-          e = c.copy_back_staged(b.host, b.dev, b.bytes);
+        if (b.bytes >= Ctx::kStagedFrom && c.stage_ready())
+          e = c.copy_staged(b.host, b.dev, b.bytes, true);
         else
           e = hipMemcpyAsync(
               b.host, b.dev, b.bytes, hipMemcpyDeviceToHost, c.stream);

@@ -618,6 +618,43 @@ def test_host_buffers_kept_on_device_between_ops(rt, oracle):
     assert np.array_equal(acc, oracle.matmul_integer(waq, W, wz, None))
 
 
+def test_large_host_buffers_both_ways(rt, oracle):
+    """Host tensors of 8 MiB and more cross PCIe in pieces through page-locked
+    slots, shared out between the calling thread and helper threads: sizes that
+    are no multiple of a piece, both piece sizes, one piece more than there are
+    lanes, and two host threads at once (one of them finds the helpers taken)."""
+    import threading
+    rng = np.random.default_rng(2024)
+    sc, zp = np.float32(0.037), np.array(9, np.uint8)
+    sizes = [(2 << 20) + 1, (2 << 20) * 3 + 17, 8 * (1 << 20) + 5, 9_000_001, 12_582_913]
+    for n in sizes:                       # x: 4n bytes in (staged), y: n bytes out (staged from 8 MiB)
+        x = rng.normal(0, 3, n).astype(np.float32)
+        q = rt.QuantizeLinear(x, sc, zp)
+        assert np.array_equal(q, oracle.quantize_linear(x, sc, zp)), n
+        y = rt.DequantizeLinear(q, sc, zp)        # n bytes in, 4n bytes out
+        assert np.array_equal(y, oracle.dequantize_linear(q, sc, zp)), n
+    xs = [rng.normal(0, 2, 5_000_003 + 999 * t).astype(np.float32) for t in range(3)]
+    want = [oracle.quantize_linear(x, sc, zp) for x in xs]
+    errors = []
+
+    def work(t):
+        try:
+            for _ in range(3):
+                q = rt.QuantizeLinear(xs[t], sc, zp)
+                assert np.array_equal(q, want[t])
+                y = rt.DequantizeLinear(q, sc, zp)
+                assert np.array_equal(y, oracle.dequantize_linear(want[t], sc, zp))
+        except Exception as e:          # noqa: BLE001
+            errors.append((t, repr(e)))
+
+    threads = [threading.Thread(target=work, args=(t,)) for t in range(3)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not errors, errors
+
+
 def test_concurrent_host_threads(rt, oracle):
     """Entry points are re-entrant: four host threads (each gets its own stream)
     run DynamicQuantizeLinear on a tensor that takes the one-launch kernel,
