@@ -1197,13 +1197,32 @@ __global__ __launch_bounds__(256, MINB) void k_gemm_i8_bs(
 // most 32 rows, zero rows above M) is read from L2 in operand layout.  The
 // eight partial 32x32 results are summed through LDS.  No LDS staging, no
 // barrier in the K loop.
-template <int A_MODE, int EPI>
+//
+// DQ: the activation arrives as f32 X[M,K] (at most kSkinnyDqBytes elements)
+// and every block quantizes it itself, exactly as DynamicQuantizeLinear
+// would: minimum and maximum over all of X, scale and zero point from them,
+// the 8-bit values minus 128 into LDS, from where the K loop takes its A
+// operands.  That is 16 KiB of reads from L2 per block for one row of 4096,
+// in place of a launch of its own in front of this one (4096 x 11008
+// weights, whole layer: 1 row 10.6 -> 9.1 us, 4 rows 12.9 -> 11.0 us, 8 rows
+// 17 -> 15.5 us).  Requesting the first Bp operands before the rows are
+// quantized did not shorten it.
+constexpr int kSkinnyDqBytes = 32768;
+
+template <int A_MODE, int EPI, bool DQ>
 __global__ __launch_bounds__(512) void k_gemm_i8_skinny_bp(
-    const uint8_t *__restrict__ A, const int8_t *__restrict__ Bp, int M, int N,
-    int K, int Kpad, EpiParams ep) {
+    const uint8_t *__restrict__ A, const float *__restrict__ X,
+    const int8_t *__restrict__ Bp, int M, int N, int K, int Kpad,
+    EpiParams ep) {
   constexpr int WAVES = 8, U = 4;
-  __shared__ int32_t part[WAVES][16][64];
+  static_assert(!DQ || A_MODE == 2, "quantized rows are stored minus 128");
+  __shared__ __attribute__((aligned(16))) int32_t part[WAVES][16][64];
   __shared__ int32_t part_rs[WAVES][64];
+  // The quantized rows share the memory of the partial sums, which are not
+  // written before every wave has left the K loop.
+  static_assert(sizeof(part) >= kSkinnyDqBytes, "quantized rows fit");
+  uint8_t *const aq = (uint8_t *)&part[0][0][0];
+  __shared__ float s_lo[WAVES], s_hi[WAVES];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -1217,8 +1236,59 @@ __global__ __launch_bounds__(512) void k_gemm_i8_skinny_bp(
   const int kt_begin = wave * per;
   const int kt_end = (kt_begin + per < KT) ? kt_begin + per : KT;
 
+  float dq_scale = 0.0f;
+  int32_t dq_zp = 0;
+  if (DQ) {
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    constexpr int NV = kSkinnyDqBytes / 4 / (WAVES * 64); // float4 per thread
+    const int nvec = (M * K) >> 2; // K % 16 == 0, M * K <= kSkinnyDqBytes
+    const f4 *__restrict__ x4 = (const f4 *)X;
+    f4 v[NV];
+    float lo = __builtin_inff(), hi = -__builtin_inff();
+    const float nan = __builtin_nanf(""); // neutral for minnum / maxnum
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const int e = j * (WAVES * 64) + tid;
+      v[j] = e < nvec ? x4[e] : (f4){nan, nan, nan, nan};
+      lo = __builtin_fminf(__builtin_fminf(lo, v[j].x),
+          __builtin_fminf(__builtin_fminf(v[j].y, v[j].z), v[j].w));
+      hi = __builtin_fmaxf(__builtin_fmaxf(hi, v[j].x),
+          __builtin_fmaxf(__builtin_fmaxf(v[j].y, v[j].z), v[j].w));
+    }
+    lo = wave_min(lo);
+    hi = wave_max(hi);
+    if (lane == 0) {
+      s_lo[wave] = lo;
+      s_hi[wave] = hi;
+    }
+    __syncthreads();
+    lo = s_lo[0];
+    hi = s_hi[0];
+#pragma unroll
+    for (int w = 1; w < WAVES; ++w) {
+      lo = __builtin_fminf(lo, s_lo[w]);
+      hi = __builtin_fmaxf(hi, s_hi[w]);
+    }
+    float zpf;
+    dynamic_params(lo, hi, dq_scale, zpf);
+    dq_zp = (int32_t)(uint32_t)zpf;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const int e = j * (WAVES * 64) + tid;
+      if (e < nvec) {
+        const uint32_t q = quant_one<false, true>(v[j].x, dq_scale, zpf) |
+                           (quant_one<false, true>(v[j].y, dq_scale, zpf) << 8) |
+                           (quant_one<false, true>(v[j].z, dq_scale, zpf) << 16) |
+                           (quant_one<false, true>(v[j].w, dq_scale, zpf) << 24);
+        ((uint32_t *)aq)[e] = q ^ 0x80808080u;
+      }
+    }
+    __syncthreads();
+  }
+
   const bool row_ok = l32 < M;
-  const uint8_t *__restrict__ ap = A + (int64_t)(row_ok ? l32 : 0) * K;
+  const uint8_t *__restrict__ ap =
+      (DQ ? (const uint8_t *)aq : A) + (int64_t)(row_ok ? l32 : 0) * K;
   const int8_t *__restrict__ bp = Bp + (int64_t)nt * KT * 2048 + lane * 16;
   constexpr int kFill = (A_MODE == 1) ? (int)0x80808080 : 0;
 
@@ -1261,6 +1331,8 @@ __global__ __launch_bounds__(512) void k_gemm_i8_skinny_bp(
       }
     }
   }
+  if (DQ)
+    __syncthreads(); // every wave is done reading the quantized rows
 #pragma unroll
   for (int r = 0; r < 16; ++r)
     part[wave][r][lane] = acc[r];
@@ -1285,7 +1357,8 @@ __global__ __launch_bounds__(512) void k_gemm_i8_skinny_bp(
   if (EPI == kEpiF32 && ep.bias != nullptr)
     bj = ep.bias[ep.bias_len > 1 ? n : 0];
   if (EPI != kEpiI32) {
-    sj = ep.a_scale[0] * ep.b_scale[ep.b_scale_len == 1 ? 0 : n];
+    sj = (DQ ? dq_scale : ep.a_scale[0]) *
+         ep.b_scale[ep.b_scale_len == 1 ? 0 : n];
     if (EPI == kEpiQ8) {
       sj = sj / ep.y_scale[0];
       yz = load_zp_i32(ep.y_zp, ep.y_unsigned, 0);
@@ -1302,7 +1375,9 @@ __global__ __launch_bounds__(512) void k_gemm_i8_skinny_bp(
     for (int w = 0; w < WAVES; ++w)
       y += (uint32_t)part[w][r][lane];
     int32_t da = oa, rs = 0;
-    if (ep.a_zp_len > 0)
+    if (DQ)
+      da = oa - dq_zp;
+    else if (ep.a_zp_len > 0)
       da = oa - load_zp_i32(ep.a_zp, A_OFF, ep.a_zp_len > 1 ? m : 0);
     if (need_rs) {
 #pragma unroll
@@ -1428,11 +1503,21 @@ hipError_t gemm_launch_cfg(
   const char *force = getenv("OM_MI355X_GEMM_TILE");
   const uint8_t *A = (const uint8_t *)g.A;
   const int M = (int)g.M, N = (int)g.N, K = (int)g.K;
+  if (g.X) {
+    // rows quantized inside the kernel (the caller asked gemm_quantizes_rows)
+    if (A_MODE != 2 || !gemm_quantizes_rows(g.M, g.K, g.X))
+      return hipErrorInvalidValue;
+    if constexpr (A_MODE == 2)
+      k_gemm_i8_skinny_bp<2, EPI, true>
+          <<<dim3((unsigned)((g.N + 31) / 32)), 512, 0, st>>>(
+              nullptr, g.X, g.Bp, M, N, K, Kpad, ep);
+    return hipGetLastError();
+  }
   if (g.M <= 32 && g.K > 0 && g.K % 16 == 0 && ((((uintptr_t)g.A) & 15) == 0) &&
       !(force && force[0])) {
-    k_gemm_i8_skinny_bp<A_MODE, EPI>
+    k_gemm_i8_skinny_bp<A_MODE, EPI, false>
         <<<dim3((unsigned)((g.N + 31) / 32)), 512, 0, st>>>(
-            A, g.Bp, M, N, K, Kpad, ep);
+            A, nullptr, g.Bp, M, N, K, Kpad, ep);
     return hipGetLastError();
   }
   const int tiles_m = (int)((g.M + 127) / 128);
@@ -1519,6 +1604,13 @@ hipError_t launch_pack_b(hipStream_t s, const void *B, bool b_unsigned,
   return hipGetLastError();
 }
 
+bool gemm_quantizes_rows(int64_t M, int64_t K, const void *x) {
+  const char *force = getenv("OM_MI355X_GEMM_TILE");
+  return M >= 1 && M <= 32 && K > 0 && K % 16 == 0 &&
+         M * K <= kSkinnyDqBytes && ((((uintptr_t)x) & 15) == 0) &&
+         !(force && force[0]);
+}
+
 hipError_t launch_gemm(hipStream_t s, const GemmArgs &g) {
   if (g.M == 0 || g.N == 0)
     return hipSuccess;
@@ -1544,7 +1636,7 @@ hipError_t launch_gemm(hipStream_t s, const GemmArgs &g) {
   ep.b_unsigned = g.b_unsigned;
   ep.y_unsigned = g.y_unsigned;
   ep.narrow = (int)g.narrow;
-  const int a_mode = g.a_preshifted ? 2 : (g.a_unsigned ? 1 : 0);
+  const int a_mode = (g.X || g.a_preshifted) ? 2 : (g.a_unsigned ? 1 : 0);
   switch (a_mode) {
   case 0:
     return gemm_launch_epi<0>(s, g, ep, Kpad);

@@ -64,6 +64,10 @@ hipError_t launch_pack_b(hipStream_t s, const void *B, bool b_unsigned,
     int64_t K, int64_t N, int8_t *Bp, int32_t *colsum);
 
 struct GemmArgs {
+  // If set (M <= 32 only, see gemm_quantizes_rows): the activation as f32
+  // [M,K]; the kernel quantizes it itself as DynamicQuantizeLinear would
+  // (A, a_zp and a_scale are then not read).
+  const float *X;
   const void *A;       // [M,K] row-major, u8 or i8
   bool a_unsigned;     // A holds u8
   bool a_preshifted;   // A already holds (u8 - 128) as int8; offsets as for u8
@@ -93,7 +97,61 @@ struct GemmArgs {
 
 hipError_t launch_gemm(hipStream_t s, const GemmArgs &g);
 
+// Whether launch_gemm can take an f32 activation of this shape in GemmArgs::X.
+bool gemm_quantizes_rows(int64_t M, int64_t K, const void *x);
+
 // Fill n 32-bit words with v.
 hipError_t launch_fill_u32(hipStream_t s, uint32_t *p, int64_t n, uint32_t v);
+
+#if defined(__HIPCC__)
+// ---- device arithmetic shared by the quantize and GEMM kernels ------------
+// One element of QuantizeLinear, operation for operation as the reference's
+// generated code (src/Conversion/ONNXToKrnl/Quantization/QuantizeLinear.cpp
+// :119-144): IEEE divide, round half to even, separate add of the zero point,
+// maxnum then minnum (NaN -> lower bound), float -> integer.
+template <bool SIGNED, bool HAS_ZP>
+__device__ __forceinline__ uint32_t quant_one(float x, float s, float zpf) {
+  float t = x / s;
+  float r = __builtin_rintf(t);
+  if (HAS_ZP)
+    r = r + zpf;
+  if (SIGNED) {
+    float c = __builtin_fminf(__builtin_fmaxf(r, -128.0f), 127.0f);
+    return (uint32_t)((int32_t)c) & 0xFFu;
+  }
+  float c = __builtin_fminf(__builtin_fmaxf(r, 0.0f), 255.0f);
+  return (uint32_t)c;
+}
+
+// minnum / maxnum from +inf / -inf (src/Conversion/ONNXToKrnl/Math/
+// Reduction.cpp:529-548); the order of a min / max reduction does not change
+// its value, so lanes, waves and blocks may combine in any order.
+__device__ __forceinline__ float wave_min(float v) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1)
+    v = __builtin_fminf(v, __shfl_xor(v, off, 64));
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1)
+    v = __builtin_fmaxf(v, __shfl_xor(v, off, 64));
+  return v;
+}
+
+// Scale and zero point of DynamicQuantizeLinear from min / max
+// (src/Conversion/ONNXToKrnl/Quantization/DynamicQuantizeLinear.cpp:43-84).
+__device__ __forceinline__ void dynamic_params(
+    float xmin, float xmax, float &scale, float &zpf) {
+  const float mx = __builtin_fmaxf(xmax, 0.0f);
+  const float mn = __builtin_fminf(xmin, 0.0f);
+  const float xdiff = mx - mn;
+  const float bound = 255.0f - 0.0f;
+  scale = xdiff / bound;
+  const float inter = 0.0f - mn / scale;
+  const float sat = __builtin_fminf(__builtin_fmaxf(inter, 0.0f), 255.0f);
+  zpf = __builtin_rintf(sat);
+}
+#endif
 
 } // namespace om

@@ -44,20 +44,6 @@ __device__ __forceinline__ float load_zp_f32(const void *zp, int64_t i) {
 }
 
 template <bool SIGNED, bool HAS_ZP>
-__device__ __forceinline__ uint32_t quant_one(float x, float s, float zpf) {
-  float t = x / s;
-  float r = __builtin_rintf(t);
-  if (HAS_ZP)
-    r = r + zpf;
-  if (SIGNED) {
-    float c = __builtin_fminf(__builtin_fmaxf(r, -128.0f), 127.0f);
-    return (uint32_t)((int32_t)c) & 0xFFu;
-  }
-  float c = __builtin_fminf(__builtin_fmaxf(r, 0.0f), 255.0f);
-  return (uint32_t)c;
-}
-
-template <bool SIGNED, bool HAS_ZP>
 __device__ __forceinline__ uint32_t quant_four(
     f4a v, float s, float zpf, uint32_t flip) {
   uint32_t b0 = quant_one<SIGNED, HAS_ZP>(v.x, s, zpf);
@@ -492,22 +478,6 @@ __global__ __launch_bounds__(kThreads) void k_dequant_general(
 }
 
 // ---- DynamicQuantizeLinear: min / max reduction ---------------------------
-// minnum / maxnum from +inf / -inf (src/Conversion/ONNXToKrnl/Math/
-// Reduction.cpp:529-548); the order of a min / max reduction does not change
-// its value, so lanes, waves and blocks may combine in any order.
-__device__ __forceinline__ float wave_min(float v) {
-#pragma unroll
-  for (int off = 32; off >= 1; off >>= 1)
-    v = __builtin_fminf(v, __shfl_xor(v, off, 64));
-  return v;
-}
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int off = 32; off >= 1; off >>= 1)
-    v = __builtin_fmaxf(v, __shfl_xor(v, off, 64));
-  return v;
-}
-
 __device__ __forceinline__ void block_minmax(float &lo, float &hi) {
   __shared__ float s_lo[kThreads / 64], s_hi[kThreads / 64];
   lo = wave_min(lo);
@@ -526,20 +496,6 @@ __device__ __forceinline__ void block_minmax(float &lo, float &hi) {
     hi = __builtin_fmaxf(hi, s_hi[w]);
   }
   __syncthreads();
-}
-
-// Scale and zero point from min / max
-// (src/Conversion/ONNXToKrnl/Quantization/DynamicQuantizeLinear.cpp:43-84).
-__device__ __forceinline__ void dynamic_params(
-    float xmin, float xmax, float &scale, float &zpf) {
-  const float mx = __builtin_fmaxf(xmax, 0.0f);
-  const float mn = __builtin_fminf(xmin, 0.0f);
-  const float xdiff = mx - mn;
-  const float bound = 255.0f - 0.0f;
-  scale = xdiff / bound;
-  const float inter = 0.0f - mn / scale;
-  const float sat = __builtin_fminf(__builtin_fmaxf(inter, 0.0f), 255.0f);
-  zpf = __builtin_rintf(sat);
 }
 
 __global__ __launch_bounds__(kThreads) void k_minmax_params(

@@ -1315,16 +1315,21 @@ void om_mi355x_DynQuantMatMulDequant(OMTensor *y_t, const OMTensor *x_t,
   if (!call.ok)
     return;
   const float *dx = (const float *)call.in(x);
-  // Quantized activations stay on the GPU, stored as (u8 - 128) so the GEMM
-  // stages them without a per-byte fix-up.
-  uint8_t *aq = (uint8_t *)call.temp((size_t)M * K);
-  call.used_dql = true;
-  if (call.ok)
-    call.check(launch_dynamic_quantize(call.c.stream, call.c.dql, dx, M * K,
-                   aq, call.c.dql_scale, call.c.dql_zp, true),
-        "dynamic quantize");
   GemmArgs g = {};
-  g.A = aq;
+  if (call.ok && gemm_quantizes_rows(M, K, dx)) {
+    // A few rows (decode): the GEMM kernel quantizes them itself.
+    g.X = dx;
+  } else {
+    // Quantized activations stay on the GPU, stored as (u8 - 128) so the GEMM
+    // stages them without a per-byte fix-up.
+    uint8_t *aq = (uint8_t *)call.temp((size_t)M * K);
+    call.used_dql = true;
+    if (call.ok)
+      call.check(launch_dynamic_quantize(call.c.stream, call.c.dql, dx, M * K,
+                     aq, call.c.dql_scale, call.c.dql_zp, true),
+          "dynamic quantize");
+    g.A = aq;
+  }
   g.a_unsigned = true;
   g.a_preshifted = true;
   g.b_unsigned = b.dtype == OM_MI355X_TYPE_UINT8;

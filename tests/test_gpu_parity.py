@@ -338,6 +338,45 @@ def test_fused_epilogue_with_bias(rt, oracle, M, K, N):
         rt.MatMulIntegerDequant(A, B, az, None, a_s, bs, np.zeros(N + 1, np.float32))
 
 
+def test_few_rows_quantized_inside_the_gemm(rt, oracle):
+    """With at most 32 rows and 32 Ki elements (a decode step) the fused layer
+    is one launch: the weight-streaming GEMM quantizes the activation rows
+    itself.  Same bits as DynamicQuantizeLinear -> MatMulInteger -> Cast -> Mul
+    (-> Add): scale and zero point over the whole activation, signed and
+    unsigned weights, weight zero points, K a multiple of 16 only, constant,
+    all-negative and extreme activations."""
+    rng = np.random.default_rng(77)
+    shapes = [(1, 4096, 1000), (4, 4096, 300), (8, 4096, 64), (3, 16, 33), (32, 1024, 96),
+              (5, 1008, 257), (1, 64, 7), (17, 1920, 130), (2, 16384, 40)]
+    for i, (M, K, N) in enumerate(shapes):
+        x = rng.normal(0, 1 + i, (M, K)).astype(np.float32)
+        if i == 2:
+            x[:] = np.float32(2.5)                      # constant: max adjusted to include 0
+        if i == 3:
+            x = -np.abs(x)                              # all negative: zero point 255
+        if i == 4:
+            x[3, 5] = np.float32(3e38)
+        bdt = np.uint8 if i % 2 else np.int8
+        B = _rand_q(rng, bdt, (K, N))
+        bz = _rand_q(rng, bdt, (N,)) if i % 3 == 0 else None
+        bs = rng.uniform(1e-3, 1e-2, N if i % 4 else 1).astype(np.float32)
+        bias = rng.normal(0, 3, N).astype(np.float32) if i % 2 == 0 else None
+        xq, xs, xz = oracle.dynamic_quantize_linear(x)
+        want = oracle.dequant_epilogue(oracle.matmul_integer(xq, B, xz, bz), xs, bs)
+        if bias is not None:
+            want = want + bias
+        got = rt.DynQuantMatMulDequant(x, B, bz, bs, bias)
+        assert same_f32(got, want), (M, K, N)
+    # one element more than the kernel takes: the two-launch path, same result
+    M, K, N = 3, 10928, 50
+    x = rng.normal(0, 1, (M, K)).astype(np.float32)
+    B = _rand_q(rng, np.int8, (K, N))
+    bs = rng.uniform(1e-3, 1e-2, N).astype(np.float32)
+    xq, xs, xz = oracle.dynamic_quantize_linear(x)
+    want = oracle.dequant_epilogue(oracle.matmul_integer(xq, B, xz, None), xs, bs)
+    assert same_f32(rt.DynQuantMatMulDequant(x, B, None, bs), want)
+
+
 def test_empty_tensors(rt, oracle):
     """A dynamic dimension can be 0 at run time: every op then returns an empty
     result (or, for K = 0, the value of an empty sum) without launching on
