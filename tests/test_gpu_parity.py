@@ -658,15 +658,15 @@ def test_host_buffers_kept_on_device_between_ops(rt, oracle):
 
 
 def test_large_host_buffers_both_ways(rt, oracle):
-    """Host tensors of 8 MiB and more cross PCIe in pieces through page-locked
+    """Large host tensors (inputs from 8 MiB, outputs from 4 MiB) cross PCIe in pieces through page-locked
     slots, shared out between the calling thread and helper threads: sizes that
     are no multiple of a piece, both piece sizes, one piece more than there are
     lanes, and two host threads at once (one of them finds the helpers taken)."""
     import threading
     rng = np.random.default_rng(2024)
     sc, zp = np.float32(0.037), np.array(9, np.uint8)
-    sizes = [(2 << 20) + 1, (2 << 20) * 3 + 17, 8 * (1 << 20) + 5, 9_000_001, 12_582_913]
-    for n in sizes:                       # x: 4n bytes in (staged), y: n bytes out (staged from 8 MiB)
+    sizes = [(1 << 20) + 1, (2 << 20) + 1, (2 << 20) * 3 + 17, 8 * (1 << 20) + 5, 9_000_001, 17_000_003]
+    for n in sizes:                       # x: 4n bytes in, y: n bytes out, then the reverse
         x = rng.normal(0, 3, n).astype(np.float32)
         q = rt.QuantizeLinear(x, sc, zp)
         assert np.array_equal(q, oracle.quantize_linear(x, sc, zp)), n
