@@ -838,8 +838,10 @@ inline int stream_grid(
 // of the unrolled loop.  Many short blocks keep more of the tensor's pages in
 // flight than few long ones.  Measured on [8192, 32768] (quantize /
 // dequantize, TB/s): 8 rows per block 6.49 / 5.97, 16 rows 6.23 / 5.94, 32
-// rows 6.02 / 5.59, 64 rows 5.62; on [8191, 32767], where a block walks
-// periods of the flat array: 8 periods 5.72 / 5.11, 16 periods 5.77 / 5.37.
+// rows 6.02 / 5.59, 64 rows 5.62 (dequantize with 4 rows in flight and 4 rows
+// per block: 5.41, with 16 in flight: 5.94); on [8191, 32767], where a block
+// walks periods of the flat array: 8 periods 5.72 / 5.11, 16 periods 5.77 /
+// 5.37.
 void rows_per_block(
     int64_t rows, int trips, int64_t &rpb, int64_t &row_blocks) {
   rpb = trips * kRowUnroll;
