@@ -367,6 +367,20 @@ def test_few_rows_quantized_inside_the_gemm(rt, oracle):
             want = want + bias
         got = rt.DynQuantMatMulDequant(x, B, bz, bs, bias)
         assert same_f32(got, want), (M, K, N)
+    # NaN is ignored by min / max and quantizes to 0; an infinite maximum makes
+    # the scale infinite (every finite element then quantizes to the zero point)
+    for special in (np.nan, np.inf):
+        M, K, N = 2, 256, 70
+        x = rng.normal(0, 1, (M, K)).astype(np.float32)
+        x[1, 17] = special
+        B = _rand_q(rng, np.int8, (K, N))
+        bs = rng.uniform(1e-3, 1e-2, N).astype(np.float32)
+        xq, xs, xz = oracle.dynamic_quantize_linear(x)
+        want = oracle.dequant_epilogue(oracle.matmul_integer(xq, B, xz, None), xs, bs)
+        got = rt.DynQuantMatMulDequant(x, B, None, bs)
+        y, s_, z_ = rt.DynamicQuantizeLinear(x)
+        assert np.array_equal(y, xq) and same_f32(np.float32(s_), xs) and z_ == xz, special
+        assert same_f32(got, want), special
     # one element more than the kernel takes: the two-launch path, same result
     M, K, N = 3, 10928, 50
     x = rng.normal(0, 1, (M, K)).astype(np.float32)
