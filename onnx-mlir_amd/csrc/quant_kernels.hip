@@ -855,21 +855,24 @@ void rows_per_block(
 }
 
 // Launch shape of the periodic kernels: `period` is the column period of the
-// 4-element vectors (C / gcd(C, 4)), repeated until it is a multiple of 8 and
-// spans at least four blocks' worth of threads; grid.x covers one period, grid.y splits the
-// periods, 16 to a block.
+// 4-element vectors (C / gcd(C, 4)), repeated until it is a multiple of 4 and
+// spans at least four blocks' worth of threads; grid.x covers one period,
+// grid.y splits the periods, `trips` * kRowUnroll to a block.  Measured on
+// [8191, 32767] (quantize / dequantize, TB/s) by the multiple the period is
+// padded to and the trips: 8 and 2: 5.76 / 5.36; 4 and 2: 5.93 / 5.49; 4 and
+// 1: 6.02 / 5.20; 2 and 1: 6.03 / 5.26; 1 and 1: 6.01 / 5.14; 1 and 2: 5.89 /
+// 4.90.  A multiple of 4 float4 keeps a thread's accesses at the same
+// position within a 64-byte segment from one period to the next; quantize
+// then does best with one trip per block, dequantize with two.
 struct PeriodicGrid {
   dim3 grid;
   int64_t period;
   int per_block;
 };
-PeriodicGrid periodic_grid(int64_t nvec, int64_t C) {
+PeriodicGrid periodic_grid(int64_t nvec, int64_t C, int trips) {
   const int64_t g = (C % 2 == 0) ? 2 : 1; // C % 4 != 0 here
   int64_t period = C / g;
-  // A multiple of 8 vectors, so that a thread's accesses keep their position
-  // within a 128-byte line from one period to the next and every wave writes
-  // whole lines.
-  while (period % 8 != 0)
+  while (period % 4 != 0)
     period *= 2;
   const int64_t want = 4 * kThreads;
   if (period < want)
@@ -877,7 +880,7 @@ PeriodicGrid periodic_grid(int64_t nvec, int64_t C) {
   const int64_t gx = (period + kThreads - 1) / kThreads;
   const int64_t periods = (nvec + period - 1) / period;
   int64_t per_block, gy;
-  rows_per_block(periods, 2, per_block, gy);
+  rows_per_block(periods, trips, per_block, gy);
   PeriodicGrid pg;
   pg.grid = dim3((unsigned)gx, (unsigned)gy);
   pg.period = period;
@@ -932,7 +935,7 @@ hipError_t quantize_dispatch(hipStream_t st, const float *x, int64_t outer,
   if (inner == 1 && channels > 1 && channels % 4 != 0 &&
       channels < ((int64_t)1 << 31) && ((((uintptr_t)x) & 15) == 0) &&
       ((((uintptr_t)y) & 3) == 0) && (n >> 2) > 0) {
-    const PeriodicGrid pg = periodic_grid(n >> 2, channels);
+    const PeriodicGrid pg = periodic_grid(n >> 2, channels, 1);
     if (has_zp)
       k_quant_periodic<SIGNED, true><<<pg.grid, kThreads, 0, st>>>(
           x, yo, n, (uint32_t)channels, pg.period, scale, zp, pg.per_block);
@@ -998,7 +1001,7 @@ hipError_t dequantize_dispatch(hipStream_t st, const void *x, int64_t outer,
   if (KIND != kI32 && inner == 1 && channels > 1 && channels % 4 != 0 &&
       channels < ((int64_t)1 << 31) && ((((uintptr_t)x) & 3) == 0) &&
       ((((uintptr_t)y) & 15) == 0) && (n >> 2) > 0) {
-    const PeriodicGrid pg = periodic_grid(n >> 2, channels);
+    const PeriodicGrid pg = periodic_grid(n >> 2, channels, 2);
     if (has_zp)
       k_dequant8_periodic<(KIND == kI32 ? kU8 : KIND), true>
           <<<pg.grid, kThreads, 0, st>>>((const uint8_t *)x, y, n,
