@@ -1402,7 +1402,7 @@ template <bool B_UNSIGNED>
 __global__ __launch_bounds__(256) void k_pack_b(const uint8_t *__restrict__ B,
     int64_t K, int64_t N, int KT, int8_t *__restrict__ Bp,
     int32_t *__restrict__ colsum) {
-  __shared__ uint8_t tile[PT][PT + 4];
+  __shared__ __attribute__((aligned(16))) uint8_t tile[PT][PT + 4];
   const int ks = blockIdx.y; // K step of 64
   const int64_t k0 = (int64_t)ks * PT;
   const int64_t n0 = (int64_t)blockIdx.x * PT;
@@ -1412,15 +1412,31 @@ __global__ __launch_bounds__(256) void k_pack_b(const uint8_t *__restrict__ B,
     const int kr = tid >> 2;
     const int nc = (tid & 3) * 16;
     const int64_t k = k0 + kr;
-#pragma unroll
-    for (int b = 0; b < 16; ++b) {
-      const int64_t n = n0 + nc + b;
-      uint8_t v = B_UNSIGNED ? 0x80 : 0;
-      if (k < K && n < N)
-        v = B[k * N + n];
+    // Rows that start on 16-byte boundaries (N % 16 == 0, aligned B): one
+    // 16-byte load per thread; otherwise, and at the edges, byte by byte.
+    const bool rows_aligned = ((N & 15) == 0) && ((((uintptr_t)B) & 15) == 0);
+    if (rows_aligned && k < K && n0 + nc + 16 <= N) {
+      v4i q = *(const v4i *)(B + k * N + n0 + nc);
       if (B_UNSIGNED)
-        v ^= 0x80;
-      tile[kr][nc + b] = v;
+        q ^= (v4i){(int)0x80808080, (int)0x80808080, (int)0x80808080,
+            (int)0x80808080};
+      // row stride 68 and nc % 16 == 0: 4-byte aligned
+      uint32_t *dst = (uint32_t *)&tile[kr][nc];
+      dst[0] = (uint32_t)q.x;
+      dst[1] = (uint32_t)q.y;
+      dst[2] = (uint32_t)q.z;
+      dst[3] = (uint32_t)q.w;
+    } else {
+#pragma unroll
+      for (int b = 0; b < 16; ++b) {
+        const int64_t n = n0 + nc + b;
+        uint8_t v = B_UNSIGNED ? 0x80 : 0;
+        if (k < K && n < N)
+          v = B[k * N + n];
+        if (B_UNSIGNED)
+          v ^= 0x80;
+        tile[kr][nc + b] = v;
+      }
     }
   }
   __syncthreads();
