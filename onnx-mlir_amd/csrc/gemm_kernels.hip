@@ -241,20 +241,38 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TM][TN],
         ((uint32_t)(4 * lh) * (uint32_t)N + (uint32_t)l32) * (uint32_t)ES;
     // One element: row tile i, register r (row 8*(r/4) + 4*lh + r%4 of the
     // tile), column tile j.  RS: add the row-sum term.
-    auto emit = [&](auto rs_c, int i, int r, int j, int32_t rs_row,
-                    char *rowp) {
+    auto emit = [&](auto rs_c, auto stream_c, int i, int r, int j,
+                    int32_t rs_row, char *rowp) {
       uint32_t y = (uint32_t)acc[i][j][r] + cj[j];
       if (decltype(rs_c)::value)
         y += (uint32_t)db[j] * (uint32_t)rs_row;
       char *const q = rowp + loff + (uint32_t)(j * 32 * ES);
       // Streaming stores: the result is not read again by this kernel, and
       // keeping it out of the way in L2 leaves the A and Bp panels cached for
-      // the blocks still in their K loop (measured faster).
+      // the blocks still in their K loop (6 % faster on 4096x768x3072) -- but
+      // only when a wave's 128-byte row pieces are whole lines.  With a row
+      // pitch that is no multiple of 128 bytes every piece straddles two
+      // lines, and streaming the parts costs far more than letting L2 put
+      // the lines together (N = 3070: 28.0 us streaming, 19.4 us plain).
+      // (The streaming hint lives in the store's memory operand, which the
+      // compiler's tail merging does not compare: without the marker below
+      // it folds the two variants into one and drops the hint.)
+      constexpr bool kStream = decltype(stream_c)::value;
       if (EPI == kEpiI32) {
-        __builtin_nontemporal_store((int32_t)y, (int32_t *)q);
+        if (kStream) {
+          __builtin_nontemporal_store((int32_t)y, (int32_t *)q);
+        } else {
+          *(int32_t *)q = (int32_t)y;
+          asm volatile("; plain store");
+        }
       } else if (EPI == kEpiF32) {
-        __builtin_nontemporal_store(
-            (float)(int32_t)y * sj[j] + bj[j], (float *)q);
+        const float f = (float)(int32_t)y * sj[j] + bj[j];
+        if (kStream) {
+          __builtin_nontemporal_store(f, (float *)q);
+        } else {
+          *(float *)q = f;
+          asm volatile("; plain store");
+        }
       } else {
         const float f = (float)(int32_t)y * sj[j];
         int32_t v =
@@ -267,7 +285,7 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TM][TN],
         *(uint8_t *)q = (uint8_t)(v & 0xFF);
       }
     };
-    auto whole = [&](auto rs_c) {
+    auto whole = [&](auto rs_c, auto stream_c) {
       // Whole grid inside the matrix: no bounds tests, and every address is
       // (scalar row base) + (one 32-bit lane offset) + constant, so a store
       // costs the few vector instructions that produce its value.
@@ -282,15 +300,23 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TM][TN],
               (int64_t)(i * 32 + 8 * (r >> 2) + (r & 3)) * N * (int64_t)ES;
 #pragma unroll
           for (int j = 0; j < TN; ++j)
-            emit(rs_c, i, r, j, rs_row, base + rowb);
+            emit(rs_c, stream_c, i, r, j, rs_row, base + rowb);
         }
       }
     };
     if (full) {
-      if (has_rs)
-        whole(std::true_type{});
-      else
-        whole(std::false_type{});
+      const bool whole_lines = ((int64_t)N * ES) % 128 == 0;
+      if (has_rs) {
+        if (whole_lines)
+          whole(std::true_type{}, std::true_type{});
+        else
+          whole(std::true_type{}, std::false_type{});
+      } else {
+        if (whole_lines)
+          whole(std::false_type{}, std::true_type{});
+        else
+          whole(std::false_type{}, std::false_type{});
+      }
       return;
     }
 #pragma unroll
