@@ -266,6 +266,66 @@ __global__ __launch_bounds__(kThreads) void k_quant_periodic(
 // One block row per (outer, channel) pair; the scale is uniform over a run of
 // `inner` elements.  Used when the axis is not the innermost dimension, and as
 // the fallback for misaligned per-tensor buffers.
+// ---- per-axis, axis not innermost, inner % 4 == 0 -------------------------
+// [outer, channels, inner] with the axis in the middle (per-channel scales of
+// an NCHW tensor): a slab of `inner` consecutive elements shares one scale and
+// the slabs lie back to back, so the tensor is walked as the flat array of
+// float4 it is.  A block takes kThreads * kUnroll consecutive float4 in one
+// trip; a thread finds the slab and channel of its first float4 by division
+// and steps on from there (kThreads float4 further = `adv` whole slabs and
+// `rem` float4), so that the other three cost a few integer operations.
+struct SlabStep {
+  uint32_t iv;       // float4 per slab
+  uint32_t channels;
+  uint32_t adv, rem; // kThreads == adv * iv + rem
+};
+
+__device__ __forceinline__ void slab_advance(
+    const SlabStep &st, uint32_t &col, uint32_t &c) {
+  col += st.rem;
+  uint32_t add = st.adv;
+  if (col >= st.iv) {
+    col -= st.iv;
+    ++add;
+  }
+  c += add;
+  if (c >= st.channels)
+    c %= st.channels;
+}
+
+template <bool SIGNED, bool HAS_ZP>
+__global__ __launch_bounds__(kThreads) void k_quant_slabs(
+    const float *__restrict__ x, uint8_t *__restrict__ y, uint32_t nvec,
+    SlabStep st, const float *__restrict__ scale,
+    const void *__restrict__ zp) {
+  const uint32_t first = blockIdx.x * (uint32_t)(kThreads * kUnroll) + threadIdx.x;
+  if (first >= nvec)
+    return;
+  const uint32_t slab = first / st.iv;
+  uint32_t col = first - slab * st.iv;
+  uint32_t c = slab % st.channels;
+  const f4a *__restrict__ x4 = (const f4a *)x;
+  uint32_t *__restrict__ y4 = (uint32_t *)y;
+  f4a v[kUnroll];
+  float s[kUnroll], z[kUnroll];
+#pragma unroll
+  for (int j = 0; j < kUnroll; ++j) {
+    const uint32_t idx = first + j * kThreads;
+    if (idx < nvec) {
+      v[j] = __builtin_nontemporal_load(&x4[idx]);
+      s[j] = scale[c];
+      z[j] = HAS_ZP ? load_zp_f32<SIGNED>(zp, c) : 0.0f;
+    }
+    slab_advance(st, col, c);
+  }
+#pragma unroll
+  for (int j = 0; j < kUnroll; ++j) {
+    const uint32_t idx = first + j * kThreads;
+    if (idx < nvec)
+      y4[idx] = quant_four<SIGNED, HAS_ZP>(v[j], s[j], z[j], 0u);
+  }
+}
+
 template <bool SIGNED, bool HAS_ZP>
 __global__ __launch_bounds__(kThreads) void k_quant_general(
     const float *__restrict__ x, uint8_t *__restrict__ y, int64_t channels,
@@ -498,6 +558,46 @@ __global__ __launch_bounds__(kThreads) void k_dequant8_periodic(
 }
 
 // Any element kind, [outer, channels, inner]: one element per lane.
+// The dequantize counterpart of k_quant_slabs (8-bit input).
+template <int KIND, bool HAS_ZP>
+__global__ __launch_bounds__(kThreads) void k_dequant8_slabs(
+    const uint8_t *__restrict__ x, float *__restrict__ y, uint32_t nvec,
+    SlabStep st, const float *__restrict__ scale,
+    const void *__restrict__ zp) {
+  const uint32_t first = blockIdx.x * (uint32_t)(kThreads * kUnroll) + threadIdx.x;
+  if (first >= nvec)
+    return;
+  const uint32_t slab = first / st.iv;
+  uint32_t col = first - slab * st.iv;
+  uint32_t c = slab % st.channels;
+  const uint32_t *__restrict__ x4 = (const uint32_t *)x;
+  f4a *__restrict__ y4 = (f4a *)y;
+  uint32_t w[kUnroll];
+  float s[kUnroll], z[kUnroll];
+#pragma unroll
+  for (int j = 0; j < kUnroll; ++j) {
+    const uint32_t idx = first + j * kThreads;
+    if (idx < nvec) {
+      w[j] = __builtin_nontemporal_load(&x4[idx]);
+      s[j] = scale[c];
+      z[j] = HAS_ZP ? load_q_zp_f32<KIND>(zp, c) : 0.0f;
+    }
+    slab_advance(st, col, c);
+  }
+#pragma unroll
+  for (int j = 0; j < kUnroll; ++j) {
+    const uint32_t idx = first + j * kThreads;
+    if (idx < nvec) {
+      f4a o;
+      o.x = dq_one<HAS_ZP>(q_to_f32<KIND>(w[j]), s[j], z[j]);
+      o.y = dq_one<HAS_ZP>(q_to_f32<KIND>(w[j] >> 8), s[j], z[j]);
+      o.z = dq_one<HAS_ZP>(q_to_f32<KIND>(w[j] >> 16), s[j], z[j]);
+      o.w = dq_one<HAS_ZP>(q_to_f32<KIND>(w[j] >> 24), s[j], z[j]);
+      __builtin_nontemporal_store(o, &y4[idx]);
+    }
+  }
+}
+
 template <int KIND, bool HAS_ZP>
 __global__ __launch_bounds__(kThreads) void k_dequant_general(
     const void *__restrict__ x, float *__restrict__ y, int64_t channels,
@@ -854,6 +954,22 @@ void rows_per_block(
     row_blocks = 1;
 }
 
+// Whether the slab kernels take [outer, channels, inner]: whole float4 per
+// slab, 32-bit indices, and slabs long enough for the thread's step from one
+// float4 to the next to stay a handful of operations.
+bool slabs_ok(int64_t n, int64_t channels, int64_t inner) {
+  return channels > 1 && inner % 4 == 0 && inner >= 64 &&
+         n < ((int64_t)1 << 32) && channels < ((int64_t)1 << 31);
+}
+SlabStep slab_step(int64_t channels, int64_t inner) {
+  SlabStep st;
+  st.iv = (uint32_t)(inner >> 2);
+  st.channels = (uint32_t)channels;
+  st.adv = (uint32_t)kThreads / st.iv;
+  st.rem = (uint32_t)kThreads % st.iv;
+  return st;
+}
+
 // Launch shape of the periodic kernels: `period` is the column period of the
 // 4-element vectors (C / gcd(C, 4)), repeated until it is a multiple of 4 and
 // spans at least four blocks' worth of threads; grid.x covers one period,
@@ -959,6 +1075,20 @@ hipError_t quantize_dispatch(hipStream_t st, const float *x, int64_t outer,
     return hipGetLastError();
   }
   // General [outer, channels, inner].
+  if (slabs_ok(n, channels, inner) && ((((uintptr_t)x) & 15) == 0) &&
+      ((((uintptr_t)y) & 3) == 0)) {
+    const SlabStep step = slab_step(channels, inner);
+    const uint32_t nvec = (uint32_t)(n >> 2);
+    const unsigned grid =
+        (unsigned)((nvec + kThreads * kUnroll - 1) / (kThreads * kUnroll));
+    if (has_zp)
+      k_quant_slabs<SIGNED, true>
+          <<<grid, kThreads, 0, st>>>(x, yo, nvec, step, scale, zp);
+    else
+      k_quant_slabs<SIGNED, false>
+          <<<grid, kThreads, 0, st>>>(x, yo, nvec, step, scale, zp);
+    return hipGetLastError();
+  }
   const int64_t oc = outer * channels;
   const int64_t gy = oc < 4096 ? oc : 4096;
   int64_t gx = (inner + kThreads - 1) / kThreads;
@@ -1029,6 +1159,20 @@ hipError_t dequantize_dispatch(hipStream_t st, const void *x, int64_t outer,
   if (channels == 1) {
     outer = 1;
     inner = n;
+  }
+  if (KIND != kI32 && slabs_ok(n, channels, inner) &&
+      ((((uintptr_t)x) & 3) == 0) && ((((uintptr_t)y) & 15) == 0)) {
+    const SlabStep step = slab_step(channels, inner);
+    const uint32_t nvec = (uint32_t)(n >> 2);
+    const unsigned grid =
+        (unsigned)((nvec + kThreads * kUnroll - 1) / (kThreads * kUnroll));
+    if (has_zp)
+      k_dequant8_slabs<(KIND == kI32 ? kU8 : KIND), true><<<grid, kThreads, 0, st>>>(
+          (const uint8_t *)x, y, nvec, step, scale, zp);
+    else
+      k_dequant8_slabs<(KIND == kI32 ? kU8 : KIND), false><<<grid, kThreads, 0, st>>>(
+          (const uint8_t *)x, y, nvec, step, scale, zp);
+    return hipGetLastError();
   }
   const int64_t oc = outer * channels;
   const int64_t gy = oc < 4096 ? oc : 4096;

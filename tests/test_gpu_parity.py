@@ -550,6 +550,31 @@ def test_quantize_random_shapes_and_axes(rt, oracle):
         assert np.array_equal(gy, wy) and same_f32(np.float32(gs), ws) and int(gz) == int(wz), tag
 
 
+def test_per_axis_with_inner_slabs(rt, oracle):
+    """Per-channel parameters on an axis that is not the innermost one (NCHW
+    activations, [C_out, C_in] weights on axis 0): slabs of `inner` elements
+    that are whole float4 take the vectorised slab kernels; the shapes cover
+    slabs shorter and longer than a block's stride, few and many channels,
+    tensors that end inside a block, and the scalar fallback (inner % 4 != 0 or
+    inner < 64)."""
+    rng = np.random.default_rng(9090)
+    cases = [((2, 3, 64), 1), ((5, 7, 8, 8), 1), ((3, 4, 100), 1), ((2, 300, 260), 1), ((1, 5, 4096), 1),
+             ((4, 2, 1028), 1), ((64, 1000), 0), ((3, 2, 5, 68), 1), ((2, 33, 7, 12), 1), ((6, 9, 1024), 0),
+             ((2, 3, 62), 1), ((2, 3, 60), 1), ((4, 16, 7, 7), 1), ((1, 1024, 1024), 1)]
+    for shape, axis in cases:
+        C = shape[axis]
+        x = rng.normal(0, 3, shape).astype(np.float32)
+        for qdt, with_zp in ((np.uint8, True), (np.int8, True), (np.uint8, False)):
+            info = np.iinfo(qdt)
+            sc = rng.uniform(0.005, 0.5, C).astype(np.float32)
+            zp = rng.integers(info.min, info.max + 1, C).astype(qdt) if with_zp else None
+            tag = (shape, axis, qdt.__name__, with_zp)
+            wq = oracle.quantize_linear(x, sc, zp, axis=axis, out_dtype=qdt)
+            assert np.array_equal(rt.QuantizeLinear(x, sc, zp, axis=axis), wq), tag
+            assert same_f32(rt.DequantizeLinear(wq, sc, zp, axis=axis),
+                            oracle.dequantize_linear(wq, sc, zp, axis=axis)), tag
+
+
 def test_large_gemm_takes_the_wide_tile_path(rt, oracle):
     # big enough for the heuristic to pick the 128 x 256 B-streaming kernel on its own
     rng = np.random.default_rng(77)
