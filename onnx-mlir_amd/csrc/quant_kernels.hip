@@ -270,10 +270,10 @@ __global__ __launch_bounds__(kThreads) void k_quant_periodic(
 // [outer, channels, inner] with the axis in the middle (per-channel scales of
 // an NCHW tensor): a slab of `inner` consecutive elements shares one scale and
 // the slabs lie back to back, so the tensor is walked as the flat array of
-// float4 it is.  A block takes kThreads * kUnroll consecutive float4 in one
+// float4 it is.  A block takes kThreads * U consecutive float4 in one
 // trip; a thread finds the slab and channel of its first float4 by division
 // and steps on from there (kThreads float4 further = `adv` whole slabs and
-// `rem` float4), so that the other three cost a few integer operations.
+// `rem` float4), so that any further ones cost a few integer operations.
 // float4 per thread: measured on 100 MB tensors, rotating over six of them,
 // quantize / dequantize in TB/s: 1: 5.0 / 5.1; 2: 4.7 / 5.2; 4: 4.1 / 4.75;
 // 8: 4.2 / 4.6.
