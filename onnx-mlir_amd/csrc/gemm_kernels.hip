@@ -1214,8 +1214,9 @@ __global__ __launch_bounds__(256, MINB) void k_gemm_i8_bs(
   gemm_epilogue<TM, TN, A_MODE, EPI>(acc, rsp, m0, ncol0, M, N, K, ep);
 }
 
-// ---- skinny GEMM (M <= 32): weight streaming -------------------------------
-// With at most 32 rows the product is bound by reading the weights once, so
+// ---- skinny GEMM (M <= 64): weight streaming -------------------------------
+// With few rows the product is bound by reading the weights once (32 rows
+// per MFMA row tile, TR = 1 or 2 tiles against the same Bp operands), so
 // the kernel is organised around keeping many KiB of Bp in flight per CU and
 // nothing else: a block owns one 32-column tile, whose operands for all of K
 // are one contiguous run of Bp (2 KiB per K step); its 8 waves take
@@ -1235,13 +1236,16 @@ __global__ __launch_bounds__(256, MINB) void k_gemm_i8_bs(
 // quantized did not shorten it.
 constexpr int kSkinnyDqBytes = 32768;
 
-template <int A_MODE, int EPI, bool DQ>
+template <int A_MODE, int EPI, bool DQ, int TR>
 __global__ __launch_bounds__(512) void k_gemm_i8_skinny_bp(
     const uint8_t *__restrict__ A, const float *__restrict__ X,
     const int8_t *__restrict__ Bp, int M, int N, int K, int Kpad,
     EpiParams ep) {
-  constexpr int WAVES = 8, U = 4;
+  // TR row tiles of 32 (M <= 32 * TR); with two of them a wave keeps half as
+  // many K steps in flight, to stay within the same registers.
+  constexpr int WAVES = 8, U = (TR == 1) ? 4 : 2;
   static_assert(!DQ || A_MODE == 2, "quantized rows are stored minus 128");
+  static_assert(TR == 1 || (TR == 2 && !DQ), "row tiles");
   __shared__ __attribute__((aligned(16))) int32_t part[WAVES][16][64];
   __shared__ int32_t part_rs[WAVES][64];
   // The quantized rows share the memory of the partial sums, which are not
@@ -1312,20 +1316,30 @@ __global__ __launch_bounds__(512) void k_gemm_i8_skinny_bp(
     __syncthreads();
   }
 
-  const bool row_ok = l32 < M;
-  const uint8_t *__restrict__ ap =
-      (DQ ? (const uint8_t *)aq : A) + (int64_t)(row_ok ? l32 : 0) * K;
+  bool row_ok[TR];
+  const uint8_t *__restrict__ ap[TR];
+#pragma unroll
+  for (int t = 0; t < TR; ++t) {
+    row_ok[t] = t * 32 + l32 < M;
+    ap[t] = (DQ ? (const uint8_t *)aq : A) +
+            (int64_t)(row_ok[t] ? t * 32 + l32 : 0) * K;
+  }
   const int8_t *__restrict__ bp = Bp + (int64_t)nt * KT * 2048 + lane * 16;
   constexpr int kFill = (A_MODE == 1) ? (int)0x80808080 : 0;
 
-  v16i acc;
+  v16i acc[TR];
 #pragma unroll
-  for (int r = 0; r < 16; ++r)
-    acc[r] = 0;
+  for (int t = 0; t < TR; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+      acc[t][r] = 0;
   const bool need_rs = ep.need_rowsum;
-  int32_t rsp = 0; // this lane's share of rowsum(A') of row lane % 32
+  int32_t rsp[TR]; // this lane's share of rowsum(A') of row t*32 + lane % 32
+#pragma unroll
+  for (int t = 0; t < TR; ++t)
+    rsp[t] = 0;
   for (int kt = kt_begin; kt < kt_end; kt += U) {
-    v4i a[U][2], b[U][2];
+    v4i a[TR][U][2], b[U][2];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       // steps past this wave's slice reload its last step and are discarded
@@ -1333,10 +1347,13 @@ __global__ __launch_bounds__(512) void k_gemm_i8_skinny_bp(
 #pragma unroll
       for (int sub = 0; sub < 2; ++sub) {
         const int k0 = s * BK + (sub * 2 + lh) * 16;
-        const bool in = row_ok && k0 < K; // K % 16 == 0: a chunk is in or out
-        a[u][sub] = *(const v4i *)(ap + (in ? k0 : 0));
-        if (!in)
-          a[u][sub] = (v4i){kFill, kFill, kFill, kFill};
+#pragma unroll
+        for (int t = 0; t < TR; ++t) {
+          const bool in = row_ok[t] && k0 < K; // K % 16 == 0: a chunk is in or out
+          a[t][u][sub] = *(const v4i *)(ap[t] + (in ? k0 : 0));
+          if (!in)
+            a[t][u][sub] = (v4i){kFill, kFill, kFill, kFill};
+        }
         b[u][sub] = *(const v4i *)(bp + (int64_t)s * 2048 + sub * 1024);
       }
     }
@@ -1345,25 +1362,23 @@ __global__ __launch_bounds__(512) void k_gemm_i8_skinny_bp(
       if (kt + u < kt_end) {
 #pragma unroll
         for (int sub = 0; sub < 2; ++sub) {
-          v4i av = a[u][sub];
-          if (A_MODE == 1)
-            av ^= (v4i){(int)0x80808080, (int)0x80808080, (int)0x80808080,
-                (int)0x80808080};
-          if (need_rs)
-            rsp += frag_rowsum(av);
-          acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(
-              av, b[u][sub], acc, 0, 0, 0);
+#pragma unroll
+          for (int t = 0; t < TR; ++t) {
+            v4i av = a[t][u][sub];
+            if (A_MODE == 1)
+              av ^= (v4i){(int)0x80808080, (int)0x80808080, (int)0x80808080,
+                  (int)0x80808080};
+            if (need_rs)
+              rsp[t] += frag_rowsum(av);
+            acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
+                av, b[u][sub], acc[t], 0, 0, 0);
+          }
         }
       }
     }
   }
   if (DQ)
     __syncthreads(); // every wave is done reading the quantized rows
-#pragma unroll
-  for (int r = 0; r < 16; ++r)
-    part[wave][r][lane] = acc[r];
-  part_rs[wave][lane] = rsp;
-  __syncthreads();
 
   // 32x32 accumulator layout: lane holds column (lane & 31); register r holds
   // row 8*(r/4) + 4*(lane/32) + r%4.  Thread t finishes elements (r, lane)
@@ -1372,48 +1387,60 @@ __global__ __launch_bounds__(512) void k_gemm_i8_skinny_bp(
   const int32_t oa = A_OFF ? 128 : 0;
   const int32_t ob = ep.b_unsigned ? 128 : 0;
   const int n = nt * 32 + l32;
-  if (n >= N)
-    return;
+  const bool col_ok = n < N;
+  const int nc = col_ok ? n : 0; // columns past N: computed on column 0, not stored
   int32_t db = ob;
   if (ep.b_zp_len > 0)
-    db = ob - load_zp_i32(ep.b_zp, ep.b_unsigned, ep.b_zp_len > 1 ? n : 0);
-  const int32_t cs = ep.colsum[n];
+    db = ob - load_zp_i32(ep.b_zp, ep.b_unsigned, ep.b_zp_len > 1 ? nc : 0);
+  const int32_t cs = ep.colsum[nc];
   float sj = 0.0f, bj = -0.0f;
   int32_t yz = 0;
   if (EPI == kEpiF32 && ep.bias != nullptr)
-    bj = ep.bias[ep.bias_len > 1 ? n : 0];
+    bj = ep.bias[ep.bias_len > 1 ? nc : 0];
   if (EPI != kEpiI32) {
     sj = (DQ ? dq_scale : ep.a_scale[0]) *
-         ep.b_scale[ep.b_scale_len == 1 ? 0 : n];
+         ep.b_scale[ep.b_scale_len == 1 ? 0 : nc];
     if (EPI == kEpiQ8) {
       sj = sj / ep.y_scale[0];
       yz = load_zp_i32(ep.y_zp, ep.y_unsigned, 0);
     }
   }
+  // One row tile at a time through the partial-sum buffers.
 #pragma unroll
-  for (int h = 0; h < 2; ++h) {
-    const int r = (tid >> 6) + h * 8;
-    const int m = 8 * (r >> 2) + 4 * lh + (r & 3);
-    if (m >= M)
-      continue;
-    uint32_t y = 0;
+  for (int t = 0; t < TR; ++t) {
+    if (t > 0)
+      __syncthreads(); // the sums of the tile before have been read
 #pragma unroll
-    for (int w = 0; w < WAVES; ++w)
-      y += (uint32_t)part[w][r][lane];
-    int32_t da = oa, rs = 0;
-    if (DQ)
-      da = oa - dq_zp;
-    else if (ep.a_zp_len > 0)
-      da = oa - load_zp_i32(ep.a_zp, A_OFF, ep.a_zp_len > 1 ? m : 0);
-    if (need_rs) {
+    for (int r = 0; r < 16; ++r)
+      part[wave][r][lane] = acc[t][r];
+    part_rs[wave][lane] = rsp[t];
+    __syncthreads();
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int r = (tid >> 6) + h * 8;
+      const int ml = 8 * (r >> 2) + 4 * lh + (r & 3); // row within the tile
+      const int m = t * 32 + ml;
+      if (m >= M || !col_ok)
+        continue;
+      uint32_t y = 0;
 #pragma unroll
       for (int w = 0; w < WAVES; ++w)
-        rs += part_rs[w][m] + part_rs[w][m + 32];
+        y += (uint32_t)part[w][r][lane];
+      int32_t da = oa, rs = 0;
+      if (DQ)
+        da = oa - dq_zp;
+      else if (ep.a_zp_len > 0)
+        da = oa - load_zp_i32(ep.a_zp, A_OFF, ep.a_zp_len > 1 ? m : 0);
+      if (need_rs) {
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w)
+          rs += part_rs[w][ml] + part_rs[w][ml + 32];
+      }
+      y += (uint32_t)da * (uint32_t)cs;
+      y += (uint32_t)db * (uint32_t)rs;
+      y += (uint32_t)K * (uint32_t)da * (uint32_t)db;
+      store_one<EPI>(ep, (int64_t)m * N + n, y, sj, yz, bj);
     }
-    y += (uint32_t)da * (uint32_t)cs;
-    y += (uint32_t)db * (uint32_t)rs;
-    y += (uint32_t)K * (uint32_t)da * (uint32_t)db;
-    store_one<EPI>(ep, (int64_t)m * N + n, y, sj, yz, bj);
   }
 }
 
@@ -1550,16 +1577,28 @@ hipError_t gemm_launch_cfg(
     if (A_MODE != 2 || !gemm_quantizes_rows(g.M, g.K, g.X))
       return hipErrorInvalidValue;
     if constexpr (A_MODE == 2)
-      k_gemm_i8_skinny_bp<2, EPI, true>
+      k_gemm_i8_skinny_bp<2, EPI, true, 1>
           <<<dim3((unsigned)((g.N + 31) / 32)), 512, 0, st>>>(
               nullptr, g.X, g.Bp, M, N, K, Kpad, ep);
     return hipGetLastError();
   }
-  if (g.M <= 32 && g.K > 0 && g.K % 16 == 0 && ((((uintptr_t)g.A) & 15) == 0) &&
+  // 33..64 rows: every block of the weight-streaming kernel reads all of A,
+  // so with many column tiles the 128x64 tile kernel overtakes it from about
+  // 48 rows (K=4096 N=11008: M=33 15.0 against 17.2 us, M=48 18.2 / 17.7,
+  // M=64 21.5 / 17.2; K=11008 N=4096 M=64: 28.5 / 37.8; K=768 N=3072 M=64:
+  // 5.0 / 5.8).
+  const bool skinny_rows =
+      g.M <= 32 || (g.M <= 64 && (g.M <= 48 || (g.N + 63) / 64 <= 128));
+  if (skinny_rows && g.K > 0 && g.K % 16 == 0 && ((((uintptr_t)g.A) & 15) == 0) &&
       !(force && force[0])) {
-    k_gemm_i8_skinny_bp<A_MODE, EPI, false>
-        <<<dim3((unsigned)((g.N + 31) / 32)), 512, 0, st>>>(
-            A, nullptr, g.Bp, M, N, K, Kpad, ep);
+    if (g.M <= 32)
+      k_gemm_i8_skinny_bp<A_MODE, EPI, false, 1>
+          <<<dim3((unsigned)((g.N + 31) / 32)), 512, 0, st>>>(
+              A, nullptr, g.Bp, M, N, K, Kpad, ep);
+    else
+      k_gemm_i8_skinny_bp<A_MODE, EPI, false, 2>
+          <<<dim3((unsigned)((g.N + 31) / 32)), 512, 0, st>>>(
+              A, nullptr, g.Bp, M, N, K, Kpad, ep);
     return hipGetLastError();
   }
   const int tiles_m = (int)((g.M + 127) / 128);

@@ -476,11 +476,11 @@ def test_every_gemm_kernel_configuration(rt, oracle, cfg, monkeypatch):
 
 def test_matmul_random_shapes_around_dispatch_boundaries(rt, oracle):
     """Seeded sweep over shapes that sit on both sides of every dispatch
-    condition (M 16/17, 32/33, 128/129; K a multiple of 64, of 16, of neither;
+    condition (M 16/17, 32/33, 64/65, 128/129; K a multiple of 64, of 16, of neither;
     N around 32, 64, 128, 256), all operand types and zero-point forms, the
     three epilogues."""
     rng = np.random.default_rng(2024)
-    Ms = [1, 2, 15, 16, 17, 31, 32, 33, 64, 127, 128, 129, 200, 257]
+    Ms = [1, 2, 15, 16, 17, 31, 32, 33, 48, 63, 64, 65, 127, 128, 129, 200, 257]
     Ks = [1, 3, 16, 17, 48, 63, 64, 65, 80, 128, 130, 192, 200, 256, 1000]
     Ns = [1, 5, 31, 32, 33, 63, 64, 65, 127, 128, 129, 255, 256, 257, 300]
     for case in range(400):
