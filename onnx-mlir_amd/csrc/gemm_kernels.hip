@@ -1230,11 +1230,14 @@ __global__ __launch_bounds__(256, MINB) void k_gemm_i8_bs(
 // would: minimum and maximum over all of X, scale and zero point from them,
 // the 8-bit values minus 128 into LDS, from where the K loop takes its A
 // operands.  That is 16 KiB of reads from L2 per block for one row of 4096,
-// in place of a launch of its own in front of this one (4096 x 11008
-// weights, whole layer: 1 row 10.6 -> 9.1 us, 4 rows 12.9 -> 11.0 us, 8 rows
-// 17 -> 15.5 us).  Requesting the first Bp operands before the rows are
-// quantized did not shorten it.
-constexpr int kSkinnyDqBytes = 32768;
+// in place of a launch of its own in front of this one.  Whole layer with
+// 4096 x 11008 weights, this kernel against DynamicQuantizeLinear (5.4 us by
+// itself at these sizes) in front of it: 1 row 8.9 / 10.6 us, 4 rows 10.7 /
+// 12.9, 5 rows 11.7 / 13.5, 6 rows 12.9 / 13.6, 8 rows 15.2 / 13.9: the cost
+// grows with every row that every block reads, so the limit is six rows of
+// 4096.  Requesting the first Bp operands before the rows are quantized did
+// not shorten it.
+constexpr int kSkinnyDqBytes = 24576;
 
 template <int A_MODE, int EPI, bool DQ, int TR>
 __global__ __launch_bounds__(512) void k_gemm_i8_skinny_bp(
