@@ -256,6 +256,8 @@ def only_mode(rt, wl, what, steps, warmup):
         return {"only": what, **r}
     if what == "decode":
         return {"only": what, **decode_case(rt, wl, 1, steps, warmup)}
+    if what == "decode16":
+        return {"only": what, **decode_case(rt, wl, 16, steps, warmup)}
     if what == "gemm_prefill_up":
         c = wl.config5("up", M=8)
         r = gemm_case(rt, wl, "config5 prefill up", 2048, 4096, 11008, c["W"], c["w_scale"], steps, warmup, "f32")
@@ -323,7 +325,7 @@ def main():
     ap.add_argument("--extras", default="gemm,fused,decode,qdq", help="which extra groups to measure")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--only", default=None,
-                    choices=["copy", "gemm_ffn_up", "gemm_prefill_up", "fused_ffn_up", "decode",
+                    choices=["copy", "gemm_ffn_up", "gemm_prefill_up", "fused_ffn_up", "decode", "decode16",
                              "quantize_per_axis", "dequantize_per_axis",
                              "quantize_per_tensor", "dequantize_per_tensor", "dynamic_quantize"],
                     help="launch just this kernel --steps times (for rocprofv3 counter runs)")
