@@ -1236,7 +1236,9 @@ __global__ __launch_bounds__(256, MINB) void k_gemm_i8_bs(
 // 12.9, 5 rows 11.7 / 13.5, 6 rows 12.9 / 13.6, 8 rows 15.2 / 13.9: the cost
 // grows with every row that every block reads, so the limit is six rows of
 // 4096.  Requesting the first Bp operands before the rows are quantized did
-// not shorten it.
+// not shorten it, and neither did rows K + 16 bytes apart in LDS (no two
+// lanes' 16-byte reads in the same banks): 4 rows 10.7 -> 11.7 us, 8 rows
+// 15.2 -> 17.1 us with the index arithmetic that takes.
 constexpr int kSkinnyDqBytes = 24576;
 
 template <int A_MODE, int EPI, bool DQ, int TR>
