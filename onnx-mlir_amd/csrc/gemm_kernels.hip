@@ -1241,7 +1241,7 @@ __global__ __launch_bounds__(256, MINB) void k_gemm_i8_bs(
 // 15.2 -> 17.1 us with the index arithmetic that takes.
 constexpr int kSkinnyDqBytes = 24576;
 
-template <int A_MODE, int EPI, bool DQ, int TR>
+template <int A_MODE, int EPI, bool DQ, int TR, bool STG>
 __global__ __launch_bounds__(512) void k_gemm_i8_skinny_bp(
     const uint8_t *__restrict__ A, const float *__restrict__ X,
     const int8_t *__restrict__ Bp, int M, int N, int K, int Kpad,
@@ -1251,12 +1251,35 @@ __global__ __launch_bounds__(512) void k_gemm_i8_skinny_bp(
   constexpr int WAVES = 8, U = (TR == 1) ? 4 : 2;
   static_assert(!DQ || A_MODE == 2, "quantized rows are stored minus 128");
   static_assert(TR == 1 || (TR == 2 && !DQ), "row tiles");
-  __shared__ __attribute__((aligned(16))) int32_t part[WAVES][16][64];
+  static_assert(!(DQ && STG), "quantized rows are in LDS already");
+  // STG: A rows from global memory pass through a piece of LDS private to
+  // the wave: a load instruction takes whole rows of the batch of U steps (CPR
+  // 16-byte chunks each, so every cache line it touches is used completely),
+  // the MFMA operands -- 32 bytes of each of 32 rows -- are read back from
+  // there.  Loading the operands straight from global memory touches 32
+  // lines per instruction for 32 bytes each, and the eight waves' lines do
+  // not stay in the CU's cache until their other three quarters are wanted
+  // (K=4096 N=11008, 32 rows: 12.6 us that way, 9.1 us with loads of whole
+  // lines).  Rows lie CPR * 16 + 16 bytes apart in LDS, which spreads the
+  // rows of one operand read over the banks.  Up to 4 rows the direct loads
+  // are kept: the lanes of the rows that are not there fetch nothing, and
+  // the way through LDS costs more than it saves (1 row 7.7 against 8.3 us,
+  // 4 rows 8.1 / 8.4, 16 rows 9.4 / 8.7, 32 rows 12.6 / 9.6).
+  constexpr int CPR = U * 4;
+  constexpr int kPitch = CPR * 16 + 16;
+  constexpr int kStageWave = 32 * TR * kPitch;
+  constexpr int kPartBytes = WAVES * 16 * 64 * 4;
+  constexpr int kLdsBytes = (STG && WAVES * kStageWave > kPartBytes)
+                                ? WAVES * kStageWave
+                                : kPartBytes;
+  // The staged rows, and the rows quantized here (DQ), share the memory of
+  // the partial sums, which are not written before every wave has left the
+  // K loop.
+  __shared__ __attribute__((aligned(16))) uint8_t lds_raw[kLdsBytes];
+  int32_t(*const part)[16][64] = (int32_t(*)[16][64])lds_raw;
   __shared__ int32_t part_rs[WAVES][64];
-  // The quantized rows share the memory of the partial sums, which are not
-  // written before every wave has left the K loop.
-  static_assert(sizeof(part) >= kSkinnyDqBytes, "quantized rows fit");
-  uint8_t *const aq = (uint8_t *)&part[0][0][0];
+  static_assert(kPartBytes >= kSkinnyDqBytes, "quantized rows fit");
+  uint8_t *const aq = lds_raw;
   __shared__ float s_lo[WAVES], s_hi[WAVES];
 
   const int tid = threadIdx.x;
@@ -1345,22 +1368,64 @@ __global__ __launch_bounds__(512) void k_gemm_i8_skinny_bp(
     rsp[t] = 0;
   for (int kt = kt_begin; kt < kt_end; kt += U) {
     v4i a[TR][U][2], b[U][2];
+    constexpr int RPI = 64 / CPR;       // rows per load instruction
+    constexpr int NLD = 32 * TR / RPI;  // load instructions per batch
+    v4i ar[NLD];
+    if (STG) {
+      const int ld_chunk = lane % CPR;
+      const int step = kt + ld_chunk / 4;
+      const int k0 = step * BK + (ld_chunk & 3) * 16;
+      const bool k_in = step < kt_end && k0 < K; // K % 16 == 0: a chunk is in or out
+#pragma unroll
+      for (int j = 0; j < NLD; ++j) {
+        const int row = j * RPI + lane / CPR;
+        const bool in = k_in && row < M;
+        ar[j] = *(const v4i *)(A + (in ? (int64_t)row * K + k0 : 0));
+        if (!in)
+          ar[j] = (v4i){kFill, kFill, kFill, kFill};
+      }
+    }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       // steps past this wave's slice reload its last step and are discarded
       const int s = (kt + u < kt_end) ? kt + u : kt_end - 1;
 #pragma unroll
       for (int sub = 0; sub < 2; ++sub) {
-        const int k0 = s * BK + (sub * 2 + lh) * 16;
+        if (!STG) {
+          const int k0 = s * BK + (sub * 2 + lh) * 16;
 #pragma unroll
-        for (int t = 0; t < TR; ++t) {
-          const bool in = row_ok[t] && k0 < K; // K % 16 == 0: a chunk is in or out
-          a[t][u][sub] = *(const v4i *)(ap[t] + (in ? k0 : 0));
-          if (!in)
-            a[t][u][sub] = (v4i){kFill, kFill, kFill, kFill};
+          for (int t = 0; t < TR; ++t) {
+            const bool in = row_ok[t] && k0 < K;
+            a[t][u][sub] = *(const v4i *)(ap[t] + (in ? k0 : 0));
+            if (!in)
+              a[t][u][sub] = (v4i){kFill, kFill, kFill, kFill};
+          }
         }
         b[u][sub] = *(const v4i *)(bp + (int64_t)s * 2048 + sub * 1024);
       }
+    }
+    if (STG) {
+      // Through the wave's own piece of LDS into operand order.  The LDS
+      // instructions of a wave execute in order; the fences keep the compiler
+      // from moving the reads above the writes of other lanes, and the next
+      // batch's writes above these reads.
+      uint8_t *const stg = lds_raw + wave * kStageWave;
+#pragma unroll
+      for (int j = 0; j < NLD; ++j)
+        *(v4i *)(stg + (j * RPI + lane / CPR) * kPitch + (lane % CPR) * 16) =
+            ar[j];
+      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+          for (int t = 0; t < TR; ++t)
+            a[t][u][sub] = *(const v4i *)(stg + (t * 32 + l32) * kPitch +
+                                          (u * 4 + sub * 2 + lh) * 16);
+      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+      __builtin_amdgcn_wave_barrier();
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -1382,8 +1447,7 @@ __global__ __launch_bounds__(512) void k_gemm_i8_skinny_bp(
       }
     }
   }
-  if (DQ)
-    __syncthreads(); // every wave is done reading the quantized rows
+  __syncthreads(); // every wave is done reading its rows from LDS
 
   // 32x32 accumulator layout: lane holds column (lane & 31); register r holds
   // row 8*(r/4) + 4*(lane/32) + r%4.  Thread t finishes elements (r, lane)
@@ -1582,28 +1646,27 @@ hipError_t gemm_launch_cfg(
     if (A_MODE != 2 || !gemm_quantizes_rows(g.M, g.K, g.X))
       return hipErrorInvalidValue;
     if constexpr (A_MODE == 2)
-      k_gemm_i8_skinny_bp<2, EPI, true, 1>
+      k_gemm_i8_skinny_bp<2, EPI, true, 1, false>
           <<<dim3((unsigned)((g.N + 31) / 32)), 512, 0, st>>>(
               nullptr, g.X, g.Bp, M, N, K, Kpad, ep);
     return hipGetLastError();
   }
-  // 33..64 rows: every block of the weight-streaming kernel reads all of A,
-  // so with many column tiles the 128x64 tile kernel overtakes it from about
-  // 48 rows (K=4096 N=11008: M=33 15.0 against 17.2 us, M=48 18.2 / 17.7,
-  // M=64 21.5 / 17.2; K=11008 N=4096 M=64: 28.5 / 37.8; K=768 N=3072 M=64:
-  // 5.0 / 5.8).
-  const bool skinny_rows =
-      g.M <= 32 || (g.M <= 64 && (g.M <= 48 || (g.N + 63) / 64 <= 128));
+  // Up to 64 rows the weight-streaming kernel is ahead of every tile kernel
+  // (K=4096 N=11008: M=33 11.6 against 17.2 us, M=48 12.3 / 17.7; K=11008
+  // N=4096 M=64: 15.0 / 37.7; K=768 N=3072 M=64: 4.2 / 6.0).
+  const bool skinny_rows = g.M <= 64;
   if (skinny_rows && g.K > 0 && g.K % 16 == 0 && ((((uintptr_t)g.A) & 15) == 0) &&
       !(force && force[0])) {
-    if (g.M <= 32)
-      k_gemm_i8_skinny_bp<A_MODE, EPI, false, 1>
-          <<<dim3((unsigned)((g.N + 31) / 32)), 512, 0, st>>>(
-              A, nullptr, g.Bp, M, N, K, Kpad, ep);
+    const dim3 grid((unsigned)((g.N + 31) / 32));
+    if (g.M <= 4)
+      k_gemm_i8_skinny_bp<A_MODE, EPI, false, 1, false>
+          <<<grid, 512, 0, st>>>(A, nullptr, g.Bp, M, N, K, Kpad, ep);
+    else if (g.M <= 32)
+      k_gemm_i8_skinny_bp<A_MODE, EPI, false, 1, true>
+          <<<grid, 512, 0, st>>>(A, nullptr, g.Bp, M, N, K, Kpad, ep);
     else
-      k_gemm_i8_skinny_bp<A_MODE, EPI, false, 2>
-          <<<dim3((unsigned)((g.N + 31) / 32)), 512, 0, st>>>(
-              A, nullptr, g.Bp, M, N, K, Kpad, ep);
+      k_gemm_i8_skinny_bp<A_MODE, EPI, false, 2, true>
+          <<<grid, 512, 0, st>>>(A, nullptr, g.Bp, M, N, K, Kpad, ep);
     return hipGetLastError();
   }
   const int tiles_m = (int)((g.M + 127) / 128);
