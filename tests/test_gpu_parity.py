@@ -438,7 +438,8 @@ def test_empty_tensors(rt, oracle):
 
 
 @pytest.mark.parametrize("M,K,N", [(128, 768, 768), (130, 200, 260), (257, 1000, 129), (64, 4096, 192),
-                                   (1, 4096, 1000), (4, 640, 11008), (16, 333, 77), (500, 48, 500)])
+                                   (1, 4096, 1000), (4, 640, 11008), (16, 333, 77), (500, 48, 500),
+                                   (5, 4112, 100), (17, 2064, 70), (40, 11008, 64), (64, 1008, 130)])
 def test_matmulinteger_shapes(rt, oracle, M, K, N):
     rng = np.random.default_rng(M * 7 + K * 3 + N)
     A, B = _rand_q(rng, np.uint8, (M, K)), _rand_q(rng, np.int8, (K, N))
@@ -448,6 +449,34 @@ def test_matmulinteger_shapes(rt, oracle, M, K, N):
     azr, bzc = _rand_q(rng, np.uint8, (M,)), _rand_q(rng, np.int8, (N,))
     want = oracle.matmul_integer(A, B, azr, bzc)
     assert np.array_equal(rt.MatMulInteger(A, B, azr, bzc), want)
+
+
+@pytest.mark.parametrize("adt", [np.int8, np.uint8])
+def test_few_rows_through_lds_all_epilogues(rt, oracle, adt):
+    """5 to 64 rows with K a multiple of 16: the weight-streaming kernel stages
+    the rows of A through LDS.  Several batches of K steps per wave, a last
+    batch that is cut short, K not a multiple of 64, row counts on both sides
+    of the 32-row tile, all three epilogues."""
+    rng = np.random.default_rng(4242 + (adt is np.int8))
+    for M, K, N in ((5, 2048 + 16, 96), (31, 4096 + 336, 40), (32, 3072, 64), (33, 2000, 33),
+                    (47, 6160, 72), (64, 4096, 31)):
+        A, B = _rand_q(rng, adt, (M, K)), _rand_q(rng, np.int8, (K, N))
+        az, bz = _rand_q(rng, adt, (M,)), _rand_q(rng, np.int8, (N,))
+        acc = oracle.matmul_integer(A, B, az, bz)
+        assert np.array_equal(rt.MatMulInteger(A, B, az, bz), acc), (M, K, N)
+        a_s = np.float32(0.0173)
+        bs = rng.uniform(1e-3, 1e-2, N).astype(np.float32)
+        bias = rng.normal(0, 2, N).astype(np.float32)
+        want = oracle.dequant_epilogue(acc, a_s, bs) + bias
+        assert same_f32(rt.MatMulIntegerDequant(A, B, az, bz, a_s, bs, bias), want), (M, K, N)
+        ydt = np.uint8 if M % 2 else np.int8
+        azq, bzq, yz = _rand_q(rng, adt, ()), _rand_q(rng, np.int8, ()), _rand_q(rng, ydt, ())
+        for mode in (rt.WRAP, rt.SATURATE):
+            wq = oracle.qlinear_matmul(A, np.float32(0.02), azq, B, np.float32(0.01), bzq,
+                                       np.float32(40.0), yz, mode)
+            gq = rt.QLinearMatMul(A, np.float32(0.02), azq, B, np.float32(0.01), bzq,
+                                  np.float32(40.0), yz, mode)
+            assert np.array_equal(gq, wq), (M, K, N, mode)
 
 
 @pytest.mark.parametrize("cfg", [0, 1, 2, 3])
