@@ -294,6 +294,12 @@ struct FusedMatMulToMI355X : public OpConversionPattern<ONNXCustomOp> {
     if (!yType)
       return failure();
 
+    // [K, N] weights only: with any other rank the last dimension of the
+    // result would not be dimension 1 of input 1.
+    auto bType = dyn_cast<MemRefType>(inputs[1].getType());
+    if (!bType || bType.getRank() != 2)
+      return failure();
+
     MultiDialectBuilder<IndexExprBuilderForKrnl, MemRefBuilder> create(
         rewriter, loc);
     IndexExprScope scope(create.krnlIE);

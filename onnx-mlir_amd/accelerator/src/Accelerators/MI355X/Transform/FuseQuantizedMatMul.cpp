@@ -88,6 +88,14 @@ bool matchChain(ONNXMulOp mul, Chain &chain) {
     auto matmul = cast.getInput().getDefiningOp<ONNXMatMulIntegerOp>();
     if (!matmul || !matmul->hasOneUse())
       continue;
+    // The fused entry points take a 2-D right-hand side (the weights of a
+    // linear layer) and a left-hand side of rank >= 1, as the unfused
+    // MatMulInteger pattern of the fused epilogue does; a batched B stays
+    // unfused.
+    auto aType = dyn_cast<RankedTensorType>(matmul.getA().getType());
+    auto bType = dyn_cast<RankedTensorType>(matmul.getB().getType());
+    if (!aType || !bType || bType.getRank() != 2 || aType.getRank() < 1)
+      continue;
     // The accumulator tensor must already have the shape of the result: a
     // scale that broadcasts the result to more dimensions is not this chain.
     auto accType = dyn_cast<RankedTensorType>(matmul.getResult().getType());

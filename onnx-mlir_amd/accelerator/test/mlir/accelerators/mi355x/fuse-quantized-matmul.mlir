@@ -98,3 +98,21 @@ func.func @other_association(%a: tensor<8x16xui8>, %w: tensor<16x4xi8>, %azp: te
 // CHECK-NOT:    onnx.Custom
 // CHECK:        onnx.MatMulInteger
 }
+
+// -----
+
+// A batched right-hand side is not a linear layer's weight matrix: the chain
+// is left as it is (the fused entry points take a 2-D B).
+func.func @batched_rhs_is_left_alone(%a: tensor<4x128x64xui8>, %b: tensor<4x64x32xi8>, %azp: tensor<ui8>, %as: tensor<f32>, %bs: tensor<32xf32>) -> tensor<*xf32> {
+  %none = "onnx.NoValue"() {value} : () -> none
+  %acc = "onnx.MatMulInteger"(%a, %b, %azp, %none) : (tensor<4x128x64xui8>, tensor<4x64x32xi8>, tensor<ui8>, none) -> tensor<*xi32>
+  %f = "onnx.Cast"(%acc) {to = f32} : (tensor<*xi32>) -> tensor<*xf32>
+  %s = "onnx.Mul"(%as, %bs) : (tensor<f32>, tensor<32xf32>) -> tensor<*xf32>
+  %y = "onnx.Mul"(%f, %s) : (tensor<*xf32>, tensor<*xf32>) -> tensor<*xf32>
+  return %y : tensor<*xf32>
+// CHECK-LABEL:  func.func @batched_rhs_is_left_alone
+// CHECK:        "onnx.MatMulInteger"
+// CHECK:        "onnx.Cast"
+// CHECK:        "onnx.Mul"
+// CHECK-NOT:    onnx.Custom
+}

@@ -27,17 +27,25 @@ hipError_t launch_dequantize(hipStream_t s, const void *x, QKind xkind,
 // first launch (the kernel leaves it zero), and the per-block slots of the
 // one-launch kernel.
 struct DqlScratch {
-  float *partial_min; // [kDqlMaxBlocks]
-  float *partial_max; // [kDqlMaxBlocks]
+  float *partial_min; // [max_blocks]
+  float *partial_max; // [max_blocks]
   unsigned *counter;  // [16], zeroed once: [0] two-pass arrivals, [8] set if
                       // the exchange of the one-launch kernel ever timed out
   int grid_blocks;    // dql_grid_blocks(), or 0 to disable the one-launch path
   unsigned spin_limit; // polls a thread of the one-launch kernel waits for
                        // another block's result before giving up
-  unsigned long long *grid_slots; // [2 * kDqlMaxBlocks], zeroed once: per
+  unsigned long long *grid_slots; // [2 * max_blocks], zeroed once: per
                       // block (launch number << 32 | float bits) of its min,
                       // then of its max
   unsigned epoch;     // launch number of the one-launch kernel (host side)
+  int max_blocks;     // capacity of partial_min / partial_max and of each half
+                      // of grid_slots (at most kDqlMaxBlocks)
+  // Two-launch path only (sets grid_blocks to 0 for the call).
+  DqlScratch two_launch() const {
+    DqlScratch s = *this;
+    s.grid_blocks = 0;
+    return s;
+  }
 };
 // Blocks of the one-launch DynamicQuantizeLinear kernel that fit the current
 // device at once (0 if it cannot run here).
@@ -50,6 +58,9 @@ constexpr int kDqlMaxBlocks = 4096;
 hipError_t launch_dynamic_quantize(hipStream_t s, DqlScratch &scratch,
     const float *x, int64_t n, uint8_t *y, float *scale, uint8_t *zp,
     bool y_shift);
+
+// Call before destroying a stream that launch_dynamic_quantize was given.
+void dql_forget_stream(hipStream_t s);
 
 // ---- int8 GEMM ------------------------------------------------------------
 // B [K,N] row-major (u8 or i8) -> Bp, Npad * Kpad bytes of int8 in MFMA

@@ -706,8 +706,11 @@ __global__ __launch_bounds__(kThreads) void k_minmax_params(
     // XCD sees them, and the last block reads them with device-scope atomic
     // loads: nothing has to be written back or invalidated in any cache.  The
     // ticket only has to be drawn after this block's two stores have
-    // completed, which the workgroup-scope fence waits for.
+    // completed.  A workgroup-scope release does not wait for that (the
+    // stores and the ticket may travel to different memory channels), so the
+    // wait is explicit: vmcnt(0) returns once both stores are acknowledged.
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
     const unsigned ticket = __hip_atomic_fetch_add(
         counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
@@ -1255,7 +1258,7 @@ hipError_t launch_dynamic_quantize(hipStream_t s, DqlScratch &scratch,
     // (64 Ki elements: 16 blocks 5.4 us, 4 blocks of 4 float4 per thread 7.0,
     // the two launches of the general path 8.1; 512 Ki: 128 blocks 7.2
     // against 8.2 for 256 blocks of 4 per thread; 96 Ki: 6.1 against 8.1).
-    int64_t blocks = scratch.grid_blocks;
+    int64_t blocks = scratch.grid_blocks; // <= scratch.max_blocks
     if (nvec <= total) {
       fn_launch = k_dql_grid<1>;
       blocks = (nvec + kGridThreads - 1) / kGridThreads;
@@ -1267,7 +1270,7 @@ hipError_t launch_dynamic_quantize(hipStream_t s, DqlScratch &scratch,
       const uint32_t flip = y_shift ? 0x80808080u : 0u;
       const unsigned spin_limit = scratch.spin_limit;
       unsigned long long *slot_lo = scratch.grid_slots;
-      unsigned long long *slot_hi = scratch.grid_slots + kDqlMaxBlocks;
+      unsigned long long *slot_hi = scratch.grid_slots + scratch.max_blocks;
       unsigned *failed = scratch.counter + 8;
       // At most one of these kernels is in flight per process: two of them
       // dispatched at the same time from different streams could each hold
@@ -1300,7 +1303,8 @@ hipError_t launch_dynamic_quantize(hipStream_t s, DqlScratch &scratch,
   // A read-only reduction streams fastest with few, long-lived blocks
   // (measured on 1 GiB: 512 blocks 6.3 TB/s for the whole op, 4096 blocks
   // 5.9), the opposite of the kernels that also store.
-  const int grid = stream_grid(n >> 2, kThreads * 8, 512);
+  const int grid = stream_grid(
+      n >> 2, kThreads * 8, scratch.max_blocks < 512 ? scratch.max_blocks : 512);
   k_minmax_params<<<grid, kThreads, 0, s>>>(x, n, scratch.partial_min,
       scratch.partial_max, scratch.counter, scale, zp);
   hipError_t e = hipGetLastError();
@@ -1311,6 +1315,12 @@ hipError_t launch_dynamic_quantize(hipStream_t s, DqlScratch &scratch,
   // the reference adds: it is an integer in [0, 255]).
   return quantize_dispatch<false>(
       s, x, 1, 1, n, scale, zp, y, y_shift ? 0x80808080u : 0u);
+}
+
+void dql_forget_stream(hipStream_t s) {
+  std::lock_guard<std::mutex> lk(g_grid_mutex);
+  if (g_grid_stream == s)
+    g_grid_stream = nullptr; // the caller has synchronised it
 }
 
 hipError_t launch_fill_u32(hipStream_t s, uint32_t *p, int64_t n, uint32_t v) {

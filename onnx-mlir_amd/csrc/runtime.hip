@@ -90,6 +90,10 @@ struct PackedB {
   bool is_unsigned;
 };
 std::unordered_map<const void *, PackedB> g_packed;
+// GPU blocks that left a cache while work on some stream may still read them
+// (a constant re-declared with another shape); freed by om_mi355x_ClearCache
+// after the device has drained.
+std::vector<void *> g_retired;
 
 // Host buffers backed by GPU memory (om_mi355x_KeepOnDevice): start address ->
 // (GPU copy, bytes).  Guarded by g_mem_mutex.
@@ -325,7 +329,7 @@ CopyHelpers *copy_helpers() {
 struct Ctx {
   bool ready = false;
   hipStream_t stream = nullptr;
-  DqlScratch dql = {nullptr, nullptr, nullptr, 0, 0, nullptr, 0};
+  DqlScratch dql = {nullptr, nullptr, nullptr, 0, 0, nullptr, 0, kDqlMaxBlocks};
   float *dql_scale = nullptr; // scale / zero point of the fused path
   uint8_t *dql_zp = nullptr;
   std::multimap<size_t, void *> pool;
@@ -359,6 +363,7 @@ struct Ctx {
     dql.grid_slots = (unsigned long long *)((char *)dql.counter + 256);
     HIP_OK(hipMemset(dql.counter, 0,
         256 + sizeof(unsigned long long) * 2 * kDqlMaxBlocks));
+    dql.max_blocks = kDqlMaxBlocks;
     dql.grid_blocks = dql_grid_blocks();
     dql.spin_limit = 1u << 20; // about a second of polling
     if (const char *v = getenv("OM_MI355X_DQL_SPIN_LIMIT"))
@@ -372,17 +377,25 @@ struct Ctx {
   // Call after the stream has been synchronised.  The one-launch
   // DynamicQuantizeLinear kernel raises a flag if its grid barrier ever timed
   // out (its output is then missing); report that and stop using the kernel.
-  bool dql_barrier_ok() {
+  // Whether a one-launch kernel of this thread gave up since the last check
+  // (call after the stream has been synchronised).  If so the flag is
+  // cleared and the one-launch kernel is not used again by this thread.
+  bool dql_gave_up() {
     if (!ready || dql.grid_blocks == 0)
-      return true;
+      return false;
     unsigned flag = 0;
     if (hipMemcpy(&flag, dql.counter + 8, sizeof(flag),
             hipMemcpyDeviceToHost) != hipSuccess)
-      return true;
+      return false;
     if (!flag)
-      return true;
+      return false;
     (void)hipMemset(dql.counter, 0, 256);
     dql.grid_blocks = 0;
+    return true;
+  }
+  bool dql_barrier_ok() {
+    if (!dql_gave_up())
+      return true;
     fail(EIO, "DynamicQuantizeLinear: the blocks of the one-launch kernel "
               "timed out waiting for one another (grid barrier); its output "
               "was not written");
@@ -515,6 +528,46 @@ struct Ctx {
     pool_bytes = 0;
   }
   std::unordered_map<void *, size_t> taken;
+
+  // A context lives as long as its host thread.  When the thread ends, what
+  // it holds on the GPU goes back to the driver: the idle pool blocks, the
+  // scratch, the page-locked copy slots, the events and the stream (after the
+  // work queued on it).  Buffers handed out by om_mi355x_malloc and backings
+  // declared with om_mi355x_KeepOnDevice are not the thread's and stay.
+  ~Ctx() {
+    if (!ready)
+      return;
+    ready = false;
+    (void)hipStreamSynchronize(stream);
+    {
+      // Backings declared by this thread no longer have a stream to wait for.
+      std::lock_guard<std::mutex> lk(g_mem_mutex);
+      for (auto &kv : g_backed)
+        if (kv.second.stream == stream)
+          kv.second.stream = nullptr;
+    }
+    dql_forget_stream(stream);
+    drop_pool();
+    for (auto &kv : taken)
+      (void)hipFree(kv.first);
+    taken.clear();
+    if (dql.partial_min)
+      (void)hipFree(dql.partial_min);
+    if (lane.ready) {
+      (void)hipHostFree(lane.slot[0]);
+      for (int i = 0; i < CopyLane::kSlots; ++i)
+        (void)hipEventDestroy(lane.ev[i]);
+      (void)hipEventDestroy(lane.done);
+    }
+    if (fork_ev)
+      (void)hipEventDestroy(fork_ev);
+    if (ev0)
+      (void)hipEventDestroy(ev0);
+    if (ev1)
+      (void)hipEventDestroy(ev1);
+    (void)hipStreamDestroy(stream);
+    (void)hipGetLastError();
+  }
 };
 
 thread_local Ctx t_ctx;
@@ -711,25 +764,24 @@ struct Call {
     return p;
   }
 
-  const void *in(const View &v) {
+  // keep_constant: a host buffer declared constant gets a GPU copy that stays
+  // (false: it is staged like any other host tensor, for this call only).
+  const void *in(const View &v, bool keep_constant = true) {
     if (!ok || v.numel == 0)
       return v.data;
     if (void *d = backed_lookup(v.data))
       return d;
     if (is_device_ptr(v.data))
       return v.data;
-    {
+    bool constant = false;
+    if (keep_constant) {
       std::lock_guard<std::mutex> lk(g_mem_mutex);
-      if (g_constants.count(v.data)) {
+      constant = g_constants.count(v.data) != 0;
+      if (constant) {
         auto it = g_const_copies.find(v.data);
         if (it != g_const_copies.end() && it->second.bytes == v.bytes)
           return it->second.dev;
       }
-    }
-    bool constant;
-    {
-      std::lock_guard<std::mutex> lk(g_mem_mutex);
-      constant = g_constants.count(v.data) != 0;
     }
     void *d = nullptr;
     if (constant) {
@@ -750,7 +802,7 @@ struct Call {
           (void)hipFree(d);
           return ins.first->second.dev;
         }
-        (void)hipFree(ins.first->second.dev);
+        g_retired.push_back(ins.first->second.dev); // may still be in use
         ins.first->second = DevCopy{d, v.bytes};
       }
       return d;
@@ -829,6 +881,41 @@ bool is_q8(int dt) {
   return dt == OM_MI355X_TYPE_UINT8 || dt == OM_MI355X_TYPE_INT8;
 }
 
+// DynamicQuantizeLinear on GPU pointers, as part of `call`.  When the call is
+// going to wait for its kernels anyway (a host tensor is involved, or one of
+// the timing modes is on), the wait happens here, and if the blocks of the
+// one-launch kernel gave up waiting for one another the two-launch path runs
+// right away: the outputs are correct when the entry point returns.  A call
+// on GPU tensors only returns without waiting; there a give-up is reported
+// (EIO) at the thread's next synchronisation.
+void run_dql(Call &call, const float *dx, int64_t n, uint8_t *dy, float *ds,
+    uint8_t *dz, bool y_shift) {
+  Ctx &c = call.c;
+  call.check(
+      launch_dynamic_quantize(c.stream, c.dql, dx, n, dy, ds, dz, y_shift),
+      "DynamicQuantizeLinear");
+  if (!call.ok || c.dql.grid_blocks == 0)
+    return;
+  if (!(call.touched_host || sync_every_call() || report_enabled())) {
+    call.used_dql = true;
+    return;
+  }
+  const hipError_t e = hipStreamSynchronize(c.stream);
+  if (e != hipSuccess) {
+    call.check(e, "stream synchronisation");
+    return;
+  }
+  if (c.dql_gave_up()) { // grid_blocks is 0 from here on: two launches
+    fprintf(stderr,
+        "om_mi355x: DynamicQuantizeLinear: the blocks of the one-launch "
+        "kernel timed out waiting for one another; redone with two launches, "
+        "which this thread uses from now on\n");
+    call.check(
+        launch_dynamic_quantize(c.stream, c.dql, dx, n, dy, ds, dz, y_shift),
+        "DynamicQuantizeLinear (two launches)");
+  }
+}
+
 // Splits `shape` around `axis` for a scale of `scale_numel` entries.
 bool axis_split(const View &x, int64_t scale_numel, int64_t axis,
     const char *op, int64_t &outer, int64_t &channels, int64_t &inner) {
@@ -903,7 +990,9 @@ bool packed_b(Call &call, const View &b, int64_t K, int64_t N,
       }
     }
   }
-  const void *db = call.in(b);
+  // A constant B is only ever read here, to be packed: its plain copy on the
+  // GPU lasts for this call, the packed form is the one that stays.
+  const void *db = call.in(b, /*keep_constant=*/false);
   if (!call.ok)
     return false;
   int8_t *pbp;
@@ -933,9 +1022,23 @@ bool packed_b(Call &call, const View &b, int64_t K, int64_t N,
     std::lock_guard<std::mutex> lk(g_mem_mutex);
     auto ins = g_packed.emplace(b.data, PackedB{pbp, pcs, K, N, uns});
     if (!ins.second) {
-      (void)hipFree(ins.first->second.bp);
-      (void)hipFree(ins.first->second.colsum);
-      ins.first->second = PackedB{pbp, pcs, K, N, uns};
+      PackedB &have = ins.first->second;
+      if (have.K == K && have.N == N && have.is_unsigned == uns) {
+        // Another thread packed the same constant first and may already be
+        // computing with its buffers: keep those, drop the ones made here
+        // (nothing but this thread's finished pack kernel has touched them).
+        (void)hipFree(pbp);
+        (void)hipFree(pcs);
+        bp = have.bp;
+        colsum = have.colsum;
+        return true;
+      }
+      // The same address declared constant with another shape: the old
+      // buffers may still be read by work in flight on any stream, so they
+      // are only retired here and freed when the cache is cleared.
+      g_retired.push_back(have.bp);
+      g_retired.push_back(have.colsum);
+      have = PackedB{pbp, pcs, K, N, uns};
     }
   }
   bp = pbp;
@@ -1246,11 +1349,8 @@ void om_mi355x_DynamicQuantizeLinear(OMTensor *y_t, OMTensor *scale_t,
   uint8_t *dy = (uint8_t *)call.out(y);
   float *ds = (float *)call.out(sc);
   uint8_t *dz = (uint8_t *)call.out(zp);
-  call.used_dql = true;
   if (call.ok)
-    call.check(launch_dynamic_quantize(
-                   call.c.stream, call.c.dql, dx, x.numel, dy, ds, dz, false),
-        "DynamicQuantizeLinear");
+    run_dql(call, dx, x.numel, dy, ds, dz, false);
   call.finish();
 }
 
@@ -1322,6 +1422,7 @@ void om_mi355x_DynQuantMatMulDequant(OMTensor *y_t, const OMTensor *x_t,
     return;
   const float *dx = (const float *)call.in(x);
   GemmArgs g = {};
+  g.out = call.out(y); // before the quantization: it decides whether to wait
   if (call.ok && gemm_quantizes_rows(M, K, dx)) {
     // A few rows (decode): the GEMM kernel quantizes them itself.
     g.X = dx;
@@ -1329,11 +1430,8 @@ void om_mi355x_DynQuantMatMulDequant(OMTensor *y_t, const OMTensor *x_t,
     // Quantized activations stay on the GPU, stored as (u8 - 128) so the GEMM
     // stages them without a per-byte fix-up.
     uint8_t *aq = (uint8_t *)call.temp((size_t)M * K);
-    call.used_dql = true;
     if (call.ok)
-      call.check(launch_dynamic_quantize(call.c.stream, call.c.dql, dx, M * K,
-                     aq, call.c.dql_scale, call.c.dql_zp, true),
-          "dynamic quantize");
+      run_dql(call, dx, M * K, aq, call.c.dql_scale, call.c.dql_zp, true);
     g.A = aq;
   }
   g.a_unsigned = true;
@@ -1360,7 +1458,6 @@ void om_mi355x_DynQuantMatMulDequant(OMTensor *y_t, const OMTensor *x_t,
     g.bias = (const float *)call.in(bias);
     g.bias_len = bias.numel;
   }
-  g.out = call.out(y);
   if (call.ok)
     call.check(launch_gemm(call.c.stream, g), op);
   call.finish();
@@ -1375,6 +1472,34 @@ void om_mi355x_MarkConstant(const OMTensor *t) {
   const void *p = omTensorGetDataPtr(t);
   std::lock_guard<std::mutex> lk(g_mem_mutex);
   g_constants.insert(p);
+}
+
+void om_mi355x_UnmarkConstant(const OMTensor *t) {
+  if (!t)
+    return;
+  const void *p = omTensorGetDataPtr(t);
+  void *drop[3] = {nullptr, nullptr, nullptr};
+  {
+    std::lock_guard<std::mutex> lk(g_mem_mutex);
+    g_constants.erase(p);
+    auto c = g_const_copies.find(p);
+    if (c != g_const_copies.end()) {
+      drop[0] = c->second.dev;
+      g_const_copies.erase(c);
+    }
+    auto k = g_packed.find(p);
+    if (k != g_packed.end()) {
+      drop[1] = k->second.bp;
+      drop[2] = k->second.colsum;
+      g_packed.erase(k);
+    }
+  }
+  if (drop[0] || drop[1]) {
+    (void)hipDeviceSynchronize(); // work on any stream may still read them
+    for (void *d : drop)
+      if (d)
+        (void)hipFree(d);
+  }
 }
 
 // The GPU blocks come from the calling thread's pool and go back to it, so a
@@ -1403,7 +1528,7 @@ void om_mi355x_KeepOnDevice(const OMTensor *t) {
     }
   }
   if (old.dev) {
-    if (old.stream != t_ctx.stream)
+    if (old.stream && old.stream != t_ctx.stream)
       (void)hipStreamSynchronize(old.stream);
     t_ctx.adopt(old.dev, old.capacity);
   }
@@ -1432,14 +1557,19 @@ void om_mi355x_Release(const OMTensor *t) {
     t_ctx.adopt(b.dev, b.capacity);
     return;
   }
-  (void)hipStreamSynchronize(b.stream);
+  if (b.stream)
+    (void)hipStreamSynchronize(b.stream);
   (void)hipFree(b.dev);
 }
 
 void om_mi355x_ClearCache(void) {
+  // Cached buffers may be in use on any thread's stream.
   if (t_ctx.ready)
-    (void)hipStreamSynchronize(t_ctx.stream);
+    (void)hipDeviceSynchronize();
   std::lock_guard<std::mutex> lk(g_mem_mutex);
+  for (void *p : g_retired)
+    (void)hipFree(p);
+  g_retired.clear();
   for (auto &kv : g_const_copies)
     (void)hipFree(kv.second.dev);
   g_const_copies.clear();

@@ -85,6 +85,7 @@ def _declare(lib, shim):
         "om_mi355x_QLinearMatMul": [P, P, P, P, P, P, P, P, P, I64],
         "om_mi355x_DynQuantMatMulDequant": [P, P, P, P, P, P],
         "om_mi355x_MarkConstant": [P],
+        "om_mi355x_UnmarkConstant": [P],
         "om_mi355x_KeepOnDevice": [P],
         "om_mi355x_Release": [P],
         "om_mi355x_ClearCache": [],
@@ -241,16 +242,33 @@ def _host(a, dtype=None) -> Tensor:
     return np.ascontiguousarray(a)
 
 
+# Arrays declared constant, by data address: the runtime keys its caches by
+# that address, so the array must stay alive (and its address taken) until
+# unmark_constant or clear_cache.
+_marked = {}
+
+
 def mark_constant(t: Tensor):
-    """Declare that ``t`` never changes (a model constant)."""
+    """Declare that ``t`` never changes (a model constant).  The binding keeps
+    ``t`` alive until :func:`unmark_constant` or :func:`clear_cache`."""
     load()
     with _OMT(t) as h:
         _lib.om_mi355x_MarkConstant(h)
+    _marked[t.ptr if isinstance(t, DeviceArray) else t.ctypes.data] = t
+
+
+def unmark_constant(t: Tensor):
+    """Take the declaration back and drop what the runtime cached for ``t``."""
+    load()
+    with _OMT(t) as h:
+        _lib.om_mi355x_UnmarkConstant(h)
+    _marked.pop(t.ptr if isinstance(t, DeviceArray) else t.ctypes.data, None)
 
 
 def clear_cache():
     load()
     _lib.om_mi355x_ClearCache()
+    _marked.clear()
 
 
 def keep_on_device(t: np.ndarray):

@@ -232,25 +232,48 @@ def test_dynamic_quantize_mid_size_with_nan_and_inf(rt, oracle):
 def test_dynamic_quantize_barrier_timeout_is_reported():
     """The one-launch kernel waits at a grid barrier for a bounded number of polls.
     With the bound forced to zero from the host every block gives up at once (and
-    exits normally); the runtime must report that instead of returning garbage,
-    and must keep working (two-launch path) afterwards."""
+    exits normally).  A call on host tensors waits for its kernels anyway: it
+    must notice, redo the op with two launches and return correct results.  A
+    call on GPU tensors returns without waiting: the give-up is reported at the
+    next synchronisation, and the runtime keeps working afterwards."""
     import subprocess, sys, textwrap
     code = textwrap.dedent("""
         import sys, numpy as np
         sys.path.insert(0, %r)
         import om_mi355x as rt
         x = np.random.default_rng(0).normal(0, 1, (4096, 768)).astype(np.float32)
-        try:
-            rt.DynamicQuantizeLinear(x)
-            print("NO-ERROR")
-        except rt.RuntimeError_ as e:
-            print("ERROR-OK" if "barrier" in str(e) else "WRONG-ERROR %%s" %% e)
-        y, s, z = rt.DynamicQuantizeLinear(x)
         lo, hi = np.float32(min(x.min(), 0)), np.float32(max(x.max(), 0))
-        print("RECOVERED" if np.float32(s) == (hi - lo) / np.float32(255) else "BAD")
+        want_s = (hi - lo) / np.float32(255)
+        mode = sys.argv[1]
+        zf = np.float32(np.rint(np.clip(np.float32(0) - lo / want_s, 0, 255)))
+        want_y = np.clip(np.rint(x / want_s) + zf, 0, 255).astype(np.uint8)
+        if mode == "host":
+            y, s, z = rt.DynamicQuantizeLinear(x)
+            print("FIRST-OK" if np.float32(s) == want_s and np.array_equal(y, want_y) else "FIRST-BAD")
+        elif mode == "fused":
+            # the fused layer goes through the same wait-and-redo
+            b = np.ones((768, 64), np.int8)
+            out = rt.DynQuantMatMulDequant(x, b, None, np.float32(1.0))
+            ref = (want_y.astype(np.int32) - np.int32(zf)) @ b.astype(np.int32)
+            print("FUSED-OK" if np.array_equal(out, ref.astype(np.float32) * (want_s * np.float32(1.0))) else "FUSED-BAD")
+        else:
+            dx = rt.DeviceArray.from_numpy(x)
+            rt.DynamicQuantizeLinear(dx)
+            try:
+                rt.synchronize()
+                print("NO-ERROR")
+            except rt.RuntimeError_ as e:
+                print("ERROR-OK" if "barrier" in str(e) else "WRONG-ERROR %%s" %% e)
+            y, s, z = rt.DynamicQuantizeLinear(dx)
+            rt.synchronize()
+            print("RECOVERED" if np.float32(s.numpy()) == want_s else "BAD")
     """ % os.path.join(os.path.dirname(HERE), "onnx-mlir_amd"))
     env = dict(os.environ, OM_MI355X_DQL_SPIN_LIMIT="0")
-    out = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=110)
+    out = subprocess.run([sys.executable, "-c", code, "host"], env=env, capture_output=True, text=True, timeout=110)
+    assert "FIRST-OK" in out.stdout and "two launches" in out.stderr, out.stdout + out.stderr
+    out = subprocess.run([sys.executable, "-c", code, "fused"], env=env, capture_output=True, text=True, timeout=110)
+    assert "FUSED-OK" in out.stdout and "two launches" in out.stderr, out.stdout + out.stderr
+    out = subprocess.run([sys.executable, "-c", code, "device"], env=env, capture_output=True, text=True, timeout=110)
     assert "ERROR-OK" in out.stdout and "RECOVERED" in out.stdout, out.stdout + out.stderr
 
 
