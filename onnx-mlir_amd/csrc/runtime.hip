@@ -37,6 +37,25 @@
 using namespace om;
 
 // ---------------------------------------------------------------------------
+// Scratch of om_mi355x_DynamicQuantizeLinearNoAlloc, the entry point that
+// allocates nothing: the per-block partial minima / maxima, the arrival
+// counter and the tagged slots that DynamicQuantizeLinear's kernels exchange
+// their results through live in this array instead of in memory from
+// hipMalloc.  Every GPU the library runs on holds its own copy until the
+// process ends.  The name below is only a host-side handle: the address a
+// kernel or a memory operation needs comes from hipGetSymbolAddress, once per
+// device (resolve_scratch), and only that address is ever used.
+// Layout: f32 partial_min[kNoAllocBlocks], f32 partial_max[kNoAllocBlocks],
+// 64 counter words ([0] arrivals of the two-launch path, [8] "the one-launch
+// kernel gave up" flag), u64 slots[2 * kNoAllocBlocks].
+// ---------------------------------------------------------------------------
+constexpr int kNoAllocBlocks = 512;
+constexpr size_t kNoAllocScratchBytes =
+    sizeof(float) * 2 * kNoAllocBlocks + 256 +
+    sizeof(unsigned long long) * 2 * kNoAllocBlocks; // 12,544 bytes
+static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
+
+// ---------------------------------------------------------------------------
 // errors
 // ---------------------------------------------------------------------------
 namespace {
@@ -105,6 +124,33 @@ struct Backing {
 };
 std::map<uintptr_t, Backing> g_backed;
 
+// Device address of `scratch` on each GPU, resolved with that GPU current
+// (each GPU has its own copy of the array at its own address), and the
+// host-side state that goes with it.  Guarded by g_scratch_mutex.
+constexpr int kMaxDevices = 16;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kMaxDevices] = {};
+unsigned g_scratch_epoch[kMaxDevices] = {};   // launch number of k_dql_grid
+bool g_scratch_no_grid[kMaxDevices] = {};     // one-launch kernel switched off
+bool g_scratch_used[kMaxDevices] = {};
+
+// Call with device `dev` current.
+bool resolve_scratch(int dev) {
+  if (dev < 0 || dev >= kMaxDevices)
+    return false;
+  std::lock_guard<std::mutex> lk(g_scratch_mutex);
+  if (g_scratch_ptr[dev])
+    return true;
+  void *p = nullptr;
+  const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+  if (e != hipSuccess || !p) {
+    (void)hipGetLastError();
+    return false;
+  }
+  g_scratch_ptr[dev] = p;
+  return true;
+}
+
 bool probe_device() {
   int count = 0;
   hipError_t e = hipGetDeviceCount(&count);
@@ -127,6 +173,10 @@ bool probe_device() {
   if (hipSetDevice(0) != hipSuccess) {
     (void)hipGetLastError();
     g_device_why = "hipSetDevice(0) failed";
+    return false;
+  }
+  if (!resolve_scratch(0)) {
+    g_device_why = "hipGetSymbolAddress(scratch) failed";
     return false;
   }
   return true;
@@ -916,6 +966,36 @@ void run_dql(Call &call, const float *dx, int64_t n, uint8_t *dy, float *ds,
   }
 }
 
+// The "gave up" flag of the static scratch on device `dev`, after a
+// synchronisation; reports and clears it.
+bool noalloc_barrier_ok() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+    return true;
+  void *sp;
+  {
+    std::lock_guard<std::mutex> lk(g_scratch_mutex);
+    if (!g_scratch_used[dev] || g_scratch_no_grid[dev])
+      return true;
+    sp = g_scratch_ptr[dev];
+  }
+  unsigned *counter = (unsigned *)((char *)sp + sizeof(float) * 2 * kNoAllocBlocks);
+  unsigned flag = 0;
+  if (hipMemcpy(&flag, counter + 8, sizeof(flag), hipMemcpyDeviceToHost) !=
+          hipSuccess ||
+      !flag)
+    return true;
+  (void)hipMemset(counter, 0, 256);
+  {
+    std::lock_guard<std::mutex> lk(g_scratch_mutex);
+    g_scratch_no_grid[dev] = true;
+  }
+  fail(EIO, "DynamicQuantizeLinearNoAlloc: the blocks of the one-launch "
+            "kernel timed out waiting for one another (grid barrier); its "
+            "output was not written");
+  return false;
+}
+
 // Splits `shape` around `axis` for a scale of `scale_numel` entries.
 bool axis_split(const View &x, int64_t scale_numel, int64_t axis,
     const char *op, int64_t &outer, int64_t &channels, int64_t &inner) {
@@ -1354,6 +1434,88 @@ void om_mi355x_DynamicQuantizeLinear(OMTensor *y_t, OMTensor *scale_t,
   call.finish();
 }
 
+void om_mi355x_DynamicQuantizeLinearNoAlloc(OMTensor *y_t, OMTensor *scale_t,
+    OMTensor *zp_t, const OMTensor *x_t) {
+  const char *op = "DynamicQuantizeLinearNoAlloc";
+  View y, sc, zp, x;
+  if (!view_of(y_t, "y", y) || !view_of(scale_t, "y_scale", sc) ||
+      !view_of(zp_t, "y_zero_point", zp) || !view_of(x_t, "x", x))
+    return;
+  if (x.dtype != OM_MI355X_TYPE_FLOAT || y.dtype != OM_MI355X_TYPE_UINT8 ||
+      sc.dtype != OM_MI355X_TYPE_FLOAT || zp.dtype != OM_MI355X_TYPE_UINT8 ||
+      sc.numel != 1 || zp.numel != 1 || y.numel != x.numel) {
+    fail(EINVAL, "%s: expected f32 x, ui8 y of x's shape, scalar f32 scale "
+                 "and scalar ui8 zero point", op);
+    return;
+  }
+  if (x.numel > OM_MI355X_NOALLOC_MAX_ELEMENTS) {
+    fail(EINVAL, "%s: x has %lld elements, the limit of this entry point is "
+                 "%lld", op, (long long)x.numel,
+        (long long)OM_MI355X_NOALLOC_MAX_ELEMENTS);
+    return;
+  }
+  // Creating the thread's stream allocates, so it must exist already.
+  Ctx &c = t_ctx;
+  if (!c.ready) {
+    fail(EINVAL, "%s: this thread has no stream yet; call "
+                 "om_mi355x_synchronize() (or any other entry point) on it "
+                 "once, outside the region that must not allocate", op);
+    return;
+  }
+  // Every tensor must be GPU memory already: staging a host tensor would take
+  // a buffer from the pool, which may allocate.
+  const View *all[4] = {&y, &sc, &zp, &x};
+  void *dev_ptr[4];
+  for (int i = 0; i < 4; ++i) {
+    dev_ptr[i] = all[i]->data;
+    if (all[i]->numel == 0)
+      continue; // never dereferenced
+    void *d = backed_lookup(all[i]->data);
+    if (!d && is_device_ptr(all[i]->data))
+      d = all[i]->data;
+    if (!d) {
+      fail(EINVAL, "%s: every tensor must be in GPU memory", op);
+      return;
+    }
+    dev_ptr[i] = d;
+  }
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || !resolve_scratch(dev)) {
+    (void)hipGetLastError();
+    fail(EIO, "%s: the scratch array has no address on this device", op);
+    return;
+  }
+  // From here on `sp`, the array's address on this device, stands for it.
+  std::lock_guard<std::mutex> lk(g_scratch_mutex);
+  char *const sp = (char *)g_scratch_ptr[dev];
+  DqlScratch s;
+  s.partial_min = (float *)sp;
+  s.partial_max = s.partial_min + kNoAllocBlocks;
+  s.counter = (unsigned *)(s.partial_max + kNoAllocBlocks);
+  s.grid_slots = (unsigned long long *)((char *)s.counter + 256);
+  s.max_blocks = kNoAllocBlocks;
+  s.grid_blocks = g_scratch_no_grid[dev]
+                      ? 0
+                      : std::min(c.dql.grid_blocks, kNoAllocBlocks);
+  s.spin_limit = c.dql.spin_limit;
+  s.epoch = g_scratch_epoch[dev];
+  g_scratch_used[dev] = true;
+  // The array keeps what the last call left.  The slots need no clearing
+  // (they carry the launch number); the arrival counter of the two-launch
+  // path must start at zero and would not be if an earlier launch had been
+  // cut short.  A fill kernel, not a memset: the caller may be recording a
+  // graph.  The "gave up" flag (word 8) is left for the next synchronisation
+  // to report.
+  hipError_t e = launch_fill_u32(c.stream, (uint32_t *)s.counter, 8, 0u);
+  if (e == hipSuccess)
+    e = launch_dynamic_quantize(c.stream, s, (const float *)dev_ptr[3],
+        x.numel, (uint8_t *)dev_ptr[0], (float *)dev_ptr[1],
+        (uint8_t *)dev_ptr[2], false);
+  g_scratch_epoch[dev] = s.epoch;
+  if (e != hipSuccess)
+    fail(EIO, "%s failed: %s", op, hipGetErrorString(e));
+}
+
 void om_mi355x_MatMulInteger(OMTensor *y, const OMTensor *a,
     const OMTensor *b, const OMTensor *a_zp, const OMTensor *b_zp) {
   MatmulSpec sp = {"MatMulInteger", kEpiI32, y, a, b, a_zp, b_zp};
@@ -1654,7 +1816,8 @@ int om_mi355x_synchronize(void) {
     fail(EIO, "stream synchronisation failed: %s", hipGetErrorString(e));
     return -1;
   }
-  return t_ctx.dql_barrier_ok() ? 0 : -1;
+  const bool mine_ok = t_ctx.dql_barrier_ok();
+  return (noalloc_barrier_ok() && mine_ok) ? 0 : -1;
 }
 
 int om_mi355x_timer_start(void) {

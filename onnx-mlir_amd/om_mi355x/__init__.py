@@ -80,6 +80,7 @@ def _declare(lib, shim):
         "om_mi355x_QuantizeLinear": [P, P, P, P, I64, I64],
         "om_mi355x_DequantizeLinear": [P, P, P, P, I64],
         "om_mi355x_DynamicQuantizeLinear": [P, P, P, P],
+        "om_mi355x_DynamicQuantizeLinearNoAlloc": [P, P, P, P],
         "om_mi355x_MatMulInteger": [P, P, P, P, P],
         "om_mi355x_MatMulIntegerDequant": [P, P, P, P, P, P, P, P],
         "om_mi355x_QLinearMatMul": [P, P, P, P, P, P, P, P, P, I64],
@@ -346,6 +347,18 @@ def DynamicQuantizeLinear(x: Tensor, out: Optional[Tuple[Tensor, Tensor, Tensor]
         z = _like(x, (), np.uint8)
     with _OMT(y) as hy, _OMT(s) as hs, _OMT(z) as hz, _OMT(x) as hx:
         _lib.om_mi355x_DynamicQuantizeLinear(hy, hs, hz, hx)
+    _check()
+    return y, s, z
+
+
+def DynamicQuantizeLinearNoAlloc(x: DeviceArray, out: Tuple[DeviceArray, DeviceArray, DeviceArray]
+                                 ) -> Tuple[DeviceArray, DeviceArray, DeviceArray]:
+    """DynamicQuantizeLinear through the entry point that allocates nothing: all
+    four tensors are GPU memory the caller allocated beforehand."""
+    load()
+    y, s, z = out
+    with _OMT(y) as hy, _OMT(s) as hs, _OMT(z) as hz, _OMT(x) as hx:
+        _lib.om_mi355x_DynamicQuantizeLinearNoAlloc(hy, hs, hz, hx)
     _check()
     return y, s, z
 
