@@ -1,0 +1,111 @@
+// Definitions shared by the int8 GEMM kernels of gemm_kernels.hip and
+// gemm_wreg.hip: vector types, the epilogue's parameter block and small device
+// helpers.  Device code only; include inside namespace om.
+#pragma once
+
+#include "om_kernels.h"
+
+#include <type_traits>
+#include <utility>
+
+namespace om {
+namespace gemm {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v4i_any __attribute__((ext_vector_type(4), aligned(1)));
+enum : int { kLoadBytes = 0, kLoadAligned = 1, kLoadAny = 2 };
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+constexpr int BK = kGemmBK;
+
+// Byte offset of 16-byte chunk `c` (0..3) of tile row `r` (row = 64 bytes).
+__device__ __forceinline__ int lds_off(int r, int c) {
+  return r * BK + ((c ^ ((r >> 2) & 3)) << 4);
+}
+
+// A pointer that is the same in every lane, pinned to scalar registers: the
+// compiler then addresses memory as (scalar base + 32-bit lane offset) and
+// cannot turn base + offset into a per-lane pointer that it advances with
+// vector adds.
+// A 32-bit lane offset whose widening to 64 bits stays next to its use: hoisted
+// out of a loop it would arrive as a 64-bit register pair, and the load would
+// then take the per-lane 64-bit address form.
+__device__ __forceinline__ uint32_t lane_offset(uint32_t o) {
+  asm volatile("" : "+v"(o));
+  return o;
+}
+
+template <typename T>
+__device__ __forceinline__ T *scalar_ptr(T *p) {
+  const uint64_t a = (uint64_t)p;
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
+  return (T *)(((uint64_t)hi << 32) | lo);
+}
+
+// Barrier that orders LDS accesses only; global loads already issued keep
+// flying across it.
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+struct EpiParams {
+  const void *a_zp;
+  int64_t a_zp_len;
+  const void *b_zp;
+  int64_t b_zp_len;
+  bool need_rowsum;      // B carries an offset: row sums of A' are needed
+  const int32_t *colsum;
+  const float *a_scale;
+  const float *b_scale;
+  int64_t b_scale_len;
+  const float *y_scale;
+  const void *y_zp;
+  const float *bias;     // kEpiF32: added after the scaling; null = none
+  int64_t bias_len;      // 1 or N
+  void *out;
+  bool b_unsigned;
+  bool y_unsigned;
+  int narrow;
+};
+
+__device__ __forceinline__ int32_t load_zp_i32(
+    const void *p, bool is_unsigned, int64_t i) {
+  return is_unsigned ? (int32_t)((const uint8_t *)p)[i]
+                     : (int32_t)((const int8_t *)p)[i];
+}
+
+// Sum of the 16 int8 values of an MFMA A operand register group (one lane:
+// one row, 16 consecutive K bytes).  Kernels add these up over K when the
+// epilogue needs rowsum(A'), i.e. when B carries an offset.
+__device__ __forceinline__ int32_t frag_rowsum(v4i f) {
+  int32_t s = __builtin_amdgcn_sdot4(f.x, 0x01010101, 0, false);
+  s = __builtin_amdgcn_sdot4(f.y, 0x01010101, s, false);
+  s = __builtin_amdgcn_sdot4(f.z, 0x01010101, s, false);
+  return __builtin_amdgcn_sdot4(f.w, 0x01010101, s, false);
+}
+
+
+// Calls f(std::integral_constant<int, 0>{}) ... f(std::integral_constant<int,
+// N - 1>{}): a loop whose index is a compile-time constant in the body.
+template <typename F, int... I>
+__device__ __forceinline__ void static_for_impl(
+    F &&f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
+// k_gemm_i8_wreg (gemm_wreg.hip): whether it takes this problem (wreg_ok),
+// whether it is the faster kernel for it (wreg_pays), and its launch.
+bool wreg_ok(const GemmArgs &g);
+bool wreg_pays(int64_t M, int64_t N);
+hipError_t launch_gemm_wreg(hipStream_t st, const GemmArgs &g,
+    const EpiParams &ep, int a_mode);
+
+} // namespace gemm
+} // namespace om

@@ -35,91 +35,15 @@
 // with bits 2..3 of the row (bank-conflict free writes and operand reads); Bp
 // tiles in LDS keep their global order.
 
-#include "om_kernels.h"
+#include "gemm_common.h"
 
 #include <stdlib.h>
 
-#include <type_traits>
-
 namespace om {
 
+using namespace gemm;
+
 namespace {
-
-typedef int v4i __attribute__((ext_vector_type(4)));
-typedef int v4i_any __attribute__((ext_vector_type(4), aligned(1)));
-enum : int { kLoadBytes = 0, kLoadAligned = 1, kLoadAny = 2 };
-typedef int v16i __attribute__((ext_vector_type(16)));
-
-constexpr int BK = kGemmBK;
-
-// Byte offset of 16-byte chunk `c` (0..3) of tile row `r` (row = 64 bytes).
-__device__ __forceinline__ int lds_off(int r, int c) {
-  return r * BK + ((c ^ ((r >> 2) & 3)) << 4);
-}
-
-// A pointer that is the same in every lane, pinned to scalar registers: the
-// compiler then addresses memory as (scalar base + 32-bit lane offset) and
-// cannot turn base + offset into a per-lane pointer that it advances with
-// vector adds.
-// A 32-bit lane offset whose widening to 64 bits stays next to its use: hoisted
-// out of a loop it would arrive as a 64-bit register pair, and the load would
-// then take the per-lane 64-bit address form.
-__device__ __forceinline__ uint32_t lane_offset(uint32_t o) {
-  asm volatile("" : "+v"(o));
-  return o;
-}
-
-template <typename T>
-__device__ __forceinline__ T *scalar_ptr(T *p) {
-  const uint64_t a = (uint64_t)p;
-  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a);
-  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
-  return (T *)(((uint64_t)hi << 32) | lo);
-}
-
-// Barrier that orders LDS accesses only; global loads already issued keep
-// flying across it.
-__device__ __forceinline__ void lds_barrier() {
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-  __builtin_amdgcn_s_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-}
-
-struct EpiParams {
-  const void *a_zp;
-  int64_t a_zp_len;
-  const void *b_zp;
-  int64_t b_zp_len;
-  bool need_rowsum;      // B carries an offset: row sums of A' are needed
-  const int32_t *colsum;
-  const float *a_scale;
-  const float *b_scale;
-  int64_t b_scale_len;
-  const float *y_scale;
-  const void *y_zp;
-  const float *bias;     // kEpiF32: added after the scaling; null = none
-  int64_t bias_len;      // 1 or N
-  void *out;
-  bool b_unsigned;
-  bool y_unsigned;
-  int narrow;
-};
-
-__device__ __forceinline__ int32_t load_zp_i32(
-    const void *p, bool is_unsigned, int64_t i) {
-  return is_unsigned ? (int32_t)((const uint8_t *)p)[i]
-                     : (int32_t)((const int8_t *)p)[i];
-}
-
-// Sum of the 16 int8 values of an MFMA A operand register group (one lane:
-// one row, 16 consecutive K bytes).  Kernels add these up over K when the
-// epilogue needs rowsum(A'), i.e. when B carries an offset.
-__device__ __forceinline__ int32_t frag_rowsum(v4i f) {
-  int32_t s = __builtin_amdgcn_sdot4(f.x, 0x01010101, 0, false);
-  s = __builtin_amdgcn_sdot4(f.y, 0x01010101, s, false);
-  s = __builtin_amdgcn_sdot4(f.z, 0x01010101, s, false);
-  return __builtin_amdgcn_sdot4(f.w, 0x01010101, s, false);
-}
 
 // Epilogue shared by the GEMM kernels: applies the zero-point correction and
 // the op's output conversion to a wave's TM x TN grid of 32x32 accumulator
@@ -1596,7 +1520,8 @@ enum TileCfg : int {
   kD128x128 = 1, // k_gemm_i8_dma: tiles copied straight into LDS
   kB128x256 = 2, // k_gemm_i8_bs: Bp straight into registers
   kD128x64 = 3,  // k_gemm_i8_dma with 128 x 64 tiles
-  kNumCfg = 4
+  kW128x384 = 4, // k_gemm_i8_wreg: weights in registers, 12 waves of 32 columns
+  kNumCfg = 5
 };
 
 // Kernel choice for problems with more than 32 rows, K % 64 == 0 and a
@@ -1684,7 +1609,13 @@ hipError_t gemm_launch_cfg(
               A, g.Bp, M, N, K, Kpad, ep, tiles_m, tiles_n128);
     return hipGetLastError();
   }
-  switch (choose_tile(g.M, g.N, g.K)) {
+  const int cfg = choose_tile(g.M, g.N, g.K);
+  // Weights in registers: K = 768 (the projections of a BERT-base layer)
+  // when the problem fills the device with its 128 x 384 blocks.
+  const bool forced = force && force[0];
+  if (wreg_ok(g) && (cfg == kW128x384 || (!forced && wreg_pays(g.M, g.N))))
+    return launch_gemm_wreg(st, g, ep, A_MODE);
+  switch (cfg) {
   case kB128x256: {
     const int tiles_n = (int)((g.N + 255) / 256);
     if (ep.need_rowsum)
@@ -1704,6 +1635,7 @@ hipError_t gemm_launch_cfg(
             A, g.Bp, M, N, K, Kpad, ep, tiles_m, tiles_n64);
     break;
   }
+  case kW128x384: // (forced, on a shape that kernel does not take)
   case kD128x128:
     k_gemm_i8_dma<128, 3, 3, A_MODE, EPI>
         <<<dim3((unsigned)(tiles_m * tiles_n128)), 256, 0, st>>>(

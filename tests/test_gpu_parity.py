@@ -502,11 +502,12 @@ def test_few_rows_through_lds_all_epilogues(rt, oracle, adt):
             assert np.array_equal(gq, wq), (M, K, N, mode)
 
 
-@pytest.mark.parametrize("cfg", [0, 1, 2, 3])
+@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 4])
 def test_every_gemm_kernel_configuration(rt, oracle, cfg, monkeypatch):
     """The kernel choice is a heuristic; force each configuration in turn (0 stages
     tiles through registers, 1 copies them straight into LDS, 2 streams B
-    straight into registers, 3 is 1 with 128 x 64 tiles) on shapes with ragged
+    straight into registers, 3 is 1 with 128 x 64 tiles, 4 keeps the weights in
+    registers where the shape allows and is 1 elsewhere) on shapes with ragged
     edges, every operand type and all zero-point forms."""
     monkeypatch.setenv("OM_MI355X_GEMM_TILE", str(cfg))
     rng = np.random.default_rng(100 + cfg)
@@ -527,6 +528,53 @@ def test_every_gemm_kernel_configuration(rt, oracle, cfg, monkeypatch):
     aq, a_s, a_zp = oracle.dynamic_quantize_linear(x)
     wantf = oracle.dequant_epilogue(oracle.matmul_integer(aq, W, a_zp, None), a_s, ws)
     assert same_f32(rt.DynQuantMatMulDequant(x, W, None, ws), wantf)
+
+
+@pytest.mark.parametrize("forced", [True, False])
+def test_weights_in_registers_kernel(rt, oracle, forced, monkeypatch):
+    """K = 768 with signed weights and no weight zero point runs k_gemm_i8_wreg
+    (weights in registers, rows through LDS) when its 128 x 384 blocks fill the
+    device, or when forced.  Shapes with ragged edges on both sides (rows and
+    column tiles past the matrix, which the kernel computes and must not store),
+    uint8 / int8 / already shifted activations, scalar zero points, both
+    epilogues it has, bias, and other shapes that must fall through to the other
+    kernels (weight zero point, unsigned weights, per-row zero point, K != 768)."""
+    if forced:
+        monkeypatch.setenv("OM_MI355X_GEMM_TILE", "4")
+        shapes = [(128, 384), (1, 32), (129, 416), (300, 800), (1000, 416), (513, 3104)]
+    else:
+        shapes = [(4096, 2304), (4097, 3104), (3000, 1536)]
+    rng = np.random.default_rng(768 + forced)
+    K = 768
+    for M, N in shapes:
+        for adt in (np.uint8, np.int8):
+            A, B = _rand_q(rng, adt, (M, K)), _rand_q(rng, np.int8, (K, N))
+            az = _rand_q(rng, adt, ())
+            acc = oracle.matmul_integer(A, B, az, None)
+            assert np.array_equal(rt.MatMulInteger(A, B, az, None), acc), (M, N, adt)
+            a_s = np.float32(0.0173)
+            bs = rng.uniform(1e-3, 1e-2, N).astype(np.float32)
+            want = oracle.dequant_epilogue(acc, a_s, bs)
+            assert same_f32(rt.MatMulIntegerDequant(A, B, az, None, a_s, bs, None), want), (M, N, adt)
+        bias = rng.normal(0, 2, N).astype(np.float32)
+        assert same_f32(rt.MatMulIntegerDequant(A, B, None, None, a_s, bs[:1], bias),
+                        oracle.dequant_epilogue(oracle.matmul_integer(A, B, None, None), a_s, bs[:1]) + bias), (M, N)
+        # the fused layer hands the kernel activations that are already minus 128
+        if M > 64:
+            x = rng.normal(0, 1, (M, K)).astype(np.float32)
+            aq, xs, xz = oracle.dynamic_quantize_linear(x)
+            wantf = oracle.dequant_epilogue(oracle.matmul_integer(aq, B, xz, None), xs, bs) + bias
+            assert same_f32(rt.DynQuantMatMulDequant(x, B, None, bs, bias), wantf), (M, N)
+    # not this kernel's: the same calls must still be right
+    M, N = (300, 800) if forced else (4096, 1536)
+    A, Bu = _rand_q(rng, np.uint8, (M, K)), _rand_q(rng, np.uint8, (K, N))
+    B = _rand_q(rng, np.int8, (K, N))
+    az, azr, bz = _rand_q(rng, np.uint8, ()), _rand_q(rng, np.uint8, (M,)), _rand_q(rng, np.int8, (N,))
+    assert np.array_equal(rt.MatMulInteger(A, Bu, az, None), oracle.matmul_integer(A, Bu, az, None))
+    assert np.array_equal(rt.MatMulInteger(A, B, az, bz), oracle.matmul_integer(A, B, az, bz))
+    assert np.array_equal(rt.MatMulInteger(A, B, azr, None), oracle.matmul_integer(A, B, azr, None))
+    A2, B2 = _rand_q(rng, np.uint8, (M, 704)), _rand_q(rng, np.int8, (704, N))
+    assert np.array_equal(rt.MatMulInteger(A2, B2, az, None), oracle.matmul_integer(A2, B2, az, None))
 
 
 def test_matmul_random_shapes_around_dispatch_boundaries(rt, oracle):
