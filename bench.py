@@ -14,6 +14,12 @@ QuantizeLinear / DequantizeLinear / DynamicQuantizeLinear rates at
 Every entry point is called through the C-ABI (include/om_mi355x.h).  Kernel
 time is measured with HIP events recorded on the runtime's own stream around
 the timed region; whole-job time with the host clock around the same region.
+The headline is timed over exactly --steps launches after --warmup untimed
+ones; before that, and before every other measurement, the same call is
+launched untimed until the device has left its idle clocks (PREHEAT_MS, the
+time spent is reported as "preheat_ms").  The other measurements time at least
+MIN_LAUNCHES launches each, in separate event brackets, and report the mean
+and the p10 / median / p90 of the bracket averages.
 """
 import argparse
 import json
@@ -32,15 +38,49 @@ INT8_PEAK_TOPS = 5000.0      # MI355X published dense int8 MFMA rate (no sparsit
 
 METRIC = "int8 MatMulInteger TOPS (% MFMA peak) + Q/DQ GB/s (% HBM), 1 MI355X"
 
-# HBM bytes per launch of the headline kernel, measured with rocprofv3 --pmc
-# (FETCH_SIZE and WRITE_SIZE, one run each, scaled by what the same counters
-# read for a 1 GiB device-to-device copy: FETCH_SIZE x2.0, WRITE_SIZE x1.0);
-# the summary of those runs is profiles/k_gemm_i8_dma_config4_ffn_up.md.
-TRAFFIC_BYTES = {"config4 FFN-up f32": int((7779.0 * 2.0 + 49190.0) * 1024)}
+# The device leaves its idle clocks only after about 100 ms of work (the headline
+# kernel measures 19.0 us after 200 launches from idle, 17.2 us in steady
+# state).  Every timed group is therefore preceded by an untimed pre-heat of the
+# same call until this much GPU time has passed; it is independent of --warmup
+# and its length is reported with every result ("preheat_ms").
+PREHEAT_MS = 120.0
+# Launches an "extras" measurement times at least, in BRACKETS separate event
+# brackets (p10 / median / p90 of the bracket averages show the spread).
+MIN_LAUNCHES = 20
+BRACKETS = 10
 
 
-def timed(rt, fn, steps, warmup):
-    """Returns (host seconds per step, event milliseconds per step)."""
+def traffic_record():
+    """HBM bytes per launch of the headline kernel, from the rocprofv3 --pmc
+    summary kept in profiles/headline_traffic.json (FETCH_SIZE and WRITE_SIZE,
+    one run each, scaled by what the same counters read for a plain copy of
+    known size).  The record names the kernel and the commit it was measured
+    at; it is only used while the headline kernel still has that name."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "headline_traffic.json")) as f:
+            return json.load(f)
+    except (OSError, ValueError):
+        return None
+
+
+def preheat(rt, fn, min_ms=PREHEAT_MS):
+    """Untimed launches of `fn` until `min_ms` of GPU time have passed.
+    Returns (milliseconds spent, milliseconds per launch of the last batch)."""
+    spent, batch, per = 0.0, 16, 1e-4
+    while spent < min_ms:
+        rt.timer_start()
+        for _ in range(batch):
+            fn()
+        ms = rt.timer_stop()
+        spent += ms
+        per = max(ms / batch, 1e-4)
+        batch = int(min(20000, max(16, (min_ms - spent) / per + 1)))
+    return spent, per
+
+
+def timed(rt, fn, steps, warmup, heat=True):
+    """Returns (host seconds per step, event milliseconds per step, pre-heat ms)."""
+    heat_ms = preheat(rt, fn)[0] if heat else 0.0
     for _ in range(warmup):
         fn()
     rt.synchronize()
@@ -51,10 +91,36 @@ def timed(rt, fn, steps, warmup):
     ev_ms = rt.timer_stop()          # waits for the last launch
     rt.synchronize()
     host = time.perf_counter() - t0
-    return host / steps, ev_ms / steps
+    return host / steps, ev_ms / steps, heat_ms
 
 
-def gemm_case(rt, wl, name, M, K, N, w_i8, w_scale, steps, warmup, epilogue="f32"):
+def measure(rt, fn, steps, warmup):
+    """One extras measurement: pre-heat, warm-up, then at least MIN_LAUNCHES
+    launches in BRACKETS event brackets of at least a millisecond each.
+    kernel_ms is the mean over all timed launches; p10 / median / p90 are of the
+    bracket averages."""
+    heat_ms, est_ms = preheat(rt, fn)
+    for _ in range(warmup):
+        fn()
+    # a bracket holds at least about a millisecond of launches: with fewer the
+    # host's submission latency shows in the events of short kernels
+    per = max(2, -(-max(steps, MIN_LAUNCHES) // BRACKETS), int(1.0 / est_ms) + 1)
+    rt.synchronize()
+    t0 = time.perf_counter()
+    times = []
+    for _ in range(BRACKETS):
+        rt.timer_start()
+        for _ in range(per):
+            fn()
+        times.append(rt.timer_stop() / per)
+    host = (time.perf_counter() - t0) / (per * BRACKETS)
+    q = np.percentile(np.array(times), [10, 50, 90])
+    return {"ms_per_step": host * 1e3, "kernel_ms": float(np.mean(times)),
+            "kernel_ms_p10": float(q[0]), "kernel_ms_median": float(q[1]), "kernel_ms_p90": float(q[2]),
+            "launches": per * BRACKETS, "preheat_ms": heat_ms}
+
+
+def gemm_case(rt, wl, name, M, K, N, w_i8, w_scale, steps, warmup, epilogue="f32", headline=False):
     rng = np.random.default_rng(0xC0FFEE00 + M + K + N)
     A = rng.integers(0, 256, (M, K), dtype=np.uint8)
     dA = rt.DeviceArray.from_numpy(A)
@@ -69,24 +135,28 @@ def gemm_case(rt, wl, name, M, K, N, w_i8, w_scale, steps, warmup, epilogue="f32
     else:
         dY = rt.DeviceArray((M, N), np.int32)
         fn = rt.PreparedCall("om_mi355x_MatMulInteger", dY, dA, dW, dAz, None)
-    host_s, ev_ms = timed(rt, fn, steps, warmup)
+    ops = 2.0 * M * N * K
+    res = {"name": name, "M": M, "K": K, "N": N, "epilogue": epilogue}
+    if headline:
+        # the contract's measurement: exactly `steps` launches in one bracket
+        host_s, ev_ms, heat_ms = timed(rt, fn, steps, warmup)
+        res.update({"ms_per_step": host_s * 1e3, "kernel_ms": ev_ms, "preheat_ms": heat_ms,
+                    "tops": ops / host_s / 1e12})
+    else:
+        res.update(measure(rt, fn, steps, warmup))
+        res["tops"] = ops / (res["ms_per_step"] * 1e-3) / 1e12
     fn.check()
     fn.close()
-    ops = 2.0 * M * N * K
-    res = {"name": name, "M": M, "K": K, "N": N, "epilogue": epilogue,
-           "ms_per_step": host_s * 1e3, "kernel_ms": ev_ms,
-           "tops": ops / host_s / 1e12, "kernel_tops": ops / (ev_ms * 1e-3) / 1e12,
-           "ops": ops, "hbm_bytes_algorithmic": M * K + K * N + 4 * M * N}
+    res.update({"kernel": rt.last_gemm_kernel(), "kernel_tops": ops / (res["kernel_ms"] * 1e-3) / 1e12,
+                "ops": ops, "hbm_bytes_algorithmic": M * K + K * N + 4 * M * N})
     for d in (dA, dW, dS, dAs, dAz, dY):
         d.free()
     return res
 
 
-def spread_case(rt, wl, M, K, N, w_i8, w_scale, steps, warmup, sets=6, chunks=20):
-    """The headline GEMM timed two more ways.  (1) In `chunks` separate event
-    brackets, to show the run-to-run spread (p10 / median / p90 of the bracket
-    averages).  (2) Rotating over `sets` activation/output buffer pairs, 320 MB
-    in all for M=4096, N=3072, so that no launch finds its output or its
+def rotated_case(rt, wl, M, K, N, w_i8, w_scale, steps, warmup, sets=6):
+    """The headline GEMM rotating over `sets` activation/output buffer pairs,
+    320 MB in all for M=4096, N=3072, so that no launch finds its output or its
     activations in the 256 MB last-level cache from the launch before."""
     rng = np.random.default_rng(0xC0FFEE00 + M + K + N)
     dW = rt.DeviceArray.from_numpy(w_i8)
@@ -100,29 +170,20 @@ def spread_case(rt, wl, M, K, N, w_i8, w_scale, steps, warmup, sets=6, chunks=20
         dY = rt.DeviceArray((M, N), np.float32)
         bufs += [dA, dY]
         calls.append(rt.PreparedCall("om_mi355x_MatMulIntegerDequant", dY, dA, dW, dAz, None, dAs, dS, None))
-    per = max(1, steps // chunks)
-    times = []
-    for i in range(chunks + 2):
-        _, ev_ms = timed(rt, calls[0], per, warmup if i == 0 else 0)
-        if i >= 2:
-            times.append(ev_ms)
     state = {"i": 0}
 
     def rotate():
         calls[state["i"] % sets]()
         state["i"] += 1
 
-    _, rot_ms = timed(rt, rotate, steps, warmup)
+    res = measure(rt, rotate, max(steps, 10 * sets), warmup)
     for c in calls:
         c.check()
         c.close()
     for d in bufs + [dW, dS, dAs, dAz]:
         d.free()
-    q = np.percentile(np.array(times), [10, 50, 90])
-    return {"launches_per_bracket": per, "brackets": chunks,
-            "kernel_ms_p10": float(q[0]), "kernel_ms_median": float(q[1]), "kernel_ms_p90": float(q[2]),
-            "buffer_sets": sets, "rotated_kernel_ms": rot_ms,
-            "rotated_tops": 2.0 * M * N * K / (rot_ms * 1e-3) / 1e12}
+    res.update({"buffer_sets": sets, "tops": 2.0 * M * N * K / (res["kernel_ms"] * 1e-3) / 1e12})
+    return res
 
 
 def decode_case(rt, wl, M, steps, warmup):
@@ -134,13 +195,13 @@ def decode_case(rt, wl, M, steps, warmup):
     dY = rt.DeviceArray((M, N), np.float32)
     rt.mark_constant(dW)
     fn = rt.PreparedCall("om_mi355x_DynQuantMatMulDequant", dY, dX, dW, None, dS, None)
-    host_s, ev_ms = timed(rt, fn, steps, warmup)
+    res = measure(rt, fn, steps, warmup)
     fn.check()
     fn.close()
     nbytes = K * N + M * K + 4 * M * N
-    res = {"name": f"config5 decode M={M}", "M": M, "K": K, "N": N, "ms_per_step": host_s * 1e3,
-           "kernel_ms": ev_ms, "gbs": nbytes / (ev_ms * 1e-3) / 1e9, "bytes": nbytes,
-           "hbm_frac": nbytes / (ev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+    res.update({"name": f"config5 decode M={M}", "M": M, "K": K, "N": N,
+                "gbs": nbytes / (res["kernel_ms"] * 1e-3) / 1e9, "bytes": nbytes,
+                "hbm_frac": nbytes / (res["kernel_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS})
     for d in (dX, dW, dS, dY):
         d.free()
     return res
@@ -158,40 +219,78 @@ def qlinear_case(rt, wl, steps, warmup):
     rt.mark_constant(d["B"])
     fn = rt.PreparedCall("om_mi355x_QLinearMatMul", dY, d["A"], d["a_scale"], d["a_zp"], d["B"],
                          d["b_scale"], d["b_zp"], d["y_scale"], d["y_zp"], rt.WRAP)
-    host_s, ev_ms = timed(rt, fn, steps, warmup)
+    res = measure(rt, fn, steps, warmup)
     fn.check()
     fn.close()
     ops = 2.0 * M * N * K
-    res = {"name": "config3 QLinearMatMul u8 x u8 -> u8", "M": M, "K": K, "N": N,
-           "ms_per_step": host_s * 1e3, "kernel_ms": ev_ms, "tops": ops / (ev_ms * 1e-3) / 1e12,
-           "hbm_bytes_algorithmic": M * K + K * N + M * N}
+    res.update({"name": "config3 QLinearMatMul u8 x u8 -> u8", "M": M, "K": K, "N": N,
+                "kernel": rt.last_gemm_kernel(), "tops": ops / (res["kernel_ms"] * 1e-3) / 1e12,
+                "hbm_bytes_algorithmic": M * K + K * N + M * N})
     for a in list(d.values()) + [dY]:
         a.free()
     return res
 
 
-def fused_case(rt, wl, name, M, K, N, w_i8, w_scale, steps, warmup):
+def fused_case(rt, wl, name, M, K, N, w_i8, w_scale, steps, warmup, X=None):
     """DynamicQuantizeLinear -> MatMulInteger -> Cast -> Mul as one call: fp32
     activations in, fp32 out (the chain the quantized models contain)."""
-    rng = np.random.default_rng(0xF00D + M + K + N)
-    X = rng.normal(0, 1, (M, K)).astype(np.float32)
+    if X is None:
+        X = np.random.default_rng(0xF00D + M + K + N).normal(0, 1, (M, K)).astype(np.float32)
     dX = rt.DeviceArray.from_numpy(X)
     dW = rt.DeviceArray.from_numpy(w_i8)
-    dS = rt.DeviceArray.from_numpy(w_scale)
+    dS = rt.DeviceArray.from_numpy(np.asarray(w_scale, np.float32))
     dY = rt.DeviceArray((M, N), np.float32)
     rt.mark_constant(dW)
     fn = rt.PreparedCall("om_mi355x_DynQuantMatMulDequant", dY, dX, dW, None, dS, None)
-    host_s, ev_ms = timed(rt, fn, steps, warmup)
+    res = measure(rt, fn, steps, warmup)
     fn.check()
     fn.close()
     ops = 2.0 * M * N * K
     nbytes = 4 * M * K + K * N + 4 * M * N
-    res = {"name": name, "M": M, "K": K, "N": N, "ms_per_step": host_s * 1e3, "kernel_ms": ev_ms,
-           "tops": ops / (ev_ms * 1e-3) / 1e12, "hbm_bytes_algorithmic": nbytes,
-           "hbm_frac_at_algorithmic_bytes": nbytes / (ev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+    res.update({"name": name, "M": M, "K": K, "N": N, "kernel": rt.last_gemm_kernel(),
+                "tops": ops / (res["kernel_ms"] * 1e-3) / 1e12, "hbm_bytes_algorithmic": nbytes,
+                "hbm_frac_at_algorithmic_bytes": nbytes / (res["kernel_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS})
     for d in (dX, dW, dS, dY):
         d.free()
     return res
+
+
+def config1_cases(rt, wl, steps, warmup):
+    """Config 1 (A f32 [128,768] -> DynamicQuantizeLinear -> MatMulInteger with
+    int8 B [768,768] -> Cast -> Mul): as the three separate calls of the
+    unfused graph, tensors resident, and as the one fused call."""
+    c = wl.config1()
+    M, K = c["A"].shape
+    N = c["B"].shape[1]
+    dA = rt.DeviceArray.from_numpy(c["A"])
+    dB = rt.DeviceArray.from_numpy(c["B"])
+    dbs = rt.DeviceArray.from_numpy(np.asarray(c["b_scale"], np.float32))
+    dbz = rt.DeviceArray.from_numpy(np.asarray(c["b_zp"]))
+    dq, ds, dz = rt.DeviceArray((M, K), np.uint8), rt.DeviceArray((), np.float32), rt.DeviceArray((), np.uint8)
+    dY = rt.DeviceArray((M, N), np.float32)
+    rt.mark_constant(dB)
+    calls = [rt.PreparedCall("om_mi355x_DynamicQuantizeLinear", dq, ds, dz, dA),
+             rt.PreparedCall("om_mi355x_MatMulIntegerDequant", dY, dq, dB, dz, dbz, ds, dbs, None)]
+
+    def separate():
+        for f in calls:
+            f()
+
+    sep = measure(rt, separate, steps, warmup)
+    sep["kernel"] = rt.last_gemm_kernel()
+    fused = rt.PreparedCall("om_mi355x_DynQuantMatMulDequant", dY, dA, dB, dbz, dbs, None)
+    fus = measure(rt, fused, steps, warmup)
+    fus["kernel"] = rt.last_gemm_kernel()
+    for f in calls + [fused]:
+        f.check()
+        f.close()
+    ops = 2.0 * M * N * K
+    for r in (sep, fus):
+        r.update({"M": M, "K": K, "N": N, "tops": ops / (r["kernel_ms"] * 1e-3) / 1e12})
+    for d in (dA, dB, dbs, dbz, dq, ds, dz, dY):
+        d.free()
+    return {"DynamicQuantizeLinear + MatMulIntegerDequant (two calls)": sep,
+            "DynQuantMatMulDequant (one call)": fus}
 
 
 def qdq_cases(rt, wl, rows, cols, steps, warmup, only=None):
@@ -212,12 +311,12 @@ def qdq_cases(rt, wl, rows, cols, steps, warmup, only=None):
         if only is not None and name != only:
             fn.close()
             return
-        host_s, ev_ms = timed(rt, fn, steps, warmup)
+        r = measure(rt, fn, steps, warmup)
         fn.check()
         fn.close()
-        out[name] = {"ms_per_step": host_s * 1e3, "kernel_ms": ev_ms, "bytes": nbytes,
-                     "gbs": nbytes / (ev_ms * 1e-3) / 1e9,
-                     "hbm_frac": nbytes / (ev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+        r.update({"bytes": nbytes, "gbs": nbytes / (r["kernel_ms"] * 1e-3) / 1e9,
+                  "hbm_frac": nbytes / (r["kernel_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS})
+        out[name] = r
 
     P = rt.PreparedCall
     run("quantize_per_axis", P("om_mi355x_QuantizeLinear", dQ, dX, dS, dZ, 1, 1), 5 * n)
@@ -246,21 +345,27 @@ def only_mode(rt, wl, what, steps, warmup):
             assert hip.hipMemcpy(b.ptr, a.ptr, n, 3) == 0
         hip.hipDeviceSynchronize()
         return {"only": what, "bytes_read": n, "bytes_written": n, "launches": steps}
-    if what == "gemm_ffn_up":
-        c = wl.config4("ffn_up", M=8)
-        r = gemm_case(rt, wl, "config4 FFN-up", 4096, 768, 3072, c["W"], c["w_scale"], steps, warmup, "f32")
+    if what in ("gemm_ffn_up", "gemm_qkv", "gemm_ffn_down", "gemm_out"):
+        layer = what[5:]
+        k, n = wl.CONFIG4_SHAPES[layer]
+        c = wl.config4(layer, M=8)
+        r = gemm_case(rt, wl, f"config4 {layer}", 4096, k, n, c["W"], c["w_scale"], steps, warmup, "f32",
+                      headline=True)
         return {"only": what, **r}
-    if what == "fused_ffn_up":
-        c = wl.config4("ffn_up", M=8)
-        r = fused_case(rt, wl, "config4 ffn_up fused layer", 4096, 768, 3072, c["W"], c["w_scale"], steps, warmup)
+    if what in ("fused_ffn_up", "fused_ffn_down"):
+        layer = what[6:]
+        k, n = wl.CONFIG4_SHAPES[layer]
+        c = wl.config4(layer, M=8)
+        r = fused_case(rt, wl, f"config4 {layer} fused layer", 4096, k, n, c["W"], c["w_scale"], steps, warmup)
         return {"only": what, **r}
-    if what == "decode":
-        return {"only": what, **decode_case(rt, wl, 1, steps, warmup)}
-    if what == "decode16":
-        return {"only": what, **decode_case(rt, wl, 16, steps, warmup)}
-    if what == "gemm_prefill_up":
-        c = wl.config5("up", M=8)
-        r = gemm_case(rt, wl, "config5 prefill up", 2048, 4096, 11008, c["W"], c["w_scale"], steps, warmup, "f32")
+    if what in ("decode", "decode4", "decode16"):
+        return {"only": what, **decode_case(rt, wl, {"decode": 1, "decode4": 4, "decode16": 16}[what], steps, warmup)}
+    if what in ("gemm_prefill_up", "gemm_prefill_down"):
+        name = what[13:]
+        k, n = wl.CONFIG5_SHAPES[name]
+        c = wl.config5(name, M=8)
+        r = gemm_case(rt, wl, f"config5 prefill {name}", 2048, k, n, c["W"], c["w_scale"], steps, warmup, "f32",
+                      headline=True)
         return {"only": what, **r}
     r = qdq_cases(rt, wl, 8192, 32768, steps, warmup, only=what)
     return {"only": what, **r[what]}
@@ -314,18 +419,17 @@ def cpu_baseline_gemm(oracle, wl, M, K, N, budget_s=20.0):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    # The device needs about 100 ms of work to leave its idle clocks: with 200
-    # warm-up launches the headline kernel measures 19.0 us, with 2000 17.9 us,
-    # with 10000 17.2 us (its steady state).
-    ap.add_argument("--steps", type=int, default=5000)
-    ap.add_argument("--warmup", type=int, default=5000)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--workload", default="config4_ffn_up",
                     choices=["config4_ffn_up", "config4_ffn_up_i32"])
     ap.add_argument("--no-extras", action="store_true", help="skip the Q/DQ and other-shape measurements")
-    ap.add_argument("--extras", default="gemm,fused,decode,qdq", help="which extra groups to measure")
+    ap.add_argument("--extras", default="config1,gemm,fused,decode,qdq", help="which extra groups to measure")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--only", default=None,
-                    choices=["copy", "gemm_ffn_up", "gemm_prefill_up", "fused_ffn_up", "decode", "decode16",
+                    choices=["copy", "gemm_ffn_up", "gemm_qkv", "gemm_out", "gemm_ffn_down",
+                             "gemm_prefill_up", "gemm_prefill_down", "fused_ffn_up", "fused_ffn_down",
+                             "decode", "decode4", "decode16",
                              "quantize_per_axis", "dequantize_per_axis",
                              "quantize_per_tensor", "dequantize_per_tensor", "dynamic_quantize"],
                     help="launch just this kernel --steps times (for rocprofv3 counter runs)")
@@ -347,49 +451,56 @@ def main():
     c = wl.config4("ffn_up", M=8)   # weights and scales only; activations are made in gemm_case
     epi = "f32" if args.workload == "config4_ffn_up" else "i32"
     main_res = gemm_case(rt, wl, "config4 FFN-up", M, K, N, c["W"], c["w_scale"],
-                         args.steps, args.warmup, epi)
+                         args.steps, args.warmup, epi, headline=True)
 
     extras = {}
     groups = set() if args.no_extras else set(args.extras.split(","))
+    esteps, ewarm = args.steps, min(args.warmup, 50)   # every extra is pre-heated as well
     # The bandwidth-bound groups run first: after the seconds of matrix-core work
     # of the gemm group the weight-streaming decode kernel takes 1.8 us longer per
     # launch (10.5 against 8.7 us at M=1, the same in a kernel trace).
     if "decode" in groups:
-        extras["decode"] = [decode_case(rt, wl, m, args.steps, args.warmup) for m in (1, 4, 16)]
+        extras["decode"] = [decode_case(rt, wl, m, esteps, ewarm) for m in (1, 4, 16)]
+    if "config1" in groups:
+        extras["config1"] = config1_cases(rt, wl, esteps, ewarm)
     if "qdq" in groups:
-        qsteps = max(5, args.steps // 10)
-        extras["qdq_8192x32768"] = qdq_cases(rt, wl, 8192, 32768, qsteps, max(2, args.warmup // 10))
-        extras["qdq_8191x32767"] = qdq_cases(rt, wl, 8191, 32767, qsteps, max(2, args.warmup // 10))
+        qsteps = min(max(MIN_LAUNCHES, args.steps // 10), 200)
+        extras["qdq_8192x32768"] = qdq_cases(rt, wl, 8192, 32768, qsteps, 2)
+        extras["qdq_8191x32767"] = qdq_cases(rt, wl, 8191, 32767, qsteps, 2)
     if "fused" in groups:
         fused = []
         for name, (k, n) in wl.CONFIG4_SHAPES.items():
             if name in ("ffn_up", "ffn_down"):
                 cc = wl.config4(name, M=8)
                 fused.append(fused_case(rt, wl, f"config4 {name} fused layer", 4096, k, n, cc["W"],
-                                        cc["w_scale"], args.steps, args.warmup))
+                                        cc["w_scale"], esteps, ewarm))
         extras["fused"] = fused
     if "gemm" in groups:
         gemms = []
         for name, (k, n) in wl.CONFIG4_SHAPES.items():
             cc = wl.config4(name, M=8)
             gemms.append(gemm_case(rt, wl, f"config4 {name}", 4096, k, n, cc["W"], cc["w_scale"],
-                                   args.steps, args.warmup, "f32"))
+                                   esteps, ewarm, "f32"))
         gemms.append(gemm_case(rt, wl, "config4 FFN-up int32 out", M, K, N, c["W"], c["w_scale"],
-                               args.steps, args.warmup, "i32"))
+                               esteps, ewarm, "i32"))
         for name, (k, n) in wl.CONFIG5_SHAPES.items():
             cc = wl.config5(name, M=8)
             gemms.append(gemm_case(rt, wl, f"config5 prefill {name}", 2048, k, n, cc["W"], cc["w_scale"],
-                                   max(10, args.steps // 10), max(2, args.warmup // 10), "f32"))
-        gemms.append(qlinear_case(rt, wl, args.steps, args.warmup))
+                                   min(max(MIN_LAUNCHES, args.steps // 10), 500), 2, "f32"))
+        gemms.append(qlinear_case(rt, wl, esteps, ewarm))
         extras["gemm"] = gemms
-        extras["headline_spread"] = spread_case(rt, wl, M, K, N, c["W"], c["w_scale"],
-                                                args.steps, args.warmup)
+        extras["headline_rotated"] = rotated_case(rt, wl, M, K, N, c["W"], c["w_scale"], esteps, ewarm)
 
     cpu = None
     if not args.no_cpu:
         import oracle_lib
         cpu = cpu_baseline_gemm(oracle_lib.load(), wl, M, K, N)
 
+    traffic = None
+    rec = traffic_record() if epi == "f32" else None
+    if rec and rec.get("kernel") == main_res["kernel"]:
+        traffic = rec.get("traffic_bytes")
+    hbm_bytes = main_res["hbm_bytes_algorithmic"]
     line = {
         "metric": METRIC,
         "value": main_res["tops"],
@@ -405,16 +516,18 @@ def main():
         "data": "synthetic",
         "config": {"workload": f"config4 FFN-up MatMulInteger M={M} K={K} N={N}, uint8 activations x int8 "
                                f"weights, a_zp scalar, {'per-column fp32 dequant' if epi == 'f32' else 'int32'} "
-                               "output, operands resident in HBM, weights packed once"},
+                               "output, operands resident in HBM, weights packed once",
+                   "preheat_ms": main_res["preheat_ms"]},
         "roofline": {"bound": "mfma", "achieved": main_res["kernel_tops"], "peak": INT8_PEAK_TOPS,
                      "unit": "TOP/s", "frac": main_res["kernel_tops"] / INT8_PEAK_TOPS,
-                     "traffic": TRAFFIC_BYTES.get("config4 FFN-up f32") if epi == "f32" else None,
-                     "kernel": "k_gemm_i8_dma<128,3,3> (128x128 tiles)", "kernel_ms": main_res["kernel_ms"],
+                     "traffic": traffic,
+                     "traffic_source": ({"file": "profiles/headline_traffic.json", "commit": rec.get("commit")}
+                                        if traffic else None),
+                     "kernel": main_res["kernel"], "kernel_ms": main_res["kernel_ms"],
                      "algorithmic_ops": main_res["ops"],
-                     "algorithmic_hbm_bytes": main_res["hbm_bytes_algorithmic"],
-                     "hbm_frac_at_algorithmic_bytes": main_res["hbm_bytes_algorithmic"]
-                     / (main_res["kernel_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                     "hbm_bound_tops": main_res["ops"] / (main_res["hbm_bytes_algorithmic"] / (HBM_PEAK_GBS * 1e9)) / 1e12},
+                     "algorithmic_hbm_bytes": hbm_bytes,
+                     "hbm_frac_at_algorithmic_bytes": hbm_bytes / (main_res["kernel_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                     "hbm_bound_tops": main_res["ops"] / (hbm_bytes / (HBM_PEAK_GBS * 1e9)) / 1e12},
         "cpu_baseline": cpu,
         "device": info,
         "extras": extras,

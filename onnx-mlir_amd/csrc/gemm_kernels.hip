@@ -1560,6 +1560,10 @@ bool gemm_fast_path(int64_t M, int64_t K, const void *A) {
   return M > 16 && K > 0 && K % 64 == 0 && ((((uintptr_t)A) & 15) == 0);
 }
 
+// Name of the kernel the calling thread's last launch_gemm chose (for tests
+// and reports).
+thread_local const char *t_last_kernel = "";
+
 template <int A_MODE, int EPI>
 hipError_t gemm_launch_cfg(
     hipStream_t st, const GemmArgs &g, const EpiParams &ep, int Kpad) {
@@ -1571,6 +1575,7 @@ hipError_t gemm_launch_cfg(
     if (A_MODE != 2 || !gemm_quantizes_rows(g.M, g.K, g.X))
       return hipErrorInvalidValue;
     if constexpr (A_MODE == 2)
+      t_last_kernel = "k_gemm_i8_skinny_bp (rows quantized in the kernel)";
       k_gemm_i8_skinny_bp<2, EPI, true, 1, false>
           <<<dim3((unsigned)((g.N + 31) / 32)), 512, 0, st>>>(
               nullptr, g.X, g.Bp, M, N, K, Kpad, ep);
@@ -1583,6 +1588,7 @@ hipError_t gemm_launch_cfg(
   if (skinny_rows && g.K > 0 && g.K % 16 == 0 && ((((uintptr_t)g.A) & 15) == 0) &&
       !(force && force[0])) {
     const dim3 grid((unsigned)((g.N + 31) / 32));
+    t_last_kernel = "k_gemm_i8_skinny_bp";
     if (g.M <= 4)
       k_gemm_i8_skinny_bp<A_MODE, EPI, false, 1, false>
           <<<grid, 512, 0, st>>>(A, nullptr, g.Bp, M, N, K, Kpad, ep);
@@ -1599,6 +1605,7 @@ hipError_t gemm_launch_cfg(
   if (!gemm_fast_path(g.M, g.K, g.A)) {
     // Any K, any alignment of A (and the forced configurations of the tests
     // when M <= 16); byte loads only for an A of fewer than 16 bytes.
+    t_last_kernel = "k_gemm_i8 (any K, any alignment)";
     if (g.M * g.K >= 16)
       k_gemm_i8<128, 128, 2, 2, 2, A_MODE, EPI, kLoadAny>
           <<<dim3((unsigned)(tiles_m * tiles_n128)), 256, 0, st>>>(
@@ -1613,11 +1620,14 @@ hipError_t gemm_launch_cfg(
   // Weights in registers: K = 768 (the projections of a BERT-base layer)
   // when the problem fills the device with its 128 x 384 blocks.
   const bool forced = force && force[0];
-  if (wreg_ok(g) && (cfg == kW128x384 || (!forced && wreg_pays(g.M, g.N))))
+  if (wreg_ok(g) && (cfg == kW128x384 || (!forced && wreg_pays(g.M, g.N)))) {
+    t_last_kernel = "k_gemm_i8_wreg (weights in registers, 128x384 blocks)";
     return launch_gemm_wreg(st, g, ep, A_MODE);
+  }
   switch (cfg) {
   case kB128x256: {
     const int tiles_n = (int)((g.N + 255) / 256);
+    t_last_kernel = "k_gemm_i8_bs (128x256 tiles)";
     if (ep.need_rowsum)
       k_gemm_i8_bs<4, 2, 4, 4, 2, true, A_MODE, EPI, true>
           <<<dim3((unsigned)(tiles_m * tiles_n)), 256, 0, st>>>(
@@ -1630,6 +1640,7 @@ hipError_t gemm_launch_cfg(
   }
   case kD128x64: {
     const int tiles_n64 = (int)((g.N + 63) / 64);
+    t_last_kernel = "k_gemm_i8_dma (128x64 tiles)";
     k_gemm_i8_dma<64, 3, 3, A_MODE, EPI>
         <<<dim3((unsigned)(tiles_m * tiles_n64)), 256, 0, st>>>(
             A, g.Bp, M, N, K, Kpad, ep, tiles_m, tiles_n64);
@@ -1637,11 +1648,13 @@ hipError_t gemm_launch_cfg(
   }
   case kW128x384: // (forced, on a shape that kernel does not take)
   case kD128x128:
+    t_last_kernel = "k_gemm_i8_dma (128x128 tiles)";
     k_gemm_i8_dma<128, 3, 3, A_MODE, EPI>
         <<<dim3((unsigned)(tiles_m * tiles_n128)), 256, 0, st>>>(
             A, g.Bp, M, N, K, Kpad, ep, tiles_m, tiles_n128);
     break;
   default:
+    t_last_kernel = "k_gemm_i8 (128x128 tiles through registers)";
     k_gemm_i8<128, 128, 2, 2, 3, A_MODE, EPI, kLoadAligned>
         <<<dim3((unsigned)(tiles_m * tiles_n128)), 256, 0, st>>>(
             A, g.Bp, M, N, K, Kpad, ep, tiles_m, tiles_n128);
@@ -1691,6 +1704,8 @@ bool gemm_quantizes_rows(int64_t M, int64_t K, const void *x) {
          M * K <= kSkinnyDqBytes && ((((uintptr_t)x) & 15) == 0) &&
          !(force && force[0]);
 }
+
+const char *last_gemm_kernel() { return t_last_kernel; }
 
 hipError_t launch_gemm(hipStream_t s, const GemmArgs &g) {
   if (g.M == 0 || g.N == 0)

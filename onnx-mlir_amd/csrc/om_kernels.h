@@ -107,6 +107,8 @@ struct GemmArgs {
 };
 
 hipError_t launch_gemm(hipStream_t s, const GemmArgs &g);
+// Name of the kernel the calling thread's last launch_gemm chose.
+const char *last_gemm_kernel();
 
 // Whether launch_gemm can take an f32 activation of this shape in GemmArgs::X.
 bool gemm_quantizes_rows(int64_t M, int64_t K, const void *x);

@@ -1853,6 +1853,8 @@ const char *om_mi355x_last_error(void) {
   return t_last_error_returned.c_str();
 }
 
+const char *om_mi355x_last_gemm_kernel(void) { return last_gemm_kernel(); }
+
 int om_mi355x_device_info(char *buf, size_t len) {
   if (!t_ctx.init())
     return -1;

@@ -111,6 +111,7 @@ def _declare(lib, shim):
     lib.om_mi355x_timer_start.restype = ctypes.c_int
     lib.om_mi355x_timer_stop.restype = ctypes.c_float
     lib.om_mi355x_last_error.restype = ctypes.c_char_p
+    lib.om_mi355x_last_gemm_kernel.restype = ctypes.c_char_p
     lib.om_mi355x_device_info.restype = ctypes.c_int
     lib.om_mi355x_device_info.argtypes = [ctypes.c_char_p, SZ]
 
@@ -130,6 +131,12 @@ def device_info() -> dict:
     name, arch, cus, mhz, gib = buf.value.decode().split("|")
     return {"name": name, "arch": arch, "cus": int(cus), "clock_mhz": int(mhz),
             "mem_gib": float(gib)}
+
+
+def last_gemm_kernel() -> str:
+    """Name of the GEMM kernel this thread's last matmul call launched."""
+    load()
+    return _lib.om_mi355x_last_gemm_kernel().decode()
 
 
 def init_compatible(version: int = 0x100) -> bool:
