@@ -60,12 +60,6 @@ bool isI32(Type t) {
 }
 bool isAbsent(Value v) { return !v || isNoneValue(v); }
 
-/// The right-hand side of every matmul entry point is one 2-D matrix.
-bool isMatrix(Value v) {
-  auto type = dyn_cast<ShapedType>(v.getType());
-  return type && type.hasRank() && type.getRank() == 2;
-}
-
 bool hasRankAtLeast(Value v, int64_t rank) {
   auto type = dyn_cast<ShapedType>(v.getType());
   return type && type.hasRank() && type.getRank() >= rank;
@@ -219,8 +213,10 @@ struct MatMulIntegerToMI355X
 
   LogicalResult matchAndRewrite(ONNXMatMulIntegerOp op, OpAdaptor adaptor,
       ConversionPatternRewriter &rewriter) const final {
-    // Batched right-hand sides ([.., K, N]) are left to the CPU.
-    if (!isEnabled(op) || !isMatrix(op.getB()) ||
+    // Any ranked pair of operands: the runtime pairs batch dimensions by the
+    // rules of ONNXMatMulOpShapeHelper (src/Dialect/ONNX/ONNXOps/Math/
+    // MatMul.cpp:200-292), the same that sized `y` here.
+    if (!isEnabled(op) || !hasRankAtLeast(op.getB(), 1) ||
         !hasRankAtLeast(op.getA(), 1))
       return failure();
     Location loc = ONNXLoc<ONNXMatMulIntegerOp>(op);
@@ -248,7 +244,7 @@ struct QLinearMatMulToMI355X
 
   LogicalResult matchAndRewrite(ONNXQLinearMatMulOp op, OpAdaptor adaptor,
       ConversionPatternRewriter &rewriter) const final {
-    if (!isEnabled(op) || !isMatrix(op.getB()) ||
+    if (!isEnabled(op) || !hasRankAtLeast(op.getB(), 1) ||
         !hasRankAtLeast(op.getA(), 1))
       return failure();
     Location loc = ONNXLoc<ONNXQLinearMatMulOp>(op);

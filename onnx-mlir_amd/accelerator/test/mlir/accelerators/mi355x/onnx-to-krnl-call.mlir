@@ -77,13 +77,16 @@ func.func @matmul_integer_constant_weight(%a: tensor<128x4xui8>, %azp: tensor<ui
 
 // -----
 
-// A batched right-hand side is not offloaded: the CPU loops remain.
+// A batched right-hand side goes to the same entry point: the runtime pairs
+// the batch dimensions itself.
 func.func @matmul_integer_batched_b(%a: tensor<2x8x4xui8>, %b: tensor<2x4x2xi8>, %azp: tensor<ui8>, %bzp: tensor<i8>) -> tensor<*xi32> {
   %y = "onnx.MatMulInteger"(%a, %b, %azp, %bzp) : (tensor<2x8x4xui8>, tensor<2x4x2xi8>, tensor<ui8>, tensor<i8>) -> tensor<*xi32>
   return %y : tensor<*xi32>
 // CHECK-LABEL:  func.func @matmul_integer_batched_b
-// CHECK-NOT:    om_mi355x_MatMulInteger
-// CHECK:        krnl.iterate
+// CHECK:        [[Y:%.+]] = memref.alloc() {{.*}}: memref<2x8x2xi32>
+// CHECK:        "krnl.call"([[Y]], {{%.+}}, {{%.+}}, {{%.+}}, {{%.+}})
+// CHECK-SAME:   funcName = "om_mi355x_MatMulInteger", numOfOutput = 1 : si64
+// CHECK-SAME:   (memref<2x8x2xi32>, memref<2x8x4xui8>, memref<2x4x2xi8>, memref<ui8>, memref<i8>) -> ()
 }
 
 // -----

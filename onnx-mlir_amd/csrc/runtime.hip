@@ -1026,26 +1026,88 @@ bool axis_split(const View &x, int64_t scale_numel, int64_t axis,
   return true;
 }
 
-// A [.., M, K] (leading dimensions folded into M) times B [K, N].
-bool matmul_dims(const View &a, const View &b, const char *op, int64_t &M,
-    int64_t &K, int64_t &N) {
-  if (b.rank != 2 || a.rank < 1) {
-    fail(EINVAL, "%s: expected A [..,M,K] and a 2-D B [K,N]", op);
+// Shape of a matrix product as onnx.MatMul defines it
+// (src/Dialect/ONNX/ONNXOps/Math/MatMul.cpp:200-292, numpy's matmul rules).
+//  - B [K, N] (or [K], taken as [K, 1]): the leading dimensions of A
+//    [.., M, K] are folded into M; one product.
+//  - B [.., K, N] with leading (batch) dimensions: A is [.., M, K] (or [K],
+//    taken as [1, K]), the batch dimensions of A and B are broadcast against
+//    each other, and there is one M x K x N product per batch entry:
+//    a_batch[i] / b_batch[i] are the matrices of A / B that entry i multiplies.
+struct MatmulShape {
+  int64_t M = 0, K = 0, N = 0;
+  int64_t batches = 1;
+  int64_t a_mats = 1, b_mats = 1; // matrices held by A and by B
+  std::vector<int64_t> a_batch, b_batch;
+};
+
+bool matmul_dims(const View &a, const View &b, const char *op, bool allow_batched_b,
+    MatmulShape &sh) {
+  if (a.rank < 1 || b.rank < 1) {
+    fail(EINVAL, "%s: A and B need at least one dimension", op);
     return false;
   }
-  K = a.shape[a.rank - 1];
-  M = (K == 0) ? 0 : a.numel / K;
-  if (a.rank >= 2 && K == 0) {
-    M = 1;
-    for (int64_t i = 0; i + 1 < a.rank; ++i)
-      M *= a.shape[i];
-  }
-  if (b.shape[0] != K) {
+  sh.K = a.shape[a.rank - 1];
+  const int64_t bk = b.rank >= 2 ? b.shape[b.rank - 2] : b.shape[0];
+  if (bk != sh.K) {
     fail(EINVAL, "%s: inner dimensions differ (%lld vs %lld)", op,
-        (long long)K, (long long)b.shape[0]);
+        (long long)sh.K, (long long)bk);
     return false;
   }
-  N = b.shape[1];
+  sh.N = b.rank >= 2 ? b.shape[b.rank - 1] : 1;
+  if (b.rank <= 2) {
+    sh.M = 1;
+    for (int64_t i = 0; i + 1 < a.rank; ++i)
+      sh.M *= a.shape[i];
+    sh.a_batch.assign(1, 0);
+    sh.b_batch.assign(1, 0);
+    return true;
+  }
+  if (!allow_batched_b) {
+    fail(EINVAL, "%s: expected a 2-D B [K,N]", op);
+    return false;
+  }
+  sh.M = a.rank >= 2 ? a.shape[a.rank - 2] : 1;
+  const int64_t ar = a.rank >= 2 ? a.rank - 2 : 0, br = b.rank - 2;
+  const int64_t r = ar > br ? ar : br;
+  std::vector<int64_t> dims(r), astr(r, 0), bstr(r, 0);
+  int64_t am = 1, bm = 1;
+  for (int64_t i = r - 1; i >= 0; --i) { // right-aligned, as numpy broadcasts
+    const int64_t ai = i - (r - ar), bi = i - (r - br);
+    const int64_t ad = ai >= 0 ? a.shape[ai] : 1, bd = bi >= 0 ? b.shape[bi] : 1;
+    if (ad != bd && ad != 1 && bd != 1) {
+      fail(EINVAL, "%s: batch dimensions %lld and %lld do not broadcast", op,
+          (long long)ad, (long long)bd);
+      return false;
+    }
+    dims[i] = ad == 1 ? bd : ad;
+    astr[i] = ad == 1 ? 0 : am;
+    bstr[i] = bd == 1 ? 0 : bm;
+    am *= ad;
+    bm *= bd;
+  }
+  sh.a_mats = am;
+  sh.b_mats = bm;
+  sh.batches = 1;
+  for (int64_t d : dims)
+    sh.batches *= d;
+  if (sh.batches > ((int64_t)1 << 20)) {
+    fail(EINVAL, "%s: more than 2^20 batch entries", op);
+    return false;
+  }
+  sh.a_batch.resize((size_t)sh.batches);
+  sh.b_batch.resize((size_t)sh.batches);
+  for (int64_t e = 0; e < sh.batches; ++e) {
+    int64_t rest = e, ai = 0, bi = 0;
+    for (int64_t i = r - 1; i >= 0; --i) {
+      const int64_t c = rest % dims[i];
+      rest /= dims[i];
+      ai += c * astr[i];
+      bi += c * bstr[i];
+    }
+    sh.a_batch[(size_t)e] = ai;
+    sh.b_batch[(size_t)e] = bi;
+  }
   return true;
 }
 
@@ -1126,19 +1188,22 @@ bool packed_b(Call &call, const View &b, int64_t K, int64_t N,
   return true;
 }
 
-bool zp_len_ok(const View *zp, int64_t full, const char *op, const char *name,
-    int64_t &len) {
+// A zero point has one entry, or one per row / column of a matrix (`per`), or
+// -- with batched operands, as [.., M, 1] / [.., 1, N] -- one per row / column
+// of every matrix of its tensor (`per * mats`).
+bool zp_len_ok(const View *zp, int64_t per, int64_t mats, const char *op,
+    const char *name, int64_t &len) {
   if (!zp) {
     len = 0;
     return true;
   }
   if (zp->numel == 1)
     len = 1;
-  else if (zp->numel == full)
-    len = full;
+  else if (zp->numel == per || zp->numel == per * mats)
+    len = zp->numel;
   else {
     fail(EINVAL, "%s: %s has %lld entries, expected 1 or %lld", op, name,
-        (long long)zp->numel, (long long)full);
+        (long long)zp->numel, (long long)per);
     return false;
   }
   return true;
@@ -1184,12 +1249,15 @@ void run_matmul(const MatmulSpec &sp) {
     fail(EINVAL, "%s: a zero point's type differs from its tensor's", sp.op);
     return;
   }
-  int64_t M, K, N;
-  if (!matmul_dims(a, b, sp.op, M, K, N))
+  MatmulShape sh;
+  // The fused epilogue of a linear layer keeps its 2-D weights; the ONNX ops
+  // themselves take batched right-hand sides.
+  if (!matmul_dims(a, b, sp.op, sp.epi != kEpiF32, sh))
     return;
-  if (y.numel != M * N) {
+  const int64_t M = sh.M, K = sh.K, N = sh.N;
+  if (y.numel != sh.batches * M * N) {
     fail(EINVAL, "%s: output has %lld elements, expected %lld", sp.op,
-        (long long)y.numel, (long long)(M * N));
+        (long long)y.numel, (long long)(sh.batches * M * N));
     return;
   }
   const int want_y = sp.epi == kEpiI32   ? OM_MI355X_TYPE_INT32
@@ -1200,8 +1268,8 @@ void run_matmul(const MatmulSpec &sp) {
     return;
   }
   int64_t azl, bzl;
-  if (!zp_len_ok(sp.a_zp ? &azp : nullptr, M, sp.op, "a_zero_point", azl) ||
-      !zp_len_ok(sp.b_zp ? &bzp : nullptr, N, sp.op, "b_zero_point", bzl))
+  if (!zp_len_ok(sp.a_zp ? &azp : nullptr, M, sh.a_mats, sp.op, "a_zero_point", azl) ||
+      !zp_len_ok(sp.b_zp ? &bzp : nullptr, N, sh.b_mats, sp.op, "b_zero_point", bzl))
     return;
   if (sp.epi != kEpiI32) {
     if (!view_of(sp.a_scale, "a_scale", as) ||
@@ -1227,7 +1295,7 @@ void run_matmul(const MatmulSpec &sp) {
       return;
     }
   }
-  if (M == 0 || N == 0)
+  if (M == 0 || N == 0 || sh.batches == 0)
     return;
 
   Call call(t_ctx, sp.op);
@@ -1244,14 +1312,37 @@ void run_matmul(const MatmulSpec &sp) {
   g.K = K;
   g.N = N;
   const int32_t *colsum = nullptr;
-  if (!packed_b(call, b, K, N, g.Bp, colsum)) {
-    call.finish();
-    return;
+  // One right-hand side: packed once (cached for a constant).  Batched: the
+  // matrices of B are packed one after the other into buffers of this call.
+  const int64_t Kpad = round_up(K > 0 ? K : 1, kGemmBK);
+  const int64_t Npad = round_up(N, kGemmBN);
+  const size_t bp_bytes = (size_t)Kpad * Npad;
+  int8_t *bp_all = nullptr;
+  int32_t *cs_all = nullptr;
+  if (b.rank <= 2) {
+    if (!packed_b(call, b, K, N, g.Bp, colsum)) {
+      call.finish();
+      return;
+    }
+  } else {
+    const uint8_t *db = (const uint8_t *)call.in(b);
+    bp_all = (int8_t *)call.temp(bp_bytes * (size_t)sh.b_mats);
+    cs_all = (int32_t *)call.temp((size_t)Npad * 4 * (size_t)sh.b_mats);
+    for (int64_t i = 0; call.ok && i < sh.b_mats; ++i)
+      call.check(launch_pack_b(call.c.stream, db + (size_t)i * K * N, b_uns, K, N,
+                     bp_all + (size_t)i * bp_bytes, cs_all + (size_t)i * Npad),
+          "pack B");
+    if (!call.ok) {
+      call.finish();
+      return;
+    }
   }
   g.colsum = colsum;
-  g.a_zp = sp.a_zp ? call.in(azp) : nullptr;
+  const uint8_t *d_azp = sp.a_zp ? (const uint8_t *)call.in(azp) : nullptr;
+  const uint8_t *d_bzp = sp.b_zp ? (const uint8_t *)call.in(bzp) : nullptr;
+  g.a_zp = d_azp;
   g.a_zp_len = azl;
-  g.b_zp = sp.b_zp ? call.in(bzp) : nullptr;
+  g.b_zp = d_bzp;
   g.b_zp_len = bzl;
   g.epi = sp.epi;
   if (sp.epi != kEpiI32) {
@@ -1270,8 +1361,34 @@ void run_matmul(const MatmulSpec &sp) {
     g.narrow = sp.narrow;
   }
   g.out = call.out(y);
-  if (call.ok)
-    call.check(launch_gemm(call.c.stream, g), sp.op);
+  if (b.rank <= 2) {
+    if (call.ok)
+      call.check(launch_gemm(call.c.stream, g), sp.op);
+    call.finish();
+    return;
+  }
+  // One product per batch entry, queued one after the other.
+  const uint8_t *d_a = (const uint8_t *)g.A;
+  char *d_y = (char *)g.out;
+  const size_t y_es = sp.epi == kEpiQ8 ? 1 : 4;
+  for (int64_t e = 0; call.ok && e < sh.batches; ++e) {
+    const int64_t ai = sh.a_batch[(size_t)e], bi = sh.b_batch[(size_t)e];
+    GemmArgs ge = g;
+    ge.A = d_a + (size_t)ai * M * K;
+    ge.Bp = bp_all + (size_t)bi * bp_bytes;
+    ge.colsum = cs_all + (size_t)bi * Npad;
+    // zero points given per matrix ([.., M, 1] / [.., 1, N]) move with it
+    if (azl > M) {
+      ge.a_zp = d_azp + (size_t)ai * M;
+      ge.a_zp_len = M;
+    }
+    if (bzl > N) {
+      ge.b_zp = d_bzp + (size_t)bi * N;
+      ge.b_zp_len = N;
+    }
+    ge.out = d_y + (size_t)e * M * N * y_es;
+    call.check(launch_gemm(call.c.stream, ge), sp.op);
+  }
   call.finish();
 }
 
@@ -1565,11 +1682,12 @@ void om_mi355x_DynQuantMatMulDequant(OMTensor *y_t, const OMTensor *x_t,
     fail(EINVAL, "%s: expected f32 x and y, ui8/i8 b, f32 b_scale", op);
     return;
   }
-  int64_t M, K, N;
-  if (!matmul_dims(x, b, op, M, K, N))
+  MatmulShape sh;
+  if (!matmul_dims(x, b, op, false, sh))
     return;
+  const int64_t M = sh.M, K = sh.K, N = sh.N;
   int64_t bzl;
-  if (!zp_len_ok(bzp_t ? &bzp : nullptr, N, op, "b_zero_point", bzl))
+  if (!zp_len_ok(bzp_t ? &bzp : nullptr, N, 1, op, "b_zero_point", bzl))
     return;
   if (y.numel != M * N || (bs.numel != 1 && bs.numel != N)) {
     fail(EINVAL, "%s: output or b_scale shape is wrong", op);

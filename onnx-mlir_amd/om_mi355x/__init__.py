@@ -371,7 +371,14 @@ def DynamicQuantizeLinearNoAlloc(x: DeviceArray, out: Tuple[DeviceArray, DeviceA
 
 
 def _mm_shape(a: Tensor, b: Tensor):
-    return tuple(a.shape[:-1]) + (b.shape[-1],)
+    """Result shape of onnx.MatMul(a, b) (numpy's matmul rules)."""
+    if len(b.shape) == 1:
+        return tuple(a.shape[:-1])
+    if len(b.shape) == 2:
+        return tuple(a.shape[:-1]) + (b.shape[-1],)
+    batch = np.broadcast_shapes(tuple(a.shape[:-2]), tuple(b.shape[:-2]))
+    rows = (a.shape[-2],) if len(a.shape) >= 2 else ()
+    return tuple(batch) + rows + (b.shape[-1],)
 
 
 def MatMulInteger(a: Tensor, b: Tensor, a_zero_point: Optional[Tensor] = None,

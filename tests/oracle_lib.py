@@ -115,8 +115,37 @@ class Oracle:
         fn(_p(x), x.size, _p(y), ctypes.byref(s), ctypes.byref(z))
         return y, np.float32(s.value), np.uint8(z.value)
 
+    @staticmethod
+    def _batched(a, b, a_zp, b_zp):
+        """Splits a product with a batched right-hand side into its 2-D
+        products, as numpy's matmul broadcasts them: yields (index of the result
+        matrix, A matrix, B matrix, a_zp for it, b_zp for it).  Zero points of
+        the forms [.., M, 1] / [.., 1, N] are sliced along with their matrix."""
+        a2 = a if a.ndim >= 2 else a.reshape(1, -1)
+        batch = np.broadcast_shapes(a2.shape[:-2], b.shape[:-2])
+        ab = np.broadcast_to(a2, batch + a2.shape[-2:])
+        bb = np.broadcast_to(b, batch + b.shape[-2:])
+        azb = bzb = None
+        if a_zp is not None and np.ndim(a_zp) > 1:
+            azb = np.broadcast_to(np.asarray(a_zp), batch + (a2.shape[-2], 1))
+        if b_zp is not None and np.ndim(b_zp) > 1:
+            bzb = np.broadcast_to(np.asarray(b_zp), batch + (1, b.shape[-1]))
+        for idx in np.ndindex(*batch):
+            yield (idx, np.ascontiguousarray(ab[idx]), np.ascontiguousarray(bb[idx]),
+                   a_zp if azb is None else np.ascontiguousarray(azb[idx]).reshape(-1),
+                   b_zp if bzb is None else np.ascontiguousarray(bzb[idx]).reshape(-1))
+
     def matmul_integer(self, a, b, a_zp=None, b_zp=None, passes=False):
         a, b = np.ascontiguousarray(a), np.ascontiguousarray(b)
+        if b.ndim > 2:     # one 2-D product per batch entry
+            batch = np.broadcast_shapes(a.shape[:-2], b.shape[:-2])
+            rows = (a.shape[-2],) if a.ndim >= 2 else ()
+            y = np.empty(batch + rows + (b.shape[-1],), np.int32)
+            for idx, am, bm, az, bz in self._batched(a, b, a_zp, b_zp):
+                y[idx] = self.matmul_integer(am, bm, az, bz, passes).reshape(y[idx].shape)
+            return y
+        if b.ndim == 1:
+            return self.matmul_integer(a, b.reshape(-1, 1), a_zp, b_zp, passes)[..., 0]
         K, N = b.shape
         M = a.size // K if K else int(np.prod(a.shape[:-1]))
         az = None if a_zp is None else np.ascontiguousarray(a_zp, a.dtype).reshape(-1)
@@ -129,6 +158,14 @@ class Oracle:
 
     def qlinear_matmul(self, a, a_scale, a_zp, b, b_scale, b_zp, y_scale, y_zp, mode=WRAP):
         a, b = np.ascontiguousarray(a), np.ascontiguousarray(b)
+        if b.ndim > 2:
+            batch = np.broadcast_shapes(a.shape[:-2], b.shape[:-2])
+            rows = (a.shape[-2],) if a.ndim >= 2 else ()
+            y = np.empty(batch + rows + (b.shape[-1],), np.asarray(y_zp).dtype)
+            for idx, am, bm, az, bz in self._batched(a, b, a_zp, b_zp):
+                y[idx] = self.qlinear_matmul(am, a_scale, az, bm, b_scale, bz, y_scale, y_zp,
+                                             mode).reshape(y[idx].shape)
+            return y
         K, N = b.shape
         M = a.size // K if K else int(np.prod(a.shape[:-1]))
         az = np.ascontiguousarray(a_zp, a.dtype).reshape(-1)

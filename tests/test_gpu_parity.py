@@ -717,6 +717,67 @@ def test_matmulinteger_batched_a(rt, oracle):
     assert got.shape == (3, 5, 24) and np.array_equal(got, oracle.matmul_integer(A, B, az, None))
 
 
+def test_matmulinteger_batched_b(rt, oracle):
+    """Right-hand sides with batch dimensions (src/Dialect/ONNX/ONNXOps/Math/MatMul.cpp
+    :200-292): equal batch dimensions, numpy-style broadcasting on either side, a 2-D
+    or 1-D A against a batched B, a 1-D B, and the zero-point forms [.., M, 1] and
+    [.., 1, N] that belong to batched operands."""
+    rng = np.random.default_rng(45)
+    cases = [((2, 3, 5, 64), (2, 3, 64, 24)), ((3, 1, 5, 64), (4, 64, 24)), ((1, 7, 40), (6, 40, 9)),
+             ((33, 100), (2, 100, 65)), ((64,), (3, 64, 10)), ((2, 130, 96), (2, 96, 300))]
+    for ashape, bshape in cases:
+        for adt, bdt in ((np.uint8, np.int8), (np.int8, np.uint8)):
+            A, B = _rand_q(rng, adt, ashape), _rand_q(rng, bdt, bshape)
+            az, bz = _rand_q(rng, adt, ()), _rand_q(rng, bdt, ())
+            want = oracle.matmul_integer(A, B, az, bz)
+            got = rt.MatMulInteger(A, B, az, bz)
+            assert got.shape == want.shape and np.array_equal(got, want), (ashape, bshape)
+            # against numpy's own batched product, in int64
+            ref = np.matmul(A.astype(np.int64) - int(az), B.astype(np.int64) - int(bz))
+            assert np.array_equal(want.astype(np.int64), ref), (ashape, bshape)
+            bzn = _rand_q(rng, bdt, bshape[:-2] + (1, bshape[-1]))
+            assert np.array_equal(rt.MatMulInteger(A, B, az, bzn), oracle.matmul_integer(A, B, az, bzn)), (ashape, bshape)
+            if len(ashape) >= 2:
+                azm = _rand_q(rng, adt, ashape[:-1] + (1,))
+                assert np.array_equal(rt.MatMulInteger(A, B, azm, bzn),
+                                      oracle.matmul_integer(A, B, azm, bzn)), (ashape, bshape)
+    # a 1-D right-hand side (the matrix-vector case of src/Conversion/ONNXToKrnl/Math/MatMul.cpp:299-304)
+    A, v = _rand_q(rng, np.uint8, (9, 50)), _rand_q(rng, np.int8, (50,))
+    got = rt.MatMulInteger(A, v, _rand_q(rng, np.uint8, ()), None)
+    assert got.shape == (9,)
+    # device-resident batched operands
+    A, B = _rand_q(rng, np.uint8, (4, 70, 128)), _rand_q(rng, np.int8, (4, 128, 96))
+    dA, dB = rt.DeviceArray.from_numpy(A), rt.DeviceArray.from_numpy(B)
+    dY = rt.MatMulInteger(dA, dB, None, None)
+    rt.synchronize()
+    assert np.array_equal(dY.numpy(), oracle.matmul_integer(A, B, None, None))
+
+
+def test_qlinearmatmul_3d(rt, oracle):
+    """QLinearMatMul with batched operands: the shapes of the ONNX node tests
+    test_qlinearmatmul_3D_{uint8,int8}_float32 that the reference enables
+    (test/backend/inference_backend.py:2549-2554) -- [2,2,4] x [2,4,3] -- built by
+    stacking the 2-D node-test matrices, so every batch entry has the published
+    2-D answer; and larger seeded shapes against the oracle, both narrowing modes."""
+    for name, dt in (("qlinearmatmul_2D_uint8_float32", np.uint8), ("qlinearmatmul_2D_int8_float32", np.int8)):
+        g = GOLD[name]
+        a, b = np.array(g["a"], dt), np.array(g["b"], dt)
+        a3, b3 = np.stack([a, a]), np.stack([b, b])
+        y = rt.QLinearMatMul(a3, np.float32(g["a_scale"]), np.array(g["a_zp"], dt), b3,
+                             np.float32(g["b_scale"]), np.array(g["b_zp"], dt),
+                             np.float32(g["y_scale"]), np.array(g["y_zp"], dt), rt.WRAP)
+        assert y.shape == (2, 2, 3)
+        assert np.array_equal(y[0], np.array(g["y"], dt)) and np.array_equal(y[1], np.array(g["y"], dt))
+    rng = np.random.default_rng(46)
+    for dt in (np.uint8, np.int8):
+        A, B = _rand_q(rng, dt, (3, 70, 192)), _rand_q(rng, dt, (3, 192, 130))
+        az, bz, yz = _rand_q(rng, dt, ()), _rand_q(rng, dt, ()), _rand_q(rng, dt, ())
+        for mode in (rt.WRAP, rt.SATURATE):
+            want = oracle.qlinear_matmul(A, np.float32(0.02), az, B, np.float32(0.01), bz, np.float32(0.7), yz, mode)
+            got = rt.QLinearMatMul(A, np.float32(0.02), az, B, np.float32(0.01), bz, np.float32(0.7), yz, mode)
+            assert np.array_equal(got, want), (dt, mode)
+
+
 def test_constant_weights_are_packed_once_and_stay_correct(rt, oracle):
     rng = np.random.default_rng(45)
     B = _rand_q(rng, np.int8, (256, 384))

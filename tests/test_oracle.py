@@ -329,3 +329,18 @@ def test_dequant_epilogue_closed_form(oracle):
     want = acc.astype(np.float32) * (a_s * bs)[None, :]   # scale product first, then one multiply
     assert np.array_equal(oracle.dequant_epilogue(acc, a_s, bs), want)
     assert np.array_equal(oracle.dequant_epilogue(acc, a_s, bs[:1]), acc.astype(np.float32) * (a_s * bs[0]))
+
+
+def test_batched_matmul_wrapper_equals_numpy_matmul(oracle):
+    """The oracle handles a batched right-hand side by looping its 2-D routine
+    over the batch entries that numpy's matmul rules pair up; the loop must
+    reproduce numpy's own batched product (in int64, no wrap at these sizes)."""
+    rng = np.random.default_rng(91)
+    for ashape, bshape in (((2, 3, 5, 16), (2, 3, 16, 7)), ((3, 1, 4, 8), (5, 8, 6)), ((6, 8), (2, 8, 3)), ((8,), (2, 8, 3))):
+        A = rng.integers(0, 256, ashape, dtype=np.uint8)
+        B = rng.integers(-128, 128, bshape).astype(np.int8)
+        az = np.array(rng.integers(0, 256), np.uint8)
+        bz = rng.integers(-128, 128, bshape[:-2] + (1, bshape[-1])).astype(np.int8)
+        want = np.matmul(A.astype(np.int64) - int(az), B.astype(np.int64) - bz.astype(np.int64))
+        got = oracle.matmul_integer(A, B, az, bz)
+        assert got.shape == want.shape and np.array_equal(got.astype(np.int64), want)
