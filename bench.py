@@ -131,7 +131,7 @@ def gemm_case(rt, wl, name, M, K, N, w_i8, w_scale, steps, warmup, epilogue="f32
     rt.mark_constant(dW)             # weights: packed once, like any model constant
     if epilogue == "f32":
         dY = rt.DeviceArray((M, N), np.float32)
-        fn = rt.PreparedCall("om_mi355x_MatMulIntegerDequant", dY, dA, dW, dAz, None, dAs, dS, None)
+        fn = rt.PreparedCall("om_mi355x_MatMulIntegerDequant", dY, dA, dW, dAz, None, dAs, dS, None, 0)
     else:
         dY = rt.DeviceArray((M, N), np.int32)
         fn = rt.PreparedCall("om_mi355x_MatMulInteger", dY, dA, dW, dAz, None)
@@ -169,7 +169,7 @@ def rotated_case(rt, wl, M, K, N, w_i8, w_scale, steps, warmup, sets=6):
         dA = rt.DeviceArray.from_numpy(rng.integers(0, 256, (M, K), dtype=np.uint8))
         dY = rt.DeviceArray((M, N), np.float32)
         bufs += [dA, dY]
-        calls.append(rt.PreparedCall("om_mi355x_MatMulIntegerDequant", dY, dA, dW, dAz, None, dAs, dS, None))
+        calls.append(rt.PreparedCall("om_mi355x_MatMulIntegerDequant", dY, dA, dW, dAz, None, dAs, dS, None, 0))
     state = {"i": 0}
 
     def rotate():
@@ -194,7 +194,7 @@ def decode_case(rt, wl, M, steps, warmup):
     dS = rt.DeviceArray.from_numpy(c["w_scale"])
     dY = rt.DeviceArray((M, N), np.float32)
     rt.mark_constant(dW)
-    fn = rt.PreparedCall("om_mi355x_DynQuantMatMulDequant", dY, dX, dW, None, dS, None)
+    fn = rt.PreparedCall("om_mi355x_DynQuantMatMulDequant", dY, dX, dW, None, dS, None, 0)
     res = measure(rt, fn, steps, warmup)
     fn.check()
     fn.close()
@@ -241,7 +241,7 @@ def fused_case(rt, wl, name, M, K, N, w_i8, w_scale, steps, warmup, X=None):
     dS = rt.DeviceArray.from_numpy(np.asarray(w_scale, np.float32))
     dY = rt.DeviceArray((M, N), np.float32)
     rt.mark_constant(dW)
-    fn = rt.PreparedCall("om_mi355x_DynQuantMatMulDequant", dY, dX, dW, None, dS, None)
+    fn = rt.PreparedCall("om_mi355x_DynQuantMatMulDequant", dY, dX, dW, None, dS, None, 0)
     res = measure(rt, fn, steps, warmup)
     fn.check()
     fn.close()
@@ -270,7 +270,7 @@ def config1_cases(rt, wl, steps, warmup):
     dY = rt.DeviceArray((M, N), np.float32)
     rt.mark_constant(dB)
     calls = [rt.PreparedCall("om_mi355x_DynamicQuantizeLinear", dq, ds, dz, dA),
-             rt.PreparedCall("om_mi355x_MatMulIntegerDequant", dY, dq, dB, dz, dbz, ds, dbs, None)]
+             rt.PreparedCall("om_mi355x_MatMulIntegerDequant", dY, dq, dB, dz, dbz, ds, dbs, None, 0)]
 
     def separate():
         for f in calls:
@@ -278,7 +278,7 @@ def config1_cases(rt, wl, steps, warmup):
 
     sep = measure(rt, separate, steps, warmup)
     sep["kernel"] = rt.last_gemm_kernel()
-    fused = rt.PreparedCall("om_mi355x_DynQuantMatMulDequant", dY, dA, dB, dbz, dbs, None)
+    fused = rt.PreparedCall("om_mi355x_DynQuantMatMulDequant", dY, dA, dB, dbz, dbs, None, 0)
     fus = measure(rt, fused, steps, warmup)
     fus["kernel"] = rt.last_gemm_kernel()
     for f in calls + [fused]:
@@ -416,6 +416,77 @@ def cpu_baseline_gemm(oracle, wl, M, K, N, budget_s=20.0):
             "seconds_per_step": best}
 
 
+def onnx_mlir_leg(A, W, az, a_scale, w_scale, gpu_y, budget_s=20.0):
+    """The reference's own CPU code for the headline op, when its compiler is
+    installed on this host: `onnx-mlir -O3 --parallel` builds
+    bench/models/cfg4_matmulinteger.mlir (MatMulInteger -> Cast -> Mul, the same
+    graph the GPU number is for) into a shared library, whose run_main_graph is
+    then called on the same operands through the OMTensor C API that every
+    compiled model exports (include/OnnxMlirRuntime.h of the reference).  Returns
+    None when there is no `onnx-mlir` on PATH -- the case on every box this was
+    written on, so this leg has never run -- and a dict with "error" when a step
+    of it fails."""
+    import ctypes, shutil, subprocess, tempfile
+    exe = shutil.which("onnx-mlir")
+    if exe is None:
+        return None
+    model = os.path.join(ROOT, "bench", "models", "cfg4_matmulinteger.mlir")
+    try:
+        with tempfile.TemporaryDirectory() as tmp:
+            base = os.path.join(tmp, "cfg4_matmulinteger")
+            r = subprocess.run([exe, "-O3", "--parallel", model, "-o", base],
+                               capture_output=True, text=True, timeout=600)
+            if r.returncode != 0:
+                return {"error": "onnx-mlir failed: " + r.stderr[-400:]}
+            so = ctypes.CDLL(base + ".so")
+            vp, i64 = ctypes.c_void_p, ctypes.c_int64
+            so.omTensorCreate.restype, so.omTensorCreate.argtypes = vp, [vp, ctypes.POINTER(i64), i64, ctypes.c_int]
+            so.omTensorListCreate.restype, so.omTensorListCreate.argtypes = vp, [ctypes.POINTER(vp), i64]
+            so.run_main_graph.restype, so.run_main_graph.argtypes = vp, [vp]
+            so.omTensorListGetOmtByIndex.restype, so.omTensorListGetOmtByIndex.argtypes = vp, [vp, i64]
+            so.omTensorGetDataPtr.restype, so.omTensorGetDataPtr.argtypes = vp, [vp]
+            so.omTensorListDestroy.restype, so.omTensorListDestroy.argtypes = None, [vp]
+            onnx_type = {np.dtype(np.float32): 1, np.dtype(np.uint8): 2, np.dtype(np.int8): 3}
+            arrays = [np.ascontiguousarray(x) for x in
+                      (A, W, az, np.array(a_scale, np.float32), np.asarray(w_scale, np.float32))]
+            tensors = (vp * len(arrays))()
+            shapes = []
+            for i, x in enumerate(arrays):
+                shp = (i64 * max(x.ndim, 1))(*x.shape)
+                shapes.append(shp)
+                tensors[i] = so.omTensorCreate(x.ctypes.data, shp, x.ndim, onnx_type[x.dtype])
+            inputs = so.omTensorListCreate(tensors, len(arrays))
+
+            def run():
+                t0 = time.perf_counter()
+                out = so.run_main_graph(inputs)
+                dt = time.perf_counter() - t0
+                if not out:
+                    raise RuntimeError("run_main_graph returned NULL")
+                return out, dt
+
+            out, first = run()
+            y = np.ctypeslib.as_array(ctypes.cast(so.omTensorGetDataPtr(so.omTensorListGetOmtByIndex(out, 0)),
+                                                  ctypes.POINTER(ctypes.c_float)), shape=gpu_y.shape)
+            same = bool(np.array_equal(y.view(np.uint32), gpu_y.view(np.uint32)))
+            so.omTensorListDestroy(out)
+            times = [first]
+            for _ in range(int(max(1, min(10, budget_s / max(first, 1e-3) - 1)))):
+                out, dt = run()
+                so.omTensorListDestroy(out)
+                times.append(dt)
+        M, K = A.shape
+        N = W.shape[1]
+        best = float(np.median(times))
+        return {"value": 2.0 * M * N * K / best / 1e12, "unit": "TOPS", "cores": host_cpu()["usable_cpus"],
+                "kind": "reference", "host": host_cpu(), "seconds_per_step": best,
+                "bit_identical_to_gpu_output": same,
+                "sample": f"full M={M} K={K} N={N} MatMulInteger+Cast+Mul, median of {len(times)} calls of "
+                          "run_main_graph of bench/models/cfg4_matmulinteger.mlir built by `onnx-mlir -O3 --parallel`"}
+    except Exception as e:                                   # noqa: BLE001 -- an optional leg must not end the bench
+        return {"error": f"{type(e).__name__}: {e}"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -495,6 +566,17 @@ def main():
     if not args.no_cpu:
         import oracle_lib
         cpu = cpu_baseline_gemm(oracle_lib.load(), wl, M, K, N)
+        # The reference's own compiled model, where its compiler is installed.
+        rng = np.random.default_rng(7)
+        A = rng.integers(0, 256, (M, K), dtype=np.uint8)
+        az, a_scale = np.array(131, np.uint8), np.float32(0.0173)
+        gpu_y = rt.MatMulIntegerDequant(A, c["W"], az, None, a_scale, c["w_scale"], None)
+        ref = onnx_mlir_leg(A, c["W"], az, a_scale, c["w_scale"], gpu_y)
+        if ref is not None and "error" not in ref:
+            ref["port"] = cpu
+            cpu = ref
+        else:
+            cpu["onnx_mlir"] = ref if ref is not None else "not on PATH"
 
     traffic = None
     rec = traffic_record() if epi == "f32" else None

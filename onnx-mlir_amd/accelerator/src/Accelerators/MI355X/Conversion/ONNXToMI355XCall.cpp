@@ -263,9 +263,10 @@ struct QLinearMatMulToMI355X
 //===----------------------------------------------------------------------===//
 // onnx.Custom created by the fusion pass.
 //   void om_mi355x_MatMulIntegerDequant(y, a, b, a_zp|NULL, b_zp|NULL,
-//                                       a_scale, b_scale, bias|NULL)
+//                                       a_scale, b_scale, bias|NULL,
+//                                       activation)
 //   void om_mi355x_DynQuantMatMulDequant(y, x, b, b_zp|NULL, b_scale,
-//                                        bias|NULL)
+//                                        bias|NULL, activation)
 // In both, input 0 is [.., M, K] and input 1 is [K, N]; the result is
 // [.., M, N].  onnx.Custom has no shape rule for that, so the dimensions are
 // taken from the operands here.
@@ -310,7 +311,10 @@ struct FusedMatMulToMI355X : public OpConversionPattern<ONNXCustomOp> {
     // uploaded once instead of with every call.
     for (size_t i = 1; i < inputs.size(); ++i)
       markIfConstant(rewriter, loc, inputs[i]);
-    emitCall(rewriter, loc, callee, {y}, inputs);
+    int64_t activation = 0;
+    if (auto attr = op->getAttrOfType<IntegerAttr>("activation"))
+      activation = attr.getInt();
+    emitCall(rewriter, loc, callee, {y}, inputs, {{"activation", activation}});
     rewriter.replaceOp(op, y);
     return success();
   }

@@ -12,14 +12,19 @@
 //   %s             = Mul(%as, %ws)
 //   %y             = Mul(%f, %s)
 //   %z             = Add(%y, %bias)          (optional)
+//   %r             = Relu(%z)                (optional)
 //
 // On the CPU that is five or six ops and as many intermediate tensors.  The
 // MI355X runtime has one entry point for everything after the quantisation
 // (the int32 accumulator never reaches memory) and one for the whole chain
 // (the 8-bit activation stays on the device).  A bias that is added to the
 // scaled result -- one value, or one per column -- goes along: the kernel
-// rounds the product to f32 and then adds, as Mul followed by Add does.  This pass replaces the chain by an `onnx.Custom` naming that entry
-// point; the ONNX-to-Krnl patterns of the accelerator lower it.
+// rounds the product to f32 and then adds, as Mul followed by Add does.  A Relu
+// that is the only user of that result goes along too, as the integer
+// attribute `activation` = 1 (max(0, x) is exact, so where it is applied does
+// not change a bit of the result).  This pass replaces the chain by an
+// `onnx.Custom` naming that entry point; the ONNX-to-Krnl patterns of the
+// accelerator lower it.
 //
 // Only the association `f32(acc) * (a_scale * b_scale)` is matched.  The other
 // one the reference knows, `(f32(acc) * a_scale) * b_scale`
@@ -158,6 +163,16 @@ struct FuseScaledMatMulInteger : public OpRewritePattern<ONNXMulOp> {
         }
       }
     }
+    // ... and so is a Relu that is the only user of what has been matched.
+    int64_t activation = 0;
+    if (root->hasOneUse()) {
+      if (auto relu = dyn_cast<ONNXReluOp>(*root->user_begin())) {
+        if (relu.getResult().getType() == root->getResult(0).getType()) {
+          root = relu;
+          activation = 1;
+        }
+      }
+    }
     rewriter.setInsertionPoint(root);
 
     SmallVector<Value, 8> inputs;
@@ -175,15 +190,17 @@ struct FuseScaledMatMulInteger : public OpRewritePattern<ONNXMulOp> {
           chain.bScale, noneIfAbsent(rewriter, loc, bias)};
     }
 
-    SmallVector<NamedAttribute, 2> attrs;
+    SmallVector<NamedAttribute, 3> attrs;
     attrs.emplace_back(
         rewriter.getNamedAttr("function_name", rewriter.getStringAttr(callee)));
+    attrs.emplace_back(rewriter.getNamedAttr(
+        "activation", rewriter.getI64IntegerAttr(activation)));
     if (Attribute nodeName = mul->getAttr("onnx_node_name"))
       attrs.emplace_back(rewriter.getNamedAttr("onnx_node_name", nodeName));
     auto fused = ONNXCustomOp::create(rewriter, loc,
         TypeRange{root->getResult(0).getType()}, ValueRange(inputs), attrs);
     rewriter.replaceOp(root, fused.getResults());
-    // Mul (when the Add was the root), Cast, MatMulInteger, the scale product
+    // Mul and Add (when a later op was the root), Cast, MatMulInteger, the scale product
     // and (for the whole layer) DynamicQuantizeLinear are now dead and pure:
     // the driver erases them.
     return success();

@@ -116,3 +116,27 @@ func.func @batched_rhs_is_left_alone(%a: tensor<4x128x64xui8>, %b: tensor<4x64x3
 // CHECK:        "onnx.Mul"
 // CHECK-NOT:    onnx.Custom
 }
+
+// -----
+
+// A Relu on the biased result, with no other user in between, becomes the
+// `activation` attribute of the same call.
+func.func @whole_layer_with_bias_and_relu(%x: tensor<128x768xf32>, %w: tensor<768x3072xi8>, %ws: tensor<3072xf32>, %bias: tensor<3072xf32>) -> tensor<*xf32> {
+  %none = "onnx.NoValue"() {value} : () -> none
+  %aq, %as, %azp = "onnx.DynamicQuantizeLinear"(%x) : (tensor<128x768xf32>) -> (tensor<*xui8>, tensor<*xf32>, tensor<*xui8>)
+  %acc = "onnx.MatMulInteger"(%aq, %w, %azp, %none) : (tensor<*xui8>, tensor<768x3072xi8>, tensor<*xui8>, none) -> tensor<*xi32>
+  %f = "onnx.Cast"(%acc) {to = f32} : (tensor<*xi32>) -> tensor<*xf32>
+  %s = "onnx.Mul"(%as, %ws) : (tensor<*xf32>, tensor<3072xf32>) -> tensor<*xf32>
+  %y = "onnx.Mul"(%f, %s) : (tensor<*xf32>, tensor<*xf32>) -> tensor<*xf32>
+  %z = "onnx.Add"(%y, %bias) : (tensor<*xf32>, tensor<3072xf32>) -> tensor<*xf32>
+  %r = "onnx.Relu"(%z) : (tensor<*xf32>) -> tensor<*xf32>
+  return %r : tensor<*xf32>
+// CHECK-LABEL:  func.func @whole_layer_with_bias_and_relu
+// CHECK-SAME:   ([[X:%.+]]: tensor<128x768xf32>, [[W:%.+]]: tensor<768x3072xi8>, [[WS:%.+]]: tensor<3072xf32>, [[BIAS:%.+]]: tensor<3072xf32>)
+// CHECK:        [[R:%.+]] = "onnx.Custom"([[X]], [[W]], {{%.+}}, [[WS]], [[BIAS]])
+// CHECK-SAME:   activation = 1 : i64
+// CHECK-SAME:   function_name = "om_mi355x_DynQuantMatMulDequant"
+// CHECK-NOT:    onnx.Relu
+// CHECK-NOT:    onnx.Add
+// CHECK:        return [[R]]
+}

@@ -18,6 +18,7 @@ func.func @whole_layer_dynamic(%x: tensor<?x768xf32>, %ws: tensor<f32>) -> tenso
 // CHECK:        "krnl.call"([[W]])
 // CHECK-SAME:   funcName = "om_mi355x_MarkConstant"
 // CHECK:        "krnl.call"([[Y]], [[X]], [[W]], {{%.+}}, [[WS]], {{%.+}})
+// CHECK-SAME:   activation = 0 : i64
 // CHECK-SAME:   funcName = "om_mi355x_DynQuantMatMulDequant", numOfOutput = 1 : si64
 // CHECK-SAME:   (memref<?x64xf32>, memref<?x768xf32>, memref<768x64xi8>, none, memref<f32>, none) -> ()
 // CHECK-NOT:    krnl.iterate

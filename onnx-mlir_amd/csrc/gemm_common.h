@@ -65,11 +65,27 @@ struct EpiParams {
   const void *y_zp;
   const float *bias;     // kEpiF32: added after the scaling; null = none
   int64_t bias_len;      // 1 or N
+  float floor;           // kEpiF32: relu_floor(whether onnx.Relu follows)
   void *out;
   bool b_unsigned;
   bool y_unsigned;
   int narrow;
 };
+
+// onnx.Relu as the reference lowers it: max(0, x) with the maximum that
+// returns the other operand for a NaN
+// (src/Conversion/ONNXToKrnl/Math/Elementwise.cpp:746-754), so NaN -> 0; a
+// negative zero becomes +0.
+// Done as one maximum per element whether or not a Relu is asked for: against
+// `floor` = 0 when it is, and against a NaN when it is not -- that maximum
+// (v_max_f32) returns its other operand unchanged, negative zero included, and
+// a NaN only when both are.
+__device__ __forceinline__ float relu_f32(float f, float floor) {
+  return __builtin_fmaxf(f, floor);
+}
+inline float relu_floor(bool relu) {
+  return relu ? 0.0f : __builtin_nanf("");
+}
 
 __device__ __forceinline__ int32_t load_zp_i32(
     const void *p, bool is_unsigned, int64_t i) {

@@ -63,7 +63,8 @@ __device__ __forceinline__ void store_one(const EpiParams &ep, int64_t o,
   if (EPI == kEpiI32) {
     ((int32_t *)ep.out)[o] = (int32_t)y;
   } else if (EPI == kEpiF32) {
-    ((float *)ep.out)[o] = (float)(int32_t)y * sj + bj;
+    const float f = (float)(int32_t)y * sj + bj;
+    ((float *)ep.out)[o] = relu_f32(f, ep.floor);
   } else {
     const float f = (float)(int32_t)y * sj;
     const int32_t q = (int32_t)__builtin_rintf(f);
@@ -190,7 +191,8 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TM][TN],
           asm volatile("; plain store");
         }
       } else if (EPI == kEpiF32) {
-        const float f = (float)(int32_t)y * sj[j] + bj[j];
+        float f = (float)(int32_t)y * sj[j] + bj[j];
+        f = relu_f32(f, ep.floor);
         if (kStream) {
           __builtin_nontemporal_store(f, (float *)q);
         } else {
@@ -1728,6 +1730,7 @@ hipError_t launch_gemm(hipStream_t s, const GemmArgs &g) {
   ep.y_zp = g.y_zp;
   ep.bias = g.epi == kEpiF32 ? g.bias : nullptr;
   ep.bias_len = g.bias_len;
+  ep.floor = relu_floor(g.epi == kEpiF32 && g.relu);
   ep.out = g.out;
   ep.b_unsigned = g.b_unsigned;
   ep.y_unsigned = g.y_unsigned;

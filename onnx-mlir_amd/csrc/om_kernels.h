@@ -101,6 +101,9 @@ struct GemmArgs {
   const void *y_zp;
   const float *bias;   // kEpiF32 only; may be null
   int64_t bias_len;    // 1 or N
+  // kEpiF32 only: onnx.Relu on the result, max(0, x) with a NaN giving 0
+  // (src/Conversion/ONNXToKrnl/Math/Elementwise.cpp:746-754).
+  bool relu;
   bool y_unsigned;
   NarrowMode narrow;
   void *out;           // i32 / f32 / u8|i8 [M,N]

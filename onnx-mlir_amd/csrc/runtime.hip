@@ -1217,7 +1217,19 @@ struct MatmulSpec {
   const OMTensor *a_scale = nullptr, *b_scale = nullptr, *y_scale = nullptr,
                  *y_zp = nullptr, *bias = nullptr;
   NarrowMode narrow = kWrap;
+  bool relu = false; // kEpiF32: onnx.Relu on the result
 };
+
+// The `activation` argument of the fused entry points: 0 = none, 1 = Relu.
+bool activation_ok(int64_t activation, const char *op, bool &relu) {
+  if (activation != 0 && activation != 1) {
+    fail(EINVAL, "%s: activation %lld is not 0 (none) or 1 (Relu)", op,
+        (long long)activation);
+    return false;
+  }
+  relu = activation == 1;
+  return true;
+}
 
 // Optional bias of the f32 epilogue: f32, one value or one per column.
 bool bias_ok(const OMTensor *bias_t, int64_t N, const char *op, View &bias) {
@@ -1354,6 +1366,7 @@ void run_matmul(const MatmulSpec &sp) {
     g.bias = (const float *)call.in(bias);
     g.bias_len = bias.numel;
   }
+  g.relu = sp.relu;
   if (sp.epi == kEpiQ8) {
     g.y_scale = (const float *)call.in(ys);
     g.y_zp = call.in(yzp);
@@ -1641,8 +1654,11 @@ void om_mi355x_MatMulInteger(OMTensor *y, const OMTensor *a,
 
 void om_mi355x_MatMulIntegerDequant(OMTensor *y, const OMTensor *a,
     const OMTensor *b, const OMTensor *a_zp, const OMTensor *b_zp,
-    const OMTensor *a_scale, const OMTensor *b_scale, const OMTensor *bias) {
+    const OMTensor *a_scale, const OMTensor *b_scale, const OMTensor *bias,
+    int64_t activation) {
   MatmulSpec sp = {"MatMulIntegerDequant", kEpiF32, y, a, b, a_zp, b_zp};
+  if (!activation_ok(activation, sp.op, sp.relu))
+    return;
   sp.a_scale = a_scale;
   sp.b_scale = b_scale;
   sp.bias = bias;
@@ -1668,9 +1684,12 @@ void om_mi355x_QLinearMatMul(OMTensor *y, const OMTensor *a,
 
 void om_mi355x_DynQuantMatMulDequant(OMTensor *y_t, const OMTensor *x_t,
     const OMTensor *b_t, const OMTensor *bzp_t, const OMTensor *bscale_t,
-    const OMTensor *bias_t) {
+    const OMTensor *bias_t, int64_t activation) {
   const char *op = "DynQuantMatMulDequant";
   View y, x, b, bzp, bs, bias;
+  bool relu;
+  if (!activation_ok(activation, op, relu))
+    return;
   if (!view_of(y_t, "y", y) || !view_of(x_t, "x", x) ||
       !view_of(b_t, "b", b) || !view_of(bscale_t, "b_scale", bs))
     return;
@@ -1738,6 +1757,7 @@ void om_mi355x_DynQuantMatMulDequant(OMTensor *y_t, const OMTensor *x_t,
     g.bias = (const float *)call.in(bias);
     g.bias_len = bias.numel;
   }
+  g.relu = relu;
   if (call.ok)
     call.check(launch_gemm(call.c.stream, g), op);
   call.finish();

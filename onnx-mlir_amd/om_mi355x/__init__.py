@@ -38,6 +38,10 @@ _NP_TO_ONNX = {
 }
 
 WRAP, SATURATE = 0, 1
+# `activation` of the fused entry points (OM_MI355X_ACTIVATION_* of the header)
+ACTIVATION_NONE, ACTIVATION_RELU = 0, 1
+# OM_MI355X_VERSION of the header this module was written against
+VERSION = 0x00010000
 
 
 class RuntimeError_(RuntimeError):
@@ -82,9 +86,9 @@ def _declare(lib, shim):
         "om_mi355x_DynamicQuantizeLinear": [P, P, P, P],
         "om_mi355x_DynamicQuantizeLinearNoAlloc": [P, P, P, P],
         "om_mi355x_MatMulInteger": [P, P, P, P, P],
-        "om_mi355x_MatMulIntegerDequant": [P, P, P, P, P, P, P, P],
+        "om_mi355x_MatMulIntegerDequant": [P, P, P, P, P, P, P, P, I64],
         "om_mi355x_QLinearMatMul": [P, P, P, P, P, P, P, P, P, I64],
-        "om_mi355x_DynQuantMatMulDequant": [P, P, P, P, P, P],
+        "om_mi355x_DynQuantMatMulDequant": [P, P, P, P, P, P, I64],
         "om_mi355x_MarkConstant": [P],
         "om_mi355x_UnmarkConstant": [P],
         "om_mi355x_KeepOnDevice": [P],
@@ -139,7 +143,7 @@ def last_gemm_kernel() -> str:
     return _lib.om_mi355x_last_gemm_kernel().decode()
 
 
-def init_compatible(version: int = 0x100) -> bool:
+def init_compatible(version: int = VERSION) -> bool:
     load()
     return bool(_lib.OMInitCompatibleAccelMI355X(version))
 
@@ -396,7 +400,8 @@ def MatMulInteger(a: Tensor, b: Tensor, a_zero_point: Optional[Tensor] = None,
 
 def MatMulIntegerDequant(a: Tensor, b: Tensor, a_zero_point: Optional[Tensor],
                          b_zero_point: Optional[Tensor], a_scale: Tensor, b_scale: Tensor,
-                         bias: Optional[Tensor] = None, out: Optional[Tensor] = None) -> Tensor:
+                         bias: Optional[Tensor] = None, out: Optional[Tensor] = None,
+                         activation: int = ACTIVATION_NONE) -> Tensor:
     load()
     a, b = _host(a), _host(b)
     a_scale, b_scale = _host(a_scale, np.float32), _host(b_scale, np.float32)
@@ -406,7 +411,7 @@ def MatMulIntegerDequant(a: Tensor, b: Tensor, a_zero_point: Optional[Tensor],
     y = out if out is not None else _like(a, _mm_shape(a, b), np.float32)
     with _OMT(y) as hy, _OMT(a) as ha, _OMT(b) as hb, _OMT(az) as haz, _OMT(bz) as hbz, \
             _OMT(a_scale) as has, _OMT(b_scale) as hbs, _OMT(bias) as hbias:
-        _lib.om_mi355x_MatMulIntegerDequant(hy, ha, hb, haz, hbz, has, hbs, hbias)
+        _lib.om_mi355x_MatMulIntegerDequant(hy, ha, hb, haz, hbz, has, hbs, hbias, int(activation))
     _check()
     return y
 
@@ -431,7 +436,7 @@ def QLinearMatMul(a: Tensor, a_scale: Tensor, a_zero_point: Tensor, b: Tensor,
 
 def DynQuantMatMulDequant(x: Tensor, b: Tensor, b_zero_point: Optional[Tensor],
                           b_scale: Tensor, bias: Optional[Tensor] = None,
-                          out: Optional[Tensor] = None) -> Tensor:
+                          out: Optional[Tensor] = None, activation: int = ACTIVATION_NONE) -> Tensor:
     load()
     x, b, b_scale = _host(x), _host(b), _host(b_scale, np.float32)
     bz = None if b_zero_point is None else _host(b_zero_point)
@@ -439,7 +444,7 @@ def DynQuantMatMulDequant(x: Tensor, b: Tensor, b_zero_point: Optional[Tensor],
     y = out if out is not None else _like(x, _mm_shape(x, b), np.float32)
     with _OMT(y) as hy, _OMT(x) as hx, _OMT(b) as hb, _OMT(bz) as hbz, _OMT(b_scale) as hbs, \
             _OMT(bias) as hbias:
-        _lib.om_mi355x_DynQuantMatMulDequant(hy, hx, hb, hbz, hbs, hbias)
+        _lib.om_mi355x_DynQuantMatMulDequant(hy, hx, hb, hbz, hbs, hbias, int(activation))
     _check()
     return y
 

@@ -436,3 +436,14 @@ void om_oracle_dequant_epilogue(const int32_t *acc, int64_t M, int64_t N,
       out[i * N + j] = (float)acc[i * N + j] * s;
     }
 }
+
+/* onnx.Relu: create.math.max(zero, x)
+ * (src/Conversion/ONNXToKrnl/Math/Elementwise.cpp:746-754), a maximum that
+ * returns the other operand when one is a NaN, so a NaN gives 0.  Which zero
+ * max(+0, -0) gives is left open by that operation; this restatement gives +0.
+ * Pinned by numpy's fmax (the same NaN rule) on random values, infinities and
+ * NaNs in tests/test_oracle.py. */
+void om_oracle_relu(const float *x, int64_t n, float *out) {
+  for (int64_t i = 0; i < n; ++i)
+    out[i] = x[i] > 0.0f ? x[i] : 0.0f;
+}

@@ -14,7 +14,7 @@
  *
  * Parity status per function (what pins it is listed in om_oracle.c):
  *   om_oracle_rne, quantize (per-tensor), dequantize (per-tensor),
- *   dynamic_quantize, matmul_integer, qlinear_matmul, dequant_epilogue:
+ *   dynamic_quantize, matmul_integer, qlinear_matmul, dequant_epilogue, relu:
  *   pinned by the reference's enabled ONNX node-test vectors, its constant-
  *   propagation lit answers and closed forms.
  *   quantize / dequantize PER-AXIS: "parity unpinned" -- the reference's CPU
@@ -91,6 +91,9 @@ void om_oracle_qlinear_matmul(const void *A, int akind, float a_scale,
 /* out[i,j] = f32(acc[i,j]) * (a_scale * b_scale[j or 0]). */
 void om_oracle_dequant_epilogue(const int32_t *acc, int64_t M, int64_t N,
     float a_scale, const float *b_scale, int64_t b_scale_len, float *out);
+
+/* out[i] = max(0, x[i]); NaN -> 0. */
+void om_oracle_relu(const float *x, int64_t n, float *out);
 
 /* The reference's pass structure for Q / DQ / DQL with OpenMP, used only as
  * the timed CPU baseline (results identical to the functions above). */

@@ -53,6 +53,8 @@ class Oracle:
             P, I, F, P, I64, P, I, F, P, I64, F, P, I, I64, I64, I64, I, P]
         lib.om_oracle_dequant_epilogue.restype = None
         lib.om_oracle_dequant_epilogue.argtypes = [P, I64, I64, F, P, I64, P]
+        lib.om_oracle_relu.restype = None
+        lib.om_oracle_relu.argtypes = [P, I64, P]
         lib.om_oracle_num_threads.restype = I
 
     # -- helpers ----------------------------------------------------------
@@ -186,6 +188,12 @@ class Oracle:
         out = np.empty(acc.shape, np.float32)
         self.lib.om_oracle_dequant_epilogue(
             _p(acc), M, N, ctypes.c_float(float(np.float32(a_scale))), _p(bs), bs.size, _p(out))
+        return out
+
+    def relu(self, x):
+        x = np.ascontiguousarray(x, np.float32)
+        out = np.empty(x.shape, np.float32)
+        self.lib.om_oracle_relu(_p(x), x.size, _p(out))
         return out
 
     def num_threads(self):

@@ -126,14 +126,15 @@ def test_argument_validation_sets_einval(rt):
 def test_incompatible_version_is_refused(rt):
     lib = rt.load()
     assert lib.OMInitCompatibleAccelMI355X(0x00020000) == 0   # newer major
-    assert lib.OMInitCompatibleAccelMI355X(0x00000101) == 0   # newer minor
+    assert lib.OMInitCompatibleAccelMI355X(0x00000100) == 0   # older major: signatures have changed since
+    assert lib.OMInitCompatibleAccelMI355X(0x00010100) == 0   # newer minor
     rt._lib.om_mi355x_last_error()
 
 
 @pytest.mark.skipif(not _no_gpu(), reason="only meaningful on a box without a GPU")
 def test_without_a_gpu_the_ops_fail_loudly(rt):
     lib = rt.load()
-    assert lib.OMInitCompatibleAccelMI355X(0x100) == 0    # run_main_graph would return NULL
+    assert lib.OMInitCompatibleAccelMI355X(rt.VERSION) == 0    # run_main_graph would return NULL
     with pytest.raises(rt.RuntimeError_, match="accelerator unavailable"):
         rt.QuantizeLinear(np.ones(8, np.float32), np.float32(0.5), np.array(3, np.uint8))
     with pytest.raises(rt.RuntimeError_, match="accelerator unavailable"):
@@ -169,8 +170,8 @@ def test_compiler_plugin_calls_only_exported_symbols(rt):
     # parameter counts: results + operands + integer attributes of each pattern
     passed = {"om_mi355x_QuantizeLinear": 1 + 3 + 2, "om_mi355x_DequantizeLinear": 1 + 3 + 1,
               "om_mi355x_DynamicQuantizeLinear": 3 + 1, "om_mi355x_MatMulInteger": 1 + 4,
-              "om_mi355x_QLinearMatMul": 1 + 8 + 1, "om_mi355x_MatMulIntegerDequant": 1 + 7,
-              "om_mi355x_DynQuantMatMulDequant": 1 + 5, "om_mi355x_MarkConstant": 1,
+              "om_mi355x_QLinearMatMul": 1 + 8 + 1, "om_mi355x_MatMulIntegerDequant": 1 + 7 + 1,
+              "om_mi355x_DynQuantMatMulDequant": 1 + 5 + 1, "om_mi355x_MarkConstant": 1,
               "om_mi355x_KeepOnDevice": 1, "om_mi355x_Release": 1}
     for name, count in passed.items():
         m = re.search(r"\b%s\s*\(([^)]*)\)" % name, header)
@@ -196,3 +197,38 @@ def test_compiler_plugin_lit_tests_name_real_entry_points(rt):
         assert "// RUN: onnx-mlir-opt --maccel=MI355X" in text
         for name in set(re.findall(r'"(om_mi355x_\w+)"', text)):
             assert hasattr(lib, name), (f, name)
+
+
+def test_benchmark_model_texts_are_what_their_generator_writes():
+    """bench/models/*.mlir are the five configurations as ONNX-dialect text for
+    the reference compiler; they must stay in step with the script beside them,
+    and their shapes with the workloads the GPU bench runs."""
+    import importlib.util
+    models = os.path.join(ROOT, "bench", "models")
+    spec = importlib.util.spec_from_file_location("make_models", os.path.join(models, "make_models.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    for n in range(1, 6):
+        assert f"cfg{n}.mlir" in mod.MODELS
+    for name, text in mod.MODELS.items():
+        with open(os.path.join(models, name)) as fh:
+            assert fh.read() == text, name
+        assert text.count("{") == text.count("}") and '"onnx.EntryPoint"() {func = @main_graph}' in text
+    assert "tensor<4096x768xui8>" in mod.MODELS["cfg4_matmulinteger.mlir"]
+    assert "tensor<768x3072xi8>" in mod.MODELS["cfg4_matmulinteger.mlir"]
+    assert "tensor<8191x32767xf32>" in mod.MODELS["cfg2_per_axis_ragged.mlir"]
+
+
+def test_reference_compiler_leg_of_the_bench_is_skipped_without_the_compiler(monkeypatch):
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("bench_main", os.path.join(ROOT, "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    monkeypatch.setenv("PATH", "/nonexistent")
+    assert bench.onnx_mlir_leg(None, None, None, None, None, None) is None
+
+
+def test_python_module_version_is_the_headers():
+    import om_mi355x
+    header = open(os.path.join(INCLUDE, "om_mi355x.h")).read()
+    assert om_mi355x.VERSION == int(re.search(r"#define\s+OM_MI355X_VERSION\s+(0x[0-9a-fA-F]+)", header).group(1), 16)

@@ -38,7 +38,7 @@ def test_device_is_gfx950(rt):
     info = rt.device_info()
     print("device:", info, flush=True)
     assert info["arch"].startswith("gfx950")
-    assert rt.init_compatible(0x100)
+    assert rt.init_compatible(rt.VERSION)
 
 
 def test_golden_vectors_on_gpu(rt):
@@ -715,6 +715,50 @@ def test_matmulinteger_batched_a(rt, oracle):
     az = _rand_q(rng, np.uint8, ())
     got = rt.MatMulInteger(A, B, az, None)
     assert got.shape == (3, 5, 24) and np.array_equal(got, oracle.matmul_integer(A, B, az, None))
+
+
+def test_fused_relu_epilogue(rt, oracle):
+    """`activation` = Relu on the two fused entry points equals onnx.Relu applied
+    to the call's own result without it (max(0, x) is exact), over the kernels a
+    shape can take: the weights-in-registers kernel (K = 768), the LDS-staged
+    ones, ragged edges, the few-row kernels with and without their own
+    quantization, per-row zero points, with and without a bias; a NaN bias
+    gives 0, as the reference's maximum does
+    (src/Conversion/ONNXToKrnl/Math/Elementwise.cpp:746-754)."""
+    rng = np.random.default_rng(47)
+    for M, K, N in ((512, 768, 3072), (300, 768, 1000), (256, 1024, 512), (130, 200, 70), (4, 4096, 256), (7, 100, 33)):
+        A, B = _rand_q(rng, np.uint8, (M, K)), _rand_q(rng, np.int8, (K, N))
+        az = _rand_q(rng, np.uint8, ())
+        a_s = np.float32(0.013)
+        bs = rng.uniform(1e-3, 1e-2, N).astype(np.float32)
+        bias = rng.standard_normal(N).astype(np.float32) * 3
+        bias[N // 2] = np.nan
+        for b in (None, bias):
+            plain = rt.MatMulIntegerDequant(A, B, az, None, a_s, bs, b)
+            got = rt.MatMulIntegerDequant(A, B, az, None, a_s, bs, b, activation=rt.ACTIVATION_RELU)
+            want = oracle.relu(plain)
+            assert same_f32(got, want), (M, K, N, b is None)
+            assert (got >= 0).all() and (got > 0).any() and (got == 0).any()
+            # and against the oracle's own chain
+            acc = oracle.matmul_integer(A, B, az, None)
+            chain = oracle.dequant_epilogue(acc, a_s, bs)
+            if b is not None:
+                chain = chain + b
+            assert same_f32(got, oracle.relu(chain)), (M, K, N)
+        x = rng.standard_normal((M, K)).astype(np.float32)
+        plain = rt.DynQuantMatMulDequant(x, B, None, bs, bias)
+        got = rt.DynQuantMatMulDequant(x, B, None, bs, bias, activation=rt.ACTIVATION_RELU)
+        assert same_f32(got, oracle.relu(plain)), (M, K, N)
+    # per-row zero points take the epilogue's other branch
+    A, B = _rand_q(rng, np.int8, (70, 96)), _rand_q(rng, np.uint8, (96, 40))
+    azm, bzn = _rand_q(rng, np.int8, (70,)), _rand_q(rng, np.uint8, (40,))
+    plain = rt.MatMulIntegerDequant(A, B, azm, bzn, np.float32(0.1), np.float32(0.2))
+    got = rt.MatMulIntegerDequant(A, B, azm, bzn, np.float32(0.1), np.float32(0.2), activation=1)
+    assert same_f32(got, oracle.relu(plain))
+    with pytest.raises(rt.RuntimeError_, match="activation"):
+        rt.MatMulIntegerDequant(A, B, azm, bzn, np.float32(0.1), np.float32(0.2), activation=2)
+    with pytest.raises(rt.RuntimeError_, match="activation"):
+        rt.DynQuantMatMulDequant(np.zeros((4, 96), np.float32), B, None, np.float32(0.2), activation=-1)
 
 
 def test_matmulinteger_batched_b(rt, oracle):

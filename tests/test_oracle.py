@@ -344,3 +344,17 @@ def test_batched_matmul_wrapper_equals_numpy_matmul(oracle):
         want = np.matmul(A.astype(np.int64) - int(az), B.astype(np.int64) - bz.astype(np.int64))
         got = oracle.matmul_integer(A, B, az, bz)
         assert got.shape == want.shape and np.array_equal(got.astype(np.int64), want)
+
+
+
+def test_relu_equals_numpy_fmax(oracle):
+    """Relu is max(0, x) with the NaN rule of maxnum / fmax (the other operand
+    wins): numpy's fmax is that operation.  Zeros compare equal whatever their
+    sign, which the reference's operation leaves open."""
+    rng = np.random.default_rng(92)
+    x = rng.standard_normal(10000).astype(np.float32)
+    x[:8] = [np.nan, -np.nan, np.inf, -np.inf, 0.0, -0.0, 1e-45, -1e-45]
+    got = oracle.relu(x)
+    assert np.array_equal(got, np.fmax(x, np.float32(0)))
+    assert got[0] == 0 and got[1] == 0 and got[2] == np.inf and got[3] == 0
+    assert not np.signbit(got[5]) and got[6] == np.float32(1e-45)
