@@ -1256,17 +1256,24 @@ __global__ __launch_bounds__(512) void k_gemm_i8_skinny_bp(
     float zpf;
     dynamic_params(lo, hi, dq_scale, zpf);
     dq_zp = (int32_t)(uint32_t)zpf;
+    const float recip = 1.0f / dq_scale;
+    auto quantize = [&](auto fast_c) {
+      constexpr bool FAST = decltype(fast_c)::value;
 #pragma unroll
-    for (int j = 0; j < NV; ++j) {
-      const int e = j * (WAVES * 64) + tid;
-      if (e < nvec) {
-        const uint32_t q = quant_one<false, true>(v[j].x, dq_scale, zpf) |
-                           (quant_one<false, true>(v[j].y, dq_scale, zpf) << 8) |
-                           (quant_one<false, true>(v[j].z, dq_scale, zpf) << 16) |
-                           (quant_one<false, true>(v[j].w, dq_scale, zpf) << 24);
-        ((uint32_t *)aq)[e] = q ^ 0x80808080u;
+      for (int j = 0; j < NV; ++j) {
+        const int e = j * (WAVES * 64) + tid;
+        if (e < nvec) {
+          const uint32_t q = quant_pack4<false, true, FAST>(v[j].x, v[j].y,
+              v[j].z, v[j].w, dq_scale, dq_scale, dq_scale, dq_scale, recip,
+              recip, recip, recip, zpf, zpf, zpf, zpf);
+          ((uint32_t *)aq)[e] = q ^ 0x80808080u;
+        }
       }
-    }
+    };
+    if (scale_is_tame(dq_scale)) // the same for every thread
+      quantize(std::true_type{});
+    else
+      quantize(std::false_type{});
     __syncthreads();
   }
 

@@ -125,18 +125,85 @@ hipError_t launch_fill_u32(hipStream_t s, uint32_t *p, int64_t n, uint32_t v);
 // generated code (src/Conversion/ONNXToKrnl/Quantization/QuantizeLinear.cpp
 // :119-144): IEEE divide, round half to even, separate add of the zero point,
 // maxnum then minnum (NaN -> lower bound), float -> integer.
-template <bool SIGNED, bool HAS_ZP>
-__device__ __forceinline__ uint32_t quant_one(float x, float s, float zpf) {
-  float t = x / s;
-  float r = __builtin_rintf(t);
+//
+// The divide.  x / s correctly rounded costs eleven vector instructions
+// (scaling of operands near the ends of the exponent range, a reciprocal
+// estimate, two refinement steps, the final correction and fix-up).  When the
+// reciprocal r = RN(1 / s) is at hand -- computed once per scale with that
+// same divide -- a single correction step gives the correctly rounded quotient:
+//     q0 = RN(x * r);  e = x - q0 * s (exact in one fma);  q = RN(q0 + e * r)
+// (Markstein's theorem: a faithful q0 and a correctly rounded r suffice), as
+// long as nothing under- or overflows on the way.  That holds for "tame"
+// scales, 2^-96 <= s <= 2^96, and quotients of magnitude 2^-3 .. 2^10; a
+// smaller quotient may be off by an ulp, which cannot change its rounding to
+// the integer 0, and q0 is clamped to +-1024 first, so that a larger one (or
+// an infinite x, for which e would be a NaN) stays beyond +-1023, where the
+// 8-bit result saturates whatever the zero point; a NaN x stays a NaN.
+// quotient<true> therefore gives the same 8-bit result as x / s for every x,
+// in four instructions.  Checked against the divide on the CPU for 2.4e9 random
+// pairs and 2.7e10 pairs next to a rounding boundary (no difference), and on
+// the GPU by the boundary test of the parity suite.  Any other scale (zero,
+// negative, denormal, huge, infinite, NaN) takes quotient<false>, the divide.
+__device__ __forceinline__ bool scale_is_tame(float s) {
+  return s >= 0x1p-96f && s <= 0x1p96f;
+}
+template <bool FAST>
+__device__ __forceinline__ float quotient(float x, float s, float r) {
+  if (!FAST)
+    return x / s;
+  const float q0 =
+      __builtin_fminf(__builtin_fmaxf(x * r, -1024.0f), 1024.0f);
+  const float e = __builtin_fmaf(-q0, s, x);
+  return __builtin_fmaf(e, r, q0);
+}
+
+// rne(x / s) + zp, not yet clamped.
+template <bool HAS_ZP, bool FAST>
+__device__ __forceinline__ float quant_value(
+    float x, float s, float r, float zpf) {
+  float v = __builtin_rintf(quotient<FAST>(x, s, r));
   if (HAS_ZP)
-    r = r + zpf;
+    v = v + zpf;
+  return v;
+}
+
+template <bool SIGNED, bool HAS_ZP, bool FAST = false>
+__device__ __forceinline__ uint32_t quant_one(
+    float x, float s, float zpf, float r = 0.0f) {
+  const float v = quant_value<HAS_ZP, FAST>(x, s, r, zpf);
   if (SIGNED) {
-    float c = __builtin_fminf(__builtin_fmaxf(r, -128.0f), 127.0f);
+    float c = __builtin_fminf(__builtin_fmaxf(v, -128.0f), 127.0f);
     return (uint32_t)((int32_t)c) & 0xFFu;
   }
-  float c = __builtin_fminf(__builtin_fmaxf(r, 0.0f), 255.0f);
+  float c = __builtin_fminf(__builtin_fmaxf(v, 0.0f), 255.0f);
   return (uint32_t)c;
+}
+
+// Four values into the bytes of one word.  Unsigned: v_cvt_pk_u8_f32 converts
+// with saturation to 0 .. 255 and writes the byte in place; its input is
+// already an integer (or an infinity, which saturates, or a NaN, which gives
+// 0 = the lower bound, as maxnum-then-minnum does), so its own rounding never
+// acts.
+template <bool SIGNED, bool HAS_ZP, bool FAST>
+__device__ __forceinline__ uint32_t quant_pack4(float x0, float x1, float x2,
+    float x3, float s0, float s1, float s2, float s3, float r0, float r1,
+    float r2, float r3, float z0, float z1, float z2, float z3) {
+  if (SIGNED) {
+    return quant_one<true, HAS_ZP, FAST>(x0, s0, z0, r0) |
+           (quant_one<true, HAS_ZP, FAST>(x1, s1, z1, r1) << 8) |
+           (quant_one<true, HAS_ZP, FAST>(x2, s2, z2, r2) << 16) |
+           (quant_one<true, HAS_ZP, FAST>(x3, s3, z3, r3) << 24);
+  }
+  uint32_t w = 0;
+  w = __builtin_amdgcn_cvt_pk_u8_f32(
+      quant_value<HAS_ZP, FAST>(x0, s0, r0, z0), 0, w);
+  w = __builtin_amdgcn_cvt_pk_u8_f32(
+      quant_value<HAS_ZP, FAST>(x1, s1, r1, z1), 1, w);
+  w = __builtin_amdgcn_cvt_pk_u8_f32(
+      quant_value<HAS_ZP, FAST>(x2, s2, r2, z2), 2, w);
+  w = __builtin_amdgcn_cvt_pk_u8_f32(
+      quant_value<HAS_ZP, FAST>(x3, s3, r3, z3), 3, w);
+  return w;
 }
 
 // minnum / maxnum from +inf / -inf (src/Conversion/ONNXToKrnl/Math/

@@ -8,7 +8,10 @@
 //
 // Arithmetic follows the reference's generated code operation for operation
 // (src/Conversion/ONNXToKrnl/Quantization/QuantizeLinear.cpp:119-144):
-//   t = x / scale          IEEE-754 correctly rounded divide (never rcp*mul)
+//   t = x / scale          IEEE-754 correctly rounded quotient: the divide, or
+//                          for scales of ordinary magnitude a reciprocal
+//                          multiply with an exact correction step that gives
+//                          the same bits (quotient<> in om_kernels.h)
 //   r = roundEven(t)       v_rndne_f32 == the reference's floor-based
 //                          emulation (src/Dialect/Mlir/DialectBuilder.cpp
 //                          :291-332) for every input, up to the sign of zero
@@ -20,6 +23,7 @@
 #include "om_kernels.h"
 
 #include <mutex>
+#include <type_traits>
 
 #include <stdlib.h>
 
@@ -43,14 +47,26 @@ __device__ __forceinline__ float load_zp_f32(const void *zp, int64_t i) {
   return (float)(uint32_t)((const uint8_t *)zp)[i];
 }
 
-template <bool SIGNED, bool HAS_ZP>
+// Four elements that share one scale; r = 1 / s is used when FAST (only for
+// a tame s, see scale_is_tame).
+template <bool SIGNED, bool HAS_ZP, bool FAST, typename V4>
 __device__ __forceinline__ uint32_t quant_four(
-    f4a v, float s, float zpf, uint32_t flip) {
-  uint32_t b0 = quant_one<SIGNED, HAS_ZP>(v.x, s, zpf);
-  uint32_t b1 = quant_one<SIGNED, HAS_ZP>(v.y, s, zpf);
-  uint32_t b2 = quant_one<SIGNED, HAS_ZP>(v.z, s, zpf);
-  uint32_t b3 = quant_one<SIGNED, HAS_ZP>(v.w, s, zpf);
-  return (b0 | (b1 << 8) | (b2 << 16) | (b3 << 24)) ^ flip;
+    V4 v, float s, float r, float zpf, uint32_t flip) {
+  return quant_pack4<SIGNED, HAS_ZP, FAST>(
+             v.x, v.y, v.z, v.w, s, s, s, s, r, r, r, r, zpf, zpf, zpf, zpf) ^
+         flip;
+}
+// Four elements with a scale each (four adjacent columns of a per-axis op).
+template <bool SIGNED, bool HAS_ZP, bool FAST, typename V4>
+__device__ __forceinline__ uint32_t quant_cols(V4 v, const float (&s)[4],
+    const float (&r)[4], const float (&z)[4]) {
+  return quant_pack4<SIGNED, HAS_ZP, FAST>(v.x, v.y, v.z, v.w, s[0], s[1], s[2],
+      s[3], r[0], r[1], r[2], r[3], z[0], z[1], z[2], z[3]);
+}
+// Whether every lane of the wave holds tame scales: the kernels pick the
+// short quotient by a branch the whole wave takes together.
+__device__ __forceinline__ bool wave_all(bool p) {
+  return __builtin_amdgcn_ballot_w64(!p) == 0;
 }
 
 // ---- per-tensor quantize over a flat array -------------------------------
@@ -66,28 +82,37 @@ __global__ __launch_bounds__(kThreads) void k_quant_flat(
     const float *__restrict__ scale_p, const void *__restrict__ zp_p,
     uint32_t flip) {
   const float s = scale_p[0];
+  const float r = 1.0f / s;
   const float zpf = HAS_ZP ? load_zp_f32<SIGNED>(zp_p, 0) : 0.0f;
   const int64_t nvec = n >> 2;
   const f4a *__restrict__ x4 = (const f4a *)x;
   uint32_t *__restrict__ y4 = (uint32_t *)y;
   const int64_t step = (int64_t)gridDim.x * (kThreads * kUnroll);
-  for (int64_t base = (int64_t)blockIdx.x * (kThreads * kUnroll); base < nvec;
-       base += step) {
-    f4a v[kUnroll];
-    int64_t idx[kUnroll];
+  auto body = [&](auto fast_c) {
+    constexpr bool FAST = decltype(fast_c)::value;
+    for (int64_t base = (int64_t)blockIdx.x * (kThreads * kUnroll);
+         base < nvec; base += step) {
+      f4a v[kUnroll];
+      int64_t idx[kUnroll];
 #pragma unroll
-    for (int j = 0; j < kUnroll; ++j) {
-      idx[j] = base + j * kThreads + threadIdx.x;
-      if (idx[j] < nvec)
-        v[j] = __builtin_nontemporal_load(&x4[idx[j]]);
-    }
+      for (int j = 0; j < kUnroll; ++j) {
+        idx[j] = base + j * kThreads + threadIdx.x;
+        if (idx[j] < nvec)
+          v[j] = __builtin_nontemporal_load(&x4[idx[j]]);
+      }
 #pragma unroll
-    for (int j = 0; j < kUnroll; ++j) {
-      if (idx[j] < nvec)
-        __builtin_nontemporal_store(
-            quant_four<SIGNED, HAS_ZP>(v[j], s, zpf, flip), &y4[idx[j]]);
+      for (int j = 0; j < kUnroll; ++j) {
+        if (idx[j] < nvec)
+          __builtin_nontemporal_store(
+              quant_four<SIGNED, HAS_ZP, FAST>(v[j], s, r, zpf, flip),
+              &y4[idx[j]]);
+      }
     }
-  }
+  };
+  if (scale_is_tame(s)) // the same for every thread
+    body(std::true_type{});
+  else
+    body(std::false_type{});
   // Up to three trailing elements.
   if (blockIdx.x == 0) {
     int64_t e = (nvec << 2) + threadIdx.x;
@@ -111,6 +136,8 @@ __global__ __launch_bounds__(kThreads) void k_quant_tiled(
     const float *__restrict__ scale_p, const void *__restrict__ zp_p,
     uint32_t flip) {
   const float s = scale_p[0];
+  const float r = 1.0f / s;
+  const bool tame = scale_is_tame(s); // the same for every thread
   const float zpf = HAS_ZP ? load_zp_f32<SIGNED>(zp_p, 0) : 0.0f;
   const int64_t nvec = n >> 2;
   const f4a *__restrict__ x4 = (const f4a *)x;
@@ -124,14 +151,21 @@ __global__ __launch_bounds__(kThreads) void k_quant_tiled(
     if (idx < nvec)
       v[j] = __builtin_nontemporal_load(&x4[idx]);
   }
+  auto store = [&](auto fast_c) {
+    constexpr bool FAST = decltype(fast_c)::value;
 #pragma unroll
-  for (int j = 0; j < kTileRows; ++j) {
-    const int64_t idx = first + (int64_t)j * kTileRun;
-    if (idx < nvec) {
-      // plain stores: streaming ones are 7 % slower here
-      y4[idx] = quant_four<SIGNED, HAS_ZP>(v[j], s, zpf, flip);
+    for (int j = 0; j < kTileRows; ++j) {
+      const int64_t idx = first + (int64_t)j * kTileRun;
+      if (idx < nvec) {
+        // plain stores: streaming ones are 7 % slower here
+        y4[idx] = quant_four<SIGNED, HAS_ZP, FAST>(v[j], s, r, zpf, flip);
+      }
     }
-  }
+  };
+  if (tame)
+    store(std::true_type{});
+  else
+    store(std::false_type{});
   if (blockIdx.x == 0 && blockIdx.y == 0) {
     int64_t e = (nvec << 2) + threadIdx.x;
     if (e < n)
@@ -153,41 +187,44 @@ __global__ __launch_bounds__(kThreads) void k_quant_lastaxis(
   if (c0 >= C)
     return;
   const int ncol = (C - c0 >= 4) ? 4 : (int)(C - c0);
-  float s[4], z[4];
+  float s[4], z[4], rc[4];
+  bool tame = true;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int64_t c = c0 + (j < ncol ? j : 0);
     s[j] = scale[c];
+    rc[j] = 1.0f / s[j];
+    tame = tame && scale_is_tame(s[j]);
     z[j] = HAS_ZP ? load_zp_f32<SIGNED>(zp, c) : 0.0f;
   }
   const int64_t r_begin = (int64_t)blockIdx.y * rows_per_block;
   const int64_t r_end =
       (r_begin + rows_per_block < rows) ? r_begin + rows_per_block : rows;
   if (ncol == 4) {
-    int64_t r = r_begin;
-    for (; r + kRowUnroll <= r_end; r += kRowUnroll) {
-      f4u v[kRowUnroll];
+    auto walk = [&](auto fast_c) {
+      constexpr bool FAST = decltype(fast_c)::value;
+      int64_t r = r_begin;
+      for (; r + kRowUnroll <= r_end; r += kRowUnroll) {
+        f4u v[kRowUnroll];
 #pragma unroll
-      for (int j = 0; j < kRowUnroll; ++j)
-        v[j] = __builtin_nontemporal_load((const f4u *)(x + (r + j) * C + c0));
+        for (int j = 0; j < kRowUnroll; ++j)
+          v[j] =
+              __builtin_nontemporal_load((const f4u *)(x + (r + j) * C + c0));
 #pragma unroll
-      for (int j = 0; j < kRowUnroll; ++j) {
-        uint32_t b0 = quant_one<SIGNED, HAS_ZP>(v[j].x, s[0], z[0]);
-        uint32_t b1 = quant_one<SIGNED, HAS_ZP>(v[j].y, s[1], z[1]);
-        uint32_t b2 = quant_one<SIGNED, HAS_ZP>(v[j].z, s[2], z[2]);
-        uint32_t b3 = quant_one<SIGNED, HAS_ZP>(v[j].w, s[3], z[3]);
-        *(u32_a1 *)(y + (r + j) * C + c0) =
-            b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
+        for (int j = 0; j < kRowUnroll; ++j)
+          *(u32_a1 *)(y + (r + j) * C + c0) =
+              quant_cols<SIGNED, HAS_ZP, FAST>(v[j], s, rc, z);
       }
-    }
-    for (; r < r_end; ++r) {
-      f4u v = *(const f4u *)(x + r * C + c0);
-      uint32_t b0 = quant_one<SIGNED, HAS_ZP>(v.x, s[0], z[0]);
-      uint32_t b1 = quant_one<SIGNED, HAS_ZP>(v.y, s[1], z[1]);
-      uint32_t b2 = quant_one<SIGNED, HAS_ZP>(v.z, s[2], z[2]);
-      uint32_t b3 = quant_one<SIGNED, HAS_ZP>(v.w, s[3], z[3]);
-      *(u32_a1 *)(y + r * C + c0) = b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
-    }
+      for (; r < r_end; ++r) {
+        f4u v = *(const f4u *)(x + r * C + c0);
+        *(u32_a1 *)(y + r * C + c0) =
+            quant_cols<SIGNED, HAS_ZP, FAST>(v, s, rc, z);
+      }
+    };
+    if (wave_all(tame))
+      walk(std::true_type{});
+    else
+      walk(std::false_type{});
   } else {
     for (int64_t r = r_begin; r < r_end; ++r)
       for (int j = 0; j < ncol; ++j)
@@ -223,43 +260,44 @@ __global__ __launch_bounds__(kThreads) void k_quant_periodic(
   }
   if (v >= period)
     return;
-  float s[4], z[4];
+  float s[4], z[4], rc[4];
+  bool tame = true;
   {
     uint32_t c = (uint32_t)(((uint64_t)v * 4) % C);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       s[e] = scale[c];
+      rc[e] = 1.0f / s[e];
+      tame = tame && scale_is_tame(s[e]);
       z[e] = HAS_ZP ? load_zp_f32<SIGNED>(zp, c) : 0.0f;
       c = (c + 1 == C) ? 0 : c + 1;
     }
   }
   const f4a *__restrict__ x4 = (const f4a *)x;
   uint32_t *__restrict__ y4 = (uint32_t *)y;
-  int64_t idx = (int64_t)blockIdx.y * periods_per_block * period + v;
-  const int64_t end = idx + (int64_t)periods_per_block * period;
+  const int64_t begin = (int64_t)blockIdx.y * periods_per_block * period + v;
+  const int64_t end = begin + (int64_t)periods_per_block * period;
   const int64_t stop = end < nvec ? end : nvec;
-  for (; idx + (kRowUnroll - 1) * period < stop; idx += kRowUnroll * period) {
-    f4a q[kRowUnroll];
+  auto walk = [&](auto fast_c) {
+    constexpr bool FAST = decltype(fast_c)::value;
+    int64_t idx = begin;
+    for (; idx + (kRowUnroll - 1) * period < stop;
+         idx += kRowUnroll * period) {
+      f4a q[kRowUnroll];
 #pragma unroll
-    for (int j = 0; j < kRowUnroll; ++j)
-      q[j] = __builtin_nontemporal_load(&x4[idx + j * period]);
+      for (int j = 0; j < kRowUnroll; ++j)
+        q[j] = __builtin_nontemporal_load(&x4[idx + j * period]);
 #pragma unroll
-    for (int j = 0; j < kRowUnroll; ++j) {
-      const uint32_t b0 = quant_one<SIGNED, HAS_ZP>(q[j].x, s[0], z[0]);
-      const uint32_t b1 = quant_one<SIGNED, HAS_ZP>(q[j].y, s[1], z[1]);
-      const uint32_t b2 = quant_one<SIGNED, HAS_ZP>(q[j].z, s[2], z[2]);
-      const uint32_t b3 = quant_one<SIGNED, HAS_ZP>(q[j].w, s[3], z[3]);
-      y4[idx + j * period] = b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
+      for (int j = 0; j < kRowUnroll; ++j)
+        y4[idx + j * period] = quant_cols<SIGNED, HAS_ZP, FAST>(q[j], s, rc, z);
     }
-  }
-  for (; idx < stop; idx += period) {
-    const f4a q = x4[idx];
-    const uint32_t b0 = quant_one<SIGNED, HAS_ZP>(q.x, s[0], z[0]);
-    const uint32_t b1 = quant_one<SIGNED, HAS_ZP>(q.y, s[1], z[1]);
-    const uint32_t b2 = quant_one<SIGNED, HAS_ZP>(q.z, s[2], z[2]);
-    const uint32_t b3 = quant_one<SIGNED, HAS_ZP>(q.w, s[3], z[3]);
-    y4[idx] = b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
-  }
+    for (; idx < stop; idx += period)
+      y4[idx] = quant_cols<SIGNED, HAS_ZP, FAST>(x4[idx], s, rc, z);
+  };
+  if (wave_all(tame))
+    walk(std::true_type{});
+  else
+    walk(std::false_type{});
 }
 
 // ---- general [outer, channels, inner] quantize ---------------------------
@@ -325,8 +363,15 @@ __global__ __launch_bounds__(kThreads) void k_quant_slabs(
 #pragma unroll
   for (int j = 0; j < U; ++j) {
     const uint32_t idx = first + j * kThreads;
-    if (idx < nvec)
-      y4[idx] = quant_four<SIGNED, HAS_ZP>(v[j], s[j], z[j], 0u);
+    if (idx < nvec) {
+      // a scale per float4: the reciprocal costs a divide, the four elements
+      // then save three
+      if (wave_all(scale_is_tame(s[j])))
+        y4[idx] = quant_four<SIGNED, HAS_ZP, true>(
+            v[j], s[j], 1.0f / s[j], z[j], 0u);
+      else
+        y4[idx] = quant_four<SIGNED, HAS_ZP, false>(v[j], s[j], 0.0f, z[j], 0u);
+    }
   }
 }
 
@@ -785,12 +830,21 @@ __global__ __launch_bounds__(kSmallThreads) void k_dql_small(
     scale_out[0] = scale;
     zp_out[0] = (uint8_t)(uint32_t)zpf;
   }
+  const float recip = 1.0f / scale;
+  auto store = [&](auto fast_c) {
+    constexpr bool FAST = decltype(fast_c)::value;
 #pragma unroll
-  for (int j = 0; j < kSmallPerThread; ++j) {
-    const int64_t e = (int64_t)j * kSmallThreads + threadIdx.x;
-    if (e < n)
-      y[e] = (uint8_t)(quant_one<false, true>(v[j], scale, zpf) ^ (flip & 0xFFu));
-  }
+    for (int j = 0; j < kSmallPerThread; ++j) {
+      const int64_t e = (int64_t)j * kSmallThreads + threadIdx.x;
+      if (e < n)
+        y[e] = (uint8_t)(quant_one<false, true, FAST>(v[j], scale, zpf, recip) ^
+                         (flip & 0xFFu));
+    }
+  };
+  if (scale_is_tame(scale)) // the same for every thread
+    store(std::true_type{});
+  else
+    store(std::false_type{});
 }
 
 // Mid-sized tensors (up to 16 float4 per thread of a grid that fills the
@@ -912,12 +966,20 @@ __global__ __launch_bounds__(kGridThreads) void k_dql_grid(
     zp_out[0] = (uint8_t)(uint32_t)zpf;
   }
   uint32_t *__restrict__ y4 = (uint32_t *)y;
+  const float recip = 1.0f / scale;
+  auto store = [&](auto fast_c) {
+    constexpr bool FAST = decltype(fast_c)::value;
 #pragma unroll
-  for (int j = 0; j < NV; ++j) {
-    const int64_t idx = (int64_t)j * total + gtid;
-    if (idx < nvec)
-      y4[idx] = quant_four<false, true>(v[j], scale, zpf, flip);
-  }
+    for (int j = 0; j < NV; ++j) {
+      const int64_t idx = (int64_t)j * total + gtid;
+      if (idx < nvec)
+        y4[idx] = quant_four<false, true, FAST>(v[j], scale, recip, zpf, flip);
+    }
+  };
+  if (scale_is_tame(scale)) // the same for every thread
+    store(std::true_type{});
+  else
+    store(std::false_type{});
   if (gtid < 3 && te < n)
     y[te] = (uint8_t)(quant_one<false, true>(tail, scale, zpf) ^ (flip & 0xFFu));
 }

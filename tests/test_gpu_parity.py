@@ -106,6 +106,86 @@ def test_quantize_zero_and_denormal_scale(rt, oracle):
         assert np.array_equal(rt.QuantizeLinear(x, np.float32(s), np.array(9, np.uint8)), want), s
 
 
+def _boundary_points(s):
+    """Inputs whose quotient by the scale s lies next to a rounding boundary:
+    the floats within three ulps of (k + 1/2) * s and of k * s for |k| <= 300
+    (beyond +-256 every 8-bit result saturates), and the special values."""
+    k = np.arange(-300, 301, dtype=np.float64)
+    with np.errstate(all="ignore"):
+        centres = np.concatenate([(k + 0.5) * float(s), k * float(s)]).astype(np.float32)
+    centres = centres[np.isfinite(centres)]
+    pts = [(centres.view(np.int32) + d).view(np.float32) for d in range(-3, 4)]
+    special = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 3e38, -3e38, 1e-45, -1e-45, 1e-38, 1.0, -1.0],
+                       np.float32)
+    return np.concatenate(pts + [special])
+
+
+# Scales whose quotients take the reciprocal-multiply-and-correct path (2^-96 ..
+# 2^96: ordinary ones, powers of two, significands of all ones or all zeros but
+# the last bit, both ends of the range) and scales that take the divide.
+_TAME_SCALES = [0.1, 1.0, 0.0173, 3.0, 2.0 ** -20, 1.0 - 2.0 ** -24, 2.0 - 2.0 ** -23, 1.0 + 2.0 ** -23,
+                0.005, 0.05, 255.0, 2.0 ** -96, 2.0 ** 96, 1.7e-20, 6.1e27]
+_OTHER_SCALES = [2.0 ** -97, 1e-38, 1e-39, 1e-45, 1e30, 3e38, 0.0, -0.5, np.inf, np.nan]
+
+
+def test_quantize_next_to_every_rounding_boundary(rt, oracle):
+    """QuantizeLinear divides by the scale either with the full divide or, for
+    scales of ordinary magnitude, with a reciprocal multiply and one exact
+    correction.  Both must give rne(x / s) as the reference's divf does
+    (src/Conversion/ONNXToKrnl/Quantization/QuantizeLinear.cpp:119-144): checked
+    where a one-ulp difference in the quotient would show, next to every
+    half-integer and integer quotient, through the per-tensor kernels (small and
+    4 Mi-element launch shapes), the per-axis kernels (aligned and ragged rows,
+    waves of only ordinary scales and waves that mix in others) and
+    DynamicQuantizeLinear's quantization."""
+    with np.errstate(all="ignore"):
+        for s in _TAME_SCALES + _OTHER_SCALES:
+            s = np.float32(s)
+            x = _boundary_points(s if np.isfinite(s) and s != 0 else np.float32(1))
+            for zp in (np.array(0, np.uint8), np.array(77, np.uint8), np.array(255, np.uint8),
+                       np.array(-128, np.int8), np.array(5, np.int8), None):
+                want = oracle.quantize_linear(x, s, zp)
+                got = rt.QuantizeLinear(x, s, zp)
+                assert np.array_equal(got, want), (float(s), zp)
+        # the launch shape of large tensors (4 Mi elements and more)
+        for s in (np.float32(0.0173), np.float32(2.0 ** -97)):
+            x = np.tile(_boundary_points(s), 500)
+            assert x.size >= 4 << 20
+            zp = np.array(131, np.uint8)
+            assert np.array_equal(rt.QuantizeLinear(x, s, zp), oracle.quantize_linear(x, s, zp)), float(s)
+        # per-axis: a column per scale, its boundary points down the rows
+        rng = np.random.default_rng(48)
+        tame = np.concatenate([np.array(_TAME_SCALES, np.float32),
+                               rng.uniform(0.005, 0.05, 600).astype(np.float32)])
+        for scales in (tame, np.concatenate([tame, np.array(_OTHER_SCALES, np.float32)]),
+                       np.concatenate([tame, np.array(_OTHER_SCALES, np.float32)])[:-1][::-1].copy()):
+            cols = [_boundary_points(s if np.isfinite(s) and s != 0 else np.float32(1)) for s in scales]
+            rows = min(c.size for c in cols)
+            x = np.stack([c[:rows] for c in cols], axis=1)
+            for qdt in (np.uint8, np.int8):
+                info = np.iinfo(qdt)
+                zp = rng.integers(info.min, info.max + 1, scales.size).astype(qdt)
+                assert np.array_equal(rt.QuantizeLinear(x, scales, zp, axis=1),
+                                      oracle.quantize_linear(x, scales, zp, axis=1)), (scales.size, qdt)
+            # the axis in the middle: one scale per slab
+            x3 = np.ascontiguousarray(x.T[:8].reshape(2, 4, -1)[:, :, :rows // 4 * 4])
+            sc3 = scales[:4]
+            assert np.array_equal(rt.QuantizeLinear(x3, sc3, None, axis=1),
+                                  oracle.quantize_linear(x3, sc3, None, axis=1))
+        # DynamicQuantizeLinear: the scale follows from the data; boundary points of that scale
+        for lo, hi, n in ((-3.1, 4.4, 1 << 12), (-0.02, 11.0, 1 << 16), (0.0, 2.55, 3 << 20), (-1e-30, 1e-30, 5000),
+                          (-3e38, 3e38, 70000), (-1e-39, 2e-39, 9000)):
+            lo, hi = np.float32(lo), np.float32(hi)
+            s = (np.maximum(hi, np.float32(0)) - np.minimum(lo, np.float32(0))) / np.float32(255)
+            pts = _boundary_points(s)
+            pts = pts[np.isfinite(pts) & (pts >= lo) & (pts <= hi)]
+            x = np.resize(np.concatenate([[lo, hi], pts]).astype(np.float32), n)
+            wy, ws, wz = oracle.dynamic_quantize_linear(x)
+            gy, gs, gz = rt.DynamicQuantizeLinear(x)
+            assert np.float32(gs).view(np.uint32) == np.float32(ws).view(np.uint32), (float(lo), float(hi), n)
+            assert int(gz) == int(wz) and np.array_equal(gy, wy), (float(lo), float(hi), n)
+
+
 @pytest.mark.parametrize("shape,axis", [((64, 1000), 1), ((37, 1023), 1), ((5, 7), 1), ((129, 4096), -1),
                                         ((3, 5, 64, 33), 1), ((6, 100), 0), ((2, 3, 4, 5), 2),
                                         ((1, 3, 3, 2), 1), ((300, 2), 1), ((1000, 6), 1), ((257, 4097), 1),
