@@ -331,6 +331,31 @@ def qdq_cases(rt, wl, rows, cols, steps, warmup, only=None):
     return out
 
 
+def dql_activation_cases(rt, steps, warmup, only=None):
+    """DynamicQuantizeLinear on activation-sized tensors (the first half of every
+    dynamically quantized layer of config 4): one launch, X read once."""
+    out = {}
+    for rows, cols in ((4096, 768), (4096, 3072)):
+        name = f"dynamic_quantize_{rows}x{cols}"
+        if only is not None and only != name:
+            continue
+        rng = np.random.default_rng(rows + cols)
+        dX = rt.DeviceArray.from_numpy(rng.standard_normal((rows, cols)).astype(np.float32))
+        dQ = rt.DeviceArray((rows, cols), np.uint8)
+        dys, dyz = rt.DeviceArray((), np.float32), rt.DeviceArray((), np.uint8)
+        fn = rt.PreparedCall("om_mi355x_DynamicQuantizeLinear", dQ, dys, dyz, dX)
+        r = measure(rt, fn, steps, warmup)
+        fn.check()
+        fn.close()
+        nbytes = 5 * rows * cols        # X once, the 8-bit result once
+        r.update({"bytes": nbytes, "gbs": nbytes / (r["kernel_ms"] * 1e-3) / 1e9,
+                  "hbm_frac": nbytes / (r["kernel_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS})
+        out[name] = r
+        for d in (dX, dQ, dys, dyz):
+            d.free()
+    return out
+
+
 def only_mode(rt, wl, what, steps, warmup):
     """One kernel, `steps` launches, nothing else on the GPU: the target of the
     rocprofv3 counter runs whose summaries are kept under profiles/."""
@@ -367,6 +392,8 @@ def only_mode(rt, wl, what, steps, warmup):
         r = gemm_case(rt, wl, f"config5 prefill {name}", 2048, k, n, c["W"], c["w_scale"], steps, warmup, "f32",
                       headline=True)
         return {"only": what, **r}
+    if what.startswith("dynamic_quantize_"):
+        return {"only": what, **dql_activation_cases(rt, steps, warmup, only=what)[what]}
     r = qdq_cases(rt, wl, 8192, 32768, steps, warmup, only=what)
     return {"only": what, **r[what]}
 
@@ -502,7 +529,8 @@ def main():
                              "gemm_prefill_up", "gemm_prefill_down", "fused_ffn_up", "fused_ffn_down",
                              "decode", "decode4", "decode16",
                              "quantize_per_axis", "dequantize_per_axis",
-                             "quantize_per_tensor", "dequantize_per_tensor", "dynamic_quantize"],
+                             "quantize_per_tensor", "dequantize_per_tensor", "dynamic_quantize",
+                             "dynamic_quantize_4096x768", "dynamic_quantize_4096x3072"],
                     help="launch just this kernel --steps times (for rocprofv3 counter runs)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -538,6 +566,8 @@ def main():
         qsteps = min(max(MIN_LAUNCHES, args.steps // 10), 200)
         extras["qdq_8192x32768"] = qdq_cases(rt, wl, 8192, 32768, qsteps, 2)
         extras["qdq_8191x32767"] = qdq_cases(rt, wl, 8191, 32767, qsteps, 2)
+    if "qdq" in groups:
+        extras["dql_activations"] = dql_activation_cases(rt, esteps, ewarm)
     if "fused" in groups:
         fused = []
         for name, (k, n) in wl.CONFIG4_SHAPES.items():

@@ -1583,11 +1583,12 @@ hipError_t gemm_launch_cfg(
     // rows quantized inside the kernel (the caller asked gemm_quantizes_rows)
     if (A_MODE != 2 || !gemm_quantizes_rows(g.M, g.K, g.X))
       return hipErrorInvalidValue;
-    if constexpr (A_MODE == 2)
+    if constexpr (A_MODE == 2) {
       t_last_kernel = "k_gemm_i8_skinny_bp (rows quantized in the kernel)";
       k_gemm_i8_skinny_bp<2, EPI, true, 1, false>
           <<<dim3((unsigned)((g.N + 31) / 32)), 512, 0, st>>>(
               nullptr, g.X, g.Bp, M, N, K, Kpad, ep);
+    }
     return hipGetLastError();
   }
   // Up to 64 rows the weight-streaming kernel is ahead of every tile kernel

@@ -34,12 +34,12 @@ struct DqlScratch {
   int grid_blocks;    // dql_grid_blocks(), or 0 to disable the one-launch path
   unsigned spin_limit; // polls a thread of the one-launch kernel waits for
                        // another block's result before giving up
-  unsigned long long *grid_slots; // [2 * max_blocks], zeroed once: per
-                      // block (launch number << 32 | float bits) of its min,
-                      // then of its max
+  unsigned long long *grid_slots; // [2 * max_blocks], 16-byte aligned,
+                      // zeroed once: per block two words, (launch number
+                      // << 32 | float bits) of its min and of its max
   unsigned epoch;     // launch number of the one-launch kernel (host side)
-  int max_blocks;     // capacity of partial_min / partial_max and of each half
-                      // of grid_slots (at most kDqlMaxBlocks)
+  int max_blocks;     // capacity of partial_min / partial_max and blocks
+                      // that grid_slots has room for (at most kDqlMaxBlocks)
   // Two-launch path only (sets grid_blocks to 0 for the call).
   DqlScratch two_launch() const {
     DqlScratch s = *this;

@@ -847,25 +847,41 @@ __global__ __launch_bounds__(kSmallThreads) void k_dql_small(
     store(std::false_type{});
 }
 
-// Mid-sized tensors (up to 16 float4 per thread of a grid that fills the
-// device once): the whole op in one launch.  Every thread keeps its elements
-// in registers while the blocks exchange their minima and maxima, so x is
-// read once, nothing but the result is written, and there is one launch
-// instead of two.  The grid is one block per CU, each of which needs a whole
-// CU's registers, and the launcher keeps at most one such kernel in flight,
-// so its blocks become resident together as soon as older work has drained
-// (a cooperative launch would guarantee that, but costs about 30 us per
-// launch on this platform).  The wait for the other blocks is bounded all the
-// same: a block that gives up raises `failed` and writes nothing.
-constexpr int kGridThreads = 1024;
+// Mid-sized tensors (up to 32 float4 per thread of a grid that fills the
+// device once, 16 Mi elements): the whole op in one launch.  Every thread keeps
+// its elements in registers while the blocks exchange their minima and maxima,
+// so x is read once, nothing but the result is written, and there is one
+// launch instead of two.  The grid is one block per CU, and the launcher keeps
+// at most one such kernel in flight, so its blocks become resident together
+// as soon as older work has drained (a cooperative launch would guarantee
+// that, but costs about 30 us per launch on this platform).  The wait for the
+// other blocks is bounded all the same: a block that gives up raises `failed`
+// and writes nothing.
+//
+// Where the time goes, [4096, 768] / [4096, 3072] on MI355X, microseconds
+// since the first block started (median block): own minimum and maximum known
+// 1.4 / 5.4 (the loads: latency, then 6 TB/s), everybody's known 3.8 / 8.1,
+// last wave done 4.6 / 10.4, next launch can start 6.1 / 15.5.  Blocks of
+// eight waves rather than sixteen start and reduce faster.  Quantizing is
+// bound by the vector units, not by memory (at sixteen instructions per
+// element the last wave finished 4 us after the first: the four-instruction
+// quotient of om_kernels.h is what shortened it).  Plain loads and stores:
+// streaming loads make a loop of nothing but this kernel on one tensor 1.5 us
+// faster at [4096, 3072], but the same kernel 5 us slower when a GEMM runs
+// between its launches (20.9 against 15.3 us in a kernel trace of the fused
+// layer), and streaming stores slow down the GEMM that reads the result next.
+constexpr int kGridThreads = 512;
+constexpr int kGridMaxPerThread = 32; // float4
 
 template <int NV>
 __global__ __launch_bounds__(kGridThreads) void k_dql_grid(
     const float *__restrict__ x, int64_t n, uint8_t *__restrict__ y,
     float *__restrict__ scale_out, uint8_t *__restrict__ zp_out, uint32_t flip,
-    unsigned long long *slot_lo, unsigned long long *slot_hi, unsigned epoch,
-    unsigned *failed, unsigned spin_limit) {
-  __shared__ float s_lo[kGridThreads / 64], s_hi[kGridThreads / 64];
+    unsigned long long *slots, unsigned epoch, unsigned *failed,
+    unsigned spin_limit) {
+  constexpr int kWaves = kGridThreads / 64;
+  __shared__ float s_lo[kWaves], s_hi[kWaves];
+  __shared__ int s_ok;
   const int64_t nvec = n >> 2;
   const int64_t total = (int64_t)gridDim.x * kGridThreads;
   const int64_t gtid = (int64_t)blockIdx.x * kGridThreads + threadIdx.x;
@@ -878,7 +894,8 @@ __global__ __launch_bounds__(kGridThreads) void k_dql_grid(
 #pragma unroll
   for (int j = 0; j < NV; ++j) {
     const int64_t idx = (int64_t)j * total + gtid;
-    v[j] = idx < nvec ? x4[idx] : nan4; // NaN is neutral for minnum / maxnum
+    // NaN is neutral for minnum / maxnum
+    v[j] = idx < nvec ? x4[idx] : nan4;
   }
   // the up to three elements after the last whole float4
   const int64_t te = (nvec << 2) + gtid;
@@ -893,71 +910,94 @@ __global__ __launch_bounds__(kGridThreads) void k_dql_grid(
   lo = __builtin_fminf(lo, tail);
   hi = __builtin_fmaxf(hi, tail);
 
-  auto block_reduce = [&](float &l, float &h) {
-    l = wave_min(l);
-    h = wave_max(h);
-    if ((threadIdx.x & 63) == 0) {
-      s_lo[threadIdx.x >> 6] = l;
-      s_hi[threadIdx.x >> 6] = h;
-    }
-    __syncthreads();
-    l = s_lo[0];
-    h = s_hi[0];
-#pragma unroll
-    for (int w = 1; w < kGridThreads / 64; ++w) {
-      l = __builtin_fminf(l, s_lo[w]);
-      h = __builtin_fmaxf(h, s_hi[w]);
-    }
-    __syncthreads();
-  };
-  block_reduce(lo, hi);
+  // The block's own result, and the flag of the exchange.
+  lo = wave_min(lo);
+  hi = wave_max(hi);
+  if ((threadIdx.x & 63) == 0) {
+    s_lo[threadIdx.x >> 6] = lo;
+    s_hi[threadIdx.x >> 6] = hi;
+  }
+  if (threadIdx.x == 0)
+    s_ok = 1;
+  __syncthreads();
 
-  // Grid-wide exchange of the block results in two memory round trips.  Block
-  // b publishes (tag, min) and (tag, max) as two 64-bit device-scope atomic
-  // stores into its own slots, where tag is this launch's number: value and
-  // "it is there" travel in one word, so no fence and no arrival counter are
-  // needed, and nothing has to be reset between launches.  Every block then
-  // reads all slots with device-scope atomic loads (served where every XCD
-  // sees them, no cache to invalidate), each thread polling one slot until it
-  // carries the tag, and folds them itself: same values, same order of
-  // operations up to the commutative min / max, so all blocks agree.  The wait
-  // is bounded: a thread that gives up makes its block raise `failed` and
-  // write nothing.
+  // Grid-wide exchange in two memory round trips.  Block b publishes
+  // (tag, min) and (tag, max), tag being this launch's number, as two 64-bit
+  // device-scope atomic stores into its own 16-byte slot: value and "it is
+  // there" travel in one word, so no fence and no arrival counter are needed,
+  // and nothing has to be reset between launches.  Every block then reads all
+  // slots, one slot per thread so that all of a block's reads are in flight
+  // together (a thread that polled four slots one after the other made the
+  // exchange 1.3 us longer), each thread polling until both words carry the
+  // tag.  The 16-byte read is one request to the slot's cache line, past the
+  // caches that other XCDs do not see (sc1); each of its 8-byte halves was
+  // written by one atomic store and is checked on its own.  All blocks fold
+  // the same values, in an order that does not matter for min / max, so all
+  // agree.  The wait is bounded: a thread that gives up makes its block raise
+  // `failed` and write nothing.
   if (threadIdx.x == 0) {
+    float bl = s_lo[0], bh = s_hi[0];
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) {
+      bl = __builtin_fminf(bl, s_lo[w]);
+      bh = __builtin_fmaxf(bh, s_hi[w]);
+    }
     const unsigned long long tag = (unsigned long long)epoch << 32;
-    __hip_atomic_store(&slot_lo[blockIdx.x], tag | __float_as_uint(lo),
+    __hip_atomic_store(&slots[2 * blockIdx.x], tag | __float_as_uint(bl),
         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __hip_atomic_store(&slot_hi[blockIdx.x], tag | __float_as_uint(hi),
+    __hip_atomic_store(&slots[2 * blockIdx.x + 1], tag | __float_as_uint(bh),
         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
+  __syncthreads(); // s_lo / s_hi are reused below
+  typedef unsigned long long u64x2 __attribute__((ext_vector_type(2)));
   bool ok = true;
   lo = __builtin_inff();
   hi = -__builtin_inff();
   for (unsigned i = threadIdx.x; i < gridDim.x; i += kGridThreads) {
-    unsigned long long a = 0, b = 0;
+    u64x2 w = {0, 0};
     bool got = false;
     for (unsigned spin = 0; spin < spin_limit; ++spin) {
-      a = __hip_atomic_load(
-          &slot_lo[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      b = __hip_atomic_load(
-          &slot_hi[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      if ((unsigned)(a >> 32) == epoch && (unsigned)(b >> 32) == epoch) {
+      asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)"
+                   : "=v"(w)
+                   : "v"(&slots[2 * i])
+                   : "memory");
+      if ((unsigned)(w.x >> 32) == epoch && (unsigned)(w.y >> 32) == epoch) {
         got = true;
         break;
       }
-      __builtin_amdgcn_s_sleep(8);
+      __builtin_amdgcn_s_sleep(1);
     }
     ok = ok && got;
-    lo = __builtin_fminf(lo, __uint_as_float((unsigned)a));
-    hi = __builtin_fmaxf(hi, __uint_as_float((unsigned)b));
+    lo = __builtin_fminf(lo, __uint_as_float((unsigned)w.x));
+    hi = __builtin_fmaxf(hi, __uint_as_float((unsigned)w.y));
   }
-  if (!__syncthreads_and(ok)) {
+  // only the waves that had a slot to poll take part in the fold
+  const unsigned pollers = gridDim.x < (unsigned)kGridThreads
+                               ? (gridDim.x + 63) / 64
+                               : (unsigned)kWaves;
+  if ((threadIdx.x >> 6) < pollers) {
+    lo = wave_min(lo);
+    hi = wave_max(hi);
+    if (!wave_all(ok) && (threadIdx.x & 63) == 0)
+      s_ok = 0;
+    if ((threadIdx.x & 63) == 0) {
+      s_lo[threadIdx.x >> 6] = lo;
+      s_hi[threadIdx.x >> 6] = hi;
+    }
+  }
+  __syncthreads();
+  if (!s_ok) {
     if (threadIdx.x == 0)
       __hip_atomic_store(
           failed, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     return;
   }
-  block_reduce(lo, hi);
+  lo = s_lo[0];
+  hi = s_hi[0];
+  for (unsigned w = 1; w < pollers; ++w) {
+    lo = __builtin_fminf(lo, s_lo[w]);
+    hi = __builtin_fmaxf(hi, s_hi[w]);
+  }
 
   float scale, zpf;
   dynamic_params(lo, hi, scale, zpf);
@@ -1313,26 +1353,25 @@ hipError_t launch_dynamic_quantize(hipStream_t s, DqlScratch &scratch,
     const int64_t total = (int64_t)scratch.grid_blocks * kGridThreads;
     const int64_t nvec = n >> 2;
     void (*fn_launch)(const float *, int64_t, uint8_t *, float *, uint8_t *,
-        uint32_t, unsigned long long *, unsigned long long *, unsigned,
-        unsigned *, unsigned) = nullptr;
-    // Up to one float4 per thread of the whole grid the launch takes only as
+        uint32_t, unsigned long long *, unsigned, unsigned *, unsigned) =
+        nullptr;
+    // Up to two float4 per thread of the whole grid the launch takes only as
     // many blocks as that needs: the fewer blocks, the shorter the exchange
     // (64 Ki elements: 16 blocks 5.4 us, 4 blocks of 4 float4 per thread 7.0,
     // the two launches of the general path 8.1; 512 Ki: 128 blocks 7.2
     // against 8.2 for 256 blocks of 4 per thread; 96 Ki: 6.1 against 8.1).
     int64_t blocks = scratch.grid_blocks; // <= scratch.max_blocks
-    if (nvec <= total) {
-      fn_launch = k_dql_grid<1>;
-      blocks = (nvec + kGridThreads - 1) / kGridThreads;
-    } else if (nvec <= 4 * total)
-      fn_launch = k_dql_grid<4>;
-    else if (nvec <= 16 * total)
-      fn_launch = k_dql_grid<16>;
+    if (nvec <= 2 * total) {
+      fn_launch = k_dql_grid<2>;
+      blocks = (nvec + 2 * kGridThreads - 1) / (2 * kGridThreads);
+    } else if (nvec <= 8 * total)
+      fn_launch = k_dql_grid<8>;
+    else if (nvec <= kGridMaxPerThread * total)
+      fn_launch = k_dql_grid<kGridMaxPerThread>;
     if (fn_launch) {
       const uint32_t flip = y_shift ? 0x80808080u : 0u;
       const unsigned spin_limit = scratch.spin_limit;
-      unsigned long long *slot_lo = scratch.grid_slots;
-      unsigned long long *slot_hi = scratch.grid_slots + scratch.max_blocks;
+      unsigned long long *slots = scratch.grid_slots; // 16-byte aligned
       unsigned *failed = scratch.counter + 8;
       // At most one of these kernels is in flight per process: two of them
       // dispatched at the same time from different streams could each hold
@@ -1349,8 +1388,8 @@ hipError_t launch_dynamic_quantize(hipStream_t s, DqlScratch &scratch,
           if (++scratch.epoch == 0) // 0 is what untouched slots hold
             scratch.epoch = 1;
           hipLaunchKernelGGL(fn_launch, dim3((unsigned)blocks),
-              dim3(kGridThreads), 0, s, x, n, y, scale, zp, flip, slot_lo,
-              slot_hi, scratch.epoch, failed, spin_limit);
+              dim3(kGridThreads), 0, s, x, n, y, scale, zp, flip, slots,
+              scratch.epoch, failed, spin_limit);
           hipError_t e = hipGetLastError();
           if (e != hipSuccess)
             return e;
@@ -1394,13 +1433,13 @@ hipError_t launch_fill_u32(hipStream_t s, uint32_t *p, int64_t n, uint32_t v) {
 
 int dql_grid_blocks() {
   // Blocks of k_dql_grid that are resident at once: one per CU if the
-  // occupancy calculator agrees that one fits (16 float4 per thread).
+  // occupancy calculator agrees that one fits (32 float4 per thread).
   int dev = 0, cus = 0, per = 0;
   if (hipGetDevice(&dev) != hipSuccess ||
       hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) !=
           hipSuccess ||
       hipOccupancyMaxActiveBlocksPerMultiprocessor(
-          &per, k_dql_grid<16>, kGridThreads, 0) != hipSuccess)
+          &per, k_dql_grid<kGridMaxPerThread>, kGridThreads, 0) != hipSuccess)
     return 0;
   if (per < 1 || cus < 1)
     return 0;
