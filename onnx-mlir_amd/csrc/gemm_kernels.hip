@@ -1160,14 +1160,28 @@ __global__ __launch_bounds__(256, MINB) void k_gemm_i8_bs(
 // 4096 x 11008 weights, this kernel against DynamicQuantizeLinear (5.4 us by
 // itself at these sizes) in front of it: 1 row 8.9 / 10.6 us, 4 rows 10.7 /
 // 12.9, 5 rows 11.7 / 13.5, 6 rows 12.9 / 13.6, 8 rows 15.2 / 13.9: the cost
-// grows with every row that every block reads, so the limit is six rows of
-// 4096.  Requesting the first Bp operands before the rows are quantized did
+// grows with every row that every block reads.  With the four-instruction
+// quotient the same comparison reads 4 rows 9.7 / 12.4, 6 rows 10.4 / 12.5,
+// 8 rows 11.2 / 12.6, 16 rows 14 / 13.2: the limit is eight rows of 4096.
+// Requesting the first Bp operands before the rows are quantized did
 // not shorten it, and neither did rows K + 16 bytes apart in LDS (no two
 // lanes' 16-byte reads in the same banks): 4 rows 10.7 -> 11.7 us, 8 rows
 // 15.2 -> 17.1 us with the index arithmetic that takes.
-constexpr int kSkinnyDqBytes = 24576;
+//
+// Tried and dropped: one launch in which the first blocks of the grid quantize
+// X between them (8192 elements each), publish the result through global
+// memory, and every block waits for it with all its weights already
+// requested.  While the 45 MB weight stream saturates HBM every dependent
+// memory step of that chain -- the load of X, the exchange of minima and
+// maxima, the acknowledgement of the quantized rows, the "done" exchange, the
+// copy of the rows into LDS, the polling wave's own weights -- takes 1.2 to
+// 2 us: 16 rows 15.0 us (rows seen at 8.0 us, K loop over at 11.4 us), 4 rows
+// 12.5 us, 1 row 11.8 us, all slower than what they would replace.
+constexpr int kSkinnyDqBytes = 32768;
 
-template <int A_MODE, int EPI, bool DQ, int TR, bool STG>
+// DQ: 0, or the float4 of X a thread takes when the block quantizes X itself
+// (4, 8 or 16: up to 8192, 16384 or kSkinnyDqBytes elements).
+template <int A_MODE, int EPI, int DQ, int TR, bool STG>
 __global__ __launch_bounds__(512) void k_gemm_i8_skinny_bp(
     const uint8_t *__restrict__ A, const float *__restrict__ X,
     const int8_t *__restrict__ Bp, int M, int N, int K, int Kpad,
@@ -1224,7 +1238,8 @@ __global__ __launch_bounds__(512) void k_gemm_i8_skinny_bp(
   int32_t dq_zp = 0;
   if (DQ) {
     typedef float f4 __attribute__((ext_vector_type(4)));
-    constexpr int NV = kSkinnyDqBytes / 4 / (WAVES * 64); // float4 per thread
+    constexpr int NV = DQ > 0 ? DQ : 1; // float4 per thread
+    static_assert(DQ * 4 * WAVES * 64 <= kSkinnyDqBytes, "quantized rows fit");
     const int nvec = (M * K) >> 2; // K % 16 == 0, M * K <= kSkinnyDqBytes
     const f4 *__restrict__ x4 = (const f4 *)X;
     f4 v[NV];
@@ -1585,9 +1600,17 @@ hipError_t gemm_launch_cfg(
       return hipErrorInvalidValue;
     if constexpr (A_MODE == 2) {
       t_last_kernel = "k_gemm_i8_skinny_bp (rows quantized in the kernel)";
-      k_gemm_i8_skinny_bp<2, EPI, true, 1, false>
-          <<<dim3((unsigned)((g.N + 31) / 32)), 512, 0, st>>>(
-              nullptr, g.X, g.Bp, M, N, K, Kpad, ep);
+      const dim3 grid((unsigned)((g.N + 31) / 32));
+      const int64_t elements = g.M * g.K;
+      if (elements <= 4 * 4 * 512)
+        k_gemm_i8_skinny_bp<2, EPI, 4, 1, false>
+            <<<grid, 512, 0, st>>>(nullptr, g.X, g.Bp, M, N, K, Kpad, ep);
+      else if (elements <= 8 * 4 * 512)
+        k_gemm_i8_skinny_bp<2, EPI, 8, 1, false>
+            <<<grid, 512, 0, st>>>(nullptr, g.X, g.Bp, M, N, K, Kpad, ep);
+      else
+        k_gemm_i8_skinny_bp<2, EPI, 16, 1, false>
+            <<<grid, 512, 0, st>>>(nullptr, g.X, g.Bp, M, N, K, Kpad, ep);
     }
     return hipGetLastError();
   }
@@ -1600,13 +1623,13 @@ hipError_t gemm_launch_cfg(
     const dim3 grid((unsigned)((g.N + 31) / 32));
     t_last_kernel = "k_gemm_i8_skinny_bp";
     if (g.M <= 4)
-      k_gemm_i8_skinny_bp<A_MODE, EPI, false, 1, false>
+      k_gemm_i8_skinny_bp<A_MODE, EPI, 0, 1, false>
           <<<grid, 512, 0, st>>>(A, nullptr, g.Bp, M, N, K, Kpad, ep);
     else if (g.M <= 32)
-      k_gemm_i8_skinny_bp<A_MODE, EPI, false, 1, true>
+      k_gemm_i8_skinny_bp<A_MODE, EPI, 0, 1, true>
           <<<grid, 512, 0, st>>>(A, nullptr, g.Bp, M, N, K, Kpad, ep);
     else
-      k_gemm_i8_skinny_bp<A_MODE, EPI, false, 2, true>
+      k_gemm_i8_skinny_bp<A_MODE, EPI, 0, 2, true>
           <<<grid, 512, 0, st>>>(A, nullptr, g.Bp, M, N, K, Kpad, ep);
     return hipGetLastError();
   }

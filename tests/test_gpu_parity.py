@@ -554,6 +554,59 @@ def test_matmulinteger_shapes(rt, oracle, M, K, N):
     assert np.array_equal(rt.MatMulInteger(A, B, azr, bzc), want)
 
 
+def test_few_rows_above_the_in_kernel_limit(rt, oracle):
+    """Up to 32 rows on both sides of the number of elements that the blocks of
+    the weight-streaming GEMM quantize for themselves (above it,
+    DynamicQuantizeLinear runs as a kernel of its own in front).  Same bits as
+    DynamicQuantizeLinear -> MatMulInteger -> Cast -> Mul (-> Add -> Relu) over:
+    rows on both sides of the staging limit of four, K a multiple of 16 only,
+    grids of two to 344 blocks, weight zero points, NaN and infinities in the
+    activation, device-resident operands, and many calls in a row on the same
+    buffers without waiting in between."""
+    rng = np.random.default_rng(78)
+    shapes = [(16, 4096, 11008), (7, 4096, 352), (8, 4096, 64), (32, 4096, 512), (32, 1024, 96), (3, 8208, 96),
+              (4, 6160, 130), (25, 1008, 1000), (32, 784, 70), (9, 2736, 33), (31, 4096 + 16, 480), (2, 16384, 64)]
+    for i, (M, K, N) in enumerate(shapes):
+        x = rng.normal(0, 1 + i, (M, K)).astype(np.float32)
+        if i == 2:
+            x[1, 7] = np.nan
+            x[5, 4000] = np.float32(-3e38)
+        if i == 3:
+            x = np.abs(x)                               # all positive: zero point 0
+        bdt = np.uint8 if i % 2 else np.int8
+        B = _rand_q(rng, bdt, (K, N))
+        bz = _rand_q(rng, bdt, (N,)) if i % 3 == 0 else None
+        bs = rng.uniform(1e-3, 1e-2, N if i % 4 else 1).astype(np.float32)
+        bias = rng.normal(0, 3, N).astype(np.float32) if i % 2 == 0 else None
+        xq, xs, xz = oracle.dynamic_quantize_linear(x)
+        want = oracle.dequant_epilogue(oracle.matmul_integer(xq, B, xz, bz), xs, bs)
+        if bias is not None:
+            want = want + bias
+        got = rt.DynQuantMatMulDequant(x, B, bz, bs, bias)
+        assert same_f32(got, want), (M, K, N)
+        if i in (0, 5):
+            got = rt.DynQuantMatMulDequant(x, B, bz, bs, bias, activation=rt.ACTIVATION_RELU)
+            assert same_f32(got, oracle.relu(want)), (M, K, N)
+    # GPU-resident operands, constant weights, calls in a row without waiting in between
+    M, K, N = 16, 4096, 2048
+    W = _rand_q(rng, np.int8, (K, N))
+    ws = rng.uniform(1e-3, 5e-3, N).astype(np.float32)
+    dW, dS = rt.DeviceArray.from_numpy(W), rt.DeviceArray.from_numpy(ws)
+    rt.mark_constant(dW)
+    try:
+        xs_ = [rng.normal(0, 1 + j, (M, K)).astype(np.float32) for j in range(6)]
+        dxs = [rt.DeviceArray.from_numpy(x) for x in xs_]
+        outs = [rt.DynQuantMatMulDequant(dx, dW, None, dS) for dx in dxs for _ in range(3)]
+        rt.synchronize()
+        for j, x in enumerate(xs_):
+            xq, xs1, xz = oracle.dynamic_quantize_linear(x)
+            want = oracle.dequant_epilogue(oracle.matmul_integer(xq, W, xz, None), xs1, ws)
+            for r in range(3):
+                assert same_f32(outs[3 * j + r].numpy(), want), (j, r)
+    finally:
+        rt.unmark_constant(dW)
+
+
 @pytest.mark.parametrize("adt", [np.int8, np.uint8])
 def test_few_rows_through_lds_all_epilogues(rt, oracle, adt):
     """5 to 64 rows with K a multiple of 16: the weight-streaming kernel stages
