@@ -7,9 +7,9 @@
  * so that no operation is fused, re-associated or replaced by a reciprocal.
  *
  * What pins each function (beyond following the cited lowering op for op):
- *  - om_oracle_rne: swept against nearbyintf over a dense set of binary32
- *    values (all exponents, tie cases); equal except the sign of zero on
- *    (-0.5, 0), which no caller can observe.
+ *  - om_oracle_rne: compared with rintf on all 2^32 binary32 bit patterns
+ *    (om_oracle_rne_sweep); equal except the sign of zero on (-0.5, 0),
+ *    which no caller can observe.
  *  - quantize / dequantize per-tensor, dynamic quantize, matmul integer,
  *    qlinear matmul: the ONNX node-test vectors the reference enables in
  *    test/backend/inference_backend.py (test_quantizelinear_cpu :2531,
@@ -51,6 +51,25 @@ float om_oracle_rne(float x) {
   float rr = y - h * 2.0f;
   float y2 = (rr == 1.0f) ? (y + 1.0f) : y;
   return (r == 0.5f) ? y2 : y1;
+}
+
+/* Checker for the function above: how many of the `count` binary32 values
+ * whose bit patterns start at `first_bits` it rounds to a different value
+ * than the C library's rintf in the default rounding mode (ties to even).
+ * Zeros compare equal whatever their sign; a NaN must give a NaN.  The test
+ * suite runs it over all 2^32 patterns. */
+int64_t om_oracle_rne_sweep(uint32_t first_bits, int64_t count) {
+  int64_t bad = 0;
+#pragma omp parallel for reduction(+ : bad) schedule(static)
+  for (int64_t i = 0; i < count; ++i) {
+    uint32_t u = first_bits + (uint32_t)i;
+    float x;
+    memcpy(&x, &u, 4);
+    float a = om_oracle_rne(x), b = rintf(x);
+    if (!(a == b || (a != a && b != b)))
+      ++bad;
+  }
+  return bad;
 }
 
 /* MathBuilder::clip = max then min, both the NaN-ignoring "num" flavours,

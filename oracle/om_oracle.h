@@ -38,6 +38,9 @@ enum { OM_ORACLE_U8 = 0, OM_ORACLE_I8 = 1, OM_ORACLE_I32 = 2 };
 enum { OM_ORACLE_WRAP = 0, OM_ORACLE_SATURATE = 1 };
 
 float om_oracle_rne(float x);
+/* Values among the `count` bit patterns from `first_bits` on that
+ * om_oracle_rne and rintf round differently (0 expected). */
+int64_t om_oracle_rne_sweep(uint32_t first_bits, int64_t count);
 
 /* y = cast(clip(rne(x / scale) + zp)).  The tensor is viewed as
  * [outer, channels, inner]; scale/zp have `channels` entries (channels == 1

@@ -32,6 +32,8 @@ class Oracle:
         P, I64, F, I = ctypes.c_void_p, ctypes.c_int64, ctypes.c_float, ctypes.c_int
         lib.om_oracle_rne.restype = F
         lib.om_oracle_rne.argtypes = [F]
+        lib.om_oracle_rne_sweep.restype = I64
+        lib.om_oracle_rne_sweep.argtypes = [ctypes.c_uint32, I64]
         for name in ("om_oracle_quantize_linear", "om_oracle_quantize_linear_omp"):
             getattr(lib, name).restype = None
             getattr(lib, name).argtypes = [P, I64, I64, I64, P, P, I, P]
@@ -68,6 +70,9 @@ class Oracle:
         inner = int(np.prod(shape[axis + 1:], dtype=np.int64))
         assert shape[axis] == scale.size
         return outer, scale.size, inner
+
+    def rne_sweep(self, first_bits: int, count: int) -> int:
+        return int(self.lib.om_oracle_rne_sweep(first_bits, count))
 
     def rne(self, x: float) -> float:
         return float(self.lib.om_oracle_rne(ctypes.c_float(x)))

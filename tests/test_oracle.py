@@ -41,6 +41,13 @@ def test_rne_matches_ieee_round_half_even(oracle):
     assert math.isnan(oracle.rne(float("nan")))
 
 
+def test_rne_equals_rintf_for_every_binary32_value(oracle):
+    """The floor-based round-half-even of the reference
+    (src/Dialect/Mlir/DialectBuilder.cpp:291-332) against the C library's rintf
+    on all 2^32 bit patterns (in C, all host threads; a few seconds)."""
+    assert oracle.rne_sweep(0, 1 << 32) == 0
+
+
 # ------------------------------------------------------------ golden: Q/DQ --
 def test_quantizelinear_node_vector(oracle):
     g = GOLD["quantizelinear"]
