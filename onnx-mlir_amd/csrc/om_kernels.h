@@ -115,6 +115,13 @@ const char *last_gemm_kernel();
 
 // Whether launch_gemm can take an f32 activation of this shape in GemmArgs::X.
 bool gemm_quantizes_rows(int64_t M, int64_t K, const void *x);
+// Whether the caller should hand `a` over as rows of round_up(K, 16) bytes
+// made by launch_pad_rows (few rows, K % 16 != 0 or a misaligned start), and
+// pass that length as K.  a_zp: the rows' zero point(s) on the GPU (null: 0),
+// one or one per row; stored_minus_128: rows hold (u8 - 128).
+bool gemm_pads_rows(int64_t M, int64_t K, const void *a);
+hipError_t launch_pad_rows(hipStream_t s, const void *a, int64_t M, int64_t K,
+    const void *a_zp, int64_t a_zp_len, bool stored_minus_128, void *out);
 
 // Fill n 32-bit words with v.
 hipError_t launch_fill_u32(hipStream_t s, uint32_t *p, int64_t n, uint32_t v);

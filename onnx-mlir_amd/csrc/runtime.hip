@@ -1375,6 +1375,17 @@ void run_matmul(const MatmulSpec &sp) {
   }
   g.out = call.out(y);
   if (b.rank <= 2) {
+    if (call.ok && gemm_pads_rows(M, K, g.A)) {
+      // few rows of an awkward length or alignment: aligned copies whose tail
+      // holds the zero point, multiplied over the padded length
+      void *padded = call.temp((size_t)M * round_up(K, 16));
+      if (call.ok)
+        call.check(launch_pad_rows(call.c.stream, g.A, M, K, d_azp, azl,
+                       /*stored_minus_128=*/false, padded),
+            "pad rows");
+      g.A = padded;
+      g.K = round_up(K, 16);
+    }
     if (call.ok)
       call.check(launch_gemm(call.c.stream, g), sp.op);
     call.finish();
@@ -1720,6 +1731,7 @@ void om_mi355x_DynQuantMatMulDequant(OMTensor *y_t, const OMTensor *x_t,
   if (!call.ok)
     return;
   const float *dx = (const float *)call.in(x);
+  int64_t padded_k = 0;
   GemmArgs g = {};
   g.out = call.out(y); // before the quantization: it decides whether to wait
   if (call.ok && gemm_quantizes_rows(M, K, dx)) {
@@ -1732,12 +1744,22 @@ void om_mi355x_DynQuantMatMulDequant(OMTensor *y_t, const OMTensor *x_t,
     if (call.ok)
       run_dql(call, dx, M * K, aq, call.c.dql_scale, call.c.dql_zp, true);
     g.A = aq;
+    if (call.ok && gemm_pads_rows(M, K, aq)) {
+      // (see run_matmul) the quantized rows are stored minus 128
+      void *padded = call.temp((size_t)M * round_up(K, 16));
+      if (call.ok)
+        call.check(launch_pad_rows(call.c.stream, aq, M, K, call.c.dql_zp, 1,
+                       /*stored_minus_128=*/true, padded),
+            "pad rows");
+      g.A = padded;
+      padded_k = round_up(K, 16);
+    }
   }
   g.a_unsigned = true;
   g.a_preshifted = true;
   g.b_unsigned = b.dtype == OM_MI355X_TYPE_UINT8;
   g.M = M;
-  g.K = K;
+  g.K = padded_k ? padded_k : K;
   g.N = N;
   const int32_t *colsum = nullptr;
   if (!call.ok || !packed_b(call, b, K, N, g.Bp, colsum)) {

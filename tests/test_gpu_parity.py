@@ -554,6 +554,52 @@ def test_matmulinteger_shapes(rt, oracle, M, K, N):
     assert np.array_equal(rt.MatMulInteger(A, B, azr, bzc), want)
 
 
+def test_few_rows_of_awkward_length_or_alignment(rt, oracle):
+    """Up to 64 rows whose length is no multiple of 16, or that start at an odd
+    address: the runtime copies them to aligned rows padded with their zero
+    point and uses the weight-streaming kernel over the padded length.  The
+    padding stands for real zeros, so every epilogue must give the bits of the
+    unpadded product: scalar, per-row and absent zero points, both operand
+    types, weight zero points (row sums of A over the padding), the fused
+    layer, a GPU view that starts one byte into its allocation."""
+    rng = np.random.default_rng(79)
+    for M, K, N in ((16, 4100, 11008), (1, 17, 40), (4, 5, 33), (33, 1001, 130), (64, 4099, 96), (7, 15, 64)):
+        for adt, bdt in ((np.uint8, np.int8), (np.int8, np.uint8)):
+            A, B = _rand_q(rng, adt, (M, K)), _rand_q(rng, bdt, (K, N))
+            bz = _rand_q(rng, bdt, (N,))
+            for az in (_rand_q(rng, adt, ()), _rand_q(rng, adt, (M,)), None):
+                want = oracle.matmul_integer(A, B, az, bz)
+                assert np.array_equal(rt.MatMulInteger(A, B, az, bz), want), (M, K, N, adt)
+                assert "skinny" in rt.last_gemm_kernel(), rt.last_gemm_kernel()
+            az = _rand_q(rng, adt, ())
+            a_s, bs = np.float32(0.02), rng.uniform(1e-3, 1e-2, N).astype(np.float32)
+            bias = rng.normal(0, 2, N).astype(np.float32)
+            want = oracle.dequant_epilogue(oracle.matmul_integer(A, B, az, None), a_s, bs) + bias
+            assert same_f32(rt.MatMulIntegerDequant(A, B, az, None, a_s, bs, bias), want), (M, K, N)
+            bzq, yz = _rand_q(rng, bdt, ()), _rand_q(rng, adt, ())
+            for mode in (rt.WRAP, rt.SATURATE):
+                wq = oracle.qlinear_matmul(A, np.float32(0.02), az, B, np.float32(0.01), bzq, np.float32(9.0), yz, mode)
+                gq = rt.QLinearMatMul(A, np.float32(0.02), az, B, np.float32(0.01), bzq, np.float32(9.0), yz, mode)
+                assert np.array_equal(gq, wq), (M, K, N, mode)
+        x = rng.normal(0, 1.5, (M, K)).astype(np.float32)
+        W, ws = _rand_q(rng, np.int8, (K, N)), rng.uniform(1e-3, 1e-2, N).astype(np.float32)
+        wz = _rand_q(rng, np.int8, (N,))
+        xq, xs, xz = oracle.dynamic_quantize_linear(x)
+        want = oracle.dequant_epilogue(oracle.matmul_integer(xq, W, xz, wz), xs, ws)
+        assert same_f32(rt.DynQuantMatMulDequant(x, W, wz, ws), want), (M, K, N)
+        assert "skinny" in rt.last_gemm_kernel(), rt.last_gemm_kernel()
+    # rows of a good length that start one byte into a GPU allocation
+    M, K, N = 8, 4096, 256
+    flat = _rand_q(rng, np.uint8, (M * K + 1,))
+    B = _rand_q(rng, np.int8, (K, N))
+    dflat = rt.DeviceArray.from_numpy(flat)
+    Av = rt.DeviceArray.view_of(dflat, 1, (M, K))
+    az = _rand_q(rng, np.uint8, ())
+    got = rt.MatMulInteger(Av, rt.DeviceArray.from_numpy(B), rt.DeviceArray.from_numpy(az), None)
+    assert np.array_equal(got.numpy(), oracle.matmul_integer(flat[1:].reshape(M, K), B, az, None))
+    assert "skinny" in rt.last_gemm_kernel()
+
+
 def test_few_rows_above_the_in_kernel_limit(rt, oracle):
     """Up to 32 rows on both sides of the number of elements that the blocks of
     the weight-streaming GEMM quantize for themselves (above it,
