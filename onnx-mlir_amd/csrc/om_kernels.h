@@ -147,9 +147,10 @@ hipError_t launch_fill_u32(hipStream_t s, uint32_t *p, int64_t n, uint32_t v);
 // an infinite x, for which e would be a NaN) stays beyond +-1023, where the
 // 8-bit result saturates whatever the zero point; a NaN x stays a NaN.
 // quotient<true> therefore gives the same 8-bit result as x / s for every x,
-// in four instructions.  Checked against the divide on the CPU for 2.4e9 random
-// pairs and 2.7e10 pairs next to a rounding boundary (no difference), and on
-// the GPU by the boundary test of the parity suite.  Any other scale (zero,
+// in four instructions.  Checked against the divide on the CPU
+// (tests/quotient_check.c: random pairs and every neighbour of a rounding
+// boundary, no difference in 2.9e10 pairs) and on the GPU by the boundary test
+// of the parity suite.  Any other scale (zero,
 // negative, denormal, huge, infinite, NaN) takes quotient<false>, the divide.
 __device__ __forceinline__ bool scale_is_tame(float s) {
   return s >= 0x1p-96f && s <= 0x1p96f;

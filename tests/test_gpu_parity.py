@@ -264,8 +264,8 @@ def test_misaligned_device_views_are_handled(rt, oracle):
 # --------------------------------------------------------------------------
 # DynamicQuantizeLinear
 # --------------------------------------------------------------------------
-# (4096, 768) and (2051, 1031) take the one-launch kernel with 4 float4 per thread,
-# (4096, 3072) and (3001, 4099) the one with 16; the last three have 1-3 tail elements.
+# (4096, 768) and (2051, 1031) take the one-launch kernel with 8 float4 per thread,
+# (4096, 3072) and (3001, 4099) the one with 32; the last three have 1-3 tail elements.
 # (16, 4096), (5, 4100), (16388,), (16385,) and (65540,) lie just above the one-block
 # kernel's 16 Ki elements and take the two-launch path.
 @pytest.mark.parametrize("shape", [(1,), (6,), (3, 4), (1023,), (128, 768), (257, 1031), (4096, 768),

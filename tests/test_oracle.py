@@ -365,3 +365,22 @@ def test_relu_equals_numpy_fmax(oracle):
     assert np.array_equal(got, np.fmax(x, np.float32(0)))
     assert got[0] == 0 and got[1] == 0 and got[2] == np.inf and got[3] == 0
     assert not np.signbit(got[5]) and got[6] == np.float32(1e-45)
+
+
+def test_four_instruction_quotient_equals_the_divide(tmp_path):
+    """The quantize kernels divide by a scale of ordinary magnitude with a
+    reciprocal multiply and one exact correction step.  tests/quotient_check.c
+    restates that sequence on the CPU (fmaf is the GPU's v_fma_f32) and compares
+    it with the IEEE divide: bit for bit where the quotient matters (random pairs,
+    and every neighbour of a half-integer or integer quotient for thousands of
+    scales), and through the 8-bit result for arbitrary x (tiny, huge, infinite,
+    NaN).  Half a billion pairs, a few seconds on all host threads."""
+    import shutil, subprocess
+    if shutil.which("gcc") is None:
+        pytest.skip("no gcc")
+    exe = str(tmp_path / "quotient_check")
+    src = os.path.join(os.path.dirname(os.path.abspath(__file__)), "quotient_check.c")
+    subprocess.check_call(["gcc", "-O2", "-march=x86-64-v3", "-fopenmp", "-ffp-contract=off", "-o", exe, src, "-lm"])
+    out = subprocess.run([exe, "20000000", "20000"], capture_output=True, text=True, timeout=600)
+    assert out.returncode == 0, out.stdout + out.stderr
+    assert "0 quotients differ, 0 8-bit results differ" in out.stdout
