@@ -445,7 +445,7 @@ def test_fused_epilogue_with_bias(rt, oracle, M, K, N):
 
 
 def test_few_rows_quantized_inside_the_gemm(rt, oracle):
-    """With at most 32 rows and 24 Ki elements (a decode step) the fused layer
+    """With at most 32 rows and 32 Ki elements (a decode step) the fused layer
     is one launch: the weight-streaming GEMM quantizes the activation rows
     itself.  Same bits as DynamicQuantizeLinear -> MatMulInteger -> Cast -> Mul
     (-> Add): scale and zero point over the whole activation, signed and
