@@ -178,7 +178,11 @@ __global__ __launch_bounds__(kThreads) void k_quant_tiled(
 // zero point in registers and walks down `rows_per_block` rows.  Row starts
 // need not be 16-byte aligned (C % 4 != 0): loads are dword-aligned float4,
 // the 4-byte store may sit at any byte address.
-template <bool SIGNED, bool HAS_ZP>
+// VEC: every thread's four columns lie inside the tensor (C % 4 == 0), `scale`
+// is 16-byte and `zp` 4-byte aligned: scale and zero point then come as one
+// load each.  Reciprocals and the conversion of the zero points wait until the
+// first rows have been requested.
+template <bool SIGNED, bool HAS_ZP, bool VEC>
 __global__ __launch_bounds__(kThreads) void k_quant_lastaxis(
     const float *__restrict__ x, uint8_t *__restrict__ y, int64_t rows,
     int64_t C, const float *__restrict__ scale, const void *__restrict__ zp,
@@ -186,46 +190,90 @@ __global__ __launch_bounds__(kThreads) void k_quant_lastaxis(
   const int64_t c0 = ((int64_t)blockIdx.x * kThreads + threadIdx.x) * 4;
   if (c0 >= C)
     return;
-  const int ncol = (C - c0 >= 4) ? 4 : (int)(C - c0);
+  const int ncol = VEC ? 4 : ((C - c0 >= 4) ? 4 : (int)(C - c0));
   float s[4], z[4], rc[4];
-  bool tame = true;
+  uint32_t zraw[4] = {0, 0, 0, 0};
+  if (VEC) {
+    const f4a sv = *(const f4a *)(scale + c0);
+    s[0] = sv.x;
+    s[1] = sv.y;
+    s[2] = sv.z;
+    s[3] = sv.w;
+    if (HAS_ZP) {
+      const uint32_t w = *(const uint32_t *)((const uint8_t *)zp + c0);
+      zraw[0] = w & 0xFFu;
+      zraw[1] = (w >> 8) & 0xFFu;
+      zraw[2] = (w >> 16) & 0xFFu;
+      zraw[3] = w >> 24;
+    }
+  } else {
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int64_t c = c0 + (j < ncol ? j : 0);
-    s[j] = scale[c];
-    rc[j] = 1.0f / s[j];
-    tame = tame && scale_is_tame(s[j]);
-    z[j] = HAS_ZP ? load_zp_f32<SIGNED>(zp, c) : 0.0f;
+    for (int j = 0; j < 4; ++j) {
+      const int64_t c = c0 + (j < ncol ? j : 0);
+      s[j] = scale[c];
+      zraw[j] = HAS_ZP ? (uint32_t)((const uint8_t *)zp)[c] : 0u;
+    }
   }
+  auto derive = [&]() { // what follows from scale and zero point
+    bool tame = true;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      rc[j] = 1.0f / s[j];
+      tame = tame && scale_is_tame(s[j]);
+      z[j] = HAS_ZP ? (SIGNED ? (float)(int32_t)(int8_t)zraw[j]
+                              : (float)zraw[j])
+                    : 0.0f;
+    }
+    return wave_all(tame);
+  };
   const int64_t r_begin = (int64_t)blockIdx.y * rows_per_block;
   const int64_t r_end =
       (r_begin + rows_per_block < rows) ? r_begin + rows_per_block : rows;
   if (ncol == 4) {
-    auto walk = [&](auto fast_c) {
+    int64_t r = r_begin;
+    f4u v[kRowUnroll];
+    auto request = [&](int64_t r0) {
+#pragma unroll
+      for (int j = 0; j < kRowUnroll; ++j)
+        v[j] = __builtin_nontemporal_load((const f4u *)(x + (r0 + j) * C + c0));
+    };
+    auto finish = [&](int64_t r0, auto fast_c) {
       constexpr bool FAST = decltype(fast_c)::value;
-      int64_t r = r_begin;
+#pragma unroll
+      for (int j = 0; j < kRowUnroll; ++j)
+        *(u32_a1 *)(y + (r0 + j) * C + c0) =
+            quant_cols<SIGNED, HAS_ZP, FAST>(v[j], s, rc, z);
+    };
+    auto rest = [&](auto fast_c) {
+      constexpr bool FAST = decltype(fast_c)::value;
       for (; r + kRowUnroll <= r_end; r += kRowUnroll) {
-        f4u v[kRowUnroll];
-#pragma unroll
-        for (int j = 0; j < kRowUnroll; ++j)
-          v[j] =
-              __builtin_nontemporal_load((const f4u *)(x + (r + j) * C + c0));
-#pragma unroll
-        for (int j = 0; j < kRowUnroll; ++j)
-          *(u32_a1 *)(y + (r + j) * C + c0) =
-              quant_cols<SIGNED, HAS_ZP, FAST>(v[j], s, rc, z);
+        request(r);
+        finish(r, fast_c);
       }
       for (; r < r_end; ++r) {
-        f4u v = *(const f4u *)(x + r * C + c0);
+        f4u v1 = *(const f4u *)(x + r * C + c0);
         *(u32_a1 *)(y + r * C + c0) =
-            quant_cols<SIGNED, HAS_ZP, FAST>(v, s, rc, z);
+            quant_cols<SIGNED, HAS_ZP, FAST>(v1, s, rc, z);
       }
     };
-    if (wave_all(tame))
-      walk(std::true_type{});
-    else
-      walk(std::false_type{});
+    const bool first = r + kRowUnroll <= r_end;
+    if (first)
+      request(r);
+    if (derive()) {
+      if (first) {
+        finish(r, std::true_type{});
+        r += kRowUnroll;
+      }
+      rest(std::true_type{});
+    } else {
+      if (first) {
+        finish(r, std::false_type{});
+        r += kRowUnroll;
+      }
+      rest(std::false_type{});
+    }
   } else {
+    derive();
     for (int64_t r = r_begin; r < r_end; ++r)
       for (int j = 0; j < ncol; ++j)
         y[r * C + c0 + j] =
@@ -243,13 +291,125 @@ __global__ __launch_bounds__(kThreads) void k_quant_lastaxis(
 // period, v + 2 period, ... meets the same four columns each time: it loads
 // their scales and zero points once, like the row-walking kernel, and every
 // data access is aligned and coalesced.
-template <bool SIGNED, bool HAS_ZP>
+// Scale and raw zero point of the four columns c, c+1, c+2, c+3 (mod C) that
+// a thread of the periodic kernels keeps to.  Unless they wrap around the end
+// of a row (one thread in C / 4 does) they are adjacent: one 16-byte load at a
+// 4-byte aligned address and one 4-byte load at any address, issued before
+// anything waits; the wrapping lanes redo theirs element by element in
+// periodic_params_fix, which the kernels call after their first vectors have
+// been requested.  Needs C >= 4 (VEC); otherwise element by element at once.
+template <bool HAS_ZP, bool VEC>
+__device__ __forceinline__ void periodic_params(const float *__restrict__ scale,
+    const void *__restrict__ zp, uint32_t c, uint32_t C, float (&s)[4],
+    uint32_t (&zraw)[4]) {
+  if (VEC) {
+    const uint32_t cb = (c + 4 > C) ? 0u : c;
+    const f4u sv = *(const f4u *)(scale + cb);
+    s[0] = sv.x;
+    s[1] = sv.y;
+    s[2] = sv.z;
+    s[3] = sv.w;
+    const uint32_t w =
+        HAS_ZP ? *(const u32_a1 *)((const uint8_t *)zp + cb) : 0u;
+    zraw[0] = w & 0xFFu;
+    zraw[1] = (w >> 8) & 0xFFu;
+    zraw[2] = (w >> 16) & 0xFFu;
+    zraw[3] = w >> 24;
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      s[e] = scale[c];
+      zraw[e] = HAS_ZP ? (uint32_t)((const uint8_t *)zp)[c] : 0u;
+      c = (c + 1 == C) ? 0 : c + 1;
+    }
+  }
+}
+template <bool HAS_ZP, bool VEC>
+__device__ __forceinline__ void periodic_params_fix(
+    const float *__restrict__ scale, const void *__restrict__ zp, uint32_t c,
+    uint32_t C, float (&s)[4], uint32_t (&zraw)[4]) {
+  if (VEC && c + 4 > C) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      s[e] = scale[c];
+      zraw[e] = HAS_ZP ? (uint32_t)((const uint8_t *)zp)[c] : 0u;
+      c = (c + 1 == C) ? 0 : c + 1;
+    }
+  }
+}
+
+template <bool SIGNED, bool HAS_ZP, bool VEC>
 __global__ __launch_bounds__(kThreads) void k_quant_periodic(
     const float *__restrict__ x, uint8_t *__restrict__ y, int64_t n, uint32_t C,
     int64_t period, const float *__restrict__ scale,
     const void *__restrict__ zp, int periods_per_block) {
   const int64_t v = (int64_t)blockIdx.x * kThreads + threadIdx.x;
   const int64_t nvec = n >> 2;
+  if (v >= period)
+    return;
+  // Scales and zero points as loaded; reciprocals and conversions wait until
+  // the first vectors have been requested.
+  float s[4], z[4], rc[4];
+  uint32_t zraw[4];
+  const uint32_t c_first = (uint32_t)(((uint64_t)v * 4) % C);
+  periodic_params<HAS_ZP, VEC>(scale, zp, c_first, C, s, zraw);
+  auto derive = [&]() {
+    periodic_params_fix<HAS_ZP, VEC>(scale, zp, c_first, C, s, zraw);
+    bool tame = true;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      rc[e] = 1.0f / s[e];
+      tame = tame && scale_is_tame(s[e]);
+      z[e] = HAS_ZP ? (SIGNED ? (float)(int32_t)(int8_t)zraw[e]
+                              : (float)zraw[e])
+                    : 0.0f;
+    }
+    return wave_all(tame);
+  };
+  const f4a *__restrict__ x4 = (const f4a *)x;
+  uint32_t *__restrict__ y4 = (uint32_t *)y;
+  int64_t idx = (int64_t)blockIdx.y * periods_per_block * period + v;
+  const int64_t end = idx + (int64_t)periods_per_block * period;
+  const int64_t stop = end < nvec ? end : nvec;
+  f4a q[kRowUnroll];
+  auto request = [&](int64_t i0) {
+#pragma unroll
+    for (int j = 0; j < kRowUnroll; ++j)
+      q[j] = __builtin_nontemporal_load(&x4[i0 + j * period]);
+  };
+  auto finish = [&](int64_t i0, auto fast_c) {
+    constexpr bool FAST = decltype(fast_c)::value;
+#pragma unroll
+    for (int j = 0; j < kRowUnroll; ++j)
+      y4[i0 + j * period] = quant_cols<SIGNED, HAS_ZP, FAST>(q[j], s, rc, z);
+  };
+  auto rest = [&](auto fast_c) {
+    constexpr bool FAST = decltype(fast_c)::value;
+    for (; idx + (kRowUnroll - 1) * period < stop;
+         idx += kRowUnroll * period) {
+      request(idx);
+      finish(idx, fast_c);
+    }
+    for (; idx < stop; idx += period)
+      y4[idx] = quant_cols<SIGNED, HAS_ZP, FAST>(x4[idx], s, rc, z);
+  };
+  const bool first = idx + (kRowUnroll - 1) * period < stop;
+  if (first)
+    request(idx);
+  if (derive()) {
+    if (first) {
+      finish(idx, std::true_type{});
+      idx += kRowUnroll * period;
+    }
+    rest(std::true_type{});
+  } else {
+    if (first) {
+      finish(idx, std::false_type{});
+      idx += kRowUnroll * period;
+    }
+    rest(std::false_type{});
+  }
+  // the up to three elements after the last whole vector
   if (blockIdx.x == 0 && blockIdx.y == 0) {
     const int64_t e = (nvec << 2) + threadIdx.x;
     if (e < n) {
@@ -258,46 +418,6 @@ __global__ __launch_bounds__(kThreads) void k_quant_periodic(
       y[e] = (uint8_t)quant_one<SIGNED, HAS_ZP>(x[e], scale[ce], zf);
     }
   }
-  if (v >= period)
-    return;
-  float s[4], z[4], rc[4];
-  bool tame = true;
-  {
-    uint32_t c = (uint32_t)(((uint64_t)v * 4) % C);
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      s[e] = scale[c];
-      rc[e] = 1.0f / s[e];
-      tame = tame && scale_is_tame(s[e]);
-      z[e] = HAS_ZP ? load_zp_f32<SIGNED>(zp, c) : 0.0f;
-      c = (c + 1 == C) ? 0 : c + 1;
-    }
-  }
-  const f4a *__restrict__ x4 = (const f4a *)x;
-  uint32_t *__restrict__ y4 = (uint32_t *)y;
-  const int64_t begin = (int64_t)blockIdx.y * periods_per_block * period + v;
-  const int64_t end = begin + (int64_t)periods_per_block * period;
-  const int64_t stop = end < nvec ? end : nvec;
-  auto walk = [&](auto fast_c) {
-    constexpr bool FAST = decltype(fast_c)::value;
-    int64_t idx = begin;
-    for (; idx + (kRowUnroll - 1) * period < stop;
-         idx += kRowUnroll * period) {
-      f4a q[kRowUnroll];
-#pragma unroll
-      for (int j = 0; j < kRowUnroll; ++j)
-        q[j] = __builtin_nontemporal_load(&x4[idx + j * period]);
-#pragma unroll
-      for (int j = 0; j < kRowUnroll; ++j)
-        y4[idx + j * period] = quant_cols<SIGNED, HAS_ZP, FAST>(q[j], s, rc, z);
-    }
-    for (; idx < stop; idx += period)
-      y4[idx] = quant_cols<SIGNED, HAS_ZP, FAST>(x4[idx], s, rc, z);
-  };
-  if (wave_all(tame))
-    walk(std::true_type{});
-  else
-    walk(std::false_type{});
 }
 
 // ---- general [outer, channels, inner] quantize ---------------------------
@@ -490,7 +610,66 @@ __device__ __forceinline__ uint32_t load_one_q(const void *x, int64_t elem) {
   return ((const uint8_t *)x)[elem];
 }
 
+// Scale and zero point of four adjacent columns.  When the four lie inside the
+// tensor and their addresses allow it they come as one 16-byte and one 4-byte
+// load (8-bit zero points), not eight loads: a block of the row-walking
+// kernels lives for eight rows only, and what it loads before its first row
+// is a visible part of its life.  The zero points are returned as loaded;
+// zp_to_f32 converts them, which the kernels do after they have requested
+// their first rows (a conversion before that would make those requests wait
+// for the zero points to arrive).
+template <int KIND>
+struct ColParams {
+  float s[4];
+  uint32_t zraw[4]; // 8-bit kinds: the byte in the low bits; i32: the word
+};
+// VEC: the launcher has checked that every thread's four columns lie inside
+// the tensor (C % 4 == 0) and that `scale` is 16-byte and `zp` 4-byte aligned,
+// so the vector loads need no test here -- a branch around them would make
+// the code after it wait for them.
+template <int KIND, bool HAS_ZP, bool VEC>
+__device__ __forceinline__ void load_col_params(const float *__restrict__ scale,
+    const void *__restrict__ zp, int64_t c0, int ncol, ColParams<KIND> &p) {
+  if (VEC) {
+    const f4a v = *(const f4a *)(scale + c0);
+    p.s[0] = v.x;
+    p.s[1] = v.y;
+    p.s[2] = v.z;
+    p.s[3] = v.w;
+  } else {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      p.s[j] = scale[c0 + (j < ncol ? j : 0)];
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    p.zraw[j] = 0;
+  if (!HAS_ZP)
+    return;
+  if (KIND != kI32 && VEC) {
+    const uint32_t w = *(const uint32_t *)((const uint8_t *)zp + c0);
+    p.zraw[0] = w & 0xFFu;
+    p.zraw[1] = (w >> 8) & 0xFFu;
+    p.zraw[2] = (w >> 16) & 0xFFu;
+    p.zraw[3] = w >> 24;
+  } else {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int64_t c = c0 + (j < ncol ? j : 0);
+      p.zraw[j] = KIND == kI32 ? (uint32_t)((const int32_t *)zp)[c]
+                               : (uint32_t)((const uint8_t *)zp)[c];
+    }
+  }
+}
 template <int KIND, bool HAS_ZP>
+__device__ __forceinline__ void zp_to_f32(
+    const ColParams<KIND> &p, float (&z)[4]) {
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    z[j] = HAS_ZP ? q_to_f32<KIND>(p.zraw[j]) : 0.0f;
+}
+
+template <int KIND, bool HAS_ZP, bool VEC>
 __global__ __launch_bounds__(kThreads) void k_dequant_lastaxis(
     const void *__restrict__ x, float *__restrict__ y, int64_t rows, int64_t C,
     const float *__restrict__ scale, const void *__restrict__ zp,
@@ -498,24 +677,23 @@ __global__ __launch_bounds__(kThreads) void k_dequant_lastaxis(
   const int64_t c0 = ((int64_t)blockIdx.x * kThreads + threadIdx.x) * 4;
   if (c0 >= C)
     return;
-  const int ncol = (C - c0 >= 4) ? 4 : (int)(C - c0);
-  float s[4], z[4];
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int64_t c = c0 + (j < ncol ? j : 0);
-    s[j] = scale[c];
-    z[j] = HAS_ZP ? load_q_zp_f32<KIND>(zp, c) : 0.0f;
-  }
+  const int ncol = VEC ? 4 : ((C - c0 >= 4) ? 4 : (int)(C - c0));
+  ColParams<KIND> cp;
+  load_col_params<KIND, HAS_ZP, VEC>(scale, zp, c0, ncol, cp);
+  const float(&s)[4] = cp.s;
+  float z[4];
   const int64_t r_begin = (int64_t)blockIdx.y * rows_per_block;
   const int64_t r_end =
       (r_begin + rows_per_block < rows) ? r_begin + rows_per_block : rows;
   if (ncol == 4) {
     int64_t r = r_begin;
-    for (; r + kRowUnroll <= r_end; r += kRowUnroll) {
-      uint32_t q[kRowUnroll][4];
+    uint32_t q[kRowUnroll][4];
+    auto request = [&](int64_t r0) {
 #pragma unroll
       for (int j = 0; j < kRowUnroll; ++j)
-        load_four_q<KIND>(x, (r + j) * C + c0, q[j]);
+        load_four_q<KIND>(x, (r0 + j) * C + c0, q[j]);
+    };
+    auto finish = [&](int64_t r0) {
 #pragma unroll
       for (int j = 0; j < kRowUnroll; ++j) {
         f4u o;
@@ -525,20 +703,34 @@ __global__ __launch_bounds__(kThreads) void k_dequant_lastaxis(
         o.w = dq_one<HAS_ZP>(q_to_f32<KIND>(q[j][3]), s[3], z[3]);
         // streaming store: measured 3.5 % faster here (and 14 % slower for
         // the 4-byte stores of the quantize kernel, which keeps plain ones)
-        __builtin_nontemporal_store(o, (f4u *)(y + (r + j) * C + c0));
+        __builtin_nontemporal_store(o, (f4u *)(y + (r0 + j) * C + c0));
       }
+    };
+    // the first rows are requested before the zero points are converted
+    const bool first = r + kRowUnroll <= r_end;
+    if (first)
+      request(r);
+    zp_to_f32<KIND, HAS_ZP>(cp, z);
+    if (first) {
+      finish(r);
+      r += kRowUnroll;
+    }
+    for (; r + kRowUnroll <= r_end; r += kRowUnroll) {
+      request(r);
+      finish(r);
     }
     for (; r < r_end; ++r) {
-      uint32_t q[4];
-      load_four_q<KIND>(x, r * C + c0, q);
+      uint32_t q1[4];
+      load_four_q<KIND>(x, r * C + c0, q1);
       f4u o;
-      o.x = dq_one<HAS_ZP>(q_to_f32<KIND>(q[0]), s[0], z[0]);
-      o.y = dq_one<HAS_ZP>(q_to_f32<KIND>(q[1]), s[1], z[1]);
-      o.z = dq_one<HAS_ZP>(q_to_f32<KIND>(q[2]), s[2], z[2]);
-      o.w = dq_one<HAS_ZP>(q_to_f32<KIND>(q[3]), s[3], z[3]);
+      o.x = dq_one<HAS_ZP>(q_to_f32<KIND>(q1[0]), s[0], z[0]);
+      o.y = dq_one<HAS_ZP>(q_to_f32<KIND>(q1[1]), s[1], z[1]);
+      o.z = dq_one<HAS_ZP>(q_to_f32<KIND>(q1[2]), s[2], z[2]);
+      o.w = dq_one<HAS_ZP>(q_to_f32<KIND>(q1[3]), s[3], z[3]);
       *(f4u *)(y + r * C + c0) = o;
     }
   } else {
+    zp_to_f32<KIND, HAS_ZP>(cp, z);
     for (int64_t r = r_begin; r < r_end; ++r)
       for (int j = 0; j < ncol; ++j)
         y[r * C + c0 + j] = dq_one<HAS_ZP>(
@@ -548,43 +740,34 @@ __global__ __launch_bounds__(kThreads) void k_dequant_lastaxis(
 
 // 8-bit input, innermost axis, C % 4 != 0: aligned vectors of the flat array,
 // each thread on a fixed set of four columns (see k_quant_periodic).
-template <int KIND, bool HAS_ZP>
+template <int KIND, bool HAS_ZP, bool VEC>
 __global__ __launch_bounds__(kThreads) void k_dequant8_periodic(
     const uint8_t *__restrict__ x, float *__restrict__ y, int64_t n, uint32_t C,
     int64_t period, const float *__restrict__ scale,
     const void *__restrict__ zp, int periods_per_block) {
   const int64_t v = (int64_t)blockIdx.x * kThreads + threadIdx.x;
   const int64_t nvec = n >> 2;
-  if (blockIdx.x == 0 && blockIdx.y == 0) {
-    const int64_t e = (nvec << 2) + threadIdx.x;
-    if (e < n) {
-      const uint32_t ce = (uint32_t)(e % C);
-      const float zf = HAS_ZP ? load_q_zp_f32<KIND>(zp, ce) : 0.0f;
-      y[e] = dq_one<HAS_ZP>(q_to_f32<KIND>(x[e]), scale[ce], zf);
-    }
-  }
   if (v >= period)
     return;
+  // Scales and zero points as loaded; the zero points are converted after the
+  // first rows have been requested (a conversion here would make those
+  // requests wait for the zero points to arrive).
   float s[4], z[4];
-  {
-    uint32_t c = (uint32_t)(((uint64_t)v * 4) % C);
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      s[e] = scale[c];
-      z[e] = HAS_ZP ? load_q_zp_f32<KIND>(zp, c) : 0.0f;
-      c = (c + 1 == C) ? 0 : c + 1;
-    }
-  }
+  uint32_t zraw[4];
+  const uint32_t c_first = (uint32_t)(((uint64_t)v * 4) % C);
+  periodic_params<HAS_ZP, VEC>(scale, zp, c_first, C, s, zraw);
   const uint32_t *__restrict__ x4 = (const uint32_t *)x;
   f4a *__restrict__ y4 = (f4a *)y;
   int64_t idx = (int64_t)blockIdx.y * periods_per_block * period + v;
   const int64_t end = idx + (int64_t)periods_per_block * period;
   const int64_t stop = end < nvec ? end : nvec;
-  for (; idx + (kRowUnroll - 1) * period < stop; idx += kRowUnroll * period) {
-    uint32_t w[kRowUnroll];
+  uint32_t w[kRowUnroll];
+  auto request = [&](int64_t i0) {
 #pragma unroll
     for (int j = 0; j < kRowUnroll; ++j)
-      w[j] = __builtin_nontemporal_load(&x4[idx + j * period]);
+      w[j] = __builtin_nontemporal_load(&x4[i0 + j * period]);
+  };
+  auto finish = [&](int64_t i0) {
 #pragma unroll
     for (int j = 0; j < kRowUnroll; ++j) {
       f4a o;
@@ -592,17 +775,41 @@ __global__ __launch_bounds__(kThreads) void k_dequant8_periodic(
       o.y = dq_one<HAS_ZP>(q_to_f32<KIND>(w[j] >> 8), s[1], z[1]);
       o.z = dq_one<HAS_ZP>(q_to_f32<KIND>(w[j] >> 16), s[2], z[2]);
       o.w = dq_one<HAS_ZP>(q_to_f32<KIND>(w[j] >> 24), s[3], z[3]);
-      __builtin_nontemporal_store(o, &y4[idx + j * period]);
+      __builtin_nontemporal_store(o, &y4[i0 + j * period]);
     }
+  };
+  const bool first = idx + (kRowUnroll - 1) * period < stop;
+  if (first)
+    request(idx);
+  periodic_params_fix<HAS_ZP, VEC>(scale, zp, c_first, C, s, zraw);
+#pragma unroll
+  for (int e = 0; e < 4; ++e)
+    z[e] = HAS_ZP ? q_to_f32<KIND>(zraw[e]) : 0.0f;
+  if (first) {
+    finish(idx);
+    idx += kRowUnroll * period;
+  }
+  for (; idx + (kRowUnroll - 1) * period < stop; idx += kRowUnroll * period) {
+    request(idx);
+    finish(idx);
   }
   for (; idx < stop; idx += period) {
-    const uint32_t w = x4[idx];
+    const uint32_t w1 = x4[idx];
     f4a o;
-    o.x = dq_one<HAS_ZP>(q_to_f32<KIND>(w), s[0], z[0]);
-    o.y = dq_one<HAS_ZP>(q_to_f32<KIND>(w >> 8), s[1], z[1]);
-    o.z = dq_one<HAS_ZP>(q_to_f32<KIND>(w >> 16), s[2], z[2]);
-    o.w = dq_one<HAS_ZP>(q_to_f32<KIND>(w >> 24), s[3], z[3]);
+    o.x = dq_one<HAS_ZP>(q_to_f32<KIND>(w1), s[0], z[0]);
+    o.y = dq_one<HAS_ZP>(q_to_f32<KIND>(w1 >> 8), s[1], z[1]);
+    o.z = dq_one<HAS_ZP>(q_to_f32<KIND>(w1 >> 16), s[2], z[2]);
+    o.w = dq_one<HAS_ZP>(q_to_f32<KIND>(w1 >> 24), s[3], z[3]);
     y4[idx] = o;
+  }
+  // the up to three elements after the last whole vector
+  if (blockIdx.x == 0 && blockIdx.y == 0) {
+    const int64_t e = (nvec << 2) + threadIdx.x;
+    if (e < n) {
+      const uint32_t ce = (uint32_t)(e % C);
+      const float zf = HAS_ZP ? load_q_zp_f32<KIND>(zp, ce) : 0.0f;
+      y[e] = dq_one<HAS_ZP>(q_to_f32<KIND>(x[e]), scale[ce], zf);
+    }
   }
 }
 
@@ -1165,11 +1372,18 @@ hipError_t quantize_dispatch(hipStream_t st, const float *x, int64_t outer,
       channels < ((int64_t)1 << 31) && ((((uintptr_t)x) & 15) == 0) &&
       ((((uintptr_t)y) & 3) == 0) && (n >> 2) > 0) {
     const PeriodicGrid pg = periodic_grid(n >> 2, channels, 1);
-    if (has_zp)
-      k_quant_periodic<SIGNED, true><<<pg.grid, kThreads, 0, st>>>(
+    const bool vec = channels >= 4 && ((((uintptr_t)scale) & 3) == 0);
+    if (has_zp && vec)
+      k_quant_periodic<SIGNED, true, true><<<pg.grid, kThreads, 0, st>>>(
+          x, yo, n, (uint32_t)channels, pg.period, scale, zp, pg.per_block);
+    else if (has_zp)
+      k_quant_periodic<SIGNED, true, false><<<pg.grid, kThreads, 0, st>>>(
+          x, yo, n, (uint32_t)channels, pg.period, scale, zp, pg.per_block);
+    else if (vec)
+      k_quant_periodic<SIGNED, false, true><<<pg.grid, kThreads, 0, st>>>(
           x, yo, n, (uint32_t)channels, pg.period, scale, zp, pg.per_block);
     else
-      k_quant_periodic<SIGNED, false><<<pg.grid, kThreads, 0, st>>>(
+      k_quant_periodic<SIGNED, false, false><<<pg.grid, kThreads, 0, st>>>(
           x, yo, n, (uint32_t)channels, pg.period, scale, zp, pg.per_block);
     return hipGetLastError();
   }
@@ -1179,11 +1393,19 @@ hipError_t quantize_dispatch(hipStream_t st, const float *x, int64_t outer,
     int64_t rpb, row_blocks;
     rows_per_block(rows, 1, rpb, row_blocks);
     dim3 grid((unsigned)col_blocks, (unsigned)row_blocks);
-    if (has_zp)
-      k_quant_lastaxis<SIGNED, true>
+    const bool vec = C % 4 == 0 && ((((uintptr_t)scale) & 15) == 0) &&
+                     (!has_zp || ((((uintptr_t)zp) & 3) == 0));
+    if (has_zp && vec)
+      k_quant_lastaxis<SIGNED, true, true>
+          <<<grid, kThreads, 0, st>>>(x, yo, rows, C, scale, zp, (int)rpb);
+    else if (has_zp)
+      k_quant_lastaxis<SIGNED, true, false>
+          <<<grid, kThreads, 0, st>>>(x, yo, rows, C, scale, zp, (int)rpb);
+    else if (vec)
+      k_quant_lastaxis<SIGNED, false, true>
           <<<grid, kThreads, 0, st>>>(x, yo, rows, C, scale, zp, (int)rpb);
     else
-      k_quant_lastaxis<SIGNED, false>
+      k_quant_lastaxis<SIGNED, false, false>
           <<<grid, kThreads, 0, st>>>(x, yo, rows, C, scale, zp, (int)rpb);
     return hipGetLastError();
   }
@@ -1245,14 +1467,24 @@ hipError_t dequantize_dispatch(hipStream_t st, const void *x, int64_t outer,
       channels < ((int64_t)1 << 31) && ((((uintptr_t)x) & 3) == 0) &&
       ((((uintptr_t)y) & 15) == 0) && (n >> 2) > 0) {
     const PeriodicGrid pg = periodic_grid(n >> 2, channels, 2);
-    if (has_zp)
-      k_dequant8_periodic<(KIND == kI32 ? kU8 : KIND), true>
-          <<<pg.grid, kThreads, 0, st>>>((const uint8_t *)x, y, n,
-              (uint32_t)channels, pg.period, scale, zp, pg.per_block);
+    constexpr int K8 = KIND == kI32 ? kU8 : KIND;
+    const bool vec = channels >= 4 && ((((uintptr_t)scale) & 3) == 0);
+    if (has_zp && vec)
+      k_dequant8_periodic<K8, true, true><<<pg.grid, kThreads, 0, st>>>(
+          (const uint8_t *)x, y, n, (uint32_t)channels, pg.period, scale, zp,
+          pg.per_block);
+    else if (has_zp)
+      k_dequant8_periodic<K8, true, false><<<pg.grid, kThreads, 0, st>>>(
+          (const uint8_t *)x, y, n, (uint32_t)channels, pg.period, scale, zp,
+          pg.per_block);
+    else if (vec)
+      k_dequant8_periodic<K8, false, true><<<pg.grid, kThreads, 0, st>>>(
+          (const uint8_t *)x, y, n, (uint32_t)channels, pg.period, scale, zp,
+          pg.per_block);
     else
-      k_dequant8_periodic<(KIND == kI32 ? kU8 : KIND), false>
-          <<<pg.grid, kThreads, 0, st>>>((const uint8_t *)x, y, n,
-              (uint32_t)channels, pg.period, scale, zp, pg.per_block);
+      k_dequant8_periodic<K8, false, false><<<pg.grid, kThreads, 0, st>>>(
+          (const uint8_t *)x, y, n, (uint32_t)channels, pg.period, scale, zp,
+          pg.per_block);
     return hipGetLastError();
   }
   if (inner == 1 && channels > 1) {
@@ -1261,11 +1493,19 @@ hipError_t dequantize_dispatch(hipStream_t st, const void *x, int64_t outer,
     int64_t rpb, row_blocks;
     rows_per_block(rows, 1, rpb, row_blocks);
     dim3 grid((unsigned)col_blocks, (unsigned)row_blocks);
-    if (has_zp)
-      k_dequant_lastaxis<KIND, true>
+    const bool vec = C % 4 == 0 && ((((uintptr_t)scale) & 15) == 0) &&
+                     (!has_zp || ((((uintptr_t)zp) & 3) == 0));
+    if (has_zp && vec)
+      k_dequant_lastaxis<KIND, true, true>
+          <<<grid, kThreads, 0, st>>>(x, y, rows, C, scale, zp, (int)rpb);
+    else if (has_zp)
+      k_dequant_lastaxis<KIND, true, false>
+          <<<grid, kThreads, 0, st>>>(x, y, rows, C, scale, zp, (int)rpb);
+    else if (vec)
+      k_dequant_lastaxis<KIND, false, true>
           <<<grid, kThreads, 0, st>>>(x, y, rows, C, scale, zp, (int)rpb);
     else
-      k_dequant_lastaxis<KIND, false>
+      k_dequant_lastaxis<KIND, false, false>
           <<<grid, kThreads, 0, st>>>(x, y, rows, C, scale, zp, (int)rpb);
     return hipGetLastError();
   }
