@@ -394,8 +394,12 @@ def only_mode(rt, wl, what, steps, warmup):
         return {"only": what, **r}
     if what.startswith("dynamic_quantize_"):
         return {"only": what, **dql_activation_cases(rt, steps, warmup, only=what)[what]}
-    r = qdq_cases(rt, wl, 8192, 32768, steps, warmup, only=what)
-    return {"only": what, **r[what]}
+    # "<op>" is the aligned config 2 tensor, "<op>_ragged" the [8191, 32767] one
+    ragged = what.endswith("_ragged")
+    op = what[:-len("_ragged")] if ragged else what
+    rows, cols = (8191, 32767) if ragged else (8192, 32768)
+    r = qdq_cases(rt, wl, rows, cols, steps, warmup, only=op)
+    return {"only": what, "shape": [rows, cols], **r[op]}
 
 
 def host_cpu():
@@ -530,6 +534,7 @@ def main():
                              "decode", "decode4", "decode16",
                              "quantize_per_axis", "dequantize_per_axis",
                              "quantize_per_tensor", "dequantize_per_tensor", "dynamic_quantize",
+                             "quantize_per_axis_ragged", "dequantize_per_axis_ragged",
                              "dynamic_quantize_4096x768", "dynamic_quantize_4096x3072"],
                     help="launch just this kernel --steps times (for rocprofv3 counter runs)")
     args = ap.parse_args()

@@ -813,6 +813,214 @@ __global__ __launch_bounds__(kThreads) void k_dequant8_periodic(
   }
 }
 
+// ---- per-axis dequantize, innermost axis, rows off the cache lines ---------
+// (k_dequant8_rowtable: 8-bit input, rows of about 4 Ki elements and more
+// whose float rows do not start on a 128-byte line, C % 32 != 0.)
+// Every access is an aligned 4-element vector of the flat array AND every
+// wave's piece of a row starts on a cache line on both sides, with the rows of
+// a block next to each other in memory.  A wave that writes its 1 KiB starting
+// 16 or 32 bytes into a line costs 12 % of the whole kernel (k_dequant_lastaxis
+// on rows that are only 16-byte aligned: 67 % of HBM peak against 76 %), and
+// so do strides of megabytes between a thread's accesses, which is what
+// keeping a thread's columns fixed takes when rows are not aligned
+// (k_dequant8_periodic).  Row r is taken to start at the next multiple of
+// kRtAlign elements at or after r * C (the elements before that go with row
+// r - 1, whose columns wrap around); block (bx, by) takes elements
+// [bx * kRtCols, + kRtCols) after that start in each of its kRowUnroll rows.
+// Which columns a thread meets therefore moves from row to row, by less than
+// kRtAlign: scale and zero point of the block's kRtCols + kRtAlign columns sit
+// in LDS and are read from there for every vector.
+constexpr int kRtCols = kThreads * 4;
+constexpr int kRtAlign = 128;
+constexpr int kRtTable = kRtCols + kRtAlign;
+// Shortest row: a block's columns wrap around at most once, and the table
+// fill per block stays small against the rows it serves.
+constexpr int64_t kRtMinC = 4 * kRtCols - kRtAlign;
+
+// Launch shape.  Blocks are numbered so that the hardware's round-robin of
+// consecutive block ids over the 8 XCDs hands each XCD whole row groups (all
+// column blocks of rows 8 by .. 8 by + 7, then those of row group by + 8, ..),
+// when a row group has at most kRtGroupedMax column blocks; longer rows run
+// column block first.  % of HBM peak, column first / row groups per XCD, on
+// one device: [8191, 32767] 62 / 74 (column first loses 10 points wherever the
+// row pitch is within a few elements of a multiple of 32 Ki, and at some other
+// pitches; DRAM write-credit stalls double there), [16384, 16380] 74 / 74.5,
+// [65528, 4095] 72 / 72, [4096, 65535] 74.5 / 73.5, [2048, 131071] 74 / 67.
+constexpr int kRtGroupedMax = 48;
+struct RtGrid {
+  int gx, gy;   // column blocks of a row group, row groups
+  int grouped;  // 1: row groups dealt to the XCDs
+};
+RtGrid rt_grid(int64_t rows, int64_t C) {
+  RtGrid g;
+  g.gx = (int)((C + kRtAlign - 1 + kRtCols - 1) / kRtCols);
+  g.gy = (int)((rows + kRowUnroll - 1) / kRowUnroll);
+  g.grouped = g.gx <= kRtGroupedMax;
+  return g;
+}
+bool rt_ok(int64_t rows, int64_t C) {
+  return C >= kRtMinC && C % 32 != 0 && rows >= kRowUnroll &&
+         C < ((int64_t)1 << 31) &&
+         ((rows + kRowUnroll - 1) / kRowUnroll) *
+                 ((C + kRtAlign - 1 + kRtCols - 1) / kRtCols) <
+             ((int64_t)1 << 31);
+}
+__device__ __forceinline__ void rt_block(const RtGrid &g, int &bx, int &by) {
+  const int id = blockIdx.x;
+  const int full = g.grouped ? g.gy / 8 * 8 : 0; // row groups in sets of 8
+  if (id < full * g.gx) {
+    by = 8 * (id / (8 * g.gx)) + (id & 7);
+    bx = (id % (8 * g.gx)) >> 3;
+  } else {
+    const int rest = id - full * g.gx;
+    by = full + rest / g.gx;
+    bx = rest % g.gx;
+  }
+}
+// First element of row r in this scheme (r == rows: the end of the last row);
+// nvec4 = the elements that whole vectors cover.
+__device__ __forceinline__ int64_t rt_row_start(int64_t r, uint32_t C, int64_t nvec4) {
+  const int64_t e = (r * (int64_t)C + (kRtAlign - 1)) & ~(int64_t)(kRtAlign - 1);
+  return e < nvec4 ? e : nvec4;
+}
+
+// Scale and zero point of the four columns from c on (a column past C - 1
+// stands for the one C before it).  rt_load_cols only issues loads, without a
+// branch, so that a caller's loads all leave before anything waits; where the
+// four columns run over the end of the row it loads the last four of the row
+// instead and rt_fix_cols then fetches the right ones.
+typedef float f4u4 __attribute__((ext_vector_type(4), aligned(4)));
+struct RtCols {
+  f4a s;
+  uint32_t z; // four bytes
+};
+__device__ __forceinline__ uint32_t rt_wrap(uint32_t c, uint32_t C) {
+  c = c >= C ? c - C : c;
+  return c >= C ? c - C : c;
+}
+template <bool HAS_ZP>
+__device__ __forceinline__ RtCols rt_load_cols(const float *__restrict__ scale,
+    const void *__restrict__ zp, uint32_t c, uint32_t C) {
+  c = rt_wrap(c, C);
+  const uint32_t cs = c + 3 < C ? c : C - 4;
+  RtCols p;
+  p.s = *(const f4u4 *)(scale + cs);
+  p.z = HAS_ZP ? *(const u32_a1 *)((const uint8_t *)zp + cs) : 0u;
+  return p;
+}
+template <bool HAS_ZP>
+__device__ __forceinline__ void rt_fix_cols(RtCols &p,
+    const float *__restrict__ scale, const void *__restrict__ zp, uint32_t c,
+    uint32_t C) {
+  c = rt_wrap(c, C);
+  if (c + 3 < C)
+    return;
+  const uint8_t *zb = (const uint8_t *)zp;
+  uint32_t ce[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e)
+    ce[e] = c + e >= C ? c + e - C : c + e;
+  p.s.x = scale[ce[0]];
+  p.s.y = scale[ce[1]];
+  p.s.z = scale[ce[2]];
+  p.s.w = scale[ce[3]];
+  if (HAS_ZP)
+    p.z = (uint32_t)zb[ce[0]] | (uint32_t)zb[ce[1]] << 8 |
+          (uint32_t)zb[ce[2]] << 16 | (uint32_t)zb[ce[3]] << 24;
+}
+// The zero points of the four columns from `first` on (counted from col0).
+template <int KIND>
+__device__ __forceinline__ void rt_zps(
+    const uint32_t *sZ, int first, float (&z)[4]) {
+  const uint32_t zw = __builtin_amdgcn_alignbyte(
+      sZ[(first >> 2) + 1], sZ[first >> 2], (uint32_t)(first & 3));
+  z[0] = q_to_f32<KIND>(zw);
+  z[1] = q_to_f32<KIND>(zw >> 8);
+  z[2] = q_to_f32<KIND>(zw >> 16);
+  z[3] = q_to_f32<KIND>(zw >> 24);
+}
+
+template <int KIND, bool HAS_ZP>
+__global__ __launch_bounds__(kThreads) void k_dequant8_rowtable(
+    const uint8_t *__restrict__ x, float *__restrict__ y, int64_t n,
+    int64_t rows, uint32_t C, const float *__restrict__ scale,
+    const void *__restrict__ zp, RtGrid g) {
+  __shared__ __attribute__((aligned(16))) float sS[kRtTable];
+  __shared__ uint32_t sZ[kRtTable / 4 + 1];
+  const int t = threadIdx.x;
+  int bx, by;
+  rt_block(g, bx, by);
+  const uint32_t col0 = bx * (uint32_t)kRtCols;
+  const int64_t nvec4 = (n >> 2) << 2;
+  const int64_t r0 = (int64_t)by * kRowUnroll;
+  const uint32_t *__restrict__ x4 = (const uint32_t *)x;
+  f4a *__restrict__ y4 = (f4a *)y;
+  uint32_t w[kRowUnroll];
+  int64_t vec[kRowUnroll]; // the thread's vector in row r0 + j, or -1
+  int first[kRowUnroll];   // its first column in that row, counted from col0
+  auto request = [&]() {
+#pragma unroll
+    for (int j = 0; j < kRowUnroll; ++j) {
+      const int64_t r = r0 + j;
+      const int64_t s0 = rt_row_start(r, C, nvec4);
+      const int64_t e = s0 + col0 + 4 * t;
+      const bool ok = r < rows && e < rt_row_start(r + 1, C, nvec4);
+      vec[j] = ok ? (e >> 2) : -1;
+      first[j] = (int)(s0 - r * (int64_t)C) + 4 * t;
+      w[j] = ok ? __builtin_nontemporal_load(&x4[e >> 2]) : 0u;
+    }
+  };
+  auto finish = [&]() {
+#pragma unroll
+    for (int j = 0; j < kRowUnroll; ++j) {
+      if (vec[j] < 0)
+        continue;
+      const f4a sv = *(const f4u4 *)&sS[first[j]];
+      float z[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+      if (HAS_ZP)
+        rt_zps<KIND>(sZ, first[j], z);
+      f4a o;
+      o.x = dq_one<HAS_ZP>(q_to_f32<KIND>(w[j]), sv.x, z[0]);
+      o.y = dq_one<HAS_ZP>(q_to_f32<KIND>(w[j] >> 8), sv.y, z[1]);
+      o.z = dq_one<HAS_ZP>(q_to_f32<KIND>(w[j] >> 16), sv.z, z[2]);
+      o.w = dq_one<HAS_ZP>(q_to_f32<KIND>(w[j] >> 24), sv.w, z[3]);
+      __builtin_nontemporal_store(o, &y4[vec[j]]);
+    }
+  };
+  // The rows are requested before the tables are: the tables' loads would
+  // otherwise stand between the block's start and its first row.
+  request();
+  // The tables: columns col0 + 4 t .. + 3 from every thread, and the
+  // kRtAlign columns after those from the first threads (plus one more word
+  // of zero points, which a read of four bytes may reach into).  Every thread
+  // issues both loads, so that no branch separates them from the rows'.
+  const int t1 = t <= kRtAlign / 4 ? t : 0;
+  RtCols p0 = rt_load_cols<HAS_ZP>(scale, zp, col0 + 4 * t, C);
+  RtCols p1 = rt_load_cols<HAS_ZP>(scale, zp, col0 + kRtCols + 4 * t1, C);
+  rt_fix_cols<HAS_ZP>(p0, scale, zp, col0 + 4 * t, C);
+  rt_fix_cols<HAS_ZP>(p1, scale, zp, col0 + kRtCols + 4 * t1, C);
+  *(f4a *)&sS[4 * t] = p0.s;
+  if (HAS_ZP)
+    sZ[t] = p0.z;
+  if (t <= kRtAlign / 4) {
+    if (t < kRtAlign / 4)
+      *(f4a *)&sS[kRtCols + 4 * t] = p1.s;
+    if (HAS_ZP)
+      sZ[kThreads + t] = p1.z;
+  }
+  __syncthreads();
+  finish();
+  // the up to three elements after the last whole vector
+  if (bx == 0 && by == 0) {
+    const int64_t e = nvec4 + t;
+    if (e < n) {
+      const uint32_t ce = (uint32_t)(e % C);
+      const float zf = HAS_ZP ? load_q_zp_f32<KIND>(zp, ce) : 0.0f;
+      y[e] = dq_one<HAS_ZP>(q_to_f32<KIND>(x[e]), scale[ce], zf);
+    }
+  }
+}
+
 // Any element kind, [outer, channels, inner]: one element per lane.
 // The dequantize counterpart of k_quant_slabs (8-bit input).
 template <int KIND, bool HAS_ZP, int U>
@@ -1463,11 +1671,25 @@ hipError_t dequantize_dispatch(hipStream_t st, const void *x, int64_t outer,
           <<<grid, kThreads, 0, st>>>(xi, y, n, scale, zp);
     return hipGetLastError();
   }
+  if (KIND != kI32 && inner == 1 && rt_ok(outer, channels) &&
+      ((((uintptr_t)x) & 3) == 0) && ((((uintptr_t)y) & 15) == 0) &&
+      ((((uintptr_t)scale) & 3) == 0)) {
+    constexpr int K8 = KIND == kI32 ? kU8 : KIND;
+    const RtGrid g = rt_grid(outer, channels);
+    const unsigned grid = (unsigned)g.gx * (unsigned)g.gy;
+    if (has_zp)
+      k_dequant8_rowtable<K8, true><<<grid, kThreads, 0, st>>>(
+          (const uint8_t *)x, y, n, outer, (uint32_t)channels, scale, zp, g);
+    else
+      k_dequant8_rowtable<K8, false><<<grid, kThreads, 0, st>>>(
+          (const uint8_t *)x, y, n, outer, (uint32_t)channels, scale, zp, g);
+    return hipGetLastError();
+  }
   if (KIND != kI32 && inner == 1 && channels > 1 && channels % 4 != 0 &&
       channels < ((int64_t)1 << 31) && ((((uintptr_t)x) & 3) == 0) &&
       ((((uintptr_t)y) & 15) == 0) && (n >> 2) > 0) {
-    const PeriodicGrid pg = periodic_grid(n >> 2, channels, 2);
     constexpr int K8 = KIND == kI32 ? kU8 : KIND;
+    const PeriodicGrid pg = periodic_grid(n >> 2, channels, 2);
     const bool vec = channels >= 4 && ((((uintptr_t)scale) & 3) == 0);
     if (has_zp && vec)
       k_dequant8_periodic<K8, true, true><<<pg.grid, kThreads, 0, st>>>(

@@ -232,6 +232,37 @@ def test_dequantize_int32_per_column(rt, oracle):
     assert same_f32(rt.DequantizeLinear(acc, sc, zp, axis=1), oracle.dequantize_linear(acc, sc, zp, axis=1))
 
 
+@pytest.mark.parametrize("rows,cols", [(8, 3968 + 4), (9, 3969), (37, 3970), (40, 3971), (23, 5001), (64, 4100),
+                                       (17, 33001), (200, 4111), (11, 51000), (70, 65537), (16, 4095), (33, 8191)])
+def test_dequantize_long_rows_off_the_cache_lines(rt, oracle, rows, cols):
+    """Rows of about 4 Ki elements and more whose starts are not 128-byte aligned in
+    the float tensor (cols % 32 != 0) take the kernel that re-aligns every row to
+    cache lines and reads scale / zero point from a per-block table: every cols % 4,
+    row counts that are no multiple of 8, rows that end inside a block's vector and
+    inside its table (the wrap to column 0), both element types, with and without
+    zero points, and operands that start 4 bytes (scale) / 1 byte (zero point) / 4
+    bytes (x) / 16 bytes (y) into their allocations."""
+    rng = np.random.default_rng(rows * 100003 + cols)
+    for qdt in (np.uint8, np.int8):
+        q = rng.integers(0, 256, (rows, cols), dtype=np.uint8).view(qdt)
+        sc = rng.uniform(0.005, 0.05, cols).astype(np.float32)
+        zp = rng.integers(0, 256, cols, dtype=np.uint8).view(qdt)
+        for z in (zp, None):
+            assert same_f32(rt.DequantizeLinear(q, sc, z, axis=1), oracle.dequantize_linear(q, sc, z, axis=1))
+    want = oracle.dequantize_linear(q, sc, zp, axis=1)
+    n = rows * cols
+    dq = rt.DeviceArray.from_numpy(np.concatenate([np.zeros(4, qdt), q.reshape(-1)]))
+    ds = rt.DeviceArray.from_numpy(np.concatenate([np.zeros(1, np.float32), sc]))
+    dz = rt.DeviceArray.from_numpy(np.concatenate([np.zeros(1, qdt), zp]))
+    dy = rt.DeviceArray.from_numpy(np.full(n + 8, -7.0, np.float32))
+    yv = rt.DeviceArray.view_of(dy, 4, (rows, cols))
+    rt.DequantizeLinear(rt.DeviceArray.view_of(dq, 4, (rows, cols)), rt.DeviceArray.view_of(ds, 1, (cols,)),
+                        rt.DeviceArray.view_of(dz, 1, (cols,)), axis=1, out=yv)
+    assert same_f32(yv.numpy(), want)
+    edge = dy.numpy()
+    assert (edge[:4] == -7.0).all() and (edge[-4:] == -7.0).all()     # nothing written outside the view
+
+
 def test_misaligned_device_views_are_handled(rt, oracle):
     # tensors that start 4 bytes (x) / 1 byte (y) into a GPU allocation: the
     # 16-byte and 4-byte alignment the fast kernels rely on is lost
@@ -1335,6 +1366,8 @@ def test_config2_full_size(rt, oracle, rows, cols):
     assert np.array_equal(q[sample], want)
     d = dD.numpy()
     assert same_f32(d[sample], oracle.dequantize_linear(want, c["scale"], c["zp"], axis=1))
+    # ... and every element against the oracle's OpenMP twin
+    assert same_f32(d, oracle.dequantize_linear(q, c["scale"], c["zp"], axis=1, omp=True))
     del d, dD, dQ2
     # dynamic quantisation of the same tensor: parameters from numpy's min / max
     dY, ds, dz = rt.DynamicQuantizeLinear(dX)
