@@ -189,7 +189,8 @@ def test_quantize_next_to_every_rounding_boundary(rt, oracle):
 @pytest.mark.parametrize("shape,axis", [((64, 1000), 1), ((37, 1023), 1), ((5, 7), 1), ((129, 4096), -1),
                                         ((3, 5, 64, 33), 1), ((6, 100), 0), ((2, 3, 4, 5), 2),
                                         ((1, 3, 3, 2), 1), ((300, 2), 1), ((1000, 6), 1), ((257, 4097), 1),
-                                        ((3, 1001), -1), ((4099, 3), 1), ((2, 40001), 1)])
+                                        ((3, 1001), -1), ((4099, 3), 1), ((2, 40001), 1),
+                                        ((5, 2048), 1), ((3, 32768), 1), ((2, 65536), 1)])
 @pytest.mark.parametrize("qdt", [np.uint8, np.int8])
 def test_quantize_dequantize_per_axis(rt, oracle, shape, axis, qdt):
     # per-axis: the oracle applies the reference's per-tensor formula per channel
