@@ -880,10 +880,11 @@ __global__ __launch_bounds__(kThreads) void k_dequant8_periodic(
 // (k_dequant8_periodic).  Row r is taken to start at the next multiple of
 // kRtAlign elements at or after r * C (the elements before that go with row
 // r - 1, whose columns wrap around); block (bx, by) takes elements
-// [bx * kRtCols, + kRtCols) after that start in each of its kRowUnroll rows.
+// [bx * kRtCols, + kRtCols) after that start in each of its kRtRows rows.
 // Which columns a thread meets therefore moves from row to row, by less than
 // kRtAlign: scale and zero point of the block's kRtCols + kRtAlign columns sit
 // in LDS and are read from there for every vector.
+constexpr int kRtRows = 8; // rows per block (4: 2 points less, 2: 8 less, 16: 6 less)
 constexpr int kRtCols = kThreads * 4;
 constexpr int kRtAlign = 128;
 constexpr int kRtTable = kRtCols + kRtAlign;
@@ -908,14 +909,14 @@ struct RtGrid {
 RtGrid rt_grid(int64_t rows, int64_t C) {
   RtGrid g;
   g.gx = (int)((C + kRtAlign - 1 + kRtCols - 1) / kRtCols);
-  g.gy = (int)((rows + kRowUnroll - 1) / kRowUnroll);
+  g.gy = (int)((rows + kRtRows - 1) / kRtRows);
   g.grouped = g.gx <= kRtGroupedMax;
   return g;
 }
 bool rt_ok(int64_t rows, int64_t C) {
-  return C >= kRtMinC && C % 32 != 0 && rows >= kRowUnroll &&
+  return C >= kRtMinC && C % 32 != 0 && rows >= kRtRows &&
          C < ((int64_t)1 << 31) &&
-         ((rows + kRowUnroll - 1) / kRowUnroll) *
+         ((rows + kRtRows - 1) / kRtRows) *
                  ((C + kRtAlign - 1 + kRtCols - 1) / kRtCols) <
              ((int64_t)1 << 31);
 }
@@ -1006,15 +1007,15 @@ __global__ __launch_bounds__(kThreads) void k_dequant8_rowtable(
   rt_block(g, bx, by);
   const uint32_t col0 = bx * (uint32_t)kRtCols;
   const int64_t nvec4 = (n >> 2) << 2;
-  const int64_t r0 = (int64_t)by * kRowUnroll;
+  const int64_t r0 = (int64_t)by * kRtRows;
   const uint32_t *__restrict__ x4 = (const uint32_t *)x;
   f4a *__restrict__ y4 = (f4a *)y;
-  uint32_t w[kRowUnroll];
-  int64_t vec[kRowUnroll]; // the thread's vector in row r0 + j, or -1
-  int first[kRowUnroll];   // its first column in that row, counted from col0
+  uint32_t w[kRtRows];
+  int64_t vec[kRtRows]; // the thread's vector in row r0 + j, or -1
+  int first[kRtRows];   // its first column in that row, counted from col0
   auto request = [&]() {
 #pragma unroll
-    for (int j = 0; j < kRowUnroll; ++j) {
+    for (int j = 0; j < kRtRows; ++j) {
       const int64_t r = r0 + j;
       const int64_t s0 = rt_row_start(r, C, nvec4);
       const int64_t e = s0 + col0 + 4 * t;
@@ -1026,7 +1027,7 @@ __global__ __launch_bounds__(kThreads) void k_dequant8_rowtable(
   };
   auto finish = [&]() {
 #pragma unroll
-    for (int j = 0; j < kRowUnroll; ++j) {
+    for (int j = 0; j < kRtRows; ++j) {
       if (vec[j] < 0)
         continue;
       const f4a sv = *(const f4u4 *)&sS[first[j]];
