@@ -133,6 +133,7 @@ void *g_scratch_ptr[kMaxDevices] = {};
 unsigned g_scratch_epoch[kMaxDevices] = {};   // launch number of k_dql_grid
 bool g_scratch_no_grid[kMaxDevices] = {};     // one-launch kernel switched off
 bool g_scratch_used[kMaxDevices] = {};
+bool g_scratch_unchecked[kMaxDevices] = {}; // launched since its flag was last fetched
 
 // Call with device `dev` current.
 bool resolve_scratch(int dev) {
@@ -430,9 +431,14 @@ struct Ctx {
   // Whether a one-launch kernel of this thread gave up since the last check
   // (call after the stream has been synchronised).  If so the flag is
   // cleared and the one-launch kernel is not used again by this thread.
+  // Whether the one-launch kernel raised its flag since the last look.  The
+  // flag is only fetched (a blocking 4-byte copy, tens of microseconds) when
+  // such a kernel has been launched since.
+  bool dql_unchecked = false;
   bool dql_gave_up() {
-    if (!ready || dql.grid_blocks == 0)
+    if (!ready || dql.grid_blocks == 0 || !dql_unchecked)
       return false;
+    dql_unchecked = false;
     unsigned flag = 0;
     if (hipMemcpy(&flag, dql.counter + 8, sizeof(flag),
             hipMemcpyDeviceToHost) != hipSuccess)
@@ -941,6 +947,7 @@ bool is_q8(int dt) {
 void run_dql(Call &call, const float *dx, int64_t n, uint8_t *dy, float *ds,
     uint8_t *dz, bool y_shift) {
   Ctx &c = call.c;
+  c.dql_unchecked = c.dql.grid_blocks != 0;
   call.check(
       launch_dynamic_quantize(c.stream, c.dql, dx, n, dy, ds, dz, y_shift),
       "DynamicQuantizeLinear");
@@ -975,8 +982,10 @@ bool noalloc_barrier_ok() {
   void *sp;
   {
     std::lock_guard<std::mutex> lk(g_scratch_mutex);
-    if (!g_scratch_used[dev] || g_scratch_no_grid[dev])
+    if (!g_scratch_used[dev] || g_scratch_no_grid[dev] ||
+        !g_scratch_unchecked[dev])
       return true;
+    g_scratch_unchecked[dev] = false;
     sp = g_scratch_ptr[dev];
   }
   unsigned *counter = (unsigned *)((char *)sp + sizeof(float) * 2 * kNoAllocBlocks);
@@ -1641,6 +1650,7 @@ void om_mi355x_DynamicQuantizeLinearNoAlloc(OMTensor *y_t, OMTensor *scale_t,
   s.spin_limit = c.dql.spin_limit;
   s.epoch = g_scratch_epoch[dev];
   g_scratch_used[dev] = true;
+  g_scratch_unchecked[dev] = true;
   // The array keeps what the last call left.  The slots need no clearing
   // (they carry the launch number); the arrival counter of the two-launch
   // path must start at zero and would not be if an earlier launch had been
@@ -1971,8 +1981,13 @@ int om_mi355x_memcpy_d2h(void *dst, const void *src, size_t bytes) {
 int om_mi355x_synchronize(void) {
   if (!t_ctx.init())
     return -1;
-  hipError_t e = hipStreamSynchronize(t_ctx.stream);
+  // A stream with nothing left to do is found idle by a query; waiting on it
+  // would still cost a round trip to the GPU (about 30 us).
+  hipError_t e = hipStreamQuery(t_ctx.stream);
+  if (e == hipErrorNotReady)
+    e = hipStreamSynchronize(t_ctx.stream);
   if (e != hipSuccess) {
+    (void)hipGetLastError();
     fail(EIO, "stream synchronisation failed: %s", hipGetErrorString(e));
     return -1;
   }
