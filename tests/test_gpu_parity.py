@@ -235,10 +235,10 @@ def test_dequantize_int32_per_column(rt, oracle):
 
 @pytest.mark.parametrize("rows,cols", [(8, 3968 + 4), (9, 3969), (37, 3970), (40, 3971), (23, 5001), (64, 4100),
                                        (17, 33001), (200, 4111), (11, 51000), (70, 65537), (16, 4095), (33, 8191)])
-def test_dequantize_long_rows_off_the_cache_lines(rt, oracle, rows, cols):
+def test_long_rows_off_the_cache_lines(rt, oracle, rows, cols):
     """Rows of about 4 Ki elements and more whose starts are not 128-byte aligned in
-    the float tensor (cols % 32 != 0) take the kernel that re-aligns every row to
-    cache lines and reads scale / zero point from a per-block table: every cols % 4,
+    the float tensor (cols % 32 != 0) take the kernels that re-align every row to
+    cache lines and read scale / zero point from a per-block table: every cols % 4,
     row counts that are no multiple of 8, rows that end inside a block's vector and
     inside its table (the wrap to column 0), both element types, with and without
     zero points, and operands that start 4 bytes (scale) / 1 byte (zero point) / 4
@@ -250,6 +250,18 @@ def test_dequantize_long_rows_off_the_cache_lines(rt, oracle, rows, cols):
         zp = rng.integers(0, 256, cols, dtype=np.uint8).view(qdt)
         for z in (zp, None):
             assert same_f32(rt.DequantizeLinear(q, sc, z, axis=1), oracle.dequantize_linear(q, sc, z, axis=1))
+        # quantize: values on and next to the rounding boundaries of their column's
+        # scale, and (second round) three columns whose scale takes the divide
+        x = ((rng.integers(-300, 300, (rows, cols)) + rng.choice(np.array([0.0, 0.5, 0.4999999, 0.5000001]),
+                                                                  (rows, cols))) * sc).astype(np.float32)
+        for wild in (False, True):
+            s2 = sc.copy()
+            if wild:
+                s2[rng.integers(0, cols, 3)] = np.float32(1e-38)
+            for z in (zp, None):
+                if z is None and qdt == np.int8:
+                    continue
+                assert np.array_equal(rt.QuantizeLinear(x, s2, z, axis=1), oracle.quantize_linear(x, s2, z, axis=1))
     want = oracle.dequantize_linear(q, sc, zp, axis=1)
     n = rows * cols
     dq = rt.DeviceArray.from_numpy(np.concatenate([np.zeros(4, qdt), q.reshape(-1)]))
@@ -262,6 +274,15 @@ def test_dequantize_long_rows_off_the_cache_lines(rt, oracle, rows, cols):
     assert same_f32(yv.numpy(), want)
     edge = dy.numpy()
     assert (edge[:4] == -7.0).all() and (edge[-4:] == -7.0).all()     # nothing written outside the view
+    # quantize with x 16 bytes, y 4 bytes, scale 4 bytes and zero point 1 byte into their allocations
+    dx = rt.DeviceArray.from_numpy(np.concatenate([np.zeros(4, np.float32), x.reshape(-1)]))
+    dq2 = rt.DeviceArray.from_numpy(np.full(n + 8, 9, qdt))
+    qv = rt.DeviceArray.view_of(dq2, 4, (rows, cols))
+    rt.QuantizeLinear(rt.DeviceArray.view_of(dx, 4, (rows, cols)), rt.DeviceArray.view_of(ds, 1, (cols,)),
+                      rt.DeviceArray.view_of(dz, 1, (cols,)), axis=1, out=qv)
+    assert np.array_equal(qv.numpy(), oracle.quantize_linear(x, sc, zp, axis=1))
+    edge = dq2.numpy()
+    assert (edge[:4] == 9).all() and (edge[-4:] == 9).all()
 
 
 def test_misaligned_device_views_are_handled(rt, oracle):
