@@ -18,6 +18,12 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 
 constexpr int BK = kGemmBK;
 
+// Cache policy operand of the buffer stores that carry results: sc1, the
+// store is written through to memory when it is issued instead of staying
+// dirty in L2 until the kernel ends (2 would be nontemporal, 0 plain).
+constexpr int kAuxThrough = 16;
+constexpr int kAuxStream = 2;
+
 // Byte offset of 16-byte chunk `c` (0..3) of tile row `r` (row = 64 bytes).
 __device__ __forceinline__ int lds_off(int r, int c) {
   return r * BK + ((c ^ ((r >> 2) & 3)) << 4);

@@ -78,7 +78,7 @@ __device__ __forceinline__ void store_one(const EpiParams &ep, int64_t o,
   }
 }
 
-template <int TM, int TN, int A_MODE, int EPI>
+template <int TM, int TN, int A_MODE, int EPI, int AUX32 = kAuxStream>
 __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TM][TN],
     const int32_t (&rsp)[TM], int mrow0, int ncol0, int M, int N, int K,
     const EpiParams &ep) {
@@ -158,7 +158,8 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TM][TN],
     // mrow0 and ncol0 are the same for every lane of the wave (callers derive
     // them from a scalar wave index), so this test and the row addresses below
     // are scalar work.
-    const bool full = (mrow0 + 32 * TM <= M) && (ncol0 + 32 * TN <= N);
+    const bool full = (mrow0 + 32 * TM <= M) && (ncol0 + 32 * TN <= N) &&
+                      (int64_t)N * (32 * TM + 8) * 4 < ((int64_t)1 << 31);
     constexpr int ES = (EPI == kEpiQ8) ? 1 : 4;
     char *const base =
         (char *)ep.out + ((int64_t)mrow0 * N + ncol0) * (int64_t)ES;
@@ -166,39 +167,42 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TM][TN],
         ((uint32_t)(4 * lh) * (uint32_t)N + (uint32_t)l32) * (uint32_t)ES;
     // One element: row tile i, register r (row 8*(r/4) + 4*lh + r%4 of the
     // tile), column tile j.  RS: add the row-sum term.
+    // Results leave through buffer stores on a descriptor that starts at the
+    // wave tile's first element (offsets then fit 32 bits: `full` below also
+    // asks for that), written through to memory as they are issued (sc1)
+    // instead of sitting in L2 until the kernel ends: the write-back of the
+    // whole result at the end of the kernel is otherwise the kernel's last
+    // microsecond or two (4096 x 768 x 3072 with f32 results, weights in
+    // registers: plain stores 15.9 us, streaming 15.0, written through 13.8;
+    // the 8-bit activations of DynamicQuantizeLinear [4096, 3072]: 15.4 ->
+    // 13.9 us, and the GEMM that reads them next is not slowed down as it is
+    // by streaming stores) -- but only when a wave's 128-byte row pieces are
+    // whole lines.  With a row pitch that is no multiple of 128 bytes every
+    // piece straddles two lines, and sending the parts to memory one by one
+    // costs far more than letting L2 put the lines together (N = 3070:
+    // 28.0 us streaming, 19.4 us plain).
+    const __amdgpu_buffer_rsrc_t orsrc =
+        __builtin_amdgcn_make_buffer_rsrc(base, 0, 0x7FFFFFFF, 0x00020000);
     auto emit = [&](auto rs_c, auto stream_c, int i, int r, int j,
-                    int32_t rs_row, char *rowp) {
+                    int32_t rs_row, int32_t rowb) {
       uint32_t y = (uint32_t)acc[i][j][r] + cj[j];
       if (decltype(rs_c)::value)
         y += (uint32_t)db[j] * (uint32_t)rs_row;
-      char *const q = rowp + loff + (uint32_t)(j * 32 * ES);
-      // Streaming stores: the result is not read again by this kernel, and
-      // keeping it out of the way in L2 leaves the A and Bp panels cached for
-      // the blocks still in their K loop (6 % faster on 4096x768x3072) -- but
-      // only when a wave's 128-byte row pieces are whole lines.  With a row
-      // pitch that is no multiple of 128 bytes every piece straddles two
-      // lines, and streaming the parts costs far more than letting L2 put
-      // the lines together (N = 3070: 28.0 us streaming, 19.4 us plain).
-      // (The streaming hint lives in the store's memory operand, which the
-      // compiler's tail merging does not compare: without the marker below
-      // it folds the two variants into one and drops the hint.)
-      constexpr bool kStream = decltype(stream_c)::value;
+      const int voff = (int)(loff + (uint32_t)(j * 32 * ES));
+      // 8-bit results: written through.  32-bit results: the caller's choice
+      // (streaming for the 128-wide tiles, 4096 x 768 x 768 7.4 us against 7.8
+      // written through; written through for k_gemm_i8_bs, 2048 x 4096 x 11008
+      // 93.9 us against 94.5 streaming).
+      constexpr int kAux = !decltype(stream_c)::value ? 0
+                           : EPI == kEpiQ8            ? kAuxThrough
+                                                      : AUX32;
       if (EPI == kEpiI32) {
-        if (kStream) {
-          __builtin_nontemporal_store((int32_t)y, (int32_t *)q);
-        } else {
-          *(int32_t *)q = (int32_t)y;
-          asm volatile("; plain store");
-        }
+        __builtin_amdgcn_raw_buffer_store_b32((int)y, orsrc, voff, rowb, kAux);
       } else if (EPI == kEpiF32) {
         float f = (float)(int32_t)y * sj[j] + bj[j];
         f = relu_f32(f, ep.floor);
-        if (kStream) {
-          __builtin_nontemporal_store(f, (float *)q);
-        } else {
-          *(float *)q = f;
-          asm volatile("; plain store");
-        }
+        __builtin_amdgcn_raw_buffer_store_b32(
+            (int)__float_as_uint(f), orsrc, voff, rowb, kAux);
       } else {
         const float f = (float)(int32_t)y * sj[j];
         int32_t v =
@@ -208,7 +212,8 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TM][TN],
           const int32_t hi = ep.y_unsigned ? 255 : 127;
           v = v < lo ? lo : (v > hi ? hi : v);
         }
-        *(uint8_t *)q = (uint8_t)(v & 0xFF);
+        __builtin_amdgcn_raw_buffer_store_b8(
+            (unsigned char)(v & 0xFF), orsrc, voff, rowb, kAux);
       }
     };
     auto whole = [&](auto rs_c, auto stream_c) {
@@ -222,11 +227,11 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TM][TN],
           const int rr = 8 * (r >> 2) + 4 * lh + (r & 3);
           const int32_t rs_row =
               decltype(rs_c)::value ? __shfl(rsf[i], rr, 64) : 0;
-          const int64_t rowb =
-              (int64_t)(i * 32 + 8 * (r >> 2) + (r & 3)) * N * (int64_t)ES;
+          const int32_t rowb =
+              (int32_t)((i * 32 + 8 * (r >> 2) + (r & 3)) * N * ES);
 #pragma unroll
           for (int j = 0; j < TN; ++j)
-            emit(rs_c, stream_c, i, r, j, rs_row, base + rowb);
+            emit(rs_c, stream_c, i, r, j, rs_row, rowb);
         }
       }
     };
@@ -1137,7 +1142,8 @@ __global__ __launch_bounds__(256, MINB) void k_gemm_i8_bs(
   // A copies past the last step are still landing in LDS.
   __builtin_amdgcn_s_waitcnt(0x0F70);
 
-  gemm_epilogue<TM, TN, A_MODE, EPI>(acc, rsp, m0, ncol0, M, N, K, ep);
+  gemm_epilogue<TM, TN, A_MODE, EPI, kAuxThrough>(
+      acc, rsp, m0, ncol0, M, N, K, ep);
 }
 
 // ---- skinny GEMM (M <= 64): weight streaming -------------------------------

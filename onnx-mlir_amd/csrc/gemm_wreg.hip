@@ -324,7 +324,7 @@ __global__ __launch_bounds__(WAVES * 64, 1) void k_gemm_i8_wreg(
     const uint32_t y = (uint32_t)accp[r] + cj;
     constexpr int row = 8 * (r >> 2) + (r & 3); // + 4 * lh
     const int soff = row * N * ES; // the same for every lane: a scalar offset
-    constexpr int kAux = STREAM ? 2 : 0; // 2: nontemporal
+    constexpr int kAux = STREAM ? kAuxThrough : 0;
     if (EPI == kEpiI32) {
       __builtin_amdgcn_raw_buffer_store_b32((int)y, out_rsrc, (int)toff, soff, kAux);
     } else if (EPI == kEpiF32) {
