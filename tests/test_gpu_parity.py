@@ -251,7 +251,7 @@ def test_long_rows_off_the_cache_lines(rt, oracle, rows, cols):
         for z in (zp, None):
             assert same_f32(rt.DequantizeLinear(q, sc, z, axis=1), oracle.dequantize_linear(q, sc, z, axis=1))
         # quantize: values on and next to the rounding boundaries of their column's
-        # scale, and (second round) three columns whose scale takes the divide
+        # scale, and (second pass) three columns whose scale takes the divide
         x = ((rng.integers(-300, 300, (rows, cols)) + rng.choice(np.array([0.0, 0.5, 0.4999999, 0.5000001]),
                                                                   (rows, cols))) * sc).astype(np.float32)
         for wild in (False, True):
