@@ -1019,8 +1019,10 @@ def test_matmulinteger_batched_b(rt, oracle):
                                       oracle.matmul_integer(A, B, azm, bzn)), (ashape, bshape)
     # a 1-D right-hand side (the matrix-vector case of src/Conversion/ONNXToKrnl/Math/MatMul.cpp:299-304)
     A, v = _rand_q(rng, np.uint8, (9, 50)), _rand_q(rng, np.int8, (50,))
-    got = rt.MatMulInteger(A, v, _rand_q(rng, np.uint8, ()), None)
-    assert got.shape == (9,)
+    az = _rand_q(rng, np.uint8, ())
+    got = rt.MatMulInteger(A, v, az, None)
+    assert got.shape == (9,) and np.array_equal(got, oracle.matmul_integer(A, v, az, None))
+    assert np.array_equal(got.astype(np.int64), (A.astype(np.int64) - int(az)) @ v.astype(np.int64))
     # device-resident batched operands
     A, B = _rand_q(rng, np.uint8, (4, 70, 128)), _rand_q(rng, np.int8, (4, 128, 96))
     dA, dB = rt.DeviceArray.from_numpy(A), rt.DeviceArray.from_numpy(B)
