@@ -885,6 +885,30 @@ def test_quantize_random_shapes_and_axes(rt, oracle):
         assert np.array_equal(gy, wy) and same_f32(np.float32(gs), ws) and int(gz) == int(wz), tag
 
 
+def test_last_axis_shapes_around_kernel_boundaries(rt, oracle):
+    """Per-axis quantize / dequantize on the innermost axis with row lengths on both
+    sides of every length the dispatch looks at (2 Ki and 32 Ki powers of two, the
+    3968 columns from which rows are re-aligned to cache lines, multiples of 4 and of
+    32 and their neighbours, rows that wrap inside a block's table), row counts on
+    both sides of 8 and of the rows a block takes, 2-D and 3-D shapes, both element
+    types, with and without zero points."""
+    rng = np.random.default_rng(777)
+    lengths = [2047, 2048, 2049, 2080, 3967, 3968, 3969, 3970, 3971, 3972, 4000, 4095, 4096, 4097, 4100, 4128,
+               5119, 5120, 5121, 6000, 8191, 8192, 8193, 16380, 16384, 32764, 32767, 32768, 32769, 33001, 65535, 65537]
+    for case, cols in enumerate(lengths):
+        rows = int(rng.choice([1, 2, 7, 8, 9, 15, 16, 17, 31]))
+        shape = (rows, cols) if case % 3 else (2, max(1, rows // 2), cols)
+        qdt = (np.uint8, np.int8)[case % 2]
+        x = rng.normal(0, 3, shape).astype(np.float32)
+        sc = rng.uniform(0.005, 0.5, cols).astype(np.float32)
+        zp = rng.integers(0, 256, cols, dtype=np.uint8).view(qdt) if case % 4 or qdt == np.int8 else None
+        tag = (shape, qdt.__name__, zp is None)
+        wq = oracle.quantize_linear(x, sc, zp, axis=-1, out_dtype=qdt)
+        assert np.array_equal(rt.QuantizeLinear(x, sc, zp, axis=-1), wq), tag
+        assert same_f32(rt.DequantizeLinear(wq, sc, zp, axis=-1), oracle.dequantize_linear(wq, sc, zp, axis=-1)), tag
+        assert same_f32(rt.DequantizeLinear(wq, sc, None, axis=-1), oracle.dequantize_linear(wq, sc, None, axis=-1)), tag
+
+
 def test_per_axis_with_inner_slabs(rt, oracle):
     """Per-channel parameters on an axis that is not the innermost one (NCHW
     activations, [C_out, C_in] weights on axis 0): slabs of `inner` elements
