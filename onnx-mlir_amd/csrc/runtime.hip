@@ -134,6 +134,7 @@ unsigned g_scratch_epoch[kMaxDevices] = {};   // launch number of k_dql_grid
 bool g_scratch_no_grid[kMaxDevices] = {};     // one-launch kernel switched off
 bool g_scratch_used[kMaxDevices] = {};
 bool g_scratch_unchecked[kMaxDevices] = {}; // launched since its flag was last fetched
+std::thread::id g_scratch_launcher[kMaxDevices]; // by this thread: the one whose synchronisation fetches it
 
 // Call with device `dev` current.
 bool resolve_scratch(int dev) {
@@ -983,7 +984,8 @@ bool noalloc_barrier_ok() {
   {
     std::lock_guard<std::mutex> lk(g_scratch_mutex);
     if (!g_scratch_used[dev] || g_scratch_no_grid[dev] ||
-        !g_scratch_unchecked[dev])
+        !g_scratch_unchecked[dev] ||
+        g_scratch_launcher[dev] != std::this_thread::get_id())
       return true;
     g_scratch_unchecked[dev] = false;
     sp = g_scratch_ptr[dev];
@@ -1651,6 +1653,7 @@ void om_mi355x_DynamicQuantizeLinearNoAlloc(OMTensor *y_t, OMTensor *scale_t,
   s.epoch = g_scratch_epoch[dev];
   g_scratch_used[dev] = true;
   g_scratch_unchecked[dev] = true;
+  g_scratch_launcher[dev] = std::this_thread::get_id();
   // The array keeps what the last call left.  The slots need no clearing
   // (they carry the launch number); the arrival counter of the two-launch
   // path must start at zero and would not be if an earlier launch had been
