@@ -194,7 +194,7 @@ def decode_case(rt, wl, M, steps, warmup):
     dS = rt.DeviceArray.from_numpy(c["w_scale"])
     dY = rt.DeviceArray((M, N), np.float32)
     rt.mark_constant(dW)
-    fn = rt.PreparedCall("om_mi355x_DynQuantMatMulDequant", dY, dX, dW, None, dS, None, 0)
+    fn = rt.PreparedCall("om_mi355x_DynQuantMatMulDequant", dY, dX, dW, None, dS, None, activation)
     res = measure(rt, fn, steps, warmup)
     fn.check()
     fn.close()
@@ -231,9 +231,10 @@ def qlinear_case(rt, wl, steps, warmup):
     return res
 
 
-def fused_case(rt, wl, name, M, K, N, w_i8, w_scale, steps, warmup, X=None):
+def fused_case(rt, wl, name, M, K, N, w_i8, w_scale, steps, warmup, X=None, activation=0):
     """DynamicQuantizeLinear -> MatMulInteger -> Cast -> Mul as one call: fp32
-    activations in, fp32 out (the chain the quantized models contain)."""
+    activations in, fp32 out (the chain the quantized models contain);
+    `activation` 1 / 2 adds the Relu / Gelu that follows an FFN-up projection."""
     if X is None:
         X = np.random.default_rng(0xF00D + M + K + N).normal(0, 1, (M, K)).astype(np.float32)
     dX = rt.DeviceArray.from_numpy(X)
@@ -241,7 +242,7 @@ def fused_case(rt, wl, name, M, K, N, w_i8, w_scale, steps, warmup, X=None):
     dS = rt.DeviceArray.from_numpy(np.asarray(w_scale, np.float32))
     dY = rt.DeviceArray((M, N), np.float32)
     rt.mark_constant(dW)
-    fn = rt.PreparedCall("om_mi355x_DynQuantMatMulDequant", dY, dX, dW, None, dS, None, 0)
+    fn = rt.PreparedCall("om_mi355x_DynQuantMatMulDequant", dY, dX, dW, None, dS, None, activation)
     res = measure(rt, fn, steps, warmup)
     fn.check()
     fn.close()
@@ -377,11 +378,13 @@ def only_mode(rt, wl, what, steps, warmup):
         r = gemm_case(rt, wl, f"config4 {layer}", 4096, k, n, c["W"], c["w_scale"], steps, warmup, "f32",
                       headline=True)
         return {"only": what, **r}
-    if what in ("fused_ffn_up", "fused_ffn_down"):
-        layer = what[6:]
+    if what in ("fused_ffn_up", "fused_ffn_down", "fused_ffn_up_relu", "fused_ffn_up_gelu"):
+        layer = "ffn_down" if what == "fused_ffn_down" else "ffn_up"
+        act = {"relu": 1, "gelu": 2}.get(what.rsplit("_", 1)[1], 0)
         k, n = wl.CONFIG4_SHAPES[layer]
         c = wl.config4(layer, M=8)
-        r = fused_case(rt, wl, f"config4 {layer} fused layer", 4096, k, n, c["W"], c["w_scale"], steps, warmup)
+        r = fused_case(rt, wl, f"config4 {layer} fused layer" + (f", activation {act}" if act else ""),
+                       4096, k, n, c["W"], c["w_scale"], steps, warmup, activation=act)
         return {"only": what, **r}
     if what in ("decode", "decode4", "decode16"):
         return {"only": what, **decode_case(rt, wl, {"decode": 1, "decode4": 4, "decode16": 16}[what], steps, warmup)}
@@ -531,6 +534,7 @@ def main():
     ap.add_argument("--only", default=None,
                     choices=["copy", "gemm_ffn_up", "gemm_qkv", "gemm_out", "gemm_ffn_down",
                              "gemm_prefill_up", "gemm_prefill_down", "fused_ffn_up", "fused_ffn_down",
+                             "fused_ffn_up_relu", "fused_ffn_up_gelu",
                              "decode", "decode4", "decode16",
                              "quantize_per_axis", "dequantize_per_axis",
                              "quantize_per_tensor", "dequantize_per_tensor", "dynamic_quantize",

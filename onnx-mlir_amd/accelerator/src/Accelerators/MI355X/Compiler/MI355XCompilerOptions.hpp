@@ -38,6 +38,7 @@ extern MI355XNarrowMode mi355xNarrowMode;
 extern bool mi355xDisableFusion;
 extern bool mi355xDisableMarkConstant;
 extern bool mi355xDisableKeepOnDevice;
+extern bool mi355xFuseGelu;
 extern std::string mi355xOps;
 
 } // namespace onnx_mlir

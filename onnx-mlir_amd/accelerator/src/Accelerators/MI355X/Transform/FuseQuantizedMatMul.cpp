@@ -12,7 +12,7 @@
 //   %s             = Mul(%as, %ws)
 //   %y             = Mul(%f, %s)
 //   %z             = Add(%y, %bias)          (optional)
-//   %r             = Relu(%z)                (optional)
+//   %r             = Relu(%z) or Gelu(%z)    (optional)
 //
 // On the CPU that is five or six ops and as many intermediate tensors.  The
 // MI355X runtime has one entry point for everything after the quantisation
@@ -22,7 +22,10 @@
 // rounds the product to f32 and then adds, as Mul followed by Add does.  A Relu
 // that is the only user of that result goes along too, as the integer
 // attribute `activation` = 1 (max(0, x) is exact, so where it is applied does
-// not change a bit of the result).  This pass replaces the chain by an
+// not change a bit of the result).  With --mi355x-fuse-gelu an onnx.Gelu with
+// approximate = "none" in that place goes along as `activation` = 2; that is
+// not the default because the runtime's erf and the polynomial the CPU code
+// evaluates differ in the last bits.  This pass replaces the chain by an
 // `onnx.Custom` naming that entry point; the ONNX-to-Krnl patterns of the
 // accelerator lower it.
 //
@@ -39,6 +42,7 @@
 #include "mlir/Pass/Pass.h"
 #include "mlir/Transforms/GreedyPatternRewriteDriver.h"
 
+#include "src/Accelerators/MI355X/Compiler/MI355XCompilerOptions.hpp"
 #include "src/Accelerators/MI355X/Transform/MI355XPasses.hpp"
 #include "src/Dialect/ONNX/ONNXOps.hpp"
 #include "src/Dialect/ONNX/ONNXOps/OpHelper.hpp"
@@ -170,6 +174,14 @@ struct FuseScaledMatMulInteger : public OpRewritePattern<ONNXMulOp> {
         if (relu.getResult().getType() == root->getResult(0).getType()) {
           root = relu;
           activation = 1;
+        }
+      } else if (auto gelu = dyn_cast<ONNXGeluOp>(*root->user_begin())) {
+        // Only on request: the entry point evaluates erf with the device
+        // library, the CPU code with a polynomial, so the last bits differ.
+        if (mi355xFuseGelu && gelu.getApproximate().equals_insensitive("none") &&
+            gelu.getResult().getType() == root->getResult(0).getType()) {
+          root = gelu;
+          activation = 2;
         }
       }
     }

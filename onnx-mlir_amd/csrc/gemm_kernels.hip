@@ -1788,6 +1788,59 @@ bool gemm_quantizes_rows(int64_t M, int64_t K, const void *x) {
 
 const char *last_gemm_kernel() { return t_last_kernel; }
 
+// onnx.Gelu with approximate = "none" as the reference lowers it
+// (src/Conversion/ONNXToKrnl/Math/Elementwise.cpp:374-388): (0.5 * x) *
+// (1 + erf(x * f32(1 / sqrt 2))), every operation rounded to f32, in this
+// order.  The reference evaluates erf by a polynomial approximation of the
+// compiler it is built with (src/Conversion/KrnlToLLVM/ConvertKrnlToLLVM.cpp:
+// 223-225), this kernel by the device library's erff: the two agree to a few
+// units in the last place of erf, not bit for bit.
+namespace {
+__device__ __forceinline__ float gelu_f32(float x) {
+  const float half_x = 0.5f * x;
+  const float e = erff(x * 0.70710678118654752440f);
+  return half_x * (1.0f + e);
+}
+// In place over n floats; y 16-byte aligned or not (the edges go one by one).
+__global__ __launch_bounds__(256) void k_gelu_inplace(float *__restrict__ y,
+    int64_t n) {
+  typedef float f4 __attribute__((ext_vector_type(4)));
+  const int64_t head = (4 - (int64_t)((((uintptr_t)y) >> 2) & 3)) & 3; // floats before the first aligned vector
+  const int64_t lead = head < n ? head : n;
+  f4 *const y4 = (f4 *)(y + lead);
+  const int64_t nvec = (n - lead) >> 2;
+  const int64_t base = (int64_t)blockIdx.x * 512 + threadIdx.x;
+  f4 v[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int64_t i = base + j * 256;
+    const f4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+    v[j] = i < nvec ? y4[i] : zero;
+  }
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int64_t i = base + j * 256;
+    if (i < nvec) {
+      f4 o;
+      o.x = gelu_f32(v[j].x);
+      o.y = gelu_f32(v[j].y);
+      o.z = gelu_f32(v[j].z);
+      o.w = gelu_f32(v[j].w);
+      y4[i] = o;
+    }
+  }
+  if (blockIdx.x == 0) {
+    // up to three floats before the first vector and after the last one
+    const int64_t t = threadIdx.x;
+    if (t < lead)
+      y[t] = gelu_f32(y[t]);
+    const int64_t tail = lead + (nvec << 2) + t;
+    if (t < 4 && tail < n)
+      y[tail] = gelu_f32(y[tail]);
+  }
+}
+} // namespace
+
 hipError_t launch_gemm(hipStream_t s, const GemmArgs &g) {
   if (g.M == 0 || g.N == 0)
     return hipSuccess;
@@ -1815,14 +1868,27 @@ hipError_t launch_gemm(hipStream_t s, const GemmArgs &g) {
   ep.y_unsigned = g.y_unsigned;
   ep.narrow = (int)g.narrow;
   const int a_mode = (g.X || g.a_preshifted) ? 2 : (g.a_unsigned ? 1 : 0);
+  hipError_t e;
   switch (a_mode) {
   case 0:
-    return gemm_launch_epi<0>(s, g, ep, Kpad);
+    e = gemm_launch_epi<0>(s, g, ep, Kpad);
+    break;
   case 1:
-    return gemm_launch_epi<1>(s, g, ep, Kpad);
+    e = gemm_launch_epi<1>(s, g, ep, Kpad);
+    break;
   default:
-    return gemm_launch_epi<2>(s, g, ep, Kpad);
+    e = gemm_launch_epi<2>(s, g, ep, Kpad);
+    break;
   }
+  if (e == hipSuccess && g.epi == kEpiF32 && g.gelu) {
+    // onnx.Gelu on the result, as a pass of its own over the f32 output
+    const int64_t n = g.M * g.N;
+    const int64_t per_block = 256 * 2 * 4;
+    k_gelu_inplace<<<(unsigned)((n + per_block - 1) / per_block), 256, 0, s>>>(
+        (float *)g.out, n);
+    e = hipGetLastError();
+  }
+  return e;
 }
 
 

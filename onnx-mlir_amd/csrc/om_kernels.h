@@ -104,6 +104,9 @@ struct GemmArgs {
   // kEpiF32 only: onnx.Relu on the result, max(0, x) with a NaN giving 0
   // (src/Conversion/ONNXToKrnl/Math/Elementwise.cpp:746-754).
   bool relu;
+  // kEpiF32 only: onnx.Gelu (approximate = "none") on the result instead,
+  // applied by a pass of its own after the product.
+  bool gelu;
   bool y_unsigned;
   NarrowMode narrow;
   void *out;           // i32 / f32 / u8|i8 [M,N]

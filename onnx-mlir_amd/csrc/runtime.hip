@@ -1229,16 +1229,19 @@ struct MatmulSpec {
                  *y_zp = nullptr, *bias = nullptr;
   NarrowMode narrow = kWrap;
   bool relu = false; // kEpiF32: onnx.Relu on the result
+  bool gelu = false; // kEpiF32: onnx.Gelu (approximate "none") on the result
 };
 
-// The `activation` argument of the fused entry points: 0 = none, 1 = Relu.
-bool activation_ok(int64_t activation, const char *op, bool &relu) {
-  if (activation != 0 && activation != 1) {
-    fail(EINVAL, "%s: activation %lld is not 0 (none) or 1 (Relu)", op,
+// The `activation` argument of the fused entry points: 0 = none, 1 = Relu,
+// 2 = Gelu.
+bool activation_ok(int64_t activation, const char *op, bool &relu, bool &gelu) {
+  if (activation < 0 || activation > 2) {
+    fail(EINVAL, "%s: activation %lld is not 0 (none), 1 (Relu) or 2 (Gelu)", op,
         (long long)activation);
     return false;
   }
   relu = activation == 1;
+  gelu = activation == 2;
   return true;
 }
 
@@ -1378,6 +1381,7 @@ void run_matmul(const MatmulSpec &sp) {
     g.bias_len = bias.numel;
   }
   g.relu = sp.relu;
+  g.gelu = sp.gelu;
   if (sp.epi == kEpiQ8) {
     g.y_scale = (const float *)call.in(ys);
     g.y_zp = call.in(yzp);
@@ -1681,7 +1685,7 @@ void om_mi355x_MatMulIntegerDequant(OMTensor *y, const OMTensor *a,
     const OMTensor *a_scale, const OMTensor *b_scale, const OMTensor *bias,
     int64_t activation) {
   MatmulSpec sp = {"MatMulIntegerDequant", kEpiF32, y, a, b, a_zp, b_zp};
-  if (!activation_ok(activation, sp.op, sp.relu))
+  if (!activation_ok(activation, sp.op, sp.relu, sp.gelu))
     return;
   sp.a_scale = a_scale;
   sp.b_scale = b_scale;
@@ -1711,8 +1715,8 @@ void om_mi355x_DynQuantMatMulDequant(OMTensor *y_t, const OMTensor *x_t,
     const OMTensor *bias_t, int64_t activation) {
   const char *op = "DynQuantMatMulDequant";
   View y, x, b, bzp, bs, bias;
-  bool relu;
-  if (!activation_ok(activation, op, relu))
+  bool relu, gelu;
+  if (!activation_ok(activation, op, relu, gelu))
     return;
   if (!view_of(y_t, "y", y) || !view_of(x_t, "x", x) ||
       !view_of(b_t, "b", b) || !view_of(bscale_t, "b_scale", bs))
@@ -1793,6 +1797,7 @@ void om_mi355x_DynQuantMatMulDequant(OMTensor *y_t, const OMTensor *x_t,
     g.bias_len = bias.numel;
   }
   g.relu = relu;
+  g.gelu = gelu;
   if (call.ok)
     call.check(launch_gemm(call.c.stream, g), op);
   call.finish();

@@ -39,7 +39,7 @@ _NP_TO_ONNX = {
 
 WRAP, SATURATE = 0, 1
 # `activation` of the fused entry points (OM_MI355X_ACTIVATION_* of the header)
-ACTIVATION_NONE, ACTIVATION_RELU = 0, 1
+ACTIVATION_NONE, ACTIVATION_RELU, ACTIVATION_GELU = 0, 1, 2
 # OM_MI355X_VERSION of the header this module was written against
 VERSION = 0x00010000
 

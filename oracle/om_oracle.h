@@ -21,6 +21,11 @@
  *   lowering asserts on per-axis scales, so there is no reference output; the
  *   per-tensor formula is applied with scale[c], zp[c] and checked against the
  *   ONNX operator specification's per-axis node vectors only.
+ *   gelu: "parity unpinned" at the bit level -- the reference expands erf
+ *   with a polynomial approximation pass of the compiler it is built on, not
+ *   held in its tree, and stores no Gelu outputs; libm's erff stands in, and
+ *   comparisons with this function carry a tolerance of a few units in the
+ *   last place of erf.
  */
 #ifndef OM_ORACLE_H
 #define OM_ORACLE_H
@@ -97,6 +102,9 @@ void om_oracle_dequant_epilogue(const int32_t *acc, int64_t M, int64_t N,
 
 /* out[i] = max(0, x[i]); NaN -> 0. */
 void om_oracle_relu(const float *x, int64_t n, float *out);
+
+/* out[i] = (0.5 * x[i]) * (1 + erf(x[i] * f32(1 / sqrt 2))), erf by libm. */
+void om_oracle_gelu(const float *x, int64_t n, float *out);
 
 /* The reference's pass structure for Q / DQ / DQL with OpenMP, used only as
  * the timed CPU baseline (results identical to the functions above). */

@@ -57,6 +57,8 @@ class Oracle:
         lib.om_oracle_dequant_epilogue.argtypes = [P, I64, I64, F, P, I64, P]
         lib.om_oracle_relu.restype = None
         lib.om_oracle_relu.argtypes = [P, I64, P]
+        lib.om_oracle_gelu.restype = None
+        lib.om_oracle_gelu.argtypes = [P, I64, P]
         lib.om_oracle_num_threads.restype = I
 
     # -- helpers ----------------------------------------------------------
@@ -199,6 +201,12 @@ class Oracle:
         x = np.ascontiguousarray(x, np.float32)
         out = np.empty(x.shape, np.float32)
         self.lib.om_oracle_relu(_p(x), x.size, _p(out))
+        return out
+
+    def gelu(self, x):
+        x = np.ascontiguousarray(x, np.float32)
+        out = np.empty(x.shape, np.float32)
+        self.lib.om_oracle_gelu(_p(x), x.size, _p(out))
         return out
 
     def num_threads(self):

@@ -1012,9 +1012,75 @@ def test_fused_relu_epilogue(rt, oracle):
     got = rt.MatMulIntegerDequant(A, B, azm, bzn, np.float32(0.1), np.float32(0.2), activation=1)
     assert same_f32(got, oracle.relu(plain))
     with pytest.raises(rt.RuntimeError_, match="activation"):
-        rt.MatMulIntegerDequant(A, B, azm, bzn, np.float32(0.1), np.float32(0.2), activation=2)
+        rt.MatMulIntegerDequant(A, B, azm, bzn, np.float32(0.1), np.float32(0.2), activation=3)
     with pytest.raises(rt.RuntimeError_, match="activation"):
         rt.DynQuantMatMulDequant(np.zeros((4, 96), np.float32), B, None, np.float32(0.2), activation=-1)
+
+
+def test_fused_gelu_epilogue(rt, oracle):
+    """`activation` = Gelu on the two fused entry points against the oracle's
+    Gelu of the call's own result without it (that result is bit-exact, see the
+    tests above).  PARITY UNPINNED at the bit level: the reference's erf is a
+    polynomial approximation its compiler expands, the oracle's is libm's and
+    the kernel's the device library's, so the comparison carries a tolerance:
+    4 units in the last place of erf (2^-22, erf lies in [-1, 1]) times
+    |0.5 x|, the factor the sum 1 + erf is multiplied by, plus one rounding of
+    the result.  Shapes as for Relu, so every GEMM kernel is followed by the
+    activation once; values from deep in the negative tail (where 1 + erf
+    cancels) to large positive ones, NaN and infinities through the bias."""
+    rng = np.random.default_rng(53)
+
+    def check(got, plain, what):
+        want = oracle.gelu(plain)
+        p64 = plain.astype(np.float64)
+        tol = np.abs(0.5 * p64) * 2.0 ** -22 + np.abs(want.astype(np.float64)) * 2.0 ** -23 + 1e-45
+        fin = np.isfinite(want)
+        assert np.array_equal(np.isnan(got), np.isnan(want)), what
+        assert np.array_equal(got[~fin & ~np.isnan(want)], want[~fin & ~np.isnan(want)]), what
+        err = np.abs(got[fin].astype(np.float64) - want[fin].astype(np.float64))
+        assert (err <= tol[fin]).all(), (what, float(err.max()))
+        # and against the definition in binary64
+        from math import erf
+        ref = np.array([0.5 * v * (1.0 + erf(v / np.sqrt(2.0))) for v in p64[fin].ravel()[:4096]])
+        assert np.allclose(got[fin].ravel()[:4096], ref, rtol=1e-5, atol=1e-6), what
+
+    for M, K, N in ((512, 768, 3072), (300, 768, 1000), (256, 1024, 512), (130, 200, 70), (4, 4096, 256), (7, 100, 33)):
+        A, B = _rand_q(rng, np.uint8, (M, K)), _rand_q(rng, np.int8, (K, N))
+        az = _rand_q(rng, np.uint8, ())
+        # products spread over about [-6, 6]: both tails and the middle of erf
+        a_s = np.float32(6.0 / (40.0 * 74.0 * np.sqrt(K)))
+        bs = rng.uniform(0.5, 1.0, N).astype(np.float32)
+        bias = rng.standard_normal(N).astype(np.float32)
+        bias[N // 2] = np.nan
+        bias[N // 3] = np.inf
+        bias[N // 4] = -np.inf
+        for b in (None, bias):
+            plain = rt.MatMulIntegerDequant(A, B, az, None, a_s, bs, b)
+            got = rt.MatMulIntegerDequant(A, B, az, None, a_s, bs, b, activation=rt.ACTIVATION_GELU)
+            check(got, plain, (M, K, N, b is None))
+            assert (plain < -3).any() and (plain > 3).any() and (np.abs(plain) < 0.5).any()
+        x = rng.standard_normal((M, K)).astype(np.float32)
+        xs = np.float32(6.0 / (0.33 * 74.0 * np.sqrt(K)))
+        plain = rt.DynQuantMatMulDequant(x, B, None, bs * xs, bias)
+        got = rt.DynQuantMatMulDequant(x, B, None, bs * xs, bias, activation=rt.ACTIVATION_GELU)
+        check(got, plain, ("dyn", M, K, N))
+    # an output the caller placed off the 16-byte grid, and batches
+    A, B = _rand_q(rng, np.uint8, (3, 37, 64)), _rand_q(rng, np.int8, (64, 23))
+    plain = rt.MatMulIntegerDequant(A, B, None, None, np.float32(0.002), np.float32(0.01))
+    got = rt.MatMulIntegerDequant(A, B, None, None, np.float32(0.002), np.float32(0.01), activation=2)
+    check(got, plain, "batched")
+    # results placed 4 and 12 bytes off the 16-byte grid, with guards either side
+    A, B = _rand_q(rng, np.uint8, (37, 64)), _rand_q(rng, np.int8, (64, 23))
+    plain = rt.MatMulIntegerDequant(A, B, None, None, np.float32(0.002), np.float32(0.01))
+    for off in (1, 3):
+        buf = rt.DeviceArray.from_numpy(np.full(37 * 23 + 8, -7.0, np.float32))
+        rt.MatMulIntegerDequant(A, B, None, None, np.float32(0.002), np.float32(0.01),
+                                out=rt.DeviceArray.view_of(buf, off, (37, 23)), activation=2)
+        rt.synchronize()
+        whole = buf.numpy()
+        assert (whole[:off] == -7.0).all() and (whole[off + 37 * 23:] == -7.0).all()
+        check(whole[off:off + 37 * 23].reshape(37, 23), plain, ("offset", off))
+        buf.free()
 
 
 def test_matmulinteger_batched_b(rt, oracle):

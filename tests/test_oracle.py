@@ -367,6 +367,27 @@ def test_relu_equals_numpy_fmax(oracle):
     assert not np.signbit(got[5]) and got[6] == np.float32(1e-45)
 
 
+def test_gelu_is_the_erf_formula(oracle):
+    """Gelu (approximate "none") against 0.5 x (1 + erf(x / sqrt 2)) evaluated
+    in binary64: pins the formula (a dropped 0.5, sqrt 2 for 1 / sqrt 2 or erf
+    for 1 + erf is off by far more than the bound), not the last bits, which
+    depend on whose erf is used.  Bound: one unit in the last place of erf
+    times |0.5 x|, plus the roundings of the products."""
+    from math import erf, sqrt
+    rng = np.random.default_rng(93)
+    x = np.concatenate([rng.standard_normal(20000) * 3, np.linspace(-9, 9, 2001),
+                        [0.0, -0.0, 1e-30, -1e-30, 40.0, -40.0]]).astype(np.float32)
+    got = oracle.gelu(x).astype(np.float64)
+    x64 = x.astype(np.float64)
+    want = np.array([0.5 * v * (1.0 + erf(v / sqrt(2.0))) for v in x64])
+    tol = np.abs(0.5 * x64) * 2.0 ** -23 + np.abs(want) * 2.0 ** -22 + 1e-45
+    assert (np.abs(got - want) <= tol).all()
+    assert got[-2] == 40.0 and got[-1] == 0.0
+    special = oracle.gelu(np.array([np.inf, -np.inf, np.nan], np.float32))
+    # 0.5 * -inf * (1 + -1) = -inf * 0 is a NaN, as the formula gives it
+    assert special[0] == np.inf and np.isnan(special[1]) and np.isnan(special[2])
+
+
 def test_four_instruction_quotient_equals_the_divide(tmp_path):
     """The quantize kernels divide by a scale of ordinary magnitude with a
     reciprocal multiply and one exact correction step.  tests/quotient_check.c
