@@ -194,7 +194,7 @@ def decode_case(rt, wl, M, steps, warmup):
     dS = rt.DeviceArray.from_numpy(c["w_scale"])
     dY = rt.DeviceArray((M, N), np.float32)
     rt.mark_constant(dW)
-    fn = rt.PreparedCall("om_mi355x_DynQuantMatMulDequant", dY, dX, dW, None, dS, None, activation)
+    fn = rt.PreparedCall("om_mi355x_DynQuantMatMulDequant", dY, dX, dW, None, dS, None, 0)
     res = measure(rt, fn, steps, warmup)
     fn.check()
     fn.close()
@@ -584,6 +584,9 @@ def main():
                 cc = wl.config4(name, M=8)
                 fused.append(fused_case(rt, wl, f"config4 {name} fused layer", 4096, k, n, cc["W"],
                                         cc["w_scale"], esteps, ewarm))
+                if name == "ffn_up":   # the projection an activation function follows
+                    fused.append(fused_case(rt, wl, f"config4 {name} fused layer, Gelu", 4096, k, n, cc["W"],
+                                            cc["w_scale"], esteps, ewarm, activation=2))
         extras["fused"] = fused
     if "gemm" in groups:
         gemms = []

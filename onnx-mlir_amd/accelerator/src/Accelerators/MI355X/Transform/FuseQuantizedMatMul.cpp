@@ -176,8 +176,8 @@ struct FuseScaledMatMulInteger : public OpRewritePattern<ONNXMulOp> {
           activation = 1;
         }
       } else if (auto gelu = dyn_cast<ONNXGeluOp>(*root->user_begin())) {
-        // Only on request: the entry point evaluates erf with the device
-        // library, the CPU code with a polynomial, so the last bits differ.
+        // Only on request: the entry point and the CPU code evaluate erf by
+        // different approximations, so the last bits differ.
         if (mi355xFuseGelu && gelu.getApproximate().equals_insensitive("none") &&
             gelu.getResult().getType() == root->getResult(0).getType()) {
           root = gelu;

@@ -93,6 +93,42 @@ inline float relu_floor(bool relu) {
   return relu ? 0.0f : __builtin_nanf("");
 }
 
+// onnx.Gelu with approximate = "none" as the reference lowers it
+// (src/Conversion/ONNXToKrnl/Math/Elementwise.cpp:374-388): (0.5 * x) *
+// (1 + erf(x * f32(1 / sqrt 2))), every operation rounded to f32, in this
+// order.  The reference's erf is a polynomial approximation that the compiler
+// it is built on expands (src/Conversion/KrnlToLLVM/ConvertKrnlToLLVM.cpp:
+// 223-225), so no erf reproduces its last bits; this one is
+//   erf(m) = sign(m) * (1 - 2^(t * p(t))),  t = min(|m|, 3.925),
+// with p of degree 7 fitted (minimax in the error of erf) to log2(erfc(t)) / t
+// on [0, 3.925] and the hardware's base-2 exponential: eight multiply-adds, an
+// exponential and a subtraction.  Past 3.925, erf rounds to 1 in f32.  Error of
+// erf: below 1.5e-7 absolute (0.63 * 2^-22) over the whole line with every
+// rounding at its worst, the exponential's one unit in the last place
+// included; Gelu needs it absolute, not relative, because the sum 1 + erf is
+// what gets multiplied.  Every kernel that applies Gelu calls this function,
+// so the result does not depend on which kernel a shape takes.  A NaN gives a
+// NaN (through 0.5 * x), +inf gives +inf and -inf gives -inf * 0 = NaN, as the
+// formula does.
+__device__ __forceinline__ float gelu_erf_f32(float m) {
+  const float t = __builtin_fminf(__builtin_fabsf(m), 3.925f);
+  float p = -0x1.740ee2p-15f;
+  p = __builtin_fmaf(p, t, 0x1.ca2b3ap-12f);
+  p = __builtin_fmaf(p, t, -0x1.7ed47ep-10f);
+  p = __builtin_fmaf(p, t, -0x1.b09ff2p-11f);
+  p = __builtin_fmaf(p, t, 0x1.cfb2b8p-6f);
+  p = __builtin_fmaf(p, t, -0x1.302440p-3f);
+  p = __builtin_fmaf(p, t, -0x1.d639d0p-1f);
+  p = __builtin_fmaf(p, t, -0x1.a0beaap+0f);
+  const float e = __builtin_amdgcn_exp2f(p * t);
+  return __builtin_copysignf(1.0f - e, m);
+}
+__device__ __forceinline__ float gelu_f32(float x) {
+  const float half_x = 0.5f * x;
+  const float e = gelu_erf_f32(x * 0.70710678118654752440f);
+  return half_x * (1.0f + e);
+}
+
 __device__ __forceinline__ int32_t load_zp_i32(
     const void *p, bool is_unsigned, int64_t i) {
   return is_unsigned ? (int32_t)((const uint8_t *)p)[i]

@@ -1593,6 +1593,9 @@ bool gemm_fast_path(int64_t M, int64_t K, const void *A) {
 // Name of the kernel the calling thread's last launch_gemm chose (for tests
 // and reports).
 thread_local const char *t_last_kernel = "";
+// Whether that kernel applied the onnx.Gelu asked for to its results itself
+// (launch_gemm runs the pass over the output when it did not).
+thread_local bool t_gelu_applied = false;
 
 template <int A_MODE, int EPI>
 hipError_t gemm_launch_cfg(
@@ -1661,6 +1664,7 @@ hipError_t gemm_launch_cfg(
   const bool forced = force && force[0];
   if (wreg_ok(g) && (cfg == kW128x384 || (!forced && wreg_pays(g.M, g.N)))) {
     t_last_kernel = "k_gemm_i8_wreg (weights in registers, 128x384 blocks)";
+    t_gelu_applied = g.epi == kEpiF32 && g.gelu; // this kernel applies it to its results
     return launch_gemm_wreg(st, g, ep, A_MODE);
   }
   switch (cfg) {
@@ -1788,20 +1792,10 @@ bool gemm_quantizes_rows(int64_t M, int64_t K, const void *x) {
 
 const char *last_gemm_kernel() { return t_last_kernel; }
 
-// onnx.Gelu with approximate = "none" as the reference lowers it
-// (src/Conversion/ONNXToKrnl/Math/Elementwise.cpp:374-388): (0.5 * x) *
-// (1 + erf(x * f32(1 / sqrt 2))), every operation rounded to f32, in this
-// order.  The reference evaluates erf by a polynomial approximation of the
-// compiler it is built with (src/Conversion/KrnlToLLVM/ConvertKrnlToLLVM.cpp:
-// 223-225), this kernel by the device library's erff: the two agree to a few
-// units in the last place of erf, not bit for bit.
 namespace {
-__device__ __forceinline__ float gelu_f32(float x) {
-  const float half_x = 0.5f * x;
-  const float e = erff(x * 0.70710678118654752440f);
-  return half_x * (1.0f + e);
-}
-// In place over n floats; y 16-byte aligned or not (the edges go one by one).
+// onnx.Gelu (gelu_f32) in place over n floats, for the kernels that do not
+// apply it to their results themselves; y 16-byte aligned or not (the edges
+// go one by one).
 __global__ __launch_bounds__(256) void k_gelu_inplace(float *__restrict__ y,
     int64_t n) {
   typedef float f4 __attribute__((ext_vector_type(4)));
@@ -1868,6 +1862,7 @@ hipError_t launch_gemm(hipStream_t s, const GemmArgs &g) {
   ep.y_unsigned = g.y_unsigned;
   ep.narrow = (int)g.narrow;
   const int a_mode = (g.X || g.a_preshifted) ? 2 : (g.a_unsigned ? 1 : 0);
+  t_gelu_applied = false;
   hipError_t e;
   switch (a_mode) {
   case 0:
@@ -1880,7 +1875,7 @@ hipError_t launch_gemm(hipStream_t s, const GemmArgs &g) {
     e = gemm_launch_epi<2>(s, g, ep, Kpad);
     break;
   }
-  if (e == hipSuccess && g.epi == kEpiF32 && g.gelu) {
+  if (e == hipSuccess && g.epi == kEpiF32 && g.gelu && !t_gelu_applied) {
     // onnx.Gelu on the result, as a pass of its own over the f32 output
     const int64_t n = g.M * g.N;
     const int64_t per_block = 256 * 2 * 4;

@@ -81,7 +81,7 @@ constexpr int wreg_younger(int s, int pf, int fix_ops, int fix_read, int fix_wri
   return x;
 }
 
-template <int KH, int WAVES, int NR, int A_MODE, int EPI, bool STREAM, bool RELU>
+template <int KH, int WAVES, int NR, int A_MODE, int EPI, bool STREAM, int ACT>
 __global__ __launch_bounds__(WAVES * 64, 1) void k_gemm_i8_wreg(
     const uint8_t *__restrict__ A, const int8_t *__restrict__ Bp, int M, int N,
     EpiParams ep, int regions_m, int regions_n, int bp_tiles) {
@@ -329,8 +329,11 @@ __global__ __launch_bounds__(WAVES * 64, 1) void k_gemm_i8_wreg(
       __builtin_amdgcn_raw_buffer_store_b32((int)y, out_rsrc, (int)toff, soff, kAux);
     } else if (EPI == kEpiF32) {
       float f = (float)(int32_t)y * sj + bj;
-      if (RELU) // compiled in only where asked for: the loop has no slot to spare
+      // compiled in only where asked for: the loop has no slot to spare
+      if (ACT == 1)
         f = relu_f32(f, 0.0f);
+      else if (ACT == 2)
+        f = gelu_f32(f);
       __builtin_amdgcn_raw_buffer_store_b32(
           (int)__float_as_uint(f), out_rsrc, (int)toff, soff, kAux);
     } else {
@@ -452,14 +455,15 @@ __global__ __launch_bounds__(WAVES * 64, 1) void k_gemm_i8_wreg(
 // Shapes the kernel is built for.
 constexpr int kWregKH = 24, kWregWaves = 12, kWregNR = 4;
 
-template <int A_MODE, int EPI, bool RELU = false>
+// ACT: 0 = none, 1 = Relu, 2 = Gelu on the f32 result
+template <int A_MODE, int EPI, int ACT = 0>
 hipError_t wreg_launch(hipStream_t st, const GemmArgs &g, const EpiParams &ep) {
   const int M = (int)g.M, N = (int)g.N;
   const int regions_m = (int)((g.M + 32 * kWregNR - 1) / (32 * kWregNR));
   const int ntiles = (int)((g.N + 31) / 32);
   const int regions_n = (ntiles + kWregWaves - 1) / kWregWaves;
   const int bp_tiles = (int)(round_up(g.N, kGemmBN) / 32);
-  k_gemm_i8_wreg<kWregKH, kWregWaves, kWregNR, A_MODE, EPI, true, RELU>
+  k_gemm_i8_wreg<kWregKH, kWregWaves, kWregNR, A_MODE, EPI, true, ACT>
       <<<dim3((unsigned)(regions_m * regions_n)), dim3(kWregWaves * 64), 0, st>>>(
           (const uint8_t *)g.A, g.Bp, M, N, ep, regions_m, regions_n, bp_tiles);
   return hipGetLastError();
@@ -497,20 +501,32 @@ hipError_t launch_gemm_wreg(hipStream_t st, const GemmArgs &g,
   return a_mode == 1 ? wreg_launch<1, kEpiF32>(st, g, ep) : hipErrorInvalidValue;
 #else
   const bool f32 = g.epi == kEpiF32;
-  const bool relu = f32 && g.relu;
-  switch (a_mode) {
+  const int act = !f32 ? 0 : g.relu ? 1 : g.gelu ? 2 : 0;
+  switch (a_mode * 4 + (f32 ? act : 3)) {
   case 0:
-    return relu  ? wreg_launch<0, kEpiF32, true>(st, g, ep)
-           : f32 ? wreg_launch<0, kEpiF32>(st, g, ep)
-                 : wreg_launch<0, kEpiI32>(st, g, ep);
+    return wreg_launch<0, kEpiF32>(st, g, ep);
   case 1:
-    return relu  ? wreg_launch<1, kEpiF32, true>(st, g, ep)
-           : f32 ? wreg_launch<1, kEpiF32>(st, g, ep)
-                 : wreg_launch<1, kEpiI32>(st, g, ep);
+    return wreg_launch<0, kEpiF32, 1>(st, g, ep);
   case 2:
-    return relu  ? wreg_launch<2, kEpiF32, true>(st, g, ep)
-           : f32 ? wreg_launch<2, kEpiF32>(st, g, ep)
-                 : wreg_launch<2, kEpiI32>(st, g, ep);
+    return wreg_launch<0, kEpiF32, 2>(st, g, ep);
+  case 3:
+    return wreg_launch<0, kEpiI32>(st, g, ep);
+  case 4:
+    return wreg_launch<1, kEpiF32>(st, g, ep);
+  case 5:
+    return wreg_launch<1, kEpiF32, 1>(st, g, ep);
+  case 6:
+    return wreg_launch<1, kEpiF32, 2>(st, g, ep);
+  case 7:
+    return wreg_launch<1, kEpiI32>(st, g, ep);
+  case 8:
+    return wreg_launch<2, kEpiF32>(st, g, ep);
+  case 9:
+    return wreg_launch<2, kEpiF32, 1>(st, g, ep);
+  case 10:
+    return wreg_launch<2, kEpiF32, 2>(st, g, ep);
+  case 11:
+    return wreg_launch<2, kEpiI32>(st, g, ep);
   default:
     return hipErrorInvalidValue;
   }

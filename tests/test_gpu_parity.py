@@ -973,7 +973,7 @@ def test_matmulinteger_batched_a(rt, oracle):
     assert got.shape == (3, 5, 24) and np.array_equal(got, oracle.matmul_integer(A, B, az, None))
 
 
-def test_fused_relu_epilogue(rt, oracle):
+def test_fused_relu_epilogue(rt, oracle, monkeypatch):
     """`activation` = Relu on the two fused entry points equals onnx.Relu applied
     to the call's own result without it (max(0, x) is exact), over the kernels a
     shape can take: the weights-in-registers kernel (K = 768), the LDS-staged
@@ -1005,6 +1005,19 @@ def test_fused_relu_epilogue(rt, oracle):
         plain = rt.DynQuantMatMulDequant(x, B, None, bs, bias)
         got = rt.DynQuantMatMulDequant(x, B, None, bs, bias, activation=rt.ACTIVATION_RELU)
         assert same_f32(got, oracle.relu(plain)), (M, K, N)
+    # the weights-in-registers kernel by choice (enough rows to fill the device)
+    # and by force, on a ragged row count
+    for M, force in ((4096, None), (300, "4")):
+        A, B = _rand_q(rng, np.uint8, (M, 768)), _rand_q(rng, np.int8, (768, 3072))
+        bs = rng.uniform(1e-3, 1e-2, 3072).astype(np.float32)
+        if force:
+            monkeypatch.setenv("OM_MI355X_GEMM_TILE", force)
+        plain = rt.MatMulIntegerDequant(A, B, None, None, np.float32(0.013), bs)
+        got = rt.MatMulIntegerDequant(A, B, None, None, np.float32(0.013), bs, activation=rt.ACTIVATION_RELU)
+        assert "wreg" in rt.last_gemm_kernel()
+        if force:
+            monkeypatch.delenv("OM_MI355X_GEMM_TILE")
+        assert same_f32(got, oracle.relu(plain)) and (got == 0).any() and (got > 0).any()
     # per-row zero points take the epilogue's other branch
     A, B = _rand_q(rng, np.int8, (70, 96)), _rand_q(rng, np.uint8, (96, 40))
     azm, bzn = _rand_q(rng, np.int8, (70,)), _rand_q(rng, np.uint8, (40,))
@@ -1017,12 +1030,12 @@ def test_fused_relu_epilogue(rt, oracle):
         rt.DynQuantMatMulDequant(np.zeros((4, 96), np.float32), B, None, np.float32(0.2), activation=-1)
 
 
-def test_fused_gelu_epilogue(rt, oracle):
+def test_fused_gelu_epilogue(rt, oracle, monkeypatch):
     """`activation` = Gelu on the two fused entry points against the oracle's
     Gelu of the call's own result without it (that result is bit-exact, see the
     tests above).  PARITY UNPINNED at the bit level: the reference's erf is a
     polynomial approximation its compiler expands, the oracle's is libm's and
-    the kernel's the device library's, so the comparison carries a tolerance:
+    the kernel's an approximation of its own, so the comparison carries a tolerance:
     4 units in the last place of erf (2^-22, erf lies in [-1, 1]) times
     |0.5 x|, the factor the sum 1 + erf is multiplied by, plus one rounding of
     the result.  Shapes as for Relu, so every GEMM kernel is followed by the
@@ -1064,6 +1077,34 @@ def test_fused_gelu_epilogue(rt, oracle):
         plain = rt.DynQuantMatMulDequant(x, B, None, bs * xs, bias)
         got = rt.DynQuantMatMulDequant(x, B, None, bs * xs, bias, activation=rt.ACTIVATION_GELU)
         check(got, plain, ("dyn", M, K, N))
+    # The weights-in-registers kernel applies Gelu to its results itself, the
+    # other kernels leave it to a pass over the output: one function, so the
+    # same bits whichever kernel a shape takes.
+    A, B = _rand_q(rng, np.uint8, (512, 768)), _rand_q(rng, np.int8, (768, 3072))
+    a_s, bs = np.float32(6.0 / (40.0 * 74.0 * np.sqrt(768))), rng.uniform(0.5, 1.0, 3072).astype(np.float32)
+    monkeypatch.setenv("OM_MI355X_GEMM_TILE", "4")
+    own = rt.MatMulIntegerDequant(A, B, None, None, a_s, bs, activation=2)
+    assert "wreg" in rt.last_gemm_kernel()
+    x = rng.standard_normal((512, 768)).astype(np.float32)
+    xs = bs * np.float32(6.0 / (0.33 * 74.0 * np.sqrt(768)))
+    layer = rt.DynQuantMatMulDequant(x, B, None, xs, None, activation=2)
+    assert "wreg" in rt.last_gemm_kernel()
+    check(layer, rt.DynQuantMatMulDequant(x, B, None, xs, None), "whole layer, weights in registers")
+    monkeypatch.setenv("OM_MI355X_GEMM_TILE", "1")
+    by_pass = rt.MatMulIntegerDequant(A, B, None, None, a_s, bs, activation=2)
+    assert "wreg" not in rt.last_gemm_kernel()
+    monkeypatch.delenv("OM_MI355X_GEMM_TILE")
+    assert same_f32(own, by_pass)
+    # the erf inside, recovered where the division is harmless, against binary64:
+    # the bound the header states (2^-22), over the 1.5 million results
+    plain = rt.MatMulIntegerDequant(A, B, None, None, a_s, bs).astype(np.float64)
+    sel = np.abs(plain) > 0.25
+    from scipy.special import erf as erf64
+    erf_got = own.astype(np.float64)[sel] / (0.5 * plain[sel]) - 1.0
+    m = (plain[sel].astype(np.float32) * np.float32(0.70710678118654752440)).astype(np.float64)
+    # (the final product's rounding, half a unit of the result, divided back)
+    slack = np.abs(own.astype(np.float64)[sel]) * 2.0 ** -24 / np.abs(0.5 * plain[sel])
+    assert (np.abs(erf_got - erf64(m)) <= 2.0 ** -22 + slack).all()
     # an output the caller placed off the 16-byte grid, and batches
     A, B = _rand_q(rng, np.uint8, (3, 37, 64)), _rand_q(rng, np.int8, (64, 23))
     plain = rt.MatMulIntegerDequant(A, B, None, None, np.float32(0.002), np.float32(0.01))
