@@ -99,6 +99,28 @@ def test_quantize_per_tensor(rt, oracle, n, qdt):
                               oracle.quantize_linear(x, np.float32(0.02), None))
 
 
+@pytest.mark.parametrize("qdt", [np.uint8, np.int8])
+def test_quantize_every_input_that_does_not_saturate(rt, oracle, qdt):
+    """Every binary32 value whose quotient by the scale has a magnitude in
+    [1/4, 512), both signs, bit pattern by bit pattern: beyond that range the
+    result is the zero point or saturated, which the sampled tests cover.  With
+    the scale 1 (the quotient is the input: the rounding alone), a scale whose
+    quotients are inexact (reciprocal-multiply path) and a scale small enough
+    to take the full divide; about 180 million inputs each."""
+    zp = np.array(3 if qdt == np.uint8 else -5, qdt)
+    for s in (np.float32(1.0), np.float32(0.0173), np.float32(5e-30)):
+        lo = int(np.float32(0.25 * float(s)).view(np.uint32))
+        hi = int(np.float32(512.0 * float(s)).view(np.uint32))
+        assert hi - lo == 11 << 23
+        for start in range(lo, hi, 1 << 24):
+            bits = np.arange(start, min(start + (1 << 24), hi), dtype=np.uint32)
+            for sign in (0, 0x80000000):
+                x = (bits | np.uint32(sign)).view(np.float32)
+                got = rt.QuantizeLinear(x, s, zp)
+                want = oracle.quantize_linear(x, s, zp, omp=True)
+                assert np.array_equal(got, want), (float(s), hex(start), sign)
+
+
 def test_quantize_zero_and_denormal_scale(rt, oracle):
     x = np.array([0.0, -0.0, 1.0, -1.0, np.nan, 3e-45, -3e-45], np.float32)
     for s in (0.0, 1e-45, 1e-39):
