@@ -822,6 +822,8 @@ __global__ __launch_bounds__(256, MINB) void k_gemm_i8_bs(
   constexpr int STAGE = BM * BK;
   constexpr int CA = BM / 64; // A copies (1 KiB each) per wave and step
   static_assert(BM % 64 == 0, "tile height");
+  // The only depths this kernel has been validated with on the device.
+  static_assert(NST == 4 && D == 4, "stages");
   __shared__ __attribute__((aligned(1024))) uint8_t sm[NST * STAGE];
 
   int pid = blockIdx.x;
