@@ -1436,12 +1436,15 @@ def test_config4_layers_reduced_m(rt, oracle, name):
 
 
 def _check_full_size_layer(rt, oracle, c, sample_rows):
-    """A layer at its benchmark size.  The oracle is too slow for the whole
-    matrix, so: (1) exact comparison of sampled rows (first, last, both sides of
-    tile edges, random ones) of the fused result; (2) two checksums over the
-    whole int32 accumulator, which every element enters: its column sums must
-    equal (sum of the rows of A - zp) x W and its row sums (A - zp) x (sum of
-    the columns of W), in arithmetic modulo 2^32."""
+    """A layer at its benchmark size, every element: the int32 accumulator
+    against the oracle's OpenMP restatement of the reference's passes (pinned to
+    the plain triple loop in tests/test_oracle.py), the fused result against
+    that accumulator scaled by the oracle.  Kept from when the oracle was the
+    triple loop only: sampled rows (first, last, both sides of tile edges,
+    random ones) against that loop, and two checksums over the accumulator
+    computed another way -- its column sums must equal (sum of the rows of
+    A - zp) x W and its row sums (A - zp) x (sum of the columns of W), in
+    arithmetic modulo 2^32."""
     X, W, ws = c["X"], c["W"], c["w_scale"]
     M, K = X.shape
     N = W.shape[1]
@@ -1464,7 +1467,8 @@ def _check_full_size_layer(rt, oracle, c, sample_rows):
     mod = 1 << 32
     assert np.array_equal(acc.sum(axis=0, dtype=np.int64) % mod, want_cols.astype(np.int64) % mod)
     assert np.array_equal(acc.sum(axis=1, dtype=np.int64) % mod, want_rows.astype(np.int64) % mod)
-    # and the fused result is that accumulator, scaled
+    # every element of the accumulator, and the fused result is it, scaled
+    assert np.array_equal(acc, oracle.matmul_integer(aq, W, a_zp, None, passes=True))
     assert same_f32(got, oracle.dequant_epilogue(acc, a_s, ws))
 
 
