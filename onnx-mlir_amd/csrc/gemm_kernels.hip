@@ -1837,6 +1837,62 @@ __global__ __launch_bounds__(256) void k_gelu_inplace(float *__restrict__ y,
 }
 } // namespace
 
+// ---- matrix-core ceiling probe ------------------------------------------------
+// Four independent accumulators per wave, MFMAs back to back, operands that
+// never leave their registers: the rate at which the matrix cores run when
+// nothing feeds them.  RANDOM: operand bytes from a per-lane generator, two
+// sets in alternation, so that the inputs toggle as a model's do; otherwise
+// ones and zeros.  The accumulators are folded into a value that is stored
+// only if it has one particular value, which keeps the loop alive.
+namespace {
+template <bool RANDOM>
+__global__ __launch_bounds__(256) void k_mfma_probe(int iters,
+    int *__restrict__ sink) {
+  unsigned seed = threadIdx.x * 7919u + blockIdx.x * 104729u + 1u;
+  auto next = [&]() {
+    seed = seed * 1664525u + 1013904223u;
+    return (int)(seed ^ (seed >> 15));
+  };
+  v4i a0 = {1, 1, 1, 1}, b0 = {1, 0, 1, 0}, a1 = a0, b1 = b0;
+  if (RANDOM) {
+    a0 = (v4i){next(), next(), next(), next()};
+    b0 = (v4i){next(), next(), next(), next()};
+    a1 = (v4i){next(), next(), next(), next()};
+    b1 = (v4i){next(), next(), next(), next()};
+  }
+  asm volatile("" : "+v"(a0), "+v"(b0), "+v"(a1), "+v"(b1));
+  v16i acc[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+      acc[i][r] = 0;
+  for (int it = 0; it < iters; ++it) {
+    acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, b0, acc[0], 0, 0, 0);
+    acc[1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, b1, acc[1], 0, 0, 0);
+    acc[2] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, b0, acc[2], 0, 0, 0);
+    acc[3] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, b1, acc[3], 0, 0, 0);
+  }
+  int fold = 0;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+      fold += acc[i][r];
+  if (fold == 0x7fffffff)
+    sink[0] = fold;
+}
+} // namespace
+
+hipError_t launch_mfma_probe(hipStream_t s, bool random_operands, int blocks,
+    int iters, int *sink) {
+  if (random_operands)
+    k_mfma_probe<true><<<(unsigned)blocks, 256, 0, s>>>(iters, sink);
+  else
+    k_mfma_probe<false><<<(unsigned)blocks, 256, 0, s>>>(iters, sink);
+  return hipGetLastError();
+}
+
 hipError_t launch_gemm(hipStream_t s, const GemmArgs &g) {
   if (g.M == 0 || g.N == 0)
     return hipSuccess;

@@ -113,6 +113,11 @@ struct GemmArgs {
 };
 
 hipError_t launch_gemm(hipStream_t s, const GemmArgs &g);
+// Matrix-core ceiling probe: `blocks` blocks of four waves, each wave issuing
+// 4 * iters v_mfma_i32_32x32x32_i8 from registers; nothing is written to
+// `sink` (it keeps the loop alive).
+hipError_t launch_mfma_probe(hipStream_t s, bool random_operands, int blocks,
+    int iters, int *sink);
 // Name of the kernel the calling thread's last launch_gemm chose.
 const char *last_gemm_kernel();
 

@@ -2030,6 +2030,67 @@ float om_mi355x_timer_stop(void) {
   return ms;
 }
 
+int om_mi355x_mfma_ceiling(int64_t random_operands, double *tops,
+    double *clock_ghz) {
+  if (!tops || !clock_ghz) {
+    fail(EINVAL, "om_mi355x_mfma_ceiling: null result pointer");
+    return -1;
+  }
+  if (!t_ctx.init())
+    return -1;
+  hipDeviceProp_t prop;
+  if (hipGetDeviceProperties(&prop, 0) != hipSuccess) {
+    fail(EIO, "om_mi355x_mfma_ceiling: no device properties");
+    return -1;
+  }
+  // Two blocks of four waves per CU (two waves per SIMD), 4 * kIters MFMAs
+  // per wave: 5 to 15 ms, long enough for the clock to settle.  The first
+  // launch brings the device to that state, the second is the one timed.
+  const int kIters = 50000;
+  const int blocks = 2 * prop.multiProcessorCount;
+  void *buf = om_mi355x_malloc(16);
+  if (!buf)
+    return -1;
+  int *sink = (int *)buf;
+  hipStream_t st = t_ctx.stream;
+  float ms = 0.0f;
+  // events of its own: a bracket opened with om_mi355x_timer_start stays valid
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  hipError_t e = hipEventCreate(&e0);
+  if (e == hipSuccess)
+    e = hipEventCreate(&e1);
+  if (e == hipSuccess)
+    e = launch_mfma_probe(st, random_operands != 0, blocks, kIters, sink);
+  if (e == hipSuccess)
+    e = hipEventRecord(e0, st);
+  if (e == hipSuccess)
+    e = launch_mfma_probe(st, random_operands != 0, blocks, kIters, sink);
+  if (e == hipSuccess)
+    e = hipEventRecord(e1, st);
+  if (e == hipSuccess)
+    e = hipEventSynchronize(e1);
+  if (e == hipSuccess)
+    e = hipEventElapsedTime(&ms, e0, e1);
+  if (e0)
+    (void)hipEventDestroy(e0);
+  if (e1)
+    (void)hipEventDestroy(e1);
+  om_mi355x_free(buf);
+  if (e != hipSuccess || ms <= 0.0f) {
+    fail(EIO, "om_mi355x_mfma_ceiling failed: %s", hipGetErrorString(e));
+    return -1;
+  }
+  // 4 waves a block, 4 * kIters MFMAs a wave, 32 * 32 * 32 multiply-adds each
+  const double ops = (double)blocks * 4.0 * 4.0 * kIters * 32768.0 * 2.0;
+  *tops = ops / ((double)ms * 1e-3) / 1e12;
+  // A SIMD issues one of these MFMAs every 32 clocks when nothing holds it
+  // up, which is the case here: the clock that this rate corresponds to.
+  const double per_simd = (double)blocks * 4.0 * 4.0 * kIters /
+                          ((double)prop.multiProcessorCount * 4.0);
+  *clock_ghz = per_simd * 32.0 / ((double)ms * 1e6);
+  return 0;
+}
+
 const char *om_mi355x_last_error(void) {
   t_last_error_returned.swap(t_last_error);
   t_last_error.clear();

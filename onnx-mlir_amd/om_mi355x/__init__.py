@@ -117,6 +117,9 @@ def _declare(lib, shim):
     lib.om_mi355x_last_error.restype = ctypes.c_char_p
     lib.om_mi355x_last_gemm_kernel.restype = ctypes.c_char_p
     lib.om_mi355x_device_info.restype = ctypes.c_int
+    lib.om_mi355x_mfma_ceiling.restype = ctypes.c_int
+    lib.om_mi355x_mfma_ceiling.argtypes = [ctypes.c_int64, ctypes.POINTER(ctypes.c_double),
+                                           ctypes.POINTER(ctypes.c_double)]
     lib.om_mi355x_device_info.argtypes = [ctypes.c_char_p, SZ]
 
 
@@ -135,6 +138,18 @@ def device_info() -> dict:
     name, arch, cus, mhz, gib = buf.value.decode().split("|")
     return {"name": name, "arch": arch, "cus": int(cus), "clock_mhz": int(mhz),
             "mem_gib": float(gib)}
+
+
+def mfma_ceiling(random_operands: bool = True) -> dict:
+    """int8 MFMA rate of the device with nothing else going on (TOPS) and the
+    shader clock it held meanwhile; see om_mi355x_mfma_ceiling in the header."""
+    load()
+    tops, ghz = ctypes.c_double(0.0), ctypes.c_double(0.0)
+    if _lib.om_mi355x_mfma_ceiling(ctypes.c_int64(1 if random_operands else 0),
+                                   ctypes.byref(tops), ctypes.byref(ghz)) != 0:
+        _check()
+        raise RuntimeError_("om_mi355x_mfma_ceiling failed")
+    return {"tops": tops.value, "clock_ghz": ghz.value}
 
 
 def last_gemm_kernel() -> str:

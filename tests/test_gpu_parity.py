@@ -995,6 +995,16 @@ def test_matmulinteger_batched_a(rt, oracle):
     assert got.shape == (3, 5, 24) and np.array_equal(got, oracle.matmul_integer(A, B, az, None))
 
 
+def test_mfma_ceiling_probe(rt):
+    """The measurement aid runs, reports a rate between a tenth of and just above
+    the published dense int8 peak (5 POP/s) and a plausible shader clock, and
+    small-constant operands are not slower than random ones by more than noise."""
+    rnd, const = rt.mfma_ceiling(True), rt.mfma_ceiling(False)
+    for r in (rnd, const):
+        assert 500.0 < r["tops"] < 5300.0 and 0.3 < r["clock_ghz"] < 2.6, r
+    assert const["tops"] > 0.9 * rnd["tops"]
+
+
 def test_fused_relu_epilogue(rt, oracle, monkeypatch):
     """`activation` = Relu on the two fused entry points equals onnx.Relu applied
     to the call's own result without it (max(0, x) is exact), over the kernels a
