@@ -93,6 +93,39 @@ void emitCall(ConversionPatternRewriter &rewriter, Location loc,
     call->setAttr(name, rewriter.getI64IntegerAttr(value));
 }
 
+/// The reference's own lowerings of QuantizeLinear, DequantizeLinear and
+/// DynamicQuantizeLinear change with two compiler options: --enable-fast-math
+/// at -O3 (the quotient becomes x * (1 / scale),
+/// src/Conversion/ONNXToKrnl/Quantization/QuantizeLinear.cpp:43-44, enabled as
+/// in src/Compiler/CompilerPasses.cpp:298-301) and
+/// --disable-quantization-zero-point (QuantizeLinear.cpp:231-237,
+/// DynamicQuantizeLinear.cpp:142, Math/Elementwise.cpp:1453).  The runtime
+/// computes either way; which one is a state of the calling thread, set by
+/// `om_mi355x_SetQuantMode(anchor, mode)`.  The call goes in front of every
+/// offloaded op that the options touch, and only when one of them is on, so a
+/// thread that runs models compiled differently is always in the right state.
+/// `anchor` (the op's first result buffer) is passed as an output for the
+/// reason given at markIfConstant; the runtime does not touch it.
+int64_t quantModeFromOptions() {
+  int64_t mode = 0;
+  if (OptimizationLevel >= OptLevel::O3 && enableFastMathOption)
+    mode |= 1; // OM_MI355X_QUANT_RECIPROCAL
+  if (disableQuantZeroPoint)
+    mode |= 2; // OM_MI355X_QUANT_NO_ZERO_POINT
+  return mode;
+}
+
+void emitQuantMode(
+    ConversionPatternRewriter &rewriter, Location loc, Value anchor) {
+  const int64_t mode = quantModeFromOptions();
+  if (mode == 0)
+    return;
+  auto call = KrnlCallOp::create(rewriter, loc,
+      std::string(kMI355XSetQuantMode),
+      /*numOfOutput=*/static_cast<int64_t>(1), ValueRange{anchor});
+  call->setAttr("mode", rewriter.getI64IntegerAttr(mode));
+}
+
 /// Tell the runtime that `v` is a model constant, so that it is copied to the
 /// device (and, as a matmul right-hand side, packed) once instead of on every
 /// call.  After conversion an `onnx.Constant` is a `krnl.global`, whose buffer
@@ -142,6 +175,7 @@ struct QuantizeLinearToMI355X
     std::vector<Value> y =
         allocResults<ONNXQuantizeLinearOp, ONNXQuantizeLinearOpShapeHelper>(
             op, adaptor.getOperands(), rewriter, typeConverter);
+    emitQuantMode(rewriter, loc, y[0]);
     emitCall(rewriter, loc, "om_mi355x_QuantizeLinear", y,
         {adaptor.getX(), adaptor.getYScale(), adaptor.getYZeroPoint()},
         {{"axis", op.getAxis()}, {"saturate", op.getSaturate()}});
@@ -170,6 +204,7 @@ struct DequantizeLinearToMI355X
     std::vector<Value> y =
         allocResults<ONNXDequantizeLinearOp, ONNXDequantizeLinearOpShapeHelper>(
             op, adaptor.getOperands(), rewriter, typeConverter);
+    emitQuantMode(rewriter, loc, y[0]);
     emitCall(rewriter, loc, "om_mi355x_DequantizeLinear", y,
         {adaptor.getX(), adaptor.getXScale(), adaptor.getXZeroPoint()},
         {{"axis", op.getAxis()}});
@@ -195,6 +230,7 @@ struct DynamicQuantizeLinearToMI355X
     std::vector<Value> results = allocResults<ONNXDynamicQuantizeLinearOp,
         ONNXDynamicQuantizeLinearOpShapeHelper>(
         op, adaptor.getOperands(), rewriter, typeConverter);
+    emitQuantMode(rewriter, loc, results[0]);
     emitCall(rewriter, loc, "om_mi355x_DynamicQuantizeLinear", results,
         {adaptor.getX()});
     rewriter.replaceOp(op, results);
@@ -314,6 +350,8 @@ struct FusedMatMulToMI355X : public OpConversionPattern<ONNXCustomOp> {
     int64_t activation = 0;
     if (auto attr = op->getAttrOfType<IntegerAttr>("activation"))
       activation = attr.getInt();
+    if (callee == kMI355XDynQuantMatMulDequant) // it quantizes; the other fused op does not
+      emitQuantMode(rewriter, loc, y);
     emitCall(rewriter, loc, callee, {y}, inputs, {{"activation", activation}});
     rewriter.replaceOp(op, y);
     return success();

@@ -23,7 +23,7 @@ namespace accel {
 
 // Must stay equal to OM_MI355X_VERSION in om_mi355x.h: the runtime refuses a
 // model compiled for a newer major.minor than its own.
-static constexpr uint64_t kRuntimeVersion = 0x010000;
+static constexpr uint64_t kRuntimeVersion = 0x010100;
 
 Accelerator *createMI355X() { return MI355XAccelerator::getInstance(); }
 

@@ -57,7 +57,8 @@ constexpr const char *kPrefix = "om_mi355x_";
 bool isOffloadedCompute(KrnlCallOp call) {
   StringRef callee = call.getFuncName();
   return callee.starts_with(kPrefix) && callee != kMI355XMarkConstant &&
-         callee != kMI355XKeepOnDevice && callee != kMI355XRelease;
+         callee != kMI355XKeepOnDevice && callee != kMI355XRelease &&
+         callee != kMI355XSetQuantMode;
 }
 
 /// First and last use of `buffer` if it qualifies (see the file header).
@@ -67,6 +68,9 @@ bool qualifies(memref::AllocOp alloc, Operation *&last) {
   last = nullptr;
   for (OpOperand &use : buffer.getUses()) {
     auto call = dyn_cast<KrnlCallOp>(use.getOwner());
+    // the buffer is only that call's anchor: neither read nor written
+    if (call && call.getFuncName() == kMI355XSetQuantMode)
+      continue;
     if (!call || call->getBlock() != alloc->getBlock() ||
         !isOffloadedCompute(call))
       return false;

@@ -24,6 +24,7 @@ constexpr const char *kMI355XDynQuantMatMulDequant =
 constexpr const char *kMI355XMarkConstant = "om_mi355x_MarkConstant";
 constexpr const char *kMI355XKeepOnDevice = "om_mi355x_KeepOnDevice";
 constexpr const char *kMI355XRelease = "om_mi355x_Release";
+constexpr const char *kMI355XSetQuantMode = "om_mi355x_SetQuantMode";
 
 /// --fuse-quantized-matmul-for-mi355x
 ///   MatMulInteger -> Cast(f32) -> Mul(a_scale * b_scale)

@@ -14,9 +14,11 @@ enum NarrowMode : int { kWrap = 0, kSaturate = 1 };
 // ---- quantize / dequantize (HBM-bound streaming kernels) ------------------
 // The tensor is viewed as [outer, channels, inner]; scale / zp have `channels`
 // entries.  channels == 1 is the per-tensor case.  zp may be null.
+// reciprocal: quantize as the reference does when compiled with
+// --enable-fast-math, x * (1 / scale) in place of x / scale.
 hipError_t launch_quantize(hipStream_t s, const float *x, int64_t outer,
     int64_t channels, int64_t inner, const float *scale, const void *zp,
-    bool is_signed, void *y);
+    bool is_signed, void *y, bool reciprocal = false);
 
 hipError_t launch_dequantize(hipStream_t s, const void *x, QKind xkind,
     int64_t outer, int64_t channels, int64_t inner, const float *scale,
@@ -55,9 +57,12 @@ constexpr int kDqlMaxBlocks = 4096;
 // y u8[n], scale f32[1], zp u8[1].  If y_shift is true the stored bytes are
 // y ^ 0x80 (the value minus 128 as int8), the form the GEMM consumes, and
 // row sums are not needed because they are not produced here.
+// mode: bits of OM_MI355X_QUANT_* (reciprocal quotient, no zero point); any
+// mode but 0 takes the small-tensor kernel or the two-launch path.
 hipError_t launch_dynamic_quantize(hipStream_t s, DqlScratch &scratch,
     const float *x, int64_t n, uint8_t *y, float *scale, uint8_t *zp,
-    bool y_shift);
+    bool y_shift, int mode = 0);
+constexpr int kQuantReciprocal = 1, kQuantNoZeroPoint = 2;
 
 // Call before destroying a stream that launch_dynamic_quantize was given.
 void dql_forget_stream(hipStream_t s);
@@ -163,10 +168,17 @@ hipError_t launch_fill_u32(hipStream_t s, uint32_t *p, int64_t n, uint32_t v);
 __device__ __forceinline__ bool scale_is_tame(float s) {
   return s >= 0x1p-96f && s <= 0x1p96f;
 }
-template <bool FAST>
+// QMODE 0: the divide; 1: the corrected reciprocal form above (same result);
+// 2: x * r and nothing else -- what the reference computes when it is
+// compiled with --enable-fast-math at -O3
+// (src/Conversion/ONNXToKrnl/Quantization/QuantizeLinear.cpp:43-44,119-132),
+// a different result by design, for any scale.
+template <int QMODE>
 __device__ __forceinline__ float quotient(float x, float s, float r) {
-  if (!FAST)
+  if (QMODE == 0)
     return x / s;
+  if (QMODE == 2)
+    return x * r;
   const float q0 =
       __builtin_fminf(__builtin_fmaxf(x * r, -1024.0f), 1024.0f);
   const float e = __builtin_fmaf(-q0, s, x);
@@ -174,19 +186,19 @@ __device__ __forceinline__ float quotient(float x, float s, float r) {
 }
 
 // rne(x / s) + zp, not yet clamped.
-template <bool HAS_ZP, bool FAST>
+template <bool HAS_ZP, int QMODE>
 __device__ __forceinline__ float quant_value(
     float x, float s, float r, float zpf) {
-  float v = __builtin_rintf(quotient<FAST>(x, s, r));
+  float v = __builtin_rintf(quotient<QMODE>(x, s, r));
   if (HAS_ZP)
     v = v + zpf;
   return v;
 }
 
-template <bool SIGNED, bool HAS_ZP, bool FAST = false>
+template <bool SIGNED, bool HAS_ZP, int QMODE = 0>
 __device__ __forceinline__ uint32_t quant_one(
     float x, float s, float zpf, float r = 0.0f) {
-  const float v = quant_value<HAS_ZP, FAST>(x, s, r, zpf);
+  const float v = quant_value<HAS_ZP, QMODE>(x, s, r, zpf);
   if (SIGNED) {
     float c = __builtin_fminf(__builtin_fmaxf(v, -128.0f), 127.0f);
     return (uint32_t)((int32_t)c) & 0xFFu;
@@ -200,7 +212,7 @@ __device__ __forceinline__ uint32_t quant_one(
 // already an integer (or an infinity, which saturates, or a NaN, which gives
 // 0 = the lower bound, as maxnum-then-minnum does), so its own rounding never
 // acts.
-template <bool SIGNED, bool HAS_ZP, bool FAST>
+template <bool SIGNED, bool HAS_ZP, int FAST>
 __device__ __forceinline__ uint32_t quant_pack4(float x0, float x1, float x2,
     float x3, float s0, float s1, float s2, float s3, float r0, float r1,
     float r2, float r3, float z0, float z1, float z2, float z3) {
@@ -240,8 +252,10 @@ __device__ __forceinline__ float wave_max(float v) {
 
 // Scale and zero point of DynamicQuantizeLinear from min / max
 // (src/Conversion/ONNXToKrnl/Quantization/DynamicQuantizeLinear.cpp:43-84).
+// no_zp: compiled with --disable-quantization-zero-point, the zero point is 0
+// (DynamicQuantizeLinear.cpp:75-84); adding that 0 changes no result.
 __device__ __forceinline__ void dynamic_params(
-    float xmin, float xmax, float &scale, float &zpf) {
+    float xmin, float xmax, float &scale, float &zpf, bool no_zp = false) {
   const float mx = __builtin_fmaxf(xmax, 0.0f);
   const float mn = __builtin_fminf(xmin, 0.0f);
   const float xdiff = mx - mn;
@@ -249,7 +263,7 @@ __device__ __forceinline__ void dynamic_params(
   scale = xdiff / bound;
   const float inter = 0.0f - mn / scale;
   const float sat = __builtin_fminf(__builtin_fmaxf(inter, 0.0f), 255.0f);
-  zpf = __builtin_rintf(sat);
+  zpf = no_zp ? 0.0f : __builtin_rintf(sat);
 }
 #endif
 

@@ -71,7 +71,7 @@ __device__ __forceinline__ float load_zp_f32(const void *zp, int64_t i) {
 
 // Four elements that share one scale; r = 1 / s is used when FAST (only for
 // a tame s, see scale_is_tame).
-template <bool SIGNED, bool HAS_ZP, bool FAST, typename V4>
+template <bool SIGNED, bool HAS_ZP, int FAST, typename V4>
 __device__ __forceinline__ uint32_t quant_four(
     V4 v, float s, float r, float zpf, uint32_t flip) {
   return quant_pack4<SIGNED, HAS_ZP, FAST>(
@@ -515,7 +515,39 @@ __global__ __launch_bounds__(kThreads) void k_quant_slabs(
   }
 }
 
+// Per-tensor quantize with the quotient taken as x * (1 / scale), the form
+// the reference's code has under --enable-fast-math (quotient<2>): blocks of
+// two float4 per thread, one trip; x 16-byte and y 4-byte aligned.
 template <bool SIGNED, bool HAS_ZP>
+__global__ __launch_bounds__(kThreads) void k_quant_flat_reciprocal(
+    const float *__restrict__ x, uint8_t *__restrict__ y, int64_t n,
+    const float *__restrict__ scale_p, const void *__restrict__ zp_p,
+    uint32_t flip) {
+  const int64_t nvec = n >> 2;
+  const f4a *__restrict__ x4 = (const f4a *)x;
+  uint32_t *__restrict__ y4 = (uint32_t *)y;
+  const int64_t base = (int64_t)blockIdx.x * (kThreads * 2) + threadIdx.x;
+  f4a v[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j)
+    if (base + j * kThreads < nvec)
+      v[j] = __builtin_nontemporal_load(&x4[base + j * kThreads]);
+  const float s = scale_p[0];
+  const float r = 1.0f / s;
+  const float zpf = HAS_ZP ? load_zp_f32<SIGNED>(zp_p, 0) : 0.0f;
+#pragma unroll
+  for (int j = 0; j < 2; ++j)
+    if (base + j * kThreads < nvec)
+      q_store(&y4[base + j * kThreads],
+          quant_four<SIGNED, HAS_ZP, 2>(v[j], s, r, zpf, flip));
+  if (blockIdx.x == 0) {
+    const int64_t e = (nvec << 2) + threadIdx.x;
+    if (e < n)
+      y[e] = (uint8_t)(quant_one<SIGNED, HAS_ZP, 2>(x[e], s, zpf, r) ^ (flip & 0xFFu));
+  }
+}
+
+template <bool SIGNED, bool HAS_ZP, bool RECIP = false>
 __global__ __launch_bounds__(kThreads) void k_quant_general(
     const float *__restrict__ x, uint8_t *__restrict__ y, int64_t channels,
     int64_t inner, const float *__restrict__ scale,
@@ -523,12 +555,13 @@ __global__ __launch_bounds__(kThreads) void k_quant_general(
   for (int64_t oc = blockIdx.y; oc < oc_total; oc += gridDim.y) {
     const int64_t c = oc % channels;
     const float s = scale[c];
+    const float r = 1.0f / s;
     const float zpf = HAS_ZP ? load_zp_f32<SIGNED>(zp, c) : 0.0f;
     const float *__restrict__ xr = x + oc * inner;
     uint8_t *__restrict__ yr = y + oc * inner;
     for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < inner;
          i += (int64_t)gridDim.x * kThreads)
-      yr[i] = (uint8_t)quant_one<SIGNED, HAS_ZP>(xr[i], s, zpf);
+      yr[i] = (uint8_t)quant_one<SIGNED, HAS_ZP, RECIP ? 2 : 0>(xr[i], s, zpf, r);
   }
 }
 
@@ -1286,7 +1319,7 @@ __device__ __forceinline__ void block_minmax(float &lo, float &hi) {
 __global__ __launch_bounds__(kThreads) void k_minmax_params(
     const float *__restrict__ x, int64_t n, float *partial_min,
     float *partial_max, unsigned *counter, float *__restrict__ scale_out,
-    uint8_t *__restrict__ zp_out) {
+    uint8_t *__restrict__ zp_out, int no_zp) {
   float lo = __builtin_inff(), hi = -__builtin_inff();
   const int64_t nvec = n >> 2;
   const f4a *__restrict__ x4 = (const f4a *)x;
@@ -1370,7 +1403,7 @@ __global__ __launch_bounds__(kThreads) void k_minmax_params(
   block_minmax(lo, hi);
   if (threadIdx.x == 0) {
     float scale, zpf;
-    dynamic_params(lo, hi, scale, zpf);
+    dynamic_params(lo, hi, scale, zpf, no_zp != 0);
     scale_out[0] = scale;
     zp_out[0] = (uint8_t)(uint32_t)zpf;
     __hip_atomic_store(
@@ -1392,7 +1425,7 @@ constexpr int64_t kSmallMax = (int64_t)kSmallThreads * kSmallPerThread;
 __global__ __launch_bounds__(kSmallThreads) void k_dql_small(
     const float *__restrict__ x, int64_t n, uint8_t *__restrict__ y,
     float *__restrict__ scale_out, uint8_t *__restrict__ zp_out,
-    uint32_t flip) {
+    uint32_t flip, int mode) {
   __shared__ float s_lo[kSmallThreads / 64], s_hi[kSmallThreads / 64];
   float v[kSmallPerThread];
   float lo = __builtin_inff(), hi = -__builtin_inff();
@@ -1418,26 +1451,29 @@ __global__ __launch_bounds__(kSmallThreads) void k_dql_small(
     hi = __builtin_fmaxf(hi, s_hi[w]);
   }
   float scale, zpf;
-  dynamic_params(lo, hi, scale, zpf);
+  dynamic_params(lo, hi, scale, zpf, (mode & kQuantNoZeroPoint) != 0);
   if (threadIdx.x == 0) {
     scale_out[0] = scale;
     zp_out[0] = (uint8_t)(uint32_t)zpf;
   }
   const float recip = 1.0f / scale;
-  auto store = [&](auto fast_c) {
-    constexpr bool FAST = decltype(fast_c)::value;
+  auto store = [&](auto qmode_c) {
+    constexpr int QMODE = decltype(qmode_c)::value;
 #pragma unroll
     for (int j = 0; j < kSmallPerThread; ++j) {
       const int64_t e = (int64_t)j * kSmallThreads + threadIdx.x;
       if (e < n)
-        y[e] = (uint8_t)(quant_one<false, true, FAST>(v[j], scale, zpf, recip) ^
+        y[e] = (uint8_t)(quant_one<false, true, QMODE>(v[j], scale, zpf, recip) ^
                          (flip & 0xFFu));
     }
   };
-  if (scale_is_tame(scale)) // the same for every thread
-    store(std::true_type{});
+  // (the same branch for every thread)
+  if (mode & kQuantReciprocal)
+    store(std::integral_constant<int, 2>{});
+  else if (scale_is_tame(scale))
+    store(std::integral_constant<int, 1>{});
   else
-    store(std::false_type{});
+    store(std::integral_constant<int, 0>{});
 }
 
 // Mid-sized tensors (up to 32 float4 per thread of a grid that fills the
@@ -1718,12 +1754,48 @@ PeriodicGrid periodic_grid(int64_t nvec, int64_t C, int trips) {
 template <bool SIGNED>
 hipError_t quantize_dispatch(hipStream_t st, const float *x, int64_t outer,
     int64_t channels, int64_t inner, const float *scale, const void *zp,
-    void *y, uint32_t flip) {
+    void *y, uint32_t flip, bool reciprocal = false) {
   const int64_t n = outer * channels * inner;
   if (n == 0)
     return hipSuccess;
   uint8_t *yo = (uint8_t *)y;
   const bool has_zp = zp != nullptr;
+  if (reciprocal) {
+    // The reference's fast-math form, x * (1 / scale): a kernel of its own
+    // for the per-tensor case, the general kernel for everything else.
+    const bool aligned =
+        ((((uintptr_t)x) & 15) == 0) && ((((uintptr_t)y) & 3) == 0);
+    const int64_t blocks = ((n >> 2) + kThreads * 2 - 1) / (kThreads * 2);
+    if (channels == 1 && aligned && blocks < ((int64_t)1 << 31)) {
+      const unsigned grid = (unsigned)(blocks > 0 ? blocks : 1);
+      if (has_zp)
+        k_quant_flat_reciprocal<SIGNED, true>
+            <<<grid, kThreads, 0, st>>>(x, yo, n, scale, zp, flip);
+      else
+        k_quant_flat_reciprocal<SIGNED, false>
+            <<<grid, kThreads, 0, st>>>(x, yo, n, scale, zp, flip);
+      return hipGetLastError();
+    }
+    if (flip != 0)
+      return hipErrorInvalidValue;
+    if (channels == 1) {
+      outer = 1;
+      inner = n;
+    }
+    const int64_t oc = outer * channels;
+    const int64_t gy = oc < 4096 ? oc : 4096;
+    int64_t gx = (inner + kThreads - 1) / kThreads;
+    const int64_t cap = (4096 + gy - 1) / gy;
+    gx = gx > cap ? cap : (gx < 1 ? 1 : gx);
+    dim3 grid((unsigned)gx, (unsigned)gy);
+    if (has_zp)
+      k_quant_general<SIGNED, true, true>
+          <<<grid, kThreads, 0, st>>>(x, yo, channels, inner, scale, zp, oc);
+    else
+      k_quant_general<SIGNED, false, true>
+          <<<grid, kThreads, 0, st>>>(x, yo, channels, inner, scale, zp, oc);
+    return hipGetLastError();
+  }
   if (channels == 1) {
     const bool aligned =
         ((((uintptr_t)x) & 15) == 0) && ((((uintptr_t)y) & 3) == 0);
@@ -1984,12 +2056,12 @@ hipError_t dequantize_dispatch(hipStream_t st, const void *x, int64_t outer,
 
 hipError_t launch_quantize(hipStream_t s, const float *x, int64_t outer,
     int64_t channels, int64_t inner, const float *scale, const void *zp,
-    bool is_signed, void *y) {
+    bool is_signed, void *y, bool reciprocal) {
   if (is_signed)
     return quantize_dispatch<true>(
-        s, x, outer, channels, inner, scale, zp, y, 0u);
+        s, x, outer, channels, inner, scale, zp, y, 0u, reciprocal);
   return quantize_dispatch<false>(
-      s, x, outer, channels, inner, scale, zp, y, 0u);
+      s, x, outer, channels, inner, scale, zp, y, 0u, reciprocal);
 }
 
 hipError_t launch_dequantize(hipStream_t s, const void *x, QKind xkind,
@@ -2013,15 +2085,15 @@ hipStream_t g_grid_stream = nullptr; // stream of the last such launch
 
 hipError_t launch_dynamic_quantize(hipStream_t s, DqlScratch &scratch,
     const float *x, int64_t n, uint8_t *y, float *scale, uint8_t *zp,
-    bool y_shift) {
+    bool y_shift, int mode) {
   if (n <= kSmallMax) { // n == 0 included: scale and zero point are written
     k_dql_small<<<1, kSmallThreads, 0, s>>>(
-        x, n, y, scale, zp, y_shift ? 0x80808080u : 0u);
+        x, n, y, scale, zp, y_shift ? 0x80808080u : 0u, mode);
     return hipGetLastError();
   }
   // One launch when the tensor fits the registers of a grid that is resident
   // all at once (one block per CU).
-  if (scratch.grid_blocks > 0 && ((((uintptr_t)x) & 15) == 0) &&
+  if (mode == 0 && scratch.grid_blocks > 0 && ((((uintptr_t)x) & 15) == 0) &&
       ((((uintptr_t)y) & 3) == 0)) {
     const int64_t total = (int64_t)scratch.grid_blocks * kGridThreads;
     const int64_t nvec = n >> 2;
@@ -2080,15 +2152,16 @@ hipError_t launch_dynamic_quantize(hipStream_t s, DqlScratch &scratch,
   const int grid = stream_grid(
       n >> 2, kThreads * 8, scratch.max_blocks < 512 ? scratch.max_blocks : 512);
   k_minmax_params<<<grid, kThreads, 0, s>>>(x, n, scratch.partial_min,
-      scratch.partial_max, scratch.counter, scale, zp);
+      scratch.partial_max, scratch.counter, scale, zp,
+      (mode & kQuantNoZeroPoint) ? 1 : 0);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess)
     return e;
   // Second pass: the ordinary per-tensor quantize with the parameters just
   // written (the u8 zero point converted back to f32 is the float zero point
   // the reference adds: it is an integer in [0, 255]).
-  return quantize_dispatch<false>(
-      s, x, 1, 1, n, scale, zp, y, y_shift ? 0x80808080u : 0u);
+  return quantize_dispatch<false>(s, x, 1, 1, n, scale, zp, y,
+      y_shift ? 0x80808080u : 0u, (mode & kQuantReciprocal) != 0);
 }
 
 void dql_forget_stream(hipStream_t s) {

@@ -60,6 +60,9 @@ static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
 // ---------------------------------------------------------------------------
 namespace {
 
+// The compiler options the calling thread's model was compiled with, as far as
+// they change this path's arithmetic (OM_MI355X_QUANT_*; om_mi355x_SetQuantMode).
+thread_local int t_quant_mode = 0;
 thread_local std::string t_last_error;
 thread_local std::string t_last_error_returned;
 
@@ -948,6 +951,13 @@ bool is_q8(int dt) {
 void run_dql(Call &call, const float *dx, int64_t n, uint8_t *dy, float *ds,
     uint8_t *dz, bool y_shift) {
   Ctx &c = call.c;
+  const int mode = t_quant_mode;
+  if (mode != 0) { // never the one-launch kernel: nothing to check afterwards
+    call.check(launch_dynamic_quantize(
+                   c.stream, c.dql, dx, n, dy, ds, dz, y_shift, mode),
+        "DynamicQuantizeLinear");
+    return;
+  }
   c.dql_unchecked = c.dql.grid_blocks != 0;
   call.check(
       launch_dynamic_quantize(c.stream, c.dql, dx, n, dy, ds, dz, y_shift),
@@ -1485,6 +1495,19 @@ void OMShutdownAccelMI355X(void) {
   }
 }
 
+void om_mi355x_SetQuantMode(OMTensor *anchor, int64_t mode) {
+  (void)anchor;
+  if (mode < 0 || mode > (OM_MI355X_QUANT_RECIPROCAL | OM_MI355X_QUANT_NO_ZERO_POINT)) {
+    fail(EINVAL, "om_mi355x_SetQuantMode: mode %lld is not a combination of "
+                 "OM_MI355X_QUANT_RECIPROCAL and OM_MI355X_QUANT_NO_ZERO_POINT",
+        (long long)mode);
+    return;
+  }
+  t_quant_mode = (int)mode;
+}
+
+int64_t om_mi355x_GetQuantMode(void) { return t_quant_mode; }
+
 // ---------------------------------------------------------------------------
 // ops
 // ---------------------------------------------------------------------------
@@ -1513,13 +1536,19 @@ void om_mi355x_QuantizeLinear(OMTensor *y_t, const OMTensor *x_t,
   Call call(t_ctx, "QuantizeLinear");
   if (!call.ok)
     return;
+  const int mode = t_quant_mode;
   const float *dx = (const float *)call.in(x);
   const float *ds = (const float *)call.in(sc);
-  const void *dz = zp_t ? call.in(zp) : nullptr;
+  // without zero points the one given only decides the output type
+  // (src/Conversion/ONNXToKrnl/Quantization/QuantizeLinear.cpp:231-237)
+  const void *dz = (zp_t && !(mode & OM_MI355X_QUANT_NO_ZERO_POINT))
+                       ? call.in(zp)
+                       : nullptr;
   void *dy = call.out(y);
   if (call.ok)
     call.check(launch_quantize(call.c.stream, dx, outer, channels, inner, ds,
-                   dz, y.dtype == OM_MI355X_TYPE_INT8, dy),
+                   dz, y.dtype == OM_MI355X_TYPE_INT8, dy,
+                   (mode & OM_MI355X_QUANT_RECIPROCAL) != 0),
         "QuantizeLinear");
   call.finish();
 }
@@ -1551,7 +1580,10 @@ void om_mi355x_DequantizeLinear(OMTensor *y_t, const OMTensor *x_t,
     return;
   const void *dx = call.in(x);
   const float *ds = (const float *)call.in(sc);
-  const void *dz = zp_t ? call.in(zp) : nullptr;
+  // (src/Conversion/ONNXToKrnl/Math/Elementwise.cpp:1453)
+  const void *dz = (zp_t && !(t_quant_mode & OM_MI355X_QUANT_NO_ZERO_POINT))
+                       ? call.in(zp)
+                       : nullptr;
   float *dy = (float *)call.out(y);
   const QKind kind = x.dtype == OM_MI355X_TYPE_UINT8  ? kU8
                      : x.dtype == OM_MI355X_TYPE_INT8 ? kI8
@@ -1668,7 +1700,7 @@ void om_mi355x_DynamicQuantizeLinearNoAlloc(OMTensor *y_t, OMTensor *scale_t,
   if (e == hipSuccess)
     e = launch_dynamic_quantize(c.stream, s, (const float *)dev_ptr[3],
         x.numel, (uint8_t *)dev_ptr[0], (float *)dev_ptr[1],
-        (uint8_t *)dev_ptr[2], false);
+        (uint8_t *)dev_ptr[2], false, t_quant_mode);
   g_scratch_epoch[dev] = s.epoch;
   if (e != hipSuccess)
     fail(EIO, "%s failed: %s", op, hipGetErrorString(e));
@@ -1751,7 +1783,7 @@ void om_mi355x_DynQuantMatMulDequant(OMTensor *y_t, const OMTensor *x_t,
   int64_t padded_k = 0;
   GemmArgs g = {};
   g.out = call.out(y); // before the quantization: it decides whether to wait
-  if (call.ok && gemm_quantizes_rows(M, K, dx)) {
+  if (call.ok && t_quant_mode == 0 && gemm_quantizes_rows(M, K, dx)) {
     // A few rows (decode): the GEMM kernel quantizes them itself.
     g.X = dx;
   } else {

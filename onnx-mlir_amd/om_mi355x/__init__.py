@@ -40,8 +40,11 @@ _NP_TO_ONNX = {
 WRAP, SATURATE = 0, 1
 # `activation` of the fused entry points (OM_MI355X_ACTIVATION_* of the header)
 ACTIVATION_NONE, ACTIVATION_RELU, ACTIVATION_GELU = 0, 1, 2
+# bits of set_quant_mode (OM_MI355X_QUANT_* of the header): the reference's
+# --enable-fast-math and --disable-quantization-zero-point
+QUANT_RECIPROCAL, QUANT_NO_ZERO_POINT = 1, 2
 # OM_MI355X_VERSION of the header this module was written against
-VERSION = 0x00010000
+VERSION = 0x00010100
 
 
 class RuntimeError_(RuntimeError):
@@ -117,6 +120,9 @@ def _declare(lib, shim):
     lib.om_mi355x_last_error.restype = ctypes.c_char_p
     lib.om_mi355x_last_gemm_kernel.restype = ctypes.c_char_p
     lib.om_mi355x_device_info.restype = ctypes.c_int
+    lib.om_mi355x_SetQuantMode.restype = None
+    lib.om_mi355x_SetQuantMode.argtypes = [ctypes.c_void_p, ctypes.c_int64]
+    lib.om_mi355x_GetQuantMode.restype = ctypes.c_int64
     lib.om_mi355x_mfma_ceiling.restype = ctypes.c_int
     lib.om_mi355x_mfma_ceiling.argtypes = [ctypes.c_int64, ctypes.POINTER(ctypes.c_double),
                                            ctypes.POINTER(ctypes.c_double)]
@@ -138,6 +144,22 @@ def device_info() -> dict:
     name, arch, cus, mhz, gib = buf.value.decode().split("|")
     return {"name": name, "arch": arch, "cus": int(cus), "clock_mhz": int(mhz),
             "mem_gib": float(gib)}
+
+
+def set_quant_mode(mode: int) -> None:
+    """How this thread's later QuantizeLinear / DequantizeLinear /
+    DynamicQuantizeLinear calls (and the fused entry points) compute: 0 as the
+    reference does by default, or QUANT_RECIPROCAL | QUANT_NO_ZERO_POINT as it
+    does when compiled with --enable-fast-math /
+    --disable-quantization-zero-point."""
+    load()
+    _lib.om_mi355x_SetQuantMode(None, ctypes.c_int64(int(mode)))
+    _check()
+
+
+def quant_mode() -> int:
+    load()
+    return int(_lib.om_mi355x_GetQuantMode())
 
 
 def mfma_ceiling(random_operands: bool = True) -> dict:

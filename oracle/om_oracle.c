@@ -250,6 +250,72 @@ void om_oracle_dynamic_quantize_linear(
     y[i] = quant_one(x[i], s, zf, 1, OM_ORACLE_U8);
 }
 
+/* ---- the two compiler options that change this path's arithmetic --------
+ * OM_ORACLE_RECIPROCAL: --enable-fast-math at -O3
+ * (src/Compiler/CompilerPasses.cpp:298-301): the quotient x / scale becomes
+ * x * (1 / scale), the reciprocal one f32 divide per scale
+ * (QuantizeLinear.cpp:43-44,119-132; op order held by
+ * test/mlir/conversion/onnx_to_krnl/Quantization/
+ * QuantizeLinear_with_fast_math_canonicalize.mlir).
+ * OM_ORACLE_NO_ZERO_POINT: --disable-quantization-zero-point
+ * (src/Compiler/CompilerOptions.cpp:255-262): QuantizeLinear and
+ * DequantizeLinear ignore a zero point they are given (QuantizeLinear.cpp
+ * :231-237, Elementwise.cpp:1453); DynamicQuantizeLinear keeps its scale
+ * formula, returns a zero point of 0 and adds none
+ * (DynamicQuantizeLinear.cpp:75-84,142-152; held by
+ * .../Quantization/QuantizationWithoutZeroPoint.mlir).
+ * Pinned in tests/test_oracle.py by numpy's binary32 arithmetic on inputs
+ * where the reciprocal form and the divide round differently. */
+static inline uint8_t quant_one_mode(
+    float x, float scale, float recip, float zpf, int has_zp, int qkind,
+    int mode) {
+  float t = (mode & OM_ORACLE_RECIPROCAL) ? x * recip : x / scale;
+  float r = om_oracle_rne(t);
+  if (has_zp)
+    r = r + zpf;
+  if (qkind == OM_ORACLE_U8) {
+    float c = clipf(r, 0.0f, 255.0f);
+    return (uint8_t)(uint32_t)c;
+  }
+  float c = clipf(r, -128.0f, 127.0f);
+  return (uint8_t)(int8_t)(int32_t)c;
+}
+
+void om_oracle_quantize_linear_mode(const float *x, int64_t outer,
+    int64_t channels, int64_t inner, const float *scale, const void *zp,
+    int qkind, void *y, int mode) {
+  uint8_t *out = (uint8_t *)y;
+  const int has_zp = zp != NULL && !(mode & OM_ORACLE_NO_ZERO_POINT);
+  for (int64_t o = 0; o < outer; ++o)
+    for (int64_t c = 0; c < channels; ++c) {
+      float s = scale[c];
+      float recip = 1.0f / s;
+      float zpf = has_zp ? load_q_as_f32(zp, qkind, c) : 0.0f;
+      int64_t base = (o * channels + c) * inner;
+#pragma omp parallel for schedule(static) if (inner > 65536)
+      for (int64_t i = 0; i < inner; ++i)
+        out[base + i] =
+            quant_one_mode(x[base + i], s, recip, zpf, has_zp, qkind, mode);
+    }
+}
+
+void om_oracle_dynamic_quantize_linear_mode(const float *x, int64_t n,
+    uint8_t *y, float *scale, uint8_t *zp, int mode) {
+  float mn, mx, s, zf;
+  om_oracle_minmax(x, n, &mn, &mx);
+  om_oracle_dynamic_params(mn, mx, &s, &zf, zp);
+  const int want_zp = !(mode & OM_ORACLE_NO_ZERO_POINT);
+  if (!want_zp) {
+    zf = 0.0f;
+    *zp = 0;
+  }
+  *scale = s;
+  const float recip = 1.0f / s;
+#pragma omp parallel for schedule(static) if (n > 65536)
+  for (int64_t i = 0; i < n; ++i)
+    y[i] = quant_one_mode(x[i], s, recip, zf, want_zp, OM_ORACLE_U8, mode);
+}
+
 /* The reference with --parallel reduces in 8 chunks and then across the 8
  * partial results (tNum = 8, src/Conversion/ONNXToKrnl/Math/Reduction.cpp
  * :466-515); the quantize loop is one more parallel pass over X. */

@@ -39,6 +39,9 @@ extern "C" {
 /* Element kinds for the quantized side. */
 enum { OM_ORACLE_U8 = 0, OM_ORACLE_I8 = 1, OM_ORACLE_I32 = 2 };
 
+/* Compiler options that change the quantize arithmetic (bits of `mode`). */
+enum { OM_ORACLE_RECIPROCAL = 1, OM_ORACLE_NO_ZERO_POINT = 2 };
+
 /* QLinearMatMul narrowing modes. */
 enum { OM_ORACLE_WRAP = 0, OM_ORACLE_SATURATE = 1 };
 
@@ -95,6 +98,15 @@ void om_oracle_qlinear_matmul(const void *A, int akind, float a_scale,
     float b_scale, const void *b_zp, int64_t b_zp_len, float y_scale,
     const void *y_zp, int ykind, int64_t M, int64_t K, int64_t N, int mode,
     void *Y);
+
+/* QuantizeLinear / DynamicQuantizeLinear as compiled with --enable-fast-math
+ * (mode & 1: x * (1 / scale)) and / or --disable-quantization-zero-point
+ * (mode & 2).  mode 0 equals the functions without the suffix. */
+void om_oracle_quantize_linear_mode(const float *x, int64_t outer,
+    int64_t channels, int64_t inner, const float *scale, const void *zp,
+    int qkind, void *y, int mode);
+void om_oracle_dynamic_quantize_linear_mode(const float *x, int64_t n,
+    uint8_t *y, float *scale, uint8_t *zp, int mode);
 
 /* out[i,j] = f32(acc[i,j]) * (a_scale * b_scale[j or 0]). */
 void om_oracle_dequant_epilogue(const int32_t *acc, int64_t M, int64_t N,

@@ -14,6 +14,7 @@ ORACLE_SO = os.path.join(ORACLE_DIR, "libom_oracle.so")
 
 U8, I8, I32 = 0, 1, 2
 WRAP, SATURATE = 0, 1
+RECIPROCAL, NO_ZERO_POINT = 1, 2   # bits of `mode` (compiler options that change the arithmetic)
 
 _KIND = {np.dtype(np.uint8): U8, np.dtype(np.int8): I8, np.dtype(np.int32): I32}
 
@@ -47,6 +48,10 @@ class Oracle:
         for name in ("om_oracle_dynamic_quantize_linear", "om_oracle_dynamic_quantize_linear_omp"):
             getattr(lib, name).restype = None
             getattr(lib, name).argtypes = [P, I64, P, P, P]
+        lib.om_oracle_quantize_linear_mode.restype = None
+        lib.om_oracle_quantize_linear_mode.argtypes = [P, I64, I64, I64, P, P, I, P, I]
+        lib.om_oracle_dynamic_quantize_linear_mode.restype = None
+        lib.om_oracle_dynamic_quantize_linear_mode.argtypes = [P, I64, P, P, P, I]
         for name in ("om_oracle_matmul_integer", "om_oracle_matmul_integer_passes"):
             getattr(lib, name).restype = None
             getattr(lib, name).argtypes = [P, I, P, I, I64, I64, I64, P, I64, P, I64, P]
@@ -90,6 +95,28 @@ class Oracle:
         fn = self.lib.om_oracle_quantize_linear_omp if omp else self.lib.om_oracle_quantize_linear
         fn(_p(x), outer, ch, inner, _p(scale), _p(zp), _KIND[np.dtype(out_dtype)], _p(y))
         return y
+
+    def quantize_linear_mode(self, x, scale, zp, mode, axis=1, out_dtype=np.uint8):
+        """QuantizeLinear as compiled with the options in `mode` (RECIPROCAL |
+        NO_ZERO_POINT); the output type still follows the zero point's."""
+        x = np.ascontiguousarray(x, np.float32)
+        scale = np.ascontiguousarray(scale, np.float32).reshape(-1)
+        if zp is not None:
+            zp = np.ascontiguousarray(zp).reshape(-1)
+            out_dtype = zp.dtype
+        y = np.empty(x.shape, out_dtype)
+        outer, ch, inner = self._split(x.shape, scale, axis)
+        self.lib.om_oracle_quantize_linear_mode(_p(x), outer, ch, inner, _p(scale), _p(zp),
+                                                _KIND[np.dtype(out_dtype)], _p(y), int(mode))
+        return y
+
+    def dynamic_quantize_linear_mode(self, x, mode):
+        x = np.ascontiguousarray(x, np.float32)
+        y = np.empty(x.shape, np.uint8)
+        s, z = ctypes.c_float(), ctypes.c_uint8()
+        self.lib.om_oracle_dynamic_quantize_linear_mode(_p(x), x.size, _p(y), ctypes.byref(s),
+                                                        ctypes.byref(z), int(mode))
+        return y, np.float32(s.value), np.uint8(z.value)
 
     def dequantize_linear(self, x, scale, zp=None, axis=1, omp=False):
         x = np.ascontiguousarray(x)

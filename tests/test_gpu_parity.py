@@ -121,6 +121,107 @@ def test_quantize_every_input_that_does_not_saturate(rt, oracle, qdt):
                 assert np.array_equal(got, want), (float(s), hex(start), sign)
 
 
+@pytest.fixture
+def quant_mode(rt):
+    """Sets the thread's quantization mode for a test and puts 0 back."""
+    def set_mode(mode):
+        rt.set_quant_mode(mode)
+    yield set_mode
+    rt.set_quant_mode(0)
+
+
+@pytest.mark.parametrize("mode", [1, 2, 3])
+def test_quantize_dequantize_under_the_compiler_options(rt, oracle, quant_mode, mode):
+    """om_mi355x_SetQuantMode: QuantizeLinear with the quotient as x * (1 / scale)
+    (--enable-fast-math) and / or without its zero point
+    (--disable-quantization-zero-point), DequantizeLinear without its zero
+    point, against the oracle's restatement of those lowerings: per-tensor at
+    sizes around the kernels' vector width, on a sample where reciprocal and
+    divide differ, with special values and scales from tiny to huge; per-axis on
+    the last and on an inner axis; misaligned device views."""
+    quant_mode(mode)
+    assert rt.quant_mode() == mode
+    rng = np.random.default_rng(300 + mode)
+    sep = np.arange(1, 1601, dtype=np.float32) * np.float32(0.15)   # x / 0.3 against x * (1 / 0.3)
+    for qdt in (np.uint8, np.int8):
+        zp = np.array(7 if qdt == np.uint8 else -9, qdt)
+        for n in (1, 3, 4, 5, 1023, 4097, (1 << 20) + 3):
+            x = rng.normal(0, 40, n).astype(np.float32)
+            x[: min(n, SPECIALS.size)] = SPECIALS[: min(n, SPECIALS.size)]
+            if n > 4000:
+                x[100:1700] = sep
+            for s in (0.3, 0.0173, 1e-38, 3e38, 2.0 ** -100):
+                want = oracle.quantize_linear_mode(x, np.float32(s), zp, mode)
+                got = rt.QuantizeLinear(x, np.float32(s), zp)
+                assert got.dtype == qdt and np.array_equal(got, want), (qdt, n, s)
+        if mode & 1:   # the sample does separate the two forms
+            a = oracle.quantize_linear_mode(sep, np.float32(0.3), zp, mode)
+            b = oracle.quantize_linear_mode(sep, np.float32(0.3), zp, mode & 2)
+            assert (a != b).any()
+        # per-axis: last axis and an inner axis
+        for shape, axis in (((37, 100), 1), ((5, 6, 70), 1), ((300, 4099), 1)):
+            x = rng.normal(0, 30, shape).astype(np.float32)
+            sc = rng.uniform(0.05, 2.0, shape[axis]).astype(np.float32)
+            z = _rand_q(rng, qdt, (shape[axis],))
+            assert np.array_equal(rt.QuantizeLinear(x, sc, z, axis=axis),
+                                  oracle.quantize_linear_mode(x, sc, z, mode, axis=axis)), (shape, axis)
+            q = _rand_q(rng, qdt, shape)
+            want = oracle.dequantize_linear(q, sc, None if mode & 2 else z, axis=axis)
+            assert same_f32(rt.DequantizeLinear(q, sc, z, axis=axis), want), (shape, axis)
+        q = _rand_q(rng, qdt, (70001,))
+        want = oracle.dequantize_linear(q, np.float32(0.02), None if mode & 2 else zp)
+        assert same_f32(rt.DequantizeLinear(q, np.float32(0.02), zp), want)
+    # a device view 4 bytes off the 16-byte grid (input) and 1 byte off (output)
+    n = 5000
+    x = rng.normal(0, 40, n + 1).astype(np.float32)
+    dx = rt.DeviceArray.from_numpy(x)
+    dy = rt.DeviceArray.from_numpy(np.full(n + 8, 0xAB, np.uint8))
+    zp = np.array(9, np.uint8)
+    rt.QuantizeLinear(rt.DeviceArray.view_of(dx, 1, (n,)), np.float32(0.3), zp, out=rt.DeviceArray.view_of(dy, 1, (n,)))
+    rt.synchronize()
+    whole = dy.numpy()
+    assert whole[0] == 0xAB and (whole[n + 1:] == 0xAB).all()
+    assert np.array_equal(whole[1:n + 1], oracle.quantize_linear_mode(x[1:], np.float32(0.3), zp, mode))
+    dx.free()
+    dy.free()
+    with pytest.raises(rt.RuntimeError_, match="SetQuantMode"):
+        rt.set_quant_mode(4)
+    assert rt.quant_mode() == mode
+
+
+@pytest.mark.parametrize("mode", [1, 2, 3])
+def test_dynamic_quantize_under_the_compiler_options(rt, oracle, quant_mode, mode):
+    """DynamicQuantizeLinear and the fused layer under om_mi355x_SetQuantMode:
+    zero point 0 and not added without zero points, reciprocal quotient with
+    fast math, the scale unchanged; sizes that take the one-block kernel and the
+    two-launch path, device-resident operands, and the whole layer
+    (DynQuantMatMulDequant) at few rows and at many."""
+    quant_mode(mode)
+    rng = np.random.default_rng(310 + mode)
+    for n, lo, hi in ((1, -1, 1), (100, 0.5, 9), (4096, -3, 5), (16385, -7, -1), (100003, -3, 5), (1 << 20, -2, 6)):
+        x = rng.uniform(lo, hi, n).astype(np.float32)
+        y, s, z = rt.DynamicQuantizeLinear(x)
+        wy, ws, wz = oracle.dynamic_quantize_linear_mode(x, mode)
+        assert s == ws and z == wz and np.array_equal(y, wy), (n, lo, hi)
+        if mode & 2:
+            assert z == 0
+    x = rng.uniform(-3, 5, (512, 768)).astype(np.float32)
+    dX = rt.DeviceArray.from_numpy(x)
+    dy, ds, dz = rt.DynamicQuantizeLinear(dX)
+    rt.synchronize()
+    wy, ws, wz = oracle.dynamic_quantize_linear_mode(x, mode)
+    assert np.array_equal(dy.numpy(), wy) and ds.numpy() == ws and dz.numpy() == wz
+    for d in (dX, dy, ds, dz):
+        d.free()
+    for M, K, N in ((4, 4096, 256), (300, 768, 1000), (512, 768, 3072)):
+        x = rng.uniform(-2, 3, (M, K)).astype(np.float32)
+        W = _rand_q(rng, np.int8, (K, N))
+        ws_ = rng.uniform(1e-3, 1e-2, N).astype(np.float32)
+        aq, a_s, a_zp = oracle.dynamic_quantize_linear_mode(x, mode)
+        want = oracle.dequant_epilogue(oracle.matmul_integer(aq, W, a_zp, None), a_s, ws_)
+        assert same_f32(rt.DynQuantMatMulDequant(x, W, None, ws_), want), (M, K, N)
+
+
 def test_quantize_zero_and_denormal_scale(rt, oracle):
     x = np.array([0.0, -0.0, 1.0, -1.0, np.nan, 3e-45, -3e-45], np.float32)
     for s in (0.0, 1e-45, 1e-39):

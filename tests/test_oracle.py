@@ -144,6 +144,62 @@ def test_quantize_uses_true_division_not_reciprocal(oracle):
     assert np.array_equal(got, want)
 
 
+def test_quantize_and_dql_under_the_two_compiler_options(oracle):
+    """--enable-fast-math (x * (1 / scale), QuantizeLinear.cpp:43-44,119-132) and
+    --disable-quantization-zero-point (QuantizeLinear.cpp:231-237,
+    DynamicQuantizeLinear.cpp:75-84,142-152) against numpy's binary32
+    arithmetic, on a sample where the reciprocal form and the divide differ
+    within the unsaturated range (so taking one for the other fails), with a
+    zero point that must be added in one mode and ignored in the other."""
+    R, NZ = oracle_lib.RECIPROCAL, oracle_lib.NO_ZERO_POINT
+    s = np.float32(0.3)
+    x = np.concatenate([np.arange(1, 1601, dtype=np.float32) * np.float32(0.15),
+                        -np.arange(1, 801, dtype=np.float32) * np.float32(0.15),
+                        np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1e30, 3e-39], np.float32)])
+    r = np.float32(1.0) / s
+    with np.errstate(all="ignore"):
+        d, m = np.rint(x / s), np.rint(x * r)
+    inside = (np.abs(d) < 120) & (d != m)
+    assert inside.any(), "sample does not separate divide from reciprocal"
+
+    def clip(v, dt):
+        lo, hi = (0, 255) if dt == np.uint8 else (-128, 127)
+        v = np.where(np.isnan(v), lo, v)          # maxnum then minnum: NaN -> lower bound
+        return np.clip(v, lo, hi).astype(np.int64).astype(dt)
+
+    for dt, zp in ((np.uint8, 7), (np.int8, -9)):
+        z = np.array(zp, dt)
+        for mode in (0, R, NZ, R | NZ):
+            t = m if mode & R else d
+            want = clip(t + (0 if mode & NZ else np.float32(zp)), dt)
+            got = oracle.quantize_linear_mode(x, s, z, mode)
+            assert got.dtype == dt and np.array_equal(got, want), (dt, mode)
+        assert np.array_equal(oracle.quantize_linear_mode(x, s, z, 0), oracle.quantize_linear(x, s, z))
+    # per-axis: scale[c], 1 / scale[c]
+    xs = np.stack([x, x * 2], axis=1)
+    sc = np.array([0.3, 0.7], np.float32)
+    got = oracle.quantize_linear_mode(xs, sc, np.array([7, 3], np.uint8), R)
+    with np.errstate(all="ignore"):
+        want = np.stack([clip(np.rint(xs[:, c] * (np.float32(1) / sc[c])) + np.float32((7, 3)[c]), np.uint8)
+                         for c in range(2)], axis=1)
+    assert np.array_equal(got, want)
+    # DynamicQuantizeLinear: the scale formula is untouched; the zero point is 0
+    # and not added without zero points; the quotient by reciprocal with fast math
+    rng = np.random.default_rng(95)
+    for lo, hi in ((-3.0, 5.0), (0.5, 9.0), (-7.0, -1.0)):
+        v = rng.uniform(lo, hi, 5000).astype(np.float32)
+        y0, s0, z0 = oracle.dynamic_quantize_linear(v)
+        for mode in (0, R, NZ, R | NZ):
+            y, sc1, z = oracle.dynamic_quantize_linear_mode(v, mode)
+            assert sc1 == s0
+            zf = np.float32(0 if mode & NZ else z0)
+            assert z == (0 if mode & NZ else z0)
+            with np.errstate(all="ignore"):
+                t = np.rint(v * (np.float32(1) / s0)) if mode & R else np.rint(v / s0)
+            assert np.array_equal(y, clip(t + zf, np.uint8)), (lo, hi, mode)
+        assert np.array_equal(oracle.dynamic_quantize_linear_mode(v, 0)[0], y0)
+
+
 def test_quantize_special_values(oracle):
     x = np.array([np.nan, np.inf, -np.inf, 1e30, -1e30, 0.0, -0.0], np.float32)
     y = oracle.quantize_linear(x, np.float32(0.1), np.array(10, np.uint8))
