@@ -547,6 +547,49 @@ __global__ __launch_bounds__(kThreads) void k_quant_flat_reciprocal(
   }
 }
 
+// The same form with a scale per column of a [rows, C] tensor (per-axis on the
+// last axis): a thread takes four consecutive elements of the flat array,
+// finds their columns (one 32-bit remainder, then steps with wrap-around) and
+// gathers scale and zero point for each; x 16-byte and y 4-byte aligned, fewer
+// than 2^32 elements.
+template <bool SIGNED, bool HAS_ZP>
+__global__ __launch_bounds__(kThreads) void k_quant_lastaxis_reciprocal(
+    const float *__restrict__ x, uint8_t *__restrict__ y, uint32_t n,
+    uint32_t C, const float *__restrict__ scale, const void *__restrict__ zp) {
+  const uint32_t nvec = n >> 2;
+  const f4a *__restrict__ x4 = (const f4a *)x;
+  uint32_t *__restrict__ y4 = (uint32_t *)y;
+  const uint32_t base = blockIdx.x * (uint32_t)(kThreads * 2) + threadIdx.x;
+  f4a v[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j)
+    if (base + j * kThreads < nvec)
+      v[j] = __builtin_nontemporal_load(&x4[base + j * kThreads]);
+  auto one = [&](float xe, uint32_t c) {
+    const float s = scale[c];
+    const float zpf = HAS_ZP ? load_zp_f32<SIGNED>(zp, c) : 0.0f;
+    return quant_one<SIGNED, HAS_ZP, 2>(xe, s, zpf, 1.0f / s);
+  };
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const uint32_t idx = base + j * kThreads;
+    if (idx < nvec) {
+      uint32_t c[4];
+      c[0] = (idx << 2) % C;
+#pragma unroll
+      for (int k = 1; k < 4; ++k)
+        c[k] = c[k - 1] + 1 == C ? 0 : c[k - 1] + 1;
+      q_store(&y4[idx], one(v[j].x, c[0]) | (one(v[j].y, c[1]) << 8) |
+                            (one(v[j].z, c[2]) << 16) | (one(v[j].w, c[3]) << 24));
+    }
+  }
+  if (blockIdx.x == 0) {
+    const uint32_t e = (nvec << 2) + threadIdx.x;
+    if (e < n)
+      y[e] = (uint8_t)one(x[e], e % C);
+  }
+}
+
 template <bool SIGNED, bool HAS_ZP, bool RECIP = false>
 __global__ __launch_bounds__(kThreads) void k_quant_general(
     const float *__restrict__ x, uint8_t *__restrict__ y, int64_t channels,
@@ -1778,6 +1821,16 @@ hipError_t quantize_dispatch(hipStream_t st, const float *x, int64_t outer,
     }
     if (flip != 0)
       return hipErrorInvalidValue;
+    if (channels > 1 && inner == 1 && aligned && n < ((int64_t)1 << 32)) {
+      const unsigned grid = (unsigned)(blocks > 0 ? blocks : 1);
+      if (has_zp)
+        k_quant_lastaxis_reciprocal<SIGNED, true><<<grid, kThreads, 0, st>>>(
+            x, yo, (uint32_t)n, (uint32_t)channels, scale, zp);
+      else
+        k_quant_lastaxis_reciprocal<SIGNED, false><<<grid, kThreads, 0, st>>>(
+            x, yo, (uint32_t)n, (uint32_t)channels, scale, zp);
+      return hipGetLastError();
+    }
     if (channels == 1) {
       outer = 1;
       inner = n;
