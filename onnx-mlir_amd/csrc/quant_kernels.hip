@@ -79,7 +79,7 @@ __device__ __forceinline__ uint32_t quant_four(
          flip;
 }
 // Four elements with a scale each (four adjacent columns of a per-axis op).
-template <bool SIGNED, bool HAS_ZP, bool FAST, typename V4>
+template <bool SIGNED, bool HAS_ZP, int FAST, typename V4>
 __device__ __forceinline__ uint32_t quant_cols(V4 v, const float (&s)[4],
     const float (&r)[4], const float (&z)[4]) {
   return quant_pack4<SIGNED, HAS_ZP, FAST>(v.x, v.y, v.z, v.w, s[0], s[1], s[2],
@@ -544,6 +544,95 @@ __global__ __launch_bounds__(kThreads) void k_quant_flat_reciprocal(
     const int64_t e = (nvec << 2) + threadIdx.x;
     if (e < n)
       y[e] = (uint8_t)(quant_one<SIGNED, HAS_ZP, 2>(x[e], s, zpf, r) ^ (flip & 0xFFu));
+  }
+}
+
+// ---- per-axis on an inner axis whose slabs are not whole float4 --------------
+// [outer, channels, inner] with inner >= 4 and inner % 4 != 0 (an NCHW
+// activation with 7 x 7 or 57 x 57 pixels a channel): the flat array is walked
+// in aligned float4 all the same; the four elements of a vector lie in at most
+// two consecutive slabs, so a thread finds the channel of its first element
+// (one 32-bit division by `inner`, one remainder by `channels`), takes the
+// parameters of that channel and of the next, and picks per element.  Blocks
+// of two vectors per thread, one trip.  x 16-byte and y 4-byte aligned (the
+// other way round for dequantize), fewer than 2^32 elements.
+struct GatherPos {
+  uint32_t ca, cb; // channel of the vector's first element, and the one after
+  uint32_t na;     // how many of the four elements belong to ca
+};
+__device__ __forceinline__ GatherPos gather_pos(
+    uint32_t e0, uint32_t channels, uint32_t inner) {
+  const uint32_t slab = e0 / inner;
+  const uint32_t left = inner - (e0 - slab * inner); // elements to the slab's end
+  GatherPos p;
+  p.ca = slab % channels;
+  p.cb = p.ca + 1 == channels ? 0 : p.ca + 1;
+  p.na = left < 4 ? left : 4;
+  return p;
+}
+
+// QMODE2: the reference's fast-math form (quotient<2>); otherwise the divide,
+// or its corrected-reciprocal equivalent when every scale in the wave is tame.
+template <bool SIGNED, bool HAS_ZP, bool QMODE2>
+__global__ __launch_bounds__(kThreads) void k_quant_gather(
+    const float *__restrict__ x, uint8_t *__restrict__ y, uint32_t n,
+    uint32_t channels, uint32_t inner, const float *__restrict__ scale,
+    const void *__restrict__ zp) {
+  const uint32_t nvec = n >> 2;
+  const f4a *__restrict__ x4 = (const f4a *)x;
+  uint32_t *__restrict__ y4 = (uint32_t *)y;
+  const uint32_t base = blockIdx.x * (uint32_t)(kThreads * 2) + threadIdx.x;
+  f4a v[2];
+  GatherPos pos[2];
+  float sa[2], sb[2], za[2], zb[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const uint32_t idx = base + j * kThreads;
+    if (idx < nvec)
+      v[j] = __builtin_nontemporal_load(&x4[idx]);
+    pos[j] = gather_pos((idx < nvec ? idx : 0) << 2, channels, inner);
+    sa[j] = scale[pos[j].ca];
+    sb[j] = scale[pos[j].cb];
+    za[j] = HAS_ZP ? load_zp_f32<SIGNED>(zp, pos[j].ca) : 0.0f;
+    zb[j] = HAS_ZP ? load_zp_f32<SIGNED>(zp, pos[j].cb) : 0.0f;
+  }
+  auto finish = [&](auto qmode_c) {
+    constexpr int QM = decltype(qmode_c)::value;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const uint32_t idx = base + j * kThreads;
+      if (idx >= nvec)
+        continue;
+      const float ra = 1.0f / sa[j], rb = 1.0f / sb[j];
+      float s[4], r[4], z[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const bool first = (uint32_t)k < pos[j].na;
+        s[k] = first ? sa[j] : sb[j];
+        r[k] = first ? ra : rb;
+        z[k] = first ? za[j] : zb[j];
+      }
+      q_store(&y4[idx], quant_cols<SIGNED, HAS_ZP, QM>(v[j], s, r, z));
+    }
+  };
+  if (QMODE2) {
+    finish(std::integral_constant<int, 2>{});
+  } else {
+    const bool tame = scale_is_tame(sa[0]) && scale_is_tame(sb[0]) &&
+                      scale_is_tame(sa[1]) && scale_is_tame(sb[1]);
+    if (wave_all(tame))
+      finish(std::integral_constant<int, 1>{});
+    else
+      finish(std::integral_constant<int, 0>{});
+  }
+  if (blockIdx.x == 0) {
+    const uint32_t e = (nvec << 2) + threadIdx.x;
+    if (e < n) {
+      const uint32_t c = (e / inner) % channels;
+      const float s1 = scale[c];
+      const float z1 = HAS_ZP ? load_zp_f32<SIGNED>(zp, c) : 0.0f;
+      y[e] = (uint8_t)quant_one<SIGNED, HAS_ZP, QMODE2 ? 2 : 0>(x[e], s1, z1, 1.0f / s1);
+    }
   }
 }
 
@@ -1316,6 +1405,54 @@ __global__ __launch_bounds__(kThreads) void k_dequant8_slabs(
   }
 }
 
+// The dequantize side of k_quant_gather: one dword of four 8-bit values in,
+// one float4 out, parameters of two consecutive channels picked per element.
+template <int KIND, bool HAS_ZP>
+__global__ __launch_bounds__(kThreads) void k_dequant8_gather(
+    const uint8_t *__restrict__ x, float *__restrict__ y, uint32_t n,
+    uint32_t channels, uint32_t inner, const float *__restrict__ scale,
+    const void *__restrict__ zp) {
+  const uint32_t nvec = n >> 2;
+  const uint32_t *__restrict__ x4 = (const uint32_t *)x;
+  f4a *__restrict__ y4 = (f4a *)y;
+  const uint32_t base = blockIdx.x * (uint32_t)(kThreads * 2) + threadIdx.x;
+  uint32_t w[2];
+  GatherPos pos[2];
+  float sa[2], sb[2], za[2], zb[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const uint32_t idx = base + j * kThreads;
+    w[j] = idx < nvec ? __builtin_nontemporal_load(&x4[idx]) : 0u;
+    pos[j] = gather_pos((idx < nvec ? idx : 0) << 2, channels, inner);
+    sa[j] = scale[pos[j].ca];
+    sb[j] = scale[pos[j].cb];
+    za[j] = HAS_ZP ? load_q_zp_f32<KIND>(zp, pos[j].ca) : 0.0f;
+    zb[j] = HAS_ZP ? load_q_zp_f32<KIND>(zp, pos[j].cb) : 0.0f;
+  }
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const uint32_t idx = base + j * kThreads;
+    if (idx >= nvec)
+      continue;
+    float o[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const bool first = (uint32_t)k < pos[j].na;
+      o[k] = dq_one<HAS_ZP>(q_to_f32<KIND>(w[j] >> (8 * k)),
+          first ? sa[j] : sb[j], first ? za[j] : zb[j]);
+    }
+    dq_store((f4a){o[0], o[1], o[2], o[3]}, &y4[idx]);
+  }
+  if (blockIdx.x == 0) {
+    const uint32_t e = (nvec << 2) + threadIdx.x;
+    if (e < n) {
+      const uint32_t c = (e / inner) % channels;
+      y[e] = dq_one<HAS_ZP>(q_to_f32<KIND>(x[e]), scale[c],
+          HAS_ZP ? load_q_zp_f32<KIND>(zp, c) : 0.0f);
+    }
+  }
+}
+
 template <int KIND, bool HAS_ZP>
 __global__ __launch_bounds__(kThreads) void k_dequant_general(
     const void *__restrict__ x, float *__restrict__ y, int64_t channels,
@@ -1794,6 +1931,17 @@ PeriodicGrid periodic_grid(int64_t nvec, int64_t C, int trips) {
   return pg;
 }
 
+// Shapes the gathering kernels take: per-axis on an inner axis, slabs of at
+// least four elements (a vector then spans two channels at most), everything
+// indexable in 32 bits.
+bool gather_ok(int64_t n, int64_t channels, int64_t inner) {
+  return channels > 1 && inner >= 4 && n < ((int64_t)1 << 32);
+}
+unsigned gather_grid(int64_t n) {
+  const int64_t blocks = ((n >> 2) + kThreads * 2 - 1) / (kThreads * 2);
+  return (unsigned)(blocks > 0 ? blocks : 1);
+}
+
 template <bool SIGNED>
 hipError_t quantize_dispatch(hipStream_t st, const float *x, int64_t outer,
     int64_t channels, int64_t inner, const float *scale, const void *zp,
@@ -1829,6 +1977,16 @@ hipError_t quantize_dispatch(hipStream_t st, const float *x, int64_t outer,
       else
         k_quant_lastaxis_reciprocal<SIGNED, false><<<grid, kThreads, 0, st>>>(
             x, yo, (uint32_t)n, (uint32_t)channels, scale, zp);
+      return hipGetLastError();
+    }
+    if (aligned && gather_ok(n, channels, inner)) {
+      const unsigned grid = gather_grid(n);
+      if (has_zp)
+        k_quant_gather<SIGNED, true, true><<<grid, kThreads, 0, st>>>(x, yo,
+            (uint32_t)n, (uint32_t)channels, (uint32_t)inner, scale, zp);
+      else
+        k_quant_gather<SIGNED, false, true><<<grid, kThreads, 0, st>>>(x, yo,
+            (uint32_t)n, (uint32_t)channels, (uint32_t)inner, scale, zp);
       return hipGetLastError();
     }
     if (channels == 1) {
@@ -1950,6 +2108,17 @@ hipError_t quantize_dispatch(hipStream_t st, const float *x, int64_t outer,
     else
       k_quant_slabs<SIGNED, false, kSlabQuantPerThread>
           <<<grid, kThreads, 0, st>>>(x, yo, nvec, step, scale, zp);
+    return hipGetLastError();
+  }
+  if (gather_ok(n, channels, inner) && ((((uintptr_t)x) & 15) == 0) &&
+      ((((uintptr_t)y) & 3) == 0)) {
+    const unsigned grid = gather_grid(n);
+    if (has_zp)
+      k_quant_gather<SIGNED, true, false><<<grid, kThreads, 0, st>>>(x, yo,
+          (uint32_t)n, (uint32_t)channels, (uint32_t)inner, scale, zp);
+    else
+      k_quant_gather<SIGNED, false, false><<<grid, kThreads, 0, st>>>(x, yo,
+          (uint32_t)n, (uint32_t)channels, (uint32_t)inner, scale, zp);
     return hipGetLastError();
   }
   const int64_t oc = outer * channels;
@@ -2085,6 +2254,18 @@ hipError_t dequantize_dispatch(hipStream_t st, const void *x, int64_t outer,
       k_dequant8_slabs<(KIND == kI32 ? kU8 : KIND), false, kSlabDequantPerThread>
           <<<grid, kThreads, 0, st>>>(
               (const uint8_t *)x, y, nvec, step, scale, zp);
+    return hipGetLastError();
+  }
+  if (KIND != kI32 && gather_ok(n, channels, inner) &&
+      ((((uintptr_t)x) & 3) == 0) && ((((uintptr_t)y) & 15) == 0)) {
+    const unsigned grid = gather_grid(n);
+    constexpr int K8 = KIND == kI32 ? kU8 : KIND;
+    if (has_zp)
+      k_dequant8_gather<K8, true><<<grid, kThreads, 0, st>>>((const uint8_t *)x,
+          y, (uint32_t)n, (uint32_t)channels, (uint32_t)inner, scale, zp);
+    else
+      k_dequant8_gather<K8, false><<<grid, kThreads, 0, st>>>((const uint8_t *)x,
+          y, (uint32_t)n, (uint32_t)channels, (uint32_t)inner, scale, zp);
     return hipGetLastError();
   }
   const int64_t oc = outer * channels;

@@ -1057,6 +1057,57 @@ def test_per_axis_with_inner_slabs(rt, oracle):
                             oracle.dequantize_linear(wq, sc, zp, axis=axis)), tag
 
 
+@pytest.mark.parametrize("mode", [0, 1])
+def test_per_axis_with_inner_slabs_that_are_not_whole_vectors(rt, oracle, quant_mode, mode):
+    """Per-channel parameters on an inner axis whose slabs are not a whole number
+    of float4 (NCHW activations with 7 x 7 or 57 x 57 pixels a channel): walked
+    as flat vectors that span two channels at most.  Slabs from four elements
+    (the shortest that kernel takes) to thousands, one to many channels per
+    block, tensors that end inside a vector, scales that take the divide, the
+    three-element slabs that stay with the general kernel, device views off the
+    alignment the kernel needs; in the default mode and with the quotient as
+    x * (1 / scale)."""
+    quant_mode(mode)
+    rng = np.random.default_rng(9191 + mode)
+    cases = [((64, 33, 7, 7), 1), ((3, 5, 7), 1), ((2, 3, 4099), 1), ((1, 2, 5), 1), ((7, 4, 4), 1), ((2, 1000, 6), 1),
+             ((5, 9, 57, 57), 1), ((17, 2, 9), 0), ((3, 300, 13), 1), ((2, 2, 70001), 1), ((4, 6, 3), 1), ((1, 3, 5, 5), 1)]
+    for shape, axis in cases:
+        C = shape[axis]
+        x = rng.normal(0, 30, shape).astype(np.float32)
+        x.reshape(-1)[: min(x.size, SPECIALS.size)] = SPECIALS[: min(x.size, SPECIALS.size)]
+        for qdt, with_zp in ((np.uint8, True), (np.int8, True), (np.int8, False)):
+            sc = rng.uniform(0.05, 2.0, C).astype(np.float32)
+            sc[0] = np.float32(1e-38)       # not "tame": the whole wave takes the divide
+            zp = _rand_q(rng, qdt, (C,)) if with_zp else None
+            tag = (shape, axis, qdt.__name__, with_zp)
+            wq = oracle.quantize_linear_mode(x, sc, zp, mode, axis=axis, out_dtype=qdt)
+            assert np.array_equal(rt.QuantizeLinear(x, sc, zp, axis=axis) if with_zp else
+                                  rt.QuantizeLinear(x, sc, None, axis=axis).view(np.uint8),
+                                  wq if with_zp else oracle.quantize_linear_mode(x, sc, None, mode, axis=axis)), tag
+            q = _rand_q(rng, qdt, shape)
+            assert same_f32(rt.DequantizeLinear(q, sc, zp, axis=axis), oracle.dequantize_linear(q, sc, zp, axis=axis)), tag
+    # device views one element off: the kernel's alignment does not hold, results must
+    shape = (6, 10, 49)
+    n = int(np.prod(shape))
+    x = rng.normal(0, 30, n + 1).astype(np.float32)
+    sc, zp = rng.uniform(0.05, 2.0, 10).astype(np.float32), _rand_q(rng, np.uint8, (10,))
+    dx = rt.DeviceArray.from_numpy(x)
+    dq = rt.DeviceArray.from_numpy(np.full(n + 8, 0xAB, np.uint8))
+    rt.QuantizeLinear(rt.DeviceArray.view_of(dx, 1, shape), sc, zp, axis=1, out=rt.DeviceArray.view_of(dq, 1, shape))
+    rt.synchronize()
+    whole = dq.numpy()
+    want = oracle.quantize_linear_mode(x[1:].reshape(shape), sc, zp, mode, axis=1)
+    assert whole[0] == 0xAB and (whole[n + 1:] == 0xAB).all() and np.array_equal(whole[1:n + 1].reshape(shape), want)
+    dy = rt.DeviceArray.from_numpy(np.full(n + 8, -7.0, np.float32))
+    rt.DequantizeLinear(rt.DeviceArray.view_of(dq, 1, shape), sc, zp, axis=1, out=rt.DeviceArray.view_of(dy, 1, shape))
+    rt.synchronize()
+    whole = dy.numpy()
+    assert whole[0] == -7.0 and (whole[n + 1:] == -7.0).all()
+    assert same_f32(whole[1:n + 1].reshape(shape), oracle.dequantize_linear(want, sc, zp, axis=1))
+    for d in (dx, dq, dy):
+        d.free()
+
+
 def test_large_gemm_takes_the_wide_tile_path(rt, oracle):
     # big enough for the heuristic to pick the 128 x 256 B-streaming kernel on its own
     rng = np.random.default_rng(77)
