@@ -1913,8 +1913,8 @@ struct PeriodicGrid {
   int per_block;
 };
 PeriodicGrid periodic_grid(int64_t nvec, int64_t C, int trips) {
-  const int64_t g = (C % 2 == 0) ? 2 : 1; // C % 4 != 0 here
-  int64_t period = C / g;
+  const int64_t g = (C % 4 == 0) ? 4 : (C % 2 == 0) ? 2 : 1; // gcd(C, 4)
+  int64_t period = C / g; // float4 until the columns repeat
   while (period % 4 != 0)
     period *= 2;
   const int64_t want = 4 * kThreads;
@@ -1930,6 +1930,12 @@ PeriodicGrid periodic_grid(int64_t nvec, int64_t C, int trips) {
   pg.per_block = (int)per_block;
   return pg;
 }
+
+// Row lengths the periodic kernels are for: rows that are not whole float4
+// (a thread's columns differ from row to row), and short rows of whole float4
+// (fewer than 256 columns), which would leave most of a block of the
+// row-walking kernels without a column to work on ([1 Mi, 4]: 0.31 TB/s there).
+bool periodic_pays(int64_t C) { return C % 4 != 0 || C < 256; }
 
 // Shapes the gathering kernels take: per-axis on an inner axis, slabs of at
 // least four elements (a vector then spans two channels at most), everything
@@ -2054,7 +2060,7 @@ hipError_t quantize_dispatch(hipStream_t st, const float *x, int64_t outer,
           x, yo, n, outer, (uint32_t)channels, scale, zp, g);
     return hipGetLastError();
   }
-  if (inner == 1 && channels > 1 && channels % 4 != 0 &&
+  if (inner == 1 && channels > 1 && periodic_pays(channels) &&
       channels < ((int64_t)1 << 31) && ((((uintptr_t)x) & 15) == 0) &&
       ((((uintptr_t)y) & 3) == 0) && (n >> 2) > 0) {
     const PeriodicGrid pg = periodic_grid(n >> 2, channels, 1);
@@ -2177,7 +2183,7 @@ hipError_t dequantize_dispatch(hipStream_t st, const void *x, int64_t outer,
           (const uint8_t *)x, y, n, outer, (uint32_t)channels, scale, zp, g);
     return hipGetLastError();
   }
-  if (KIND != kI32 && inner == 1 && channels > 1 && channels % 4 != 0 &&
+  if (KIND != kI32 && inner == 1 && channels > 1 && periodic_pays(channels) &&
       channels < ((int64_t)1 << 31) && ((((uintptr_t)x) & 3) == 0) &&
       ((((uintptr_t)y) & 15) == 0) && (n >> 2) > 0) {
     constexpr int K8 = KIND == kI32 ? kU8 : KIND;

@@ -1108,6 +1108,27 @@ def test_per_axis_with_inner_slabs_that_are_not_whole_vectors(rt, oracle, quant_
         d.free()
 
 
+def test_per_axis_short_rows_of_whole_vectors(rt, oracle):
+    """Rows of 4 .. 252 columns (whole float4, fewer than a block of the
+    row-walking kernels covers) take the kernels whose threads keep their
+    columns from one period of the flat array to the next; 256 columns is the
+    first length that stays with the row-walking kernels.  Few rows and many,
+    row counts that end inside a period."""
+    rng = np.random.default_rng(9292)
+    for C in (4, 8, 12, 64, 128, 252, 256):
+        for rows in (1, 7, 1000, 65537):
+            x = rng.normal(0, 30, (rows, C)).astype(np.float32)
+            x.reshape(-1)[: min(x.size, SPECIALS.size)] = SPECIALS[: min(x.size, SPECIALS.size)]
+            sc = rng.uniform(0.05, 2.0, C).astype(np.float32)
+            for qdt in (np.uint8, np.int8):
+                zp = _rand_q(rng, qdt, (C,))
+                wq = oracle.quantize_linear(x, sc, zp, axis=1)
+                assert np.array_equal(rt.QuantizeLinear(x, sc, zp, axis=1), wq), (C, rows, qdt.__name__)
+                assert same_f32(rt.DequantizeLinear(wq, sc, zp, axis=1),
+                                oracle.dequantize_linear(wq, sc, zp, axis=1)), (C, rows, qdt.__name__)
+            assert np.array_equal(rt.QuantizeLinear(x, sc, None, axis=1), oracle.quantize_linear(x, sc, None, axis=1))
+
+
 def test_large_gemm_takes_the_wide_tile_path(rt, oracle):
     # big enough for the heuristic to pick the 128 x 256 B-streaming kernel on its own
     rng = np.random.default_rng(77)
