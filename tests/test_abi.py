@@ -164,7 +164,7 @@ def test_compiler_plugin_calls_only_exported_symbols(rt):
             "om_mi355x_DynamicQuantizeLinear", "om_mi355x_MatMulInteger",
             "om_mi355x_QLinearMatMul", "om_mi355x_MatMulIntegerDequant",
             "om_mi355x_DynQuantMatMulDequant", "om_mi355x_MarkConstant",
-            "om_mi355x_KeepOnDevice", "om_mi355x_Release"} <= callees
+            "om_mi355x_KeepOnDevice", "om_mi355x_Release", "om_mi355x_SetQuantMode"} <= callees
     for name in callees:
         assert hasattr(lib, name), f"plug-in calls {name}, which the runtime lacks"
     # parameter counts: results + operands + integer attributes of each pattern
@@ -172,11 +172,29 @@ def test_compiler_plugin_calls_only_exported_symbols(rt):
               "om_mi355x_DynamicQuantizeLinear": 3 + 1, "om_mi355x_MatMulInteger": 1 + 4,
               "om_mi355x_QLinearMatMul": 1 + 8 + 1, "om_mi355x_MatMulIntegerDequant": 1 + 7 + 1,
               "om_mi355x_DynQuantMatMulDequant": 1 + 5 + 1, "om_mi355x_MarkConstant": 1,
-              "om_mi355x_KeepOnDevice": 1, "om_mi355x_Release": 1}
+              "om_mi355x_KeepOnDevice": 1, "om_mi355x_Release": 1,
+              "om_mi355x_SetQuantMode": 1 + 1}   # the anchor buffer + `mode`
     for name, count in passed.items():
         m = re.search(r"\b%s\s*\(([^)]*)\)" % name, header)
         assert m, name
         assert len([p for p in m.group(1).split(",") if p.strip()]) == count, name
+
+
+def test_quant_mode_constants_agree_everywhere():
+    """The two bits of om_mi355x_SetQuantMode are spelled in the header, the
+    Python mirror, the oracle and (as literals) the plug-in: same values."""
+    import om_mi355x
+    import oracle_lib
+    header = open(os.path.join(INCLUDE, "om_mi355x.h")).read()
+    recip = int(re.search(r"#define\s+OM_MI355X_QUANT_RECIPROCAL\s+(\d+)", header).group(1))
+    no_zp = int(re.search(r"#define\s+OM_MI355X_QUANT_NO_ZERO_POINT\s+(\d+)", header).group(1))
+    assert (recip, no_zp) == (1, 2)
+    assert (om_mi355x.QUANT_RECIPROCAL, om_mi355x.QUANT_NO_ZERO_POINT) == (recip, no_zp)
+    assert (oracle_lib.RECIPROCAL, oracle_lib.NO_ZERO_POINT) == (recip, no_zp)
+    oracle_h = open(os.path.join(ROOT, "oracle", "om_oracle.h")).read()
+    assert re.search(r"OM_ORACLE_RECIPROCAL\s*=\s*1\s*,\s*OM_ORACLE_NO_ZERO_POINT\s*=\s*2", oracle_h)
+    conv = open(os.path.join(PLUGIN, "src", "Accelerators", "MI355X", "Conversion", "ONNXToMI355XCall.cpp")).read()
+    assert "mode |= 1; // OM_MI355X_QUANT_RECIPROCAL" in conv and "mode |= 2; // OM_MI355X_QUANT_NO_ZERO_POINT" in conv
 
 
 def test_compiler_plugin_version_matches_runtime():
