@@ -357,6 +357,34 @@ def dql_activation_cases(rt, steps, warmup, only=None):
     return out
 
 
+def per_axis_layout_cases(rt, steps, warmup):
+    """Per-axis QuantizeLinear / DequantizeLinear on layouts other than config 2's:
+    an inner axis with slabs that are / are not whole float4, short rows, rows
+    that are not whole float4.  Small tensors (cache-resident): the figures
+    compare dispatch paths, they are not HBM rates."""
+    rng = np.random.default_rng(0xA715)
+    out = {}
+    for shape in ((64, 2048, 7, 7), (256, 512, 14, 14), (8, 256, 57, 57), (1 << 20, 4), (1 << 18, 64),
+                  (1 << 16, 256), (1 << 18, 65), (1 << 13, 2048)):
+        C = shape[1]
+        x = rng.normal(0, 1, shape).astype(np.float32)
+        dX = rt.DeviceArray.from_numpy(x)
+        dS = rt.DeviceArray.from_numpy(rng.uniform(0.01, 0.1, C).astype(np.float32))
+        dZ = rt.DeviceArray.from_numpy(rng.integers(0, 255, C).astype(np.uint8))
+        dQ, dY = rt.DeviceArray(shape, np.uint8), rt.DeviceArray(shape, np.float32)
+        res = {}
+        for name, fn in (("quantize", rt.PreparedCall("om_mi355x_QuantizeLinear", dQ, dX, dS, dZ, 1, 1)),
+                         ("dequantize", rt.PreparedCall("om_mi355x_DequantizeLinear", dY, dQ, dS, dZ, 1))):
+            r = measure(rt, fn, steps, warmup)
+            fn.check()
+            fn.close()
+            res[name] = {"kernel_us": r["kernel_ms"] * 1e3, "gb_per_s": 5 * x.size / (r["kernel_ms"] * 1e-3) / 1e9}
+        out["x".join(str(d) for d in shape)] = res
+        for d in (dX, dS, dZ, dQ, dY):
+            d.free()
+    return out
+
+
 def only_mode(rt, wl, what, steps, warmup):
     """One kernel, `steps` launches, nothing else on the GPU: the target of the
     rocprofv3 counter runs whose summaries are kept under profiles/."""
@@ -378,6 +406,8 @@ def only_mode(rt, wl, what, steps, warmup):
         r = gemm_case(rt, wl, f"config4 {layer}", 4096, k, n, c["W"], c["w_scale"], steps, warmup, "f32",
                       headline=True)
         return {"only": what, **r}
+    if what == "per_axis_layouts":
+        return {"only": what, **per_axis_layout_cases(rt, steps, warmup)}
     if what == "mfma_ceiling":
         return {"only": what, "random_operands": rt.mfma_ceiling(True),
                 "small_constant_operands": rt.mfma_ceiling(False)}
@@ -535,7 +565,7 @@ def main():
     ap.add_argument("--extras", default="config1,gemm,fused,decode,qdq", help="which extra groups to measure")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--only", default=None,
-                    choices=["copy", "mfma_ceiling", "gemm_ffn_up", "gemm_qkv", "gemm_out", "gemm_ffn_down",
+                    choices=["copy", "mfma_ceiling", "per_axis_layouts", "gemm_ffn_up", "gemm_qkv", "gemm_out", "gemm_ffn_down",
                              "gemm_prefill_up", "gemm_prefill_down", "fused_ffn_up", "fused_ffn_down",
                              "fused_ffn_up_relu", "fused_ffn_up_gelu",
                              "decode", "decode4", "decode16",
