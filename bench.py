@@ -256,7 +256,7 @@ def fused_case(rt, wl, name, M, K, N, w_i8, w_scale, steps, warmup, X=None, acti
     return res
 
 
-def config1_cases(rt, wl, steps, warmup):
+def config1_cases(rt, wl, steps, warmup, only=None):
     """Config 1 (A f32 [128,768] -> DynamicQuantizeLinear -> MatMulInteger with
     int8 B [768,768] -> Cast -> Mul): as the three separate calls of the
     unfused graph, tensors resident, and as the one fused call."""
@@ -277,21 +277,27 @@ def config1_cases(rt, wl, steps, warmup):
         for f in calls:
             f()
 
-    sep = measure(rt, separate, steps, warmup)
-    sep["kernel"] = rt.last_gemm_kernel()
     fused = rt.PreparedCall("om_mi355x_DynQuantMatMulDequant", dY, dA, dB, dbz, dbs, None, 0)
-    fus = measure(rt, fused, steps, warmup)
-    fus["kernel"] = rt.last_gemm_kernel()
+    out = {}
+    if only in (None, "separate"):
+        sep = measure(rt, separate, steps, warmup)
+        sep["kernel"] = rt.last_gemm_kernel()
+        out["DynamicQuantizeLinear + MatMulIntegerDequant (two calls)"] = sep
+    if only in (None, "fused"):
+        fus = measure(rt, fused, steps, warmup)
+        fus["kernel"] = rt.last_gemm_kernel()
+        out["DynQuantMatMulDequant (one call)"] = fus
     for f in calls + [fused]:
         f.check()
         f.close()
     ops = 2.0 * M * N * K
-    for r in (sep, fus):
-        r.update({"M": M, "K": K, "N": N, "tops": ops / (r["kernel_ms"] * 1e-3) / 1e12})
+    nbytes = 4 * M * K + K * N + 4 * M * N
+    for r in out.values():
+        r.update({"M": M, "K": K, "N": N, "tops": ops / (r["kernel_ms"] * 1e-3) / 1e12,
+                  "hbm_bytes_algorithmic": nbytes})
     for d in (dA, dB, dbs, dbz, dq, ds, dz, dY):
         d.free()
-    return {"DynamicQuantizeLinear + MatMulIntegerDequant (two calls)": sep,
-            "DynQuantMatMulDequant (one call)": fus}
+    return out
 
 
 def qdq_cases(rt, wl, rows, cols, steps, warmup, only=None):
@@ -428,6 +434,11 @@ def only_mode(rt, wl, what, steps, warmup):
         r = gemm_case(rt, wl, f"config5 prefill {name}", 2048, k, n, c["W"], c["w_scale"], steps, warmup, "f32",
                       headline=True)
         return {"only": what, **r}
+    if what == "config3":
+        return {"only": what, **qlinear_case(rt, wl, steps, warmup)}
+    if what in ("config1", "config1_two_calls"):
+        r = config1_cases(rt, wl, steps, warmup, only="fused" if what == "config1" else "separate")
+        return {"only": what, **r}
     if what.startswith("dynamic_quantize_"):
         return {"only": what, **dql_activation_cases(rt, steps, warmup, only=what)[what]}
     # "<op>" is the aligned config 2 tensor, "<op>_ragged" the [8191, 32767] one
@@ -436,6 +447,90 @@ def only_mode(rt, wl, what, steps, warmup):
     rows, cols = (8191, 32767) if ragged else (8192, 32768)
     r = qdq_cases(rt, wl, rows, cols, steps, warmup, only=op)
     return {"only": what, "shape": [rows, cols], **r[op]}
+
+
+def sig(x, digits=5):
+    """Floats to `digits` significant digits, through any nesting."""
+    if isinstance(x, float):
+        return float(f"{x:.{digits}g}")
+    if isinstance(x, dict):
+        return {k: sig(v, digits) for k, v in x.items()}
+    if isinstance(x, (list, tuple)):
+        return [sig(v, digits) for v in x]
+    return x
+
+
+# What a measurement keeps in the one JSON line; everything else (percentiles,
+# launch counts, pre-heat times, byte counts) goes to the detail file.
+_LINE_KEYS = ("name", "M", "K", "N", "kernel_us", "tops", "gbs", "hbm_frac", "hbm_frac_at_algorithmic_bytes",
+              "kernel", "buffer_sets")
+
+
+def for_line(x):
+    """A measurement (or a nesting of them) reduced to the fields of _LINE_KEYS,
+    the kernel time in microseconds."""
+    if isinstance(x, list):
+        return [for_line(v) for v in x]
+    if isinstance(x, dict) and "kernel_ms" in x:
+        y = dict(x, kernel_us=x["kernel_ms"] * 1e3)
+        if "kernel" in y:
+            y["kernel"] = y["kernel"].split(" (")[0]
+        return {k: y[k] for k in _LINE_KEYS if k in y}
+    if isinstance(x, dict):
+        return {k: for_line(v) for k, v in x.items()}
+    return x
+
+
+def config_summary(main_res, extras):
+    """The figures of the five benchmark configurations, compact enough to sit
+    at the very end of the line (a reader that keeps only the line's last 2000
+    characters still sees every configuration): kernel time in microseconds by
+    HIP events, with TOP/s and the fraction of the 5 POP/s int8 peak for the
+    GEMMs, GB/s and the fraction of 8 TB/s for the bandwidth-bound ops."""
+    def us(r):
+        return r["kernel_ms"] * 1e3
+
+    def gemm(r):
+        t = r.get("kernel_tops", r.get("tops"))
+        return [us(r), t, t / INT8_PEAK_TOPS]
+
+    def bw(r):
+        return [us(r), r["gbs"], r["hbm_frac"]]
+
+    out = {"units": "GEMM [us, TOP/s, frac of 5 POP/s]; Q/DQ and decode [us, GB/s, frac of 8 TB/s]"}
+    c1 = extras.get("config1", {})
+    if c1:
+        out["c1_128x768x768"] = {("fused_one_call" if "one call" in k else "two_calls"): gemm(v) for k, v in c1.items()}
+    for key, name in (("qdq_8192x32768", "c2_8192x32768"), ("qdq_8191x32767", "c2_8191x32767")):
+        if key in extras:
+            short = {"quantize_per_axis": "q_axis", "dequantize_per_axis": "dq_axis", "quantize_per_tensor": "q_tensor",
+                     "dequantize_per_tensor": "dq_tensor", "dynamic_quantize": "dql"}
+            out[name] = {short[k]: bw(v) for k, v in extras[key].items()}
+    gemms = {g["name"]: g for g in extras.get("gemm", [])}
+    fused = {g["name"]: g for g in extras.get("fused", [])}
+    for k, g in gemms.items():
+        if k.startswith("config3"):
+            out["c3_512x1024x4096_qlinear"] = gemm(g)
+    c4 = {"ffn_up": gemm(main_res)}
+    for k, g in gemms.items():
+        if k.startswith("config4") and "int32" not in k and "QLinear" not in k:
+            c4.setdefault(k.split()[1], gemm(g))
+        elif k.startswith("config4") and "QLinear" in k:
+            c4["ffn_up_qlinear_u8_out"] = gemm(g)
+    for k, g in fused.items():
+        c4["fused_" + k.split()[1] + ("_gelu" if "Gelu" in k else "")] = gemm(g)
+    if "ffn_block" in extras:
+        c4["ffn_block_us"] = {k: v["kernel_ms"] * 1e3 for k, v in extras["ffn_block"].items()}
+    out["c4_M4096"] = c4
+    c5 = {}
+    for k, g in gemms.items():
+        if k.startswith("config5"):
+            c5["prefill_" + k.split()[2]] = gemm(g)
+    for d in extras.get("decode", []):
+        c5[f"decode_M{d['M']}"] = bw(d)
+    if c5:
+        out["c5"] = c5
+    return sig(out, 4)
 
 
 def host_cpu():
@@ -568,7 +663,7 @@ def main():
                     choices=["copy", "mfma_ceiling", "per_axis_layouts", "gemm_ffn_up", "gemm_qkv", "gemm_out", "gemm_ffn_down",
                              "gemm_prefill_up", "gemm_prefill_down", "fused_ffn_up", "fused_ffn_down",
                              "fused_ffn_up_relu", "fused_ffn_up_gelu",
-                             "decode", "decode4", "decode16",
+                             "decode", "decode4", "decode16", "config1", "config1_two_calls", "config3",
                              "quantize_per_axis", "dequantize_per_axis",
                              "quantize_per_tensor", "dequantize_per_tensor", "dynamic_quantize",
                              "quantize_per_axis_ragged", "dequantize_per_axis_ragged",
@@ -692,9 +787,20 @@ def main():
                      "measured_mfma_ceiling": ceiling},
         "cpu_baseline": cpu,
         "device": info,
-        "extras": extras,
     }
-    print(json.dumps(line))
+    # Everything measured, in full, beside the line; the line itself carries the
+    # extras reduced to their figures and ends with the per-configuration summary.
+    detail = dict(line, extras=extras)
+    try:
+        os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
+        with open(os.path.join(ROOT, "gpurun_out", "bench_detail.json"), "w") as f:
+            json.dump(detail, f)
+        line["detail_file"] = "gpurun_out/bench_detail.json"
+    except OSError:
+        line["detail_file"] = None
+    line["extras"] = for_line(extras)
+    line["configs"] = config_summary(main_res, extras)
+    print(json.dumps(sig(line), separators=(",", ":")))
 
 
 if __name__ == "__main__":

@@ -65,15 +65,25 @@ void OMShutdownAccelMI355X(void);
  *     the 8-bit type; QuantizeLinear.cpp:231-237, Elementwise.cpp:1453), and
  *     DynamicQuantizeLinear returns a zero point of 0 and adds none
  *     (DynamicQuantizeLinear.cpp:75-84,142-152).
- * om_mi355x_SetQuantMode(anchor, mode) makes every later call of the calling
- * thread compute that way (mode: 0, the default, or a combination of the
- * two); code compiled with either option calls it in front of each of these
+ * The form is a property of the compiled model in the reference, so here it
+ * is a property of each op, never a lasting state of the thread:
+ * om_mi355x_SetQuantMode(anchor, mode) applies to the NEXT call of
+ * om_mi355x_QuantizeLinear, om_mi355x_DequantizeLinear,
+ * om_mi355x_DynamicQuantizeLinear[NoAlloc] or om_mi355x_DynQuantMatMulDequant
+ * that the calling thread makes.  That call takes the mode (mode: 0, the
+ * default, or a combination of the two bits) when it is entered -- also when
+ * it then fails -- and leaves 0 behind, so an op that no SetQuantMode call
+ * precedes always computes the default form, whatever model ran on the thread
+ * before.  Code compiled with either option calls it in front of each of these
  * ops ("krnl.call"(%y) {funcName = "om_mi355x_SetQuantMode", mode = 3 : si64,
- * numOfOutput = 1 : si64}).  `anchor` is not used: generated code names the
- * op's result buffer there, as an output, because a krnl.call without an
- * operand it writes counts as dead and is removed; other callers pass NULL.
- * The fused entry points follow the mode as the ops they stand for would.
- * Any other value is refused (EINVAL). */
+ * numOfOutput = 1 : si64}); code compiled without them calls nothing.  The
+ * other entry points neither read nor change the pending mode.  `anchor` is
+ * not used: generated code names the op's result buffer there, as an output,
+ * because a krnl.call without an operand it writes counts as dead and is
+ * removed (and writing the same buffer keeps the pair in order); other callers
+ * pass NULL.  om_mi355x_GetQuantMode returns the mode the thread's next such
+ * op would take.  Any value outside 0..3 is refused (EINVAL) and leaves the
+ * pending mode as it was. */
 #define OM_MI355X_QUANT_RECIPROCAL 1
 #define OM_MI355X_QUANT_NO_ZERO_POINT 2
 void om_mi355x_SetQuantMode(OMTensor *anchor, int64_t mode);
@@ -240,19 +250,6 @@ int om_mi355x_synchronize(void);
  * milliseconds, or a negative value on error. */
 int om_mi355x_timer_start(void);
 float om_mi355x_timer_stop(void);
-
-/* What the matrix cores of device 0 deliver with nothing else going on: every
- * SIMD of every CU issues v_mfma_i32_32x32x32_i8 back to back from registers
- * for a few milliseconds, no memory traffic.  random_operands = 0: operands
- * of small constants (few bits toggle); 1: operands of random bytes, as a
- * quantized model's are.  Returns 0 and fills *tops (10^12 int8 operations
- * per second over the device) and *clock_ghz (the shader clock that rate
- * corresponds to at one such MFMA per 32 clocks and SIMD), or -1 with the
- * error kept for om_mi355x_last_error().  A measurement aid for roofline
- * figures: under random operands the device lowers its clock, and no int8
- * GEMM can exceed what this reports.  No counterpart in the reference. */
-int om_mi355x_mfma_ceiling(int64_t random_operands, double *tops,
-    double *clock_ghz);
 
 /* Last error message of the calling thread ("" if none); clears it. */
 const char *om_mi355x_last_error(void);

@@ -100,12 +100,17 @@ void emitCall(ConversionPatternRewriter &rewriter, Location loc,
 /// in src/Compiler/CompilerPasses.cpp:298-301) and
 /// --disable-quantization-zero-point (QuantizeLinear.cpp:231-237,
 /// DynamicQuantizeLinear.cpp:142, Math/Elementwise.cpp:1453).  The runtime
-/// computes either way; which one is a state of the calling thread, set by
-/// `om_mi355x_SetQuantMode(anchor, mode)`.  The call goes in front of every
-/// offloaded op that the options touch, and only when one of them is on, so a
-/// thread that runs models compiled differently is always in the right state.
+/// computes either way.  Which one is a property of the compiled model, as in
+/// the reference, so it travels with each op: `om_mi355x_SetQuantMode(anchor,
+/// mode)` applies to the calling thread's next quantize / dequantize /
+/// dynamic-quantize / fused-layer entry point only, which takes the mode and
+/// leaves the default behind.  The call therefore goes directly in front of
+/// every offloaded op that the options touch when one of them is on; code
+/// compiled with default options emits nothing and cannot inherit a mode from
+/// a model that ran on the thread before it.
 /// `anchor` (the op's first result buffer) is passed as an output for the
-/// reason given at markIfConstant; the runtime does not touch it.
+/// reason given at markIfConstant, and because two calls that write the same
+/// buffer keep their order; the runtime does not touch it.
 int64_t quantModeFromOptions() {
   int64_t mode = 0;
   if (OptimizationLevel >= OptLevel::O3 && enableFastMathOption)

@@ -14,7 +14,7 @@ namespace onnx_mlir {
 
 /// Patterns for the ONNX-to-Krnl conversion that replace the quantisation ops
 /// (and the `onnx.Custom` ops the MI355X fusion pass creates) by `krnl.call`s
-/// to libom_mi355x.so.  Their benefit is above that of the CPU patterns, and
+/// to libRuntimeMI355X.a.  Their benefit is above that of the CPU patterns, and
 /// they fail to match whatever the runtime does not implement, which then goes
 /// to the CPU lowering.
 void populateONNXToMI355XCallPatterns(mlir::RewritePatternSet &patterns,

@@ -40,8 +40,12 @@ MI355XAccelerator::MI355XAccelerator()
   acceleratorTargets.push_back(this);
 
   // Libraries a compiled model is linked against, in dependency order
-  // (the option mechanism is src/Compiler/CompilerOptions.cpp:1559-1575).
-  addCompilerConfig(CCM_SHARED_LIB_DEPS, {"om_mi355x", "amdhip64"},
+  // (the option mechanism is src/Compiler/CompilerOptions.cpp:1559-1575): the
+  // runtime as a static archive, libRuntimeMI355X.a, the way
+  // src/Accelerators/NNPA/NNPAAccelerator.cpp:60-81 names libRuntimeNNPA.a,
+  // then the HIP runtime it calls.  The archive leaves the omTensor*
+  // accessors undefined; the model's libcruntime provides them.
+  addCompilerConfig(CCM_SHARED_LIB_DEPS, {"RuntimeMI355X", "amdhip64"},
       /*exclusive=*/true);
   std::vector<std::string> libDirs;
 #ifdef OM_MI355X_RUNTIME_DIR

@@ -5,7 +5,7 @@
 //===------------------------ MI355XAccelerator.hpp -----------------------===//
 //
 // Accelerator plug-in that sends the 8-bit quantisation ops of a model to an
-// AMD Instinct MI355X through the C entry points of libom_mi355x.so.
+// AMD Instinct MI355X through the C entry points of libRuntimeMI355X.a.
 //
 // It introduces no dialect: the ops stay in the ONNX dialect until the
 // ONNX-to-Krnl conversion, where patterns of a higher benefit than the CPU ones

@@ -3,7 +3,10 @@
 
 // The reference's CPU code for these ops changes with --enable-fast-math (at
 // -O3) and --disable-quantization-zero-point; the offloaded ops are told which
-// form to compute by a call in front of each of them, and only then.
+// form to compute by a call directly in front of each of them.  The runtime
+// applies that call to the very next such op of the thread and to no other, so
+// code compiled with default options (DEFAULT) needs no call: an op that none
+// precedes computes the default form whatever ran on the thread before.
 func.func @quantize_then_dequantize(%x: tensor<64x768xf32>, %s: tensor<f32>, %z: tensor<ui8>) -> tensor<64x768xf32> {
   %q = "onnx.QuantizeLinear"(%x, %s, %z) {axis = 1 : si64, saturate = 1 : si64} : (tensor<64x768xf32>, tensor<f32>, tensor<ui8>) -> tensor<64x768xui8>
   %y = "onnx.DequantizeLinear"(%q, %s, %z) {axis = 1 : si64} : (tensor<64x768xui8>, tensor<f32>, tensor<ui8>) -> tensor<64x768xf32>

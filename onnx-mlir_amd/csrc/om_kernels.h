@@ -64,6 +64,24 @@ hipError_t launch_dynamic_quantize(hipStream_t s, DqlScratch &scratch,
     bool y_shift, int mode = 0);
 constexpr int kQuantReciprocal = 1, kQuantNoZeroPoint = 2;
 
+// The tagged-slot exchange between the blocks of one launch (k_dql_grid, the
+// fused layer of k_gemm_i8_flight).  At most one kernel that uses it may be in
+// flight per process: two of them dispatched at the same time from different
+// streams could each hold part of the device and wait for the rest.
+// dql_exchange_begin returns false when the exchange is switched off
+// (scratch.grid_blocks == 0) or the last such kernel was launched on another
+// stream that is still busy; otherwise it fills `x` with this launch's number
+// and the slots, and holds a lock until dql_exchange_end, which the caller
+// calls right after queuing its kernel on `s` (launched: whether it did).
+struct GridExchange {
+  unsigned long long *slots;
+  unsigned epoch;
+  unsigned *failed;
+  unsigned spin_limit;
+};
+bool dql_exchange_begin(hipStream_t s, DqlScratch &scratch, GridExchange &x);
+void dql_exchange_end(hipStream_t s, bool launched);
+
 // Call before destroying a stream that launch_dynamic_quantize was given.
 void dql_forget_stream(hipStream_t s);
 
@@ -80,10 +98,12 @@ hipError_t launch_pack_b(hipStream_t s, const void *B, bool b_unsigned,
     int64_t K, int64_t N, int8_t *Bp, int32_t *colsum);
 
 struct GemmArgs {
-  // If set (M <= 32 only, see gemm_quantizes_rows): the activation as f32
-  // [M,K]; the kernel quantizes it itself as DynamicQuantizeLinear would
-  // (A, a_zp and a_scale are then not read).
+  // If set (see gemm_quantizes_rows): the activation as f32 [M,K]; the kernel
+  // quantizes it itself as DynamicQuantizeLinear would (A, a_zp and a_scale
+  // are then not read).  `dql`: the scratch whose exchange slots the blocks
+  // use where they have to agree on minimum and maximum across the grid.
   const float *X;
+  DqlScratch *dql;
   const void *A;       // [M,K] row-major, u8 or i8
   bool a_unsigned;     // A holds u8
   bool a_preshifted;   // A already holds (u8 - 128) as int8; offsets as for u8
@@ -118,16 +138,17 @@ struct GemmArgs {
 };
 
 hipError_t launch_gemm(hipStream_t s, const GemmArgs &g);
-// Matrix-core ceiling probe: `blocks` blocks of four waves, each wave issuing
-// 4 * iters v_mfma_i32_32x32x32_i8 from registers; nothing is written to
-// `sink` (it keeps the loop alive).
-hipError_t launch_mfma_probe(hipStream_t s, bool random_operands, int blocks,
-    int iters, int *sink);
 // Name of the kernel the calling thread's last launch_gemm chose.
 const char *last_gemm_kernel();
 
-// Whether launch_gemm can take an f32 activation of this shape in GemmArgs::X.
-bool gemm_quantizes_rows(int64_t M, int64_t K, const void *x);
+// Whether launch_gemm can take an f32 activation of this shape in GemmArgs::X:
+// 0 no; 1 yes, every block quantizes the rows for itself; 2 yes, the blocks
+// agree on minimum and maximum through the exchange slots of GemmArgs::dql
+// (one-launch rules of DynamicQuantizeLinear apply: launch_gemm answers
+// hipErrorNotReady when the exchange cannot be used right now -- the caller
+// then quantizes with DynamicQuantizeLinear and passes A -- and a block that
+// gives up waiting raises the scratch's flag).
+int gemm_quantizes_rows(int64_t M, int64_t K, int64_t N, const void *x);
 // Whether the caller should hand `a` over as rows of round_up(K, 16) bytes
 // made by launch_pad_rows (few rows, K % 16 != 0 or a misaligned start), and
 // pass that length as K.  a_zp: the rows' zero point(s) on the GPU (null: 0),

@@ -2355,35 +2355,17 @@ hipError_t launch_dynamic_quantize(hipStream_t s, DqlScratch &scratch,
       fn_launch = k_dql_grid<kGridMaxPerThread>;
     if (fn_launch) {
       const uint32_t flip = y_shift ? 0x80808080u : 0u;
-      const unsigned spin_limit = scratch.spin_limit;
-      unsigned long long *slots = scratch.grid_slots; // 16-byte aligned
-      unsigned *failed = scratch.counter + 8;
-      // At most one of these kernels is in flight per process: two of them
-      // dispatched at the same time from different streams could each hold
-      // part of the device and wait for the rest.  If the previous one was
-      // launched on another stream and that stream is still busy, this call
-      // takes the two-launch path.  (Streams of this library live as long as
-      // the process.)
-      bool mine = false;
-      {
-        std::lock_guard<std::mutex> lk(g_grid_mutex);
-        // (same stream: the previous one finishes before this one starts)
-        if (!g_grid_stream || g_grid_stream == s ||
-            hipStreamQuery(g_grid_stream) == hipSuccess) {
-          if (++scratch.epoch == 0) // 0 is what untouched slots hold
-            scratch.epoch = 1;
-          hipLaunchKernelGGL(fn_launch, dim3((unsigned)blocks),
-              dim3(kGridThreads), 0, s, x, n, y, scale, zp, flip, slots,
-              scratch.epoch, failed, spin_limit);
-          hipError_t e = hipGetLastError();
-          if (e != hipSuccess)
-            return e;
-          g_grid_stream = s;
-          mine = true;
-        }
+      // If the previous kernel of this kind was launched on another stream and
+      // that stream is still busy, this call takes the two-launch path.
+      GridExchange ex;
+      if (dql_exchange_begin(s, scratch, ex)) {
+        hipLaunchKernelGGL(fn_launch, dim3((unsigned)blocks),
+            dim3(kGridThreads), 0, s, x, n, y, scale, zp, flip, ex.slots,
+            ex.epoch, ex.failed, ex.spin_limit);
+        const hipError_t e = hipGetLastError();
+        dql_exchange_end(s, e == hipSuccess);
+        return e;
       }
-      if (mine)
-        return hipSuccess;
     }
   }
   // A read-only reduction streams fastest with few, long-lived blocks
@@ -2402,6 +2384,33 @@ hipError_t launch_dynamic_quantize(hipStream_t s, DqlScratch &scratch,
   // the reference adds: it is an integer in [0, 255]).
   return quantize_dispatch<false>(s, x, 1, 1, n, scale, zp, y,
       y_shift ? 0x80808080u : 0u, (mode & kQuantReciprocal) != 0);
+}
+
+bool dql_exchange_begin(hipStream_t s, DqlScratch &scratch, GridExchange &x) {
+  if (scratch.grid_blocks <= 0)
+    return false;
+  g_grid_mutex.lock();
+  // (same stream: the previous kernel finishes before the next one starts;
+  // streams of this library live as long as their threads)
+  if (g_grid_stream && g_grid_stream != s &&
+      hipStreamQuery(g_grid_stream) != hipSuccess) {
+    (void)hipGetLastError();
+    g_grid_mutex.unlock();
+    return false;
+  }
+  if (++scratch.epoch == 0) // 0 is what untouched slots hold
+    scratch.epoch = 1;
+  x.slots = scratch.grid_slots; // 16-byte aligned
+  x.epoch = scratch.epoch;
+  x.failed = scratch.counter + 8;
+  x.spin_limit = scratch.spin_limit;
+  return true;
+}
+
+void dql_exchange_end(hipStream_t s, bool launched) {
+  if (launched)
+    g_grid_stream = s;
+  g_grid_mutex.unlock();
 }
 
 void dql_forget_stream(hipStream_t s) {

@@ -60,9 +60,24 @@ static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
 // ---------------------------------------------------------------------------
 namespace {
 
-// The compiler options the calling thread's model was compiled with, as far as
-// they change this path's arithmetic (OM_MI355X_QUANT_*; om_mi355x_SetQuantMode).
+// The compiler options that change this path's arithmetic (OM_MI355X_QUANT_*).
+// In the reference they are a property of each compiled model
+// (src/Compiler/CompilerPasses.cpp:298-301), so here they are a property of
+// each op: om_mi355x_SetQuantMode leaves its mode in t_quant_mode_next, the
+// next QuantizeLinear / DequantizeLinear / DynamicQuantizeLinear / fused-layer
+// entry point of the thread takes it (QuantModeScope) and leaves 0 behind.  An
+// op that no SetQuantMode call precedes therefore always computes the default
+// form, whatever ran on the thread before it.
+thread_local int t_quant_mode_next = 0;
+// Mode of the entry point that is running on this thread; 0 outside one.
 thread_local int t_quant_mode = 0;
+struct QuantModeScope {
+  QuantModeScope() {
+    t_quant_mode = t_quant_mode_next;
+    t_quant_mode_next = 0;
+  }
+  ~QuantModeScope() { t_quant_mode = 0; }
+};
 thread_local std::string t_last_error;
 thread_local std::string t_last_error_returned;
 
@@ -1503,10 +1518,10 @@ void om_mi355x_SetQuantMode(OMTensor *anchor, int64_t mode) {
         (long long)mode);
     return;
   }
-  t_quant_mode = (int)mode;
+  t_quant_mode_next = (int)mode;
 }
 
-int64_t om_mi355x_GetQuantMode(void) { return t_quant_mode; }
+int64_t om_mi355x_GetQuantMode(void) { return t_quant_mode_next; }
 
 // ---------------------------------------------------------------------------
 // ops
@@ -1514,6 +1529,7 @@ int64_t om_mi355x_GetQuantMode(void) { return t_quant_mode; }
 void om_mi355x_QuantizeLinear(OMTensor *y_t, const OMTensor *x_t,
     const OMTensor *scale_t, const OMTensor *zp_t, int64_t axis,
     int64_t saturate) {
+  const QuantModeScope quant_mode_of_this_op;
   (void)saturate;
   View y, x, sc, zp;
   if (!view_of(y_t, "y", y) || !view_of(x_t, "x", x) ||
@@ -1555,6 +1571,7 @@ void om_mi355x_QuantizeLinear(OMTensor *y_t, const OMTensor *x_t,
 
 void om_mi355x_DequantizeLinear(OMTensor *y_t, const OMTensor *x_t,
     const OMTensor *scale_t, const OMTensor *zp_t, int64_t axis) {
+  const QuantModeScope quant_mode_of_this_op;
   View y, x, sc, zp;
   if (!view_of(y_t, "y", y) || !view_of(x_t, "x", x) ||
       !view_of(scale_t, "x_scale", sc))
@@ -1597,6 +1614,7 @@ void om_mi355x_DequantizeLinear(OMTensor *y_t, const OMTensor *x_t,
 
 void om_mi355x_DynamicQuantizeLinear(OMTensor *y_t, OMTensor *scale_t,
     OMTensor *zp_t, const OMTensor *x_t) {
+  const QuantModeScope quant_mode_of_this_op;
   View y, sc, zp, x;
   if (!view_of(y_t, "y", y) || !view_of(scale_t, "y_scale", sc) ||
       !view_of(zp_t, "y_zero_point", zp) || !view_of(x_t, "x", x))
@@ -1624,6 +1642,7 @@ void om_mi355x_DynamicQuantizeLinear(OMTensor *y_t, OMTensor *scale_t,
 
 void om_mi355x_DynamicQuantizeLinearNoAlloc(OMTensor *y_t, OMTensor *scale_t,
     OMTensor *zp_t, const OMTensor *x_t) {
+  const QuantModeScope quant_mode_of_this_op;
   const char *op = "DynamicQuantizeLinearNoAlloc";
   View y, sc, zp, x;
   if (!view_of(y_t, "y", y) || !view_of(scale_t, "y_scale", sc) ||
@@ -1745,6 +1764,7 @@ void om_mi355x_QLinearMatMul(OMTensor *y, const OMTensor *a,
 void om_mi355x_DynQuantMatMulDequant(OMTensor *y_t, const OMTensor *x_t,
     const OMTensor *b_t, const OMTensor *bzp_t, const OMTensor *bscale_t,
     const OMTensor *bias_t, int64_t activation) {
+  const QuantModeScope quant_mode_of_this_op;
   const char *op = "DynQuantMatMulDequant";
   View y, x, b, bzp, bs, bias;
   bool relu, gelu;
@@ -1780,58 +1800,100 @@ void om_mi355x_DynQuantMatMulDequant(OMTensor *y_t, const OMTensor *x_t,
   if (!call.ok)
     return;
   const float *dx = (const float *)call.in(x);
-  int64_t padded_k = 0;
-  GemmArgs g = {};
-  g.out = call.out(y); // before the quantization: it decides whether to wait
-  if (call.ok && t_quant_mode == 0 && gemm_quantizes_rows(M, K, dx)) {
-    // A few rows (decode): the GEMM kernel quantizes them itself.
-    g.X = dx;
-  } else {
-    // Quantized activations stay on the GPU, stored as (u8 - 128) so the GEMM
-    // stages them without a per-byte fix-up.
-    uint8_t *aq = (uint8_t *)call.temp((size_t)M * K);
-    if (call.ok)
-      run_dql(call, dx, M * K, aq, call.c.dql_scale, call.c.dql_zp, true);
-    g.A = aq;
-    if (call.ok && gemm_pads_rows(M, K, aq)) {
-      // (see run_matmul) the quantized rows are stored minus 128
-      void *padded = call.temp((size_t)M * round_up(K, 16));
-      if (call.ok)
-        call.check(launch_pad_rows(call.c.stream, aq, M, K, call.c.dql_zp, 1,
-                       /*stored_minus_128=*/true, padded),
-            "pad rows");
-      g.A = padded;
-      padded_k = round_up(K, 16);
-    }
-  }
-  g.a_unsigned = true;
-  g.a_preshifted = true;
-  g.b_unsigned = b.dtype == OM_MI355X_TYPE_UINT8;
-  g.M = M;
-  g.K = padded_k ? padded_k : K;
-  g.N = N;
+  void *dy = call.out(y); // before the quantization: it decides whether to wait
   const int32_t *colsum = nullptr;
-  if (!call.ok || !packed_b(call, b, K, N, g.Bp, colsum)) {
+  const int8_t *bp = nullptr;
+  if (!call.ok || !packed_b(call, b, K, N, bp, colsum)) {
     call.finish();
     return;
   }
-  g.colsum = colsum;
-  g.a_zp = call.c.dql_zp;
-  g.a_zp_len = 1;
-  g.b_zp = bzp_t ? call.in(bzp) : nullptr;
-  g.b_zp_len = bzl;
-  g.epi = kEpiF32;
-  g.a_scale = call.c.dql_scale;
-  g.b_scale = (const float *)call.in(bs);
-  g.b_scale_len = bs.numel;
-  if (bias_t) {
-    g.bias = (const float *)call.in(bias);
-    g.bias_len = bias.numel;
+  const void *d_bzp = bzp_t ? call.in(bzp) : nullptr;
+  const float *d_bs = (const float *)call.in(bs);
+  const float *d_bias = bias_t ? (const float *)call.in(bias) : nullptr;
+  // in_kernel: the GEMM kernel quantizes the rows itself (a few rows: every
+  // block on its own; up to one round of 32-row blocks: the blocks agree on
+  // minimum and maximum through the exchange slots).  Otherwise
+  // DynamicQuantizeLinear is a launch of its own and the quantized
+  // activations stay on the GPU, stored as (u8 - 128) so that the GEMM stages
+  // them without a per-byte fix-up.
+  auto run = [&](bool in_kernel) -> hipError_t {
+    int64_t padded_k = 0;
+    GemmArgs g = {};
+    g.out = dy;
+    if (in_kernel) {
+      g.X = dx;
+      g.dql = &call.c.dql;
+    } else {
+      uint8_t *aq = (uint8_t *)call.temp((size_t)M * K);
+      if (call.ok)
+        run_dql(call, dx, M * K, aq, call.c.dql_scale, call.c.dql_zp, true);
+      g.A = aq;
+      if (call.ok && gemm_pads_rows(M, K, aq)) {
+        // (see run_matmul) the quantized rows are stored minus 128
+        void *padded = call.temp((size_t)M * round_up(K, 16));
+        if (call.ok)
+          call.check(launch_pad_rows(call.c.stream, aq, M, K, call.c.dql_zp, 1,
+                         /*stored_minus_128=*/true, padded),
+              "pad rows");
+        g.A = padded;
+        padded_k = round_up(K, 16);
+      }
+      if (!call.ok)
+        return hipSuccess; // already reported
+    }
+    g.a_unsigned = true;
+    g.a_preshifted = true;
+    g.b_unsigned = b.dtype == OM_MI355X_TYPE_UINT8;
+    g.M = M;
+    g.K = padded_k ? padded_k : K;
+    g.N = N;
+    g.Bp = bp;
+    g.colsum = colsum;
+    g.a_zp = call.c.dql_zp;
+    g.a_zp_len = 1;
+    g.b_zp = d_bzp;
+    g.b_zp_len = bzl;
+    g.epi = kEpiF32;
+    g.a_scale = call.c.dql_scale;
+    g.b_scale = d_bs;
+    g.b_scale_len = bs.numel;
+    g.bias = d_bias;
+    g.bias_len = bias_t ? bias.numel : 0;
+    g.relu = relu;
+    g.gelu = gelu;
+    return launch_gemm(call.c.stream, g);
+  };
+  const int kind = (call.ok && t_quant_mode == 0 && call.c.dql.grid_blocks >= 0)
+                       ? gemm_quantizes_rows(M, K, N, dx)
+                       : 0;
+  // Blocks that wait for one another (more rows than one block quantizes for
+  // itself) raise the same flag as DynamicQuantizeLinear's one-launch kernel
+  // when they give up; checked like that kernel's.
+  const bool exchanges = kind == 2;
+  const bool in_kernel = kind == 1 || (kind == 2 && call.c.dql.grid_blocks > 0);
+  hipError_t e = hipSuccess;
+  if (call.ok) {
+    e = run(in_kernel);
+    if (e == hipErrorNotReady && exchanges) // the exchange is taken or off
+      e = run(false);
+    else if (e == hipSuccess && exchanges) {
+      call.c.dql_unchecked = true;
+      if (!(call.touched_host || sync_every_call() || report_enabled()))
+        call.used_dql = true;
+      else {
+        e = hipStreamSynchronize(call.c.stream);
+        if (e == hipSuccess && call.c.dql_gave_up()) {
+          fprintf(stderr,
+              "om_mi355x: DynQuantMatMulDequant: the blocks of the one-launch "
+              "kernel timed out waiting for one another; redone with separate "
+              "launches, which this thread uses from now on\n");
+          e = run(false);
+        }
+      }
+    }
+    if (call.ok)
+      call.check(e, op);
   }
-  g.relu = relu;
-  g.gelu = gelu;
-  if (call.ok)
-    call.check(launch_gemm(call.c.stream, g), op);
   call.finish();
 }
 
@@ -2060,67 +2122,6 @@ float om_mi355x_timer_stop(void) {
     return -1.0f;
   }
   return ms;
-}
-
-int om_mi355x_mfma_ceiling(int64_t random_operands, double *tops,
-    double *clock_ghz) {
-  if (!tops || !clock_ghz) {
-    fail(EINVAL, "om_mi355x_mfma_ceiling: null result pointer");
-    return -1;
-  }
-  if (!t_ctx.init())
-    return -1;
-  hipDeviceProp_t prop;
-  if (hipGetDeviceProperties(&prop, 0) != hipSuccess) {
-    fail(EIO, "om_mi355x_mfma_ceiling: no device properties");
-    return -1;
-  }
-  // Two blocks of four waves per CU (two waves per SIMD), 4 * kIters MFMAs
-  // per wave: 5 to 15 ms, long enough for the clock to settle.  The first
-  // launch brings the device to that state, the second is the one timed.
-  const int kIters = 50000;
-  const int blocks = 2 * prop.multiProcessorCount;
-  void *buf = om_mi355x_malloc(16);
-  if (!buf)
-    return -1;
-  int *sink = (int *)buf;
-  hipStream_t st = t_ctx.stream;
-  float ms = 0.0f;
-  // events of its own: a bracket opened with om_mi355x_timer_start stays valid
-  hipEvent_t e0 = nullptr, e1 = nullptr;
-  hipError_t e = hipEventCreate(&e0);
-  if (e == hipSuccess)
-    e = hipEventCreate(&e1);
-  if (e == hipSuccess)
-    e = launch_mfma_probe(st, random_operands != 0, blocks, kIters, sink);
-  if (e == hipSuccess)
-    e = hipEventRecord(e0, st);
-  if (e == hipSuccess)
-    e = launch_mfma_probe(st, random_operands != 0, blocks, kIters, sink);
-  if (e == hipSuccess)
-    e = hipEventRecord(e1, st);
-  if (e == hipSuccess)
-    e = hipEventSynchronize(e1);
-  if (e == hipSuccess)
-    e = hipEventElapsedTime(&ms, e0, e1);
-  if (e0)
-    (void)hipEventDestroy(e0);
-  if (e1)
-    (void)hipEventDestroy(e1);
-  om_mi355x_free(buf);
-  if (e != hipSuccess || ms <= 0.0f) {
-    fail(EIO, "om_mi355x_mfma_ceiling failed: %s", hipGetErrorString(e));
-    return -1;
-  }
-  // 4 waves a block, 4 * kIters MFMAs a wave, 32 * 32 * 32 multiply-adds each
-  const double ops = (double)blocks * 4.0 * 4.0 * kIters * 32768.0 * 2.0;
-  *tops = ops / ((double)ms * 1e-3) / 1e12;
-  // A SIMD issues one of these MFMAs every 32 clocks when nothing holds it
-  // up, which is the case here: the clock that this rate corresponds to.
-  const double per_simd = (double)blocks * 4.0 * 4.0 * kIters /
-                          ((double)prop.multiProcessorCount * 4.0);
-  *clock_ghz = per_simd * 32.0 / ((double)ms * 1e6);
-  return 0;
 }
 
 const char *om_mi355x_last_error(void) {

@@ -27,6 +27,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _CSRC = os.path.normpath(os.path.join(_HERE, "..", "csrc"))
 LIB_PATH = os.path.join(_CSRC, "libom_mi355x.so")
 SHIM_PATH = os.path.join(_CSRC, "libom_tensor_shim.so")
+# measurement aids (csrc/measure), outside the runtime's C-ABI
+MEASURE_PATH = os.path.join(_CSRC, "libom_mi355x_measure.so")
 
 # ONNX element-type codes (include/onnx-mlir/Runtime/OnnxDataTypeMetaData.inc:22-44)
 ONNX_FLOAT, ONNX_UINT8, ONNX_INT8, ONNX_INT32 = 1, 2, 3, 6
@@ -123,9 +125,6 @@ def _declare(lib, shim):
     lib.om_mi355x_SetQuantMode.restype = None
     lib.om_mi355x_SetQuantMode.argtypes = [ctypes.c_void_p, ctypes.c_int64]
     lib.om_mi355x_GetQuantMode.restype = ctypes.c_int64
-    lib.om_mi355x_mfma_ceiling.restype = ctypes.c_int
-    lib.om_mi355x_mfma_ceiling.argtypes = [ctypes.c_int64, ctypes.POINTER(ctypes.c_double),
-                                           ctypes.POINTER(ctypes.c_double)]
     lib.om_mi355x_device_info.argtypes = [ctypes.c_char_p, SZ]
 
 
@@ -146,31 +145,63 @@ def device_info() -> dict:
             "mem_gib": float(gib)}
 
 
+# The compiler options this binding "compiles" its calls with.  In the runtime
+# the mode belongs to one op (om_mi355x_SetQuantMode applies to the thread's
+# next quantize / dequantize / dynamic-quantize / fused-layer call only), so
+# the binding does what generated code does: while the mode is non-zero it puts
+# om_mi355x_SetQuantMode in front of each such call, and nothing otherwise.
+_compiled_mode = 0
+
+
 def set_quant_mode(mode: int) -> None:
-    """How this thread's later QuantizeLinear / DequantizeLinear /
-    DynamicQuantizeLinear calls (and the fused entry points) compute: 0 as the
-    reference does by default, or QUANT_RECIPROCAL | QUANT_NO_ZERO_POINT as it
-    does when compiled with --enable-fast-math /
+    """How the QuantizeLinear / DequantizeLinear / DynamicQuantizeLinear calls
+    (and the whole-layer fused call) made through this module from now on
+    compute: 0 as the reference does by default, or QUANT_RECIPROCAL |
+    QUANT_NO_ZERO_POINT as it does when compiled with --enable-fast-math /
     --disable-quantization-zero-point."""
+    global _compiled_mode
     load()
-    _lib.om_mi355x_SetQuantMode(None, ctypes.c_int64(int(mode)))
+    _lib.om_mi355x_SetQuantMode(None, ctypes.c_int64(int(mode)))   # validates
     _check()
+    _lib.om_mi355x_SetQuantMode(None, ctypes.c_int64(0))
+    _compiled_mode = int(mode)
 
 
 def quant_mode() -> int:
+    return _compiled_mode
+
+
+def pending_quant_mode() -> int:
+    """The mode the calling thread's next such op would take in the runtime
+    (om_mi355x_GetQuantMode): non-zero only between om_mi355x_SetQuantMode and
+    the op it precedes."""
     load()
     return int(_lib.om_mi355x_GetQuantMode())
 
 
+def _emit_quant_mode():
+    if _compiled_mode:
+        _lib.om_mi355x_SetQuantMode(None, ctypes.c_int64(_compiled_mode))
+
+
+_measure = None
+
+
 def mfma_ceiling(random_operands: bool = True) -> dict:
     """int8 MFMA rate of the device with nothing else going on (TOPS) and the
-    shader clock it held meanwhile; see om_mi355x_mfma_ceiling in the header."""
-    load()
+    shader clock it held meanwhile (csrc/measure/mfma_ceiling.h; a library of
+    its own, not part of the runtime)."""
+    global _measure
+    if _measure is None:
+        _measure = ctypes.CDLL(MEASURE_PATH)
+        _measure.om_mi355x_measure_mfma_ceiling.restype = ctypes.c_int
+        _measure.om_mi355x_measure_mfma_ceiling.argtypes = [
+            ctypes.c_int64, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]
     tops, ghz = ctypes.c_double(0.0), ctypes.c_double(0.0)
-    if _lib.om_mi355x_mfma_ceiling(ctypes.c_int64(1 if random_operands else 0),
-                                   ctypes.byref(tops), ctypes.byref(ghz)) != 0:
-        _check()
-        raise RuntimeError_("om_mi355x_mfma_ceiling failed")
+    rc = _measure.om_mi355x_measure_mfma_ceiling(ctypes.c_int64(1 if random_operands else 0),
+                                                 ctypes.byref(tops), ctypes.byref(ghz))
+    if rc != 0:
+        raise RuntimeError_(f"om_mi355x_measure_mfma_ceiling failed: HIP error {rc}")
     return {"tops": tops.value, "clock_ghz": ghz.value}
 
 
@@ -365,6 +396,7 @@ def QuantizeLinear(x: Tensor, y_scale: Tensor, y_zero_point: Optional[Tensor] = 
         y_zero_point = _host(y_zero_point)
     y = out if out is not None else _like(x, x.shape, ydt)
     with _OMT(y) as hy, _OMT(x) as hx, _OMT(y_scale) as hs, _OMT(y_zero_point) as hz:
+        _emit_quant_mode()
         _lib.om_mi355x_QuantizeLinear(hy, hx, hs, hz, axis, saturate)
     _check()
     return y
@@ -378,6 +410,7 @@ def DequantizeLinear(x: Tensor, x_scale: Tensor, x_zero_point: Optional[Tensor] 
         x_zero_point = _host(x_zero_point)
     y = out if out is not None else _like(x, x.shape, np.float32)
     with _OMT(y) as hy, _OMT(x) as hx, _OMT(x_scale) as hs, _OMT(x_zero_point) as hz:
+        _emit_quant_mode()
         _lib.om_mi355x_DequantizeLinear(hy, hx, hs, hz, axis)
     _check()
     return y
@@ -394,6 +427,7 @@ def DynamicQuantizeLinear(x: Tensor, out: Optional[Tuple[Tensor, Tensor, Tensor]
         s = _like(x, (), np.float32)
         z = _like(x, (), np.uint8)
     with _OMT(y) as hy, _OMT(s) as hs, _OMT(z) as hz, _OMT(x) as hx:
+        _emit_quant_mode()
         _lib.om_mi355x_DynamicQuantizeLinear(hy, hs, hz, hx)
     _check()
     return y, s, z
@@ -406,6 +440,7 @@ def DynamicQuantizeLinearNoAlloc(x: DeviceArray, out: Tuple[DeviceArray, DeviceA
     load()
     y, s, z = out
     with _OMT(y) as hy, _OMT(s) as hs, _OMT(z) as hz, _OMT(x) as hx:
+        _emit_quant_mode()
         _lib.om_mi355x_DynamicQuantizeLinearNoAlloc(hy, hs, hz, hx)
     _check()
     return y, s, z
@@ -481,6 +516,7 @@ def DynQuantMatMulDequant(x: Tensor, b: Tensor, b_zero_point: Optional[Tensor],
     y = out if out is not None else _like(x, _mm_shape(x, b), np.float32)
     with _OMT(y) as hy, _OMT(x) as hx, _OMT(b) as hb, _OMT(bz) as hbz, _OMT(b_scale) as hbs, \
             _OMT(bias) as hbias:
+        _emit_quant_mode()
         _lib.om_mi355x_DynQuantMatMulDequant(hy, hx, hb, hbz, hbs, hbias, int(activation))
     _check()
     return y

@@ -43,6 +43,55 @@ def test_runtime_library_does_not_define_tensor_accessors(rt):
     assert "omTensorGetDataPtr" in und
 
 
+def test_runtime_does_not_depend_on_the_test_shim(rt):
+    """Neither form of the runtime names libom_tensor_shim.so: the omTensor*
+    accessors are resolved by whatever provides them in the process (a
+    compiled model's libcruntime; the shim in these tests)."""
+    import subprocess
+    dyn = subprocess.check_output(["readelf", "-d", rt.LIB_PATH], text=True)
+    needed = re.findall(r"\(NEEDED\).*\[(.*?)\]", dyn)
+    assert needed and not any("tensor_shim" in n for n in needed), needed
+    assert any(n.startswith("libamdhip64") for n in needed)
+
+
+def test_static_archive_links_into_a_model_library(rt, tmp_path):
+    """libRuntimeMI355X.a is what a compiled model links against, as the
+    reference's accelerators package their runtimes
+    (src/Accelerators/NNPA/Runtime/CMakeLists.txt:5-35; added to the link line
+    by CCM_SHARED_LIB_DEPS, src/Accelerators/NNPA/NNPAAccelerator.cpp:60-81).
+    A stand-in for a model -- one C function that references every entry point
+    of include/om_mi355x.h -- is linked into a shared library against the
+    archive and libamdhip64 the way src/Compiler/CompilerUtils.cpp links
+    models (C++ driver, -shared, -l<dep> after the object), loaded beside an
+    OMTensor provider, and called: the version handshake answers."""
+    import subprocess
+    archive = os.path.join(os.path.dirname(rt.LIB_PATH), "libRuntimeMI355X.a")
+    assert os.path.exists(archive), "libRuntimeMI355X.a is not built"
+    names = _declared("om_mi355x.h", r"\b(om_mi355x_\w+|OM\w+AccelMI355X)\s*\(")
+    stub = tmp_path / "model_stub.c"
+    stub.write_text(
+        '#include "om_mi355x.h"\n'
+        "const void *model_entry_points[] = {\n"
+        + "".join(f"  (const void *){n},\n" for n in names)
+        + "};\nunsigned long long model_handshake(unsigned long long v) {\n"
+          "  return OMInitCompatibleAccelMI355X(v);\n}\n")
+    obj, lib = tmp_path / "model_stub.o", tmp_path / "model.so"
+    subprocess.check_call(["gcc", "-c", "-fPIC", "-I", INCLUDE, str(stub), "-o", str(obj)])
+    subprocess.check_call(["g++", "-shared", "-fPIC", str(obj), "-o", str(lib),
+                           "-L", os.path.dirname(archive), "-lRuntimeMI355X",
+                           "-L", "/opt/rocm/lib", "-lamdhip64", "-Wl,-rpath,/opt/rocm/lib"])
+    defined = subprocess.check_output(["nm", "-D", "--defined-only", str(lib)], text=True)
+    assert "om_mi355x_QLinearMatMul" in defined and "omTensorGetDataPtr" not in defined
+    ctypes.CDLL(rt.SHIM_PATH, mode=ctypes.RTLD_GLOBAL)
+    model = ctypes.CDLL(str(lib))
+    model.model_handshake.restype = ctypes.c_uint64
+    model.model_handshake.argtypes = [ctypes.c_uint64]
+    # another major version is refused with or without a GPU
+    assert model.model_handshake(0x00FF0000) == 0
+    if not _no_gpu():
+        assert model.model_handshake(rt.VERSION) == 1
+
+
 @pytest.mark.skipif(not os.path.exists(REF_RUNTIME), reason="oracle/_ref not built (no reference tree)")
 def test_omtensor_layout_matches_reference_runtime(rt):
     """A tensor built by the reference's own C runtime is read correctly by our

@@ -1,0 +1,147 @@
+"""Parity of k_gemm_i8_flight -- the kernel for products that one round of
+blocks covers (K = 512, 768 or 1024), and the dynamically quantized layer in
+one launch -- with the CPU oracle, through the C-ABI.  Bit-exact, fp32
+included (same sequence of correctly rounded operations)."""
+import numpy as np
+import pytest
+
+import oracle_lib
+from om_mi355x import workloads as wl
+
+pytestmark = pytest.mark.gpu
+
+
+def _rand_q(rng, dt, shape):
+    info = np.iinfo(dt)
+    return rng.integers(info.min, info.max + 1, shape, dtype=dt)
+
+
+def bits(a):
+    return np.ascontiguousarray(a).view(np.uint32)
+
+
+def same_f32(a, b):
+    a, b = np.asarray(a, np.float32), np.asarray(b, np.float32)
+    return a.shape == b.shape and bool(np.all((bits(a) == bits(b)) | (np.isnan(a) & np.isnan(b))))
+
+
+def mm(oracle, A, B, a_zp, b_zp):
+    """The oracle's MatMulInteger; large products through its OpenMP restatement
+    of the reference's passes (pinned to the triple loop in test_oracle.py)."""
+    big = A.shape[0] * A.shape[1] * B.shape[1] > 1 << 27
+    return oracle.matmul_integer(A, B, a_zp, b_zp, passes=big)
+
+
+SHAPES = [(65, 512, 100), (128, 768, 768), (200, 1024, 1000), (512, 1024, 4096), (1000, 768, 416),
+          (4096, 768, 768), (97, 768, 33), (3000, 512, 1024)]
+
+
+@pytest.mark.parametrize("M,K,N", SHAPES)
+def test_one_round_kernel_all_operand_types_and_epilogues(rt, oracle, M, K, N):
+    """Every pair of operand types, zero points absent / scalar / per row and per
+    column, and the three epilogues (int32; f32 with per-column scale, bias and
+    Relu; 8-bit requantize, wrapping and saturating) on shapes with ragged edges
+    in both directions that the dispatch gives to k_gemm_i8_flight."""
+    rng = np.random.default_rng(M * 7 + K + N)
+    for adt, bdt in ((np.uint8, np.int8), (np.int8, np.uint8), (np.uint8, np.uint8), (np.int8, np.int8)):
+        A, B = _rand_q(rng, adt, (M, K)), _rand_q(rng, bdt, (K, N))
+        az, bz = _rand_q(rng, adt, (M,)), _rand_q(rng, bdt, (N,))
+        for a_zp, b_zp in ((None, None), (az[:1], None), (az[:1], bz[:1]), (az, bz)):
+            want = mm(oracle, A, B, a_zp, b_zp)
+            got = rt.MatMulInteger(A, B, a_zp, b_zp)
+            assert "flight" in rt.last_gemm_kernel(), rt.last_gemm_kernel()
+            assert np.array_equal(got, want), (adt, bdt, a_zp is not None, b_zp is not None)
+        acc = mm(oracle, A, B, az[:1], bz[:1])
+        a_s = np.float32(0.0173)
+        bs = rng.uniform(1e-3, 1e-2, N).astype(np.float32)
+        bias = rng.normal(0, 2, N).astype(np.float32)
+        want = oracle.dequant_epilogue(acc, a_s, bs) + bias
+        assert same_f32(rt.MatMulIntegerDequant(A, B, az[:1], bz[:1], a_s, bs, bias), want)
+        assert same_f32(rt.MatMulIntegerDequant(A, B, az[:1], bz[:1], a_s, bs, bias, activation=1),
+                        np.fmax(want, np.float32(0)))
+        assert "flight" in rt.last_gemm_kernel()
+        if adt == bdt:
+            ys = np.float32(0.37)
+            yz = _rand_q(rng, adt, ())
+            for mode, omode in ((rt.WRAP, oracle_lib.WRAP), (rt.SATURATE, oracle_lib.SATURATE)):
+                want = oracle.qlinear_matmul(A, a_s, az[:1], B, np.float32(0.005), bz[:1], ys, yz, omode)
+                got = rt.QLinearMatMul(A, a_s, az[:1], B, np.float32(0.005), bz[:1], ys, yz, mode)
+                assert "flight" in rt.last_gemm_kernel()
+                assert np.array_equal(got, want), (adt, mode)
+
+
+def test_one_round_kernel_is_forced_and_falls_through(rt, oracle, monkeypatch):
+    """OM_MI355X_GEMM_TILE=5 names the kernel; a shape it does not take (K no
+    multiple of 256, more blocks than one round) still computes, with another
+    kernel."""
+    monkeypatch.setenv("OM_MI355X_GEMM_TILE", "5")
+    rng = np.random.default_rng(55)
+    for (M, K, N), mine in (((300, 768, 500), True), ((300, 704, 500), False), ((8192, 768, 3072), False)):
+        A, B = _rand_q(rng, np.uint8, (M, K)), _rand_q(rng, np.int8, (K, N))
+        az = _rand_q(rng, np.uint8, ())
+        assert np.array_equal(rt.MatMulInteger(A, B, az, None), mm(oracle, A, B, az, None)), (M, K, N)
+        assert ("flight" in rt.last_gemm_kernel()) == mine, (M, K, N, rt.last_gemm_kernel())
+
+
+@pytest.mark.parametrize("M,K,N", [(33, 768, 768), (128, 768, 768), (100, 512, 200), (512, 1024, 1024), (65, 1024, 97),
+                                   (1024, 768, 768), (2048, 512, 100), (40, 768, 3072)])
+def test_dynamically_quantized_layer_in_one_launch(rt, oracle, M, K, N):
+    """DynamicQuantizeLinear -> MatMulInteger -> Cast -> Mul (-> Add -> Relu) as
+    one launch of k_gemm_i8_flight: the blocks agree on minimum and maximum
+    through the exchange slots, every block quantizes its own 32 rows.  Against
+    the oracle's chain of the separate ops, bit for bit; host and GPU-resident
+    operands; signed and unsigned weights, weight zero points; inputs whose
+    minimum or maximum sits in the last (ragged) row block, NaN and infinities
+    among the activations."""
+    rng = np.random.default_rng(M + K * 3 + N)
+    x = rng.normal(0, 1, (M, K)).astype(np.float32)
+    x[M - 1, K - 1] = 7.5            # the maximum in the last row
+    x[0, 0] = -6.25
+    for bdt in (np.int8, np.uint8):
+        W = _rand_q(rng, bdt, (K, N))
+        ws = rng.uniform(1e-3, 1e-2, N).astype(np.float32)
+        bias = rng.normal(0, 1, N).astype(np.float32)
+        bz = _rand_q(rng, bdt, (N,))
+        aq, a_s, a_zp = oracle.dynamic_quantize_linear(x)
+        for b_zp in (None, bz[:1], bz):
+            acc = mm(oracle, aq, W, a_zp, b_zp)
+            want = oracle.dequant_epilogue(acc, a_s, ws)
+            got = rt.DynQuantMatMulDequant(x, W, b_zp, ws)
+            assert "flight (rows quantized" in rt.last_gemm_kernel(), rt.last_gemm_kernel()
+            assert same_f32(got, want), (bdt, b_zp is not None)
+        wantb = np.fmax(oracle.dequant_epilogue(mm(oracle, aq, W, a_zp, None), a_s, ws[:1]) + bias,
+                        np.float32(0))
+        assert same_f32(rt.DynQuantMatMulDequant(x, W, None, ws[:1], bias, activation=1), wantb)
+    # GPU-resident operands, called repeatedly (the launch number in the slots moves on)
+    dX, dW, dS = rt.DeviceArray.from_numpy(x), rt.DeviceArray.from_numpy(W), rt.DeviceArray.from_numpy(ws)
+    dY = rt.DeviceArray((M, N), np.float32)
+    rt.mark_constant(dW)
+    acc = mm(oracle, aq, W, a_zp, None)
+    want = oracle.dequant_epilogue(acc, a_s, ws)
+    for _ in range(5):
+        rt.DynQuantMatMulDequant(dX, dW, None, dS, out=dY)
+    rt.synchronize()
+    assert same_f32(dY.numpy(), want)
+    rt.unmark_constant(dW)
+    for d in (dX, dW, dS, dY):
+        d.free()
+    # special values: NaN is ignored by the minimum / maximum and quantizes to
+    # the lower bound, infinities saturate (and make the scale infinite)
+    x2 = x.copy()
+    x2[3, 5] = np.nan
+    aq, a_s, a_zp = oracle.dynamic_quantize_linear(x2)
+    W = _rand_q(rng, np.int8, (K, N))
+    want = oracle.dequant_epilogue(mm(oracle, aq, W, a_zp, None), a_s, ws)
+    assert same_f32(rt.DynQuantMatMulDequant(x2, W, None, ws), want)
+    x2[M // 2, 7] = np.inf
+    aq, a_s, a_zp = oracle.dynamic_quantize_linear(x2)
+    want = oracle.dequant_epilogue(mm(oracle, aq, W, a_zp, None), a_s, ws)
+    assert same_f32(rt.DynQuantMatMulDequant(x2, W, None, ws), want)
+
+
+def test_config1_is_one_launch(rt, oracle):
+    c = wl.config1()
+    aq, a_s, a_zp = oracle.dynamic_quantize_linear(c["A"])
+    want = oracle.dequant_epilogue(oracle.matmul_integer(aq, c["B"], a_zp, c["b_zp"]), a_s, c["b_scale"])
+    assert same_f32(rt.DynQuantMatMulDequant(c["A"], c["B"], c["b_zp"], c["b_scale"]), want)
+    assert rt.last_gemm_kernel() == "k_gemm_i8_flight (rows quantized in the kernel)"
