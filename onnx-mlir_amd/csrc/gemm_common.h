@@ -166,12 +166,11 @@ hipError_t launch_gemm_wreg(hipStream_t st, const GemmArgs &g,
     const EpiParams &ep, int a_mode);
 
 // k_gemm_i8_flight (gemm_flight.hip): problems that one round of blocks covers,
-// K a multiple of 256 up to 1024.  flight_row_tiles: 0 if the kernel does not
-// take the problem.  The _dq forms take the f32 activation of a dynamically
+// K a multiple of 256 up to 1024.  The _dq forms take the f32 activation of a dynamically
 // quantized layer (GemmArgs::X) and quantize it in the same launch; the launch
 // returns hipErrorNotReady when the exchange between blocks cannot be used
 // right now (the caller quantizes with a launch of its own instead).
-int flight_row_tiles(const GemmArgs &g);
+bool flight_ok(const GemmArgs &g, int a_mode);
 hipError_t launch_gemm_flight(hipStream_t st, const GemmArgs &g,
     const EpiParams &ep, int a_mode);
 bool flight_quantizes_rows(int64_t M, int64_t K, int64_t N, const void *x);

@@ -1,9 +1,10 @@
 // int8 GEMM for gfx950 for problems that one round of blocks covers
-// (k_gemm_i8_flight): everything a block needs is requested at once.
+// (k_gemm_i8_flight, k_gemm_i8_flight_dq): everything a block needs is
+// requested at once.
 //
 // A small product -- a [128, 768] activation against [768, 768] weights, a
-// 512 x 1024 x 4096 QLinearMatMul -- is one tile per CU and a dozen K steps.
-// A pipelined K loop that keeps two or three steps in flight then pays the
+// 512 x 1024 x 4096 QLinearMatMul -- is at most one tile per CU and a dozen K
+// steps.  A pipelined K loop that keeps two or three steps in flight pays the
 // memory latency once per step or two (16 steps of ~0.35 us on top of the
 // launch: 8 us for work that the matrix cores do in under one).  Here a block
 // asks for all of its operands before it waits for any of them: the weights of
@@ -13,18 +14,27 @@
 // follows touches LDS and registers only.  K is limited by the registers (K <=
 // 1024: 128 per lane for the weights) and must be a multiple of 256.
 //
-// DQ: the whole dynamically quantized layer in one launch
+// What bounds such a launch is the path into the CU: it takes in about 64
+// bytes per clock (130 B/ns), and a load instruction is not issued before the
+// ones in front of it have been through.  512 x 1024 x 4096 on 256 CUs is
+// 192 KB per CU however it is tiled -- 1.45 us -- so the launcher picks, among
+// the block shapes that cover the problem in one round, the one with the
+// fewest bytes per block, and the K loop of the first row tile runs while the
+// weights are still arriving.
+//
+// k_gemm_i8_flight_dq: the whole dynamically quantized layer in one launch
 // (DynamicQuantizeLinear -> MatMulInteger -> Cast -> Mul,
 // src/Conversion/ONNXToKrnl/Quantization/DynamicQuantizeLinear.cpp:86-158 and
 // src/Conversion/ONNXToKrnl/Math/MatMulInteger.cpp:59-90).  The activation
-// arrives as f32 X[M,K].  A block loads its 32 rows into registers; the
-// blocks of a row region split those rows between them for the minimum and
-// maximum (a block reduces the K columns c with (c / 32) % G == its share),
-// publish them in the tagged slots that DynamicQuantizeLinear's one-launch
-// kernel uses, read everybody's, derive scale and zero point (every block the
-// same), quantize their rows into LDS and multiply.  No block reads more of X
-// than the rows it multiplies, and the weights arrive while the blocks wait
-// for one another.
+// arrives as f32 X[M,K].  A block of w waves owns 4 w rows and 32 w columns.
+// It first loads only its share of its rows (the blocks of a row region split
+// the region's columns between them), reduces it and publishes minimum and
+// maximum in the tagged slots that DynamicQuantizeLinear's one-launch kernel
+// uses; only then does it request the rest of its rows and its weights, which
+// arrive while the blocks wait for one another; then every block reads all
+// slots, derives scale and zero point (every block the same), quantizes its
+// rows into LDS and multiplies.  No block reads more of X than the rows it
+// multiplies.
 //
 // A in LDS: [row tile of 32][K group of 256 bytes][row][256 bytes]; within a
 // row's 256 bytes the 16-byte chunk c sits at position c ^ (row % 16), so the
@@ -40,251 +50,469 @@ namespace gemm {
 
 namespace {
 
-constexpr int kFlightKH = 32;   // K steps of 32 bytes a wave's registers hold
-constexpr int kFlightWaves = 4; // column tiles (of 32) per block
-constexpr int kFlightGroup = 8; // operand reads issued together
+#ifdef FLIGHT_TIMING
+// Development build: readings of the 100 MHz clock by wave 0 of every block at
+// fixed points, written out when the kernel ends (om_dev_flight_ts reads them).
+__device__ unsigned long long flight_ts[1024 * 10];
+#define FLIGHT_TS(i)                                                           \
+  if (wave == 0)                                                               \
+  ts[i] = __builtin_amdgcn_s_memrealtime()
+#define FLIGHT_TS_DECL                                                         \
+  unsigned long long ts[10] = {};                                              \
+  ts[8] = __builtin_readcyclecounter()
+#define FLIGHT_TS_WRITE                                                        \
+  ts[9] = __builtin_readcyclecounter();                                        \
+  if (wave == 0 && lane == 0 && blockIdx.x < 1024)                             \
+    for (int i_ = 0; i_ < 10; ++i_)                                            \
+  flight_ts[blockIdx.x * 10 + i_] = ts[i_]
+#else
+#define FLIGHT_TS(i)
+#define FLIGHT_TS_DECL
+#define FLIGHT_TS_WRITE
+#endif
 
-struct FlightDq {
-  const float *X;            // [M, K] f32
-  unsigned long long *slots; // tagged (launch number, value) slots
-  unsigned epoch;
-  unsigned *failed;
-  unsigned spin_limit;
-  int share_groups; // G: blocks of a row region that split its min / max
-  int col_blocks;   // blocks per row region
+constexpr int kFlightMaxKG = 4;  // K / 256 at most: 128 registers of weights
+constexpr int kFlightMaxTiles = 4;
+
+typedef __attribute__((address_space(3))) void *lds_ptr;
+typedef const __attribute__((address_space(1))) void *glb_ptr;
+
+// Block-wide barrier that orders LDS accesses and nothing else: this wave's LDS
+// operations have completed, and memory operations on global memory (loads
+// still arriving, copies into LDS of later pieces, stores on their way out)
+// keep flying across it.  (A workgroup fence, even one restricted to LDS, makes
+// the compiler wait for every outstanding vector memory operation as soon as
+// the kernel contains copies from global memory into LDS.)
+__device__ __forceinline__ void lds_sync() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" : : : "memory");
+}
+
+// Sum over the 16 lanes of a DPP row (lanes 16 k .. 16 k + 15); every lane
+// gets the total.
+__device__ __forceinline__ int32_t row16_sum(int32_t v) {
+  v += __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, true);  // quad_perm [1,0,3,2]
+  v += __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xF, 0xF, true);  // quad_perm [2,3,0,1]
+  v += __builtin_amdgcn_update_dpp(0, v, 0x141, 0xF, 0xF, true); // row_half_mirror
+  v += __builtin_amdgcn_update_dpp(0, v, 0x140, 0xF, 0xF, true); // row_mirror
+  return v;
+}
+
+// Minimum / maximum over the wave, every lane gets the result: within the
+// rows of 16 lanes by DPP, across the four rows through scalar registers (a
+// butterfly of __shfl_xor is six dependent LDS-crossbar round trips).
+template <bool MAX>
+__device__ __forceinline__ float wave_fold(float v) {
+  auto op = [](float a, float b) {
+    return MAX ? __builtin_fmaxf(a, b) : __builtin_fminf(a, b);
+  };
+  auto dpp = [](float a, auto ctrl) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(
+        0, __float_as_int(a), decltype(ctrl)::value, 0xF, 0xF, true));
+  };
+  v = op(v, dpp(v, std::integral_constant<int, 0xB1>{}));  // quad_perm [1,0,3,2]
+  v = op(v, dpp(v, std::integral_constant<int, 0x4E>{}));  // quad_perm [2,3,0,1]
+  v = op(v, dpp(v, std::integral_constant<int, 0x141>{})); // row_half_mirror
+  v = op(v, dpp(v, std::integral_constant<int, 0x140>{})); // row_mirror
+  const float r0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
+  const float r1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
+  const float r2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
+  const float r3 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
+  return op(op(r0, r1), op(r2, r3));
+}
+
+// The per-column operands of the epilogue and its scalars, as they come out
+// of memory.  Loaded before everything else so that their latency is spent
+// behind the operand loads; turned into FlightEpi once they are needed.
+struct FlightRaw {
+  float as, bs, ys, bias;
+  int32_t yz, az, bz, cs;
+  int yz_sh, az_sh, bz_sh; // where in the loaded word each zero point's byte is
 };
 
+// The aligned word that holds the byte at p + i: a byte load would be widened
+// right behind the load, which is a use of it, and the wave would wait there.
+__device__ __forceinline__ int32_t flight_load_byte_word(
+    const void *p, int i, int &shift) {
+  // (pointer arithmetic only: through an integer the pointer would lose its
+  // address space and the load become a flat one)
+  const int at = (int)(((uintptr_t)p + (uintptr_t)(uint32_t)i) & 3);
+  shift = at * 8;
+  return *(const int32_t *)((const char *)p + (i - at));
+}
+
+template <int EPI>
+__device__ __forceinline__ FlightRaw flight_load_params(
+    const EpiParams &ep, bool a_off, int nc) {
+  // absent operands read from colsum (always valid) and are masked later
+  const bool has_bzp = ep.b_zp_len > 0;
+  const void *bzp_ptr = has_bzp ? ep.b_zp : (const void *)ep.colsum;
+  const bool has_azp = ep.a_zp_len > 0;
+  const void *azp_ptr = has_azp ? ep.a_zp : (const void *)ep.colsum;
+  const bool has_bias = EPI == kEpiF32 && ep.bias != nullptr;
+  const float *bias_ptr = has_bias ? ep.bias : (const float *)ep.colsum;
+  const float *as_ptr =
+      (EPI != kEpiI32 && ep.a_scale) ? ep.a_scale : (const float *)ep.colsum;
+  const float *bs_ptr = EPI != kEpiI32 ? ep.b_scale : (const float *)ep.colsum;
+  const float *ys_ptr = EPI == kEpiQ8 ? ep.y_scale : (const float *)ep.colsum;
+  const void *yz_ptr = EPI == kEpiQ8 ? ep.y_zp : (const void *)ep.colsum;
+  // A zero the compiler cannot see through: a value loaded from an address
+  // that is the same in every lane would be moved to a scalar register right
+  // after the load, and the wave would wait there for every load it has
+  // issued.  These stay vector registers until the epilogue.
+  int vz = 0;
+  asm volatile("" : "+v"(vz));
+  FlightRaw r;
+  r.as = as_ptr[vz];
+  r.bs = bs_ptr[(EPI != kEpiI32 && ep.b_scale_len > 1) ? nc : vz];
+  r.ys = ys_ptr[vz];
+  // (the zero points as the bytes they are; flight_epi gives them their sign)
+  r.yz = flight_load_byte_word(yz_ptr, vz, r.yz_sh);
+  r.az = flight_load_byte_word(azp_ptr, vz, r.az_sh);
+  r.bz = flight_load_byte_word(bzp_ptr, ep.b_zp_len > 1 ? nc : vz, r.bz_sh);
+  r.cs = ep.colsum[nc];
+  r.bias = bias_ptr[has_bias && ep.bias_len > 1 ? nc : 0];
+  return r;
+}
+
+// Keeps every use of the parameters behind this point (the compiler would
+// otherwise decode them, and wait for them, as early as it can: in front of
+// the K loop, where that wait covers the weights as well).
+__device__ __forceinline__ void flight_params_not_before(FlightRaw &r) {
+  asm volatile(""
+               : "+v"(r.as), "+v"(r.bs), "+v"(r.ys), "+v"(r.bias), "+v"(r.yz),
+               "+v"(r.az), "+v"(r.bz), "+v"(r.cs));
+  r.yz = (r.yz >> r.yz_sh) & 0xff;
+  r.az = (r.az >> r.az_sh) & 0xff;
+  r.bz = (r.bz >> r.bz_sh) & 0xff;
+}
+
+// What the epilogue needs per lane (its column) once the parameters are in.
+struct FlightEpi {
+  uint32_t cj; // da0 * colsum[j] + K * da0 * db[j]
+  int32_t db;  // offset of B's column: its -128 shift minus its zero point
+  float sj;    // a_scale * b_scale[j] (/ y_scale)
+  float bj;    // bias[j], or -0.0f
+  int32_t yz;
+};
+
+// a_scale / a_zp: the values to use (the fused layer computes them itself).
+template <int EPI>
+__device__ __forceinline__ FlightEpi flight_epi(const EpiParams &ep,
+    const FlightRaw &r, bool a_off, int K, float a_scale, int32_t a_zp) {
+  FlightEpi e;
+  const int32_t oa = a_off ? 128 : 0;
+  const int32_t ob = ep.b_unsigned ? 128 : 0;
+  const int32_t da0 = oa - a_zp;
+  const int32_t bz = ep.b_unsigned ? r.bz : (int32_t)(int8_t)r.bz;
+  e.db = ob - (ep.b_zp_len > 0 ? bz : 0);
+  e.cj = (uint32_t)da0 * (uint32_t)r.cs +
+         (uint32_t)K * (uint32_t)da0 * (uint32_t)e.db;
+  e.sj = 0.0f;
+  e.yz = 0;
+  if (EPI != kEpiI32) {
+    // a_scale * b_scale[j] first, then one multiply per element; for the
+    // requantize (a_scale * b_scale) / y_scale, in this order
+    // (src/Conversion/ONNXToKrnl/Math/QLinearMatMul.cpp:127).
+    e.sj = a_scale * r.bs;
+    if (EPI == kEpiQ8) {
+      e.sj = e.sj / r.ys;
+      e.yz = ep.y_unsigned ? r.yz : (int32_t)(int8_t)r.yz;
+    }
+  }
+  e.bj = (EPI == kEpiF32 && ep.bias != nullptr) ? r.bias : -0.0f;
+  return e;
+}
+
+// One finished 32 x 32 tile of a wave: zero-point correction, the op's output
+// conversion, store.  Lane (column n = ncol0 + lane % 32, half lh) holds in
+// register r the row 8 (r / 4) + 4 lh + r % 4 of the tile.  Only the first
+// `rows` rows of the tile are the block's.  rs: LDS words with rowsum(A') of
+// the tile's 32 rows (read only if B carries an offset).  Results leave
+// through range-checked buffer stores on a descriptor that covers exactly the
+// M x N output: rows past M fall off its end, columns past N and rows that are
+// not the block's get an offset that is out of range for every row (the
+// hardware checks the sum of the lane's offset and the scalar row offset).
+// act: 0 none / Relu by EpiParams::floor, 2 Gelu.
+// 8-bit results in whole 16-byte pieces (N % 16 == 0, aligned output) pass
+// through `stage` (32 rows x 32 * waves bytes) so that a lane stores 16 bytes
+// of one row and the block's waves together write whole lines; every wave of
+// the block must then call this together.
+template <int EPI, bool RS>
+__device__ __forceinline__ void flight_store_tile(const v16i &acc,
+    const FlightEpi &e, const EpiParams &ep, const int32_t *rs, int mrow0,
+    int rows, int ncol0_block, int wave, int waves, int lane, int M, int N,
+    int act, uint8_t *stage, bool q8_lines) {
+  constexpr int ES = (EPI == kEpiQ8) ? 1 : 4;
+  const int l32 = lane & 31, lh = lane >> 5;
+  const int n = ncol0_block + wave * 32 + l32;
+  const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      ep.out, 0, (int)((uint32_t)M * (uint32_t)N * (uint32_t)ES), 0x00020000);
+  const uint32_t toff =
+      n < N ? ((uint32_t)(mrow0 + 4 * lh) * (uint32_t)N + (uint32_t)n) * (uint32_t)ES
+            : 0x80000000u;
+  // rowsum(A') of this lane's rows: four words per group of four registers
+  int32_t rsv[16];
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    v4i w = {0, 0, 0, 0};
+    if (RS)
+      w = *(const v4i *)(rs + 8 * g + 4 * lh);
+    rsv[4 * g + 0] = w.x;
+    rsv[4 * g + 1] = w.y;
+    rsv[4 * g + 2] = w.z;
+    rsv[4 * g + 3] = w.w;
+  }
+  const bool sat = EPI == kEpiQ8 && ep.narrow == kSaturate;
+  const int32_t sat_lo = ep.y_unsigned ? 0 : -128, sat_hi = ep.y_unsigned ? 255 : 127;
+  const int pitch = 32 * waves;
+  uint8_t *const my_stage = stage + 4 * lh * pitch + wave * 32 + l32;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int rr = 8 * (r >> 2) + (r & 3); // + 4 lh: the row within the tile
+    if (8 * (r >> 2) >= rows) // (the same for every lane) not the block's rows
+      continue;
+    // |rowsum| <= 128 K and |db| < 512 fit 24 bits: a full-rate multiply
+    uint32_t y = (uint32_t)acc[r] + e.cj;
+    if (RS)
+      y += (uint32_t)__mul24(e.db, rsv[r]);
+    const bool mine = rr + 4 * lh < rows;
+    const int voff = (int)(mine ? toff : 0x80000000u);
+    const int soff = rr * N * ES; // the same for every lane
+    if (EPI == kEpiI32) {
+      __builtin_amdgcn_raw_buffer_store_b32((int)y, rsrc, voff, soff, kAuxThrough);
+    } else if (EPI == kEpiF32) {
+      float f = (float)(int32_t)y * e.sj + e.bj;
+      f = act == 2 ? gelu_f32(f) : relu_f32(f, ep.floor);
+      __builtin_amdgcn_raw_buffer_store_b32(
+          (int)__float_as_uint(f), rsrc, voff, soff, kAuxThrough);
+    } else {
+      const float f = (float)(int32_t)y * e.sj;
+      int32_t v = (int32_t)((uint32_t)(int32_t)__builtin_rintf(f) + (uint32_t)e.yz);
+      if (sat)
+        v = v < sat_lo ? sat_lo : (v > sat_hi ? sat_hi : v);
+      if (q8_lines)
+        my_stage[rr * pitch] = (uint8_t)v;
+      else
+        __builtin_amdgcn_raw_buffer_store_b8((uint8_t)v, rsrc, voff, soff, 0);
+    }
+  }
+  if (EPI == kEpiQ8 && q8_lines) {
+    lds_sync();
+    // lane -> 16 bytes of one row: 2 * waves lanes a row, 32 / waves rows a wave
+    const int row = wave * (32 / waves) + lane / (2 * waves);
+    const int c16 = lane % (2 * waves);
+    const v4i w = *(const v4i *)(stage + row * pitch + c16 * 16);
+    const int col = ncol0_block + c16 * 16;
+    const uint32_t off = (col < N && row < rows)
+                             ? (uint32_t)(mrow0 + row) * (uint32_t)N + (uint32_t)col
+                             : 0x80000000u;
+    __builtin_amdgcn_raw_buffer_store_b128(w, rsrc, (int)off, 0, kAuxThrough);
+  }
+}
+
+// The K loop of one wave: LDS and registers only -- one LDS read and one MFMA a
+// step and nothing else.  (A wave does not issue while one of its MFMAs is being
+// fed, 32 clocks; vector instructions between the MFMAs of a wave add their
+// time to the loop instead of hiding in it.  Measured with one wave per SIMD:
+// 32 clocks an MFMA with two independent accumulators, 44 with one, 71 with
+// eight vector instructions in between.)
+//
+// Lane (row l32, half lh) takes chunk 2 s + lh of its row in step s.  With
+// s = 8 g + v that is chunk 2 v + lh of K group g, at byte 8192 g + 256 l32 +
+// ((32 v + 16 lh) ^ (16 (l32 % 16))) of the row tile: eight lane addresses
+// (aaddr), one per v, and an immediate per g.
+//
+// Two independent accumulators, because an MFMA that adds to the result of
+// the one before it waits for that result.  NT == 2: two row tiles (the second
+// KG * 8 KiB after the first), each over all of K, sharing the weights.
+// NT == 1: one row tile, even steps into acc[0], odd steps into acc[1]; the
+// caller adds them.  Operand reads run a batch of four steps ahead; they
+// complete in order, and the counts below say how many may still be
+// outstanding when one is used.
+// The weights may still be arriving when the loop starts: they were requested
+// in order of K, and the compiler puts the wait for each in front of its MFMA.
+template <int KG, int NT>
+__device__ __forceinline__ void flight_kloop(const unsigned (&aaddr)[8],
+    const v4i (&b)[8 * KG], v16i (&acc)[2]) {
+  constexpr int BS = 4, NB = 8 * KG / BS;
+  v4i fa[2][NT][BS];
+  auto read_batch = [&](auto kc) {
+    constexpr int k = decltype(kc)::value;
+    static_for<BS>([&](auto vc) {
+      static_for<NT>([&](auto tc) {
+        constexpr int s = BS * k + decltype(vc)::value, t = decltype(tc)::value;
+        v4i &f = fa[k & 1][t][decltype(vc)::value];
+        const unsigned addr = aaddr[s % 8];
+        asm volatile("ds_read_b128 %0, %1 offset:%2"
+                     : "=v"(f)
+                     : "v"(addr), "n"(8192 * (s / 8) + t * KG * 8192)
+                     : "memory");
+      });
+    });
+  };
+  read_batch(std::integral_constant<int, 0>{});
+  static_for<NB>([&](auto kc) {
+    constexpr int k = decltype(kc)::value;
+    constexpr bool more = k + 1 < NB;
+    if constexpr (more)
+      read_batch(std::integral_constant<int, k + 1>{});
+    static_for<BS>([&](auto vc) {
+      static_for<NT>([&](auto tc) {
+        constexpr int v = decltype(vc)::value, t = decltype(tc)::value;
+        constexpr int s = BS * k + v;
+        constexpr int c = NT == 2 ? t : (s & 1);
+        v4i &f = fa[k & 1][t][v];
+        asm volatile("s_waitcnt lgkmcnt(%1)"
+                     : "+v"(f)
+                     : "n"((BS - 1 - v) * NT + (NT - 1 - t) + (more ? BS * NT : 0))
+                     : "memory");
+        acc[c] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f, b[s], acc[c], 0, 0, 0);
+      });
+    });
+  });
+}
+
+// ---------------------------------------------------------------------------
 // KG: K / 256 (a template argument: every loop over K is unrolled and has no
-// branch).  nr: row tiles of 32 per block; the block's LDS, nr * KG * 8 KiB, is
-// sized at launch.
-template <int KG, bool A_OFF, bool DQ, int EPI>
-__global__ __launch_bounds__(kFlightWaves * 64, 1) void k_gemm_i8_flight(
+// branch).  A_MODE: 0 int8 as is, 1 uint8, 2 already stored minus 128.
+// The rows of A are copied into LDS without passing through registers.  When
+// they hold uint8, or when B carries an offset, every wave then goes once over
+// the pieces it copied: uint8 becomes int8 (minus 128) in place, and the row
+// sums of A' are taken -- vector work that is done while the weights are still
+// arriving, so that the K loop stays free of it.
+// Launch: waves = blockDim.x / 64 column tiles side by side, nr row tiles of 32
+// one after the other (1, 2 or 4); LDS nr * KG * 8 KiB + 512 + 2 * waves KiB.
+// ---------------------------------------------------------------------------
+template <int KG, int A_MODE, int EPI>
+__global__ __launch_bounds__(256, 1) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void k_gemm_i8_flight(
     const uint8_t *__restrict__ A, const int8_t *__restrict__ Bp, int M, int N,
-    EpiParams ep, uint32_t flip, int nr, int regions_n, int bp_tiles,
-    FlightDq dq) {
-  constexpr int WAVES = kFlightWaves, KH = 8 * KG, K = 256 * KG, G8 = kFlightGroup;
-  constexpr int KHMAX = KH;
-  static_assert(KH <= kFlightKH, "registers");
-  static_assert(!DQ || (A_OFF && EPI == kEpiF32), "fused layer");
+    EpiParams ep, int nr, int regions_n, int bp_tiles) {
+  constexpr int KH = 8 * KG, K = 256 * KG;
+  constexpr bool A_OFF = A_MODE != 0;
+  static_assert(KG >= 1 && KG <= kFlightMaxKG, "registers");
   extern __shared__ __attribute__((aligned(1024))) uint8_t sA[];
-  const int ROWS = 32 * nr;
-  __shared__ float s_lo[WAVES], s_hi[WAVES];
-  __shared__ int s_ok;
-  __shared__ float s_scale;
-  __shared__ __attribute__((aligned(4))) uint8_t s_zp[4];
+  int32_t *const s_rs = (int32_t *)(sA + nr * KG * 8192); // [32 * nr] row sums
+  uint8_t *const stage = (uint8_t *)(s_rs + 32 * kFlightMaxTiles);
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int waves = blockDim.x >> 6;
   const int l32 = lane & 31;
   const int lh = lane >> 5;
   const int rm = blockIdx.x / regions_n, rn = blockIdx.x % regions_n;
-  const int row0 = rm * ROWS;
-  const int ct = rn * WAVES + wave; // the wave's column tile
-
-  typedef __attribute__((address_space(3))) void *lds_ptr;
-  typedef const __attribute__((address_space(1))) void *glb_ptr;
+  const int row0 = rm * 32 * nr;
+  const int ct = rn * waves + wave; // the wave's column tile
+  FLIGHT_TS_DECL;
+  FLIGHT_TS(0);
 
   // ---- everything is requested here ----------------------------------------
-  typedef float f4 __attribute__((ext_vector_type(4)));
-  f4 x[DQ ? KHMAX : 1];
-  if (DQ) {
-    // Thread (row r = tid / 8, position p = tid % 8) takes float4 p + 8 j of
-    // its row, j < K / 32: a wave instruction reads 8 rows x 128 bytes, whole
-    // cache lines.  Register slot i holds j = ((i / S + share) % G) + G * (i % S)
-    // with S = (K / 32) / G, so that slots 0 .. S-1 are the block's own share
-    // of the minimum / maximum and arrive first.
-    const int r = tid >> 3;
-    const int row = row0 + r < M ? row0 + r : M - 1;
-    const f4 *__restrict__ xr = (const f4 *)(dq.X + (int64_t)row * K) + (tid & 7);
-    const int G = dq.share_groups, S = KH / G;
-    int a = 0, b = 0; // i / S, i % S
-#pragma unroll
-    for (int i = 0; i < KHMAX; ++i) {
-      int g = a + (rn % G);
-      g = g >= G ? g - G : g;
-      x[i] = xr[8 * (g + G * b)];
-      if (++b == S) {
-        b = 0;
-        ++a;
-      }
-    }
-  } else {
-    // A copy instruction fills 1 KiB of consecutive LDS, 16 bytes per lane:
-    // rows 4 q .. 4 q + 3 (q < 8) of K group cg of row tile t.  Lane l is
-    // position l % 16 of row 4 q + l / 16 and fetches the chunk that belongs
-    // there.  Wave w issues q = w and w + 4 of every (t, cg).  Rows past M
-    // are copies of the last row and are never stored.
-    const int rl = lane >> 4;
-#pragma unroll 1
-    for (int t = 0; t < nr; ++t) {
-#pragma unroll
-      for (int cg = 0; cg < KG; ++cg) {
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-          const int q = wave + 4 * h;
+  const bool need_rs = ep.need_rowsum;
+  // A piece of 1 KiB of LDS, 16 bytes per lane, is rows 4 q .. 4 q + 3 (q < 8)
+  // of K group cg of row tile t: lane l is position l % 16 of row 4 q + l / 16
+  // and holds the chunk that belongs there.  Wave w handles q = w, w + waves,
+  // ..  Rows past M are copies of the last row and are never stored.
+  // (Spelled out piece by piece rather than as loops, so that the compiler can
+  // count the copies on every path.)
+  // (Buffer loads, not global ones: the compiler takes a global load into LDS
+  // for an access that may touch both memories, and would from then on wait
+  // for every outstanding load at the first use of any.)  The block's rows
+  // start the buffer, so that offsets stay far below 2^31 whatever M is.
+  const int rl = lane >> 4;
+  const int rows_here = M - row0 < 32 * nr ? M - row0 : 32 * nr;
+  const __amdgpu_buffer_rsrc_t arsrc = __builtin_amdgcn_make_buffer_rsrc(
+      (void *)(A + (int64_t)row0 * K), 0, rows_here * K, 0x00020000);
+  static_for<kFlightMaxTiles>([&](auto tc) {
+    constexpr int t = decltype(tc)::value;
+    if (t < nr) {
+      static_for<8>([&](auto hc) {
+        const int q = wave + decltype(hc)::value * waves;
+        if (q < 8) { // (the same for the whole wave)
           const int r = 4 * q + rl; // row within the tile
           const int c = (lane & 15) ^ (r & 15);
-          int row = row0 + 32 * t + r;
-          row = row < M ? row : M - 1;
-          __builtin_amdgcn_global_load_lds(
-              (glb_ptr)(A + (int64_t)row * K + cg * 256 + c * 16),
-              (lds_ptr)(sA + ((t * KG + cg) * 8 + q) * 1024), 16, 0, 0);
+          int row = 32 * t + r;
+          row = row < rows_here ? row : rows_here - 1;
+          const int voff = row * K + c * 16;
+          static_for<KG>([&](auto cgc) {
+            constexpr int cg = decltype(cgc)::value;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(arsrc,
+                (lds_ptr)(sA + ((t * KG + cg) * 8 + q) * 1024), 16, voff,
+                cg * 256, 0, 0); // (an immediate offset would move the LDS side too)
+          });
         }
-      }
+      });
     }
-  }
-  v4i b[KHMAX];
+  });
+  __builtin_amdgcn_sched_barrier(0);
+  v4i b[KH];
   {
     // column tiles past the packed weights (the last region of a ragged N)
     // read the last tile and are not stored
     const int ctc = ct < bp_tiles ? ct : bp_tiles - 1;
     const int8_t *const bp = Bp + (int64_t)ctc * KH * 1024 + lane * 16;
+    // (the last 8 KG memory operations of the wave, in order of K: the K loop
+    // of the first tiles starts while the later ones are still arriving)
 #pragma unroll
-    for (int s = 0; s < KH; ++s)
+    for (int s = 0; s < KH; ++s) {
       b[s] = *(const v4i *)(bp + s * 1024);
-  }
-
-  if (DQ) {
-    // ---- minimum / maximum of the block's share, exchange, quantize ---------
-    const int G = dq.share_groups, S = KH / G;
-    const bool row_in = row0 + (tid >> 3) < M;
-    float lo = __builtin_inff(), hi = -__builtin_inff();
-#pragma unroll
-    for (int i = 0; i < KHMAX; ++i) {
-      if (i < S) {
-        lo = __builtin_fminf(lo, __builtin_fminf(__builtin_fminf(x[i].x, x[i].y),
-                                     __builtin_fminf(x[i].z, x[i].w)));
-        hi = __builtin_fmaxf(hi, __builtin_fmaxf(__builtin_fmaxf(x[i].x, x[i].y),
-                                     __builtin_fmaxf(x[i].z, x[i].w)));
-      }
+      __builtin_amdgcn_sched_barrier(0); // in this order
     }
-    if (!row_in) { // a copy of the last row: in another block's share already
-      lo = __builtin_inff();
-      hi = -__builtin_inff();
-    }
-    lo = wave_min(lo);
-    hi = wave_max(hi);
-    if (lane == 0) {
-      s_lo[wave] = lo;
-      s_hi[wave] = hi;
-    }
-    if (tid == 0)
-      s_ok = 1;
-    __syncthreads();
-    // Publishers: the first G blocks of every row region (with G == 1 every
-    // block of the region holds the same values and the first one publishes).
-    const int nslots = (int)(gridDim.x / dq.col_blocks) * G;
-    if (tid == 0 && rn < G) {
-      float bl = s_lo[0], bh = s_hi[0];
-#pragma unroll
-      for (int w = 1; w < WAVES; ++w) {
-        bl = __builtin_fminf(bl, s_lo[w]);
-        bh = __builtin_fmaxf(bh, s_hi[w]);
-      }
-      const unsigned long long tag = (unsigned long long)dq.epoch << 32;
-      const int slot = rm * G + rn;
-      __hip_atomic_store(&dq.slots[2 * slot], tag | __float_as_uint(bl),
-          __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      __hip_atomic_store(&dq.slots[2 * slot + 1], tag | __float_as_uint(bh),
-          __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    __syncthreads();
-    // Everybody's: one slot per thread (nslots <= 256), polled until both
-    // words carry this launch's number; bounded (see k_dql_grid).
-    typedef unsigned long long u64x2 __attribute__((ext_vector_type(2)));
-    bool ok = true;
-    lo = __builtin_inff();
-    hi = -__builtin_inff();
-    if (tid < nslots) {
-      u64x2 w = {0, 0};
-      bool got = false;
-      for (unsigned spin = 0; spin < dq.spin_limit; ++spin) {
-        asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)"
-                     : "=v"(w)
-                     : "v"(&dq.slots[2 * tid])
-                     : "memory");
-        if ((unsigned)(w.x >> 32) == dq.epoch && (unsigned)(w.y >> 32) == dq.epoch) {
-          got = true;
-          break;
-        }
-        __builtin_amdgcn_s_sleep(1);
-      }
-      ok = got;
-      lo = __uint_as_float((unsigned)w.x);
-      hi = __uint_as_float((unsigned)w.y);
-    }
-    lo = wave_min(lo);
-    hi = wave_max(hi);
-    const bool all_ok = __builtin_amdgcn_ballot_w64(!ok) == 0;
-    if (lane == 0) {
-      s_lo[wave] = lo;
-      s_hi[wave] = hi;
-      if (!all_ok)
-        s_ok = 0;
-    }
-    __syncthreads();
-    if (!s_ok) {
-      if (tid == 0)
-        __hip_atomic_store(
-            dq.failed, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      return;
-    }
-    lo = s_lo[0];
-    hi = s_hi[0];
-#pragma unroll
-    for (int w = 1; w < WAVES; ++w) {
-      lo = __builtin_fminf(lo, s_lo[w]);
-      hi = __builtin_fmaxf(hi, s_hi[w]);
-    }
-    float scale, zpf;
-    dynamic_params(lo, hi, scale, zpf);
-    if (tid == 0) {
-      s_scale = scale;
-      s_zp[0] = (uint8_t)(uint32_t)zpf;
-    }
-    // The 8-bit rows, minus 128, into LDS at the operand layout's positions.
-    const float recip = 1.0f / scale;
-    const int r = tid >> 3;
-    const int p = tid & 7;
-    uint8_t *const rowp = sA + r * 256 + (p & 3) * 4;
-    auto quantize = [&](auto fast_c) {
-      constexpr int FAST = decltype(fast_c)::value ? 1 : 0;
-      int a = 0, bq = 0;
-#pragma unroll
-      for (int i = 0; i < KHMAX; ++i) {
-        int g = a + (rn % G);
-        g = g >= G ? g - G : g;
-        const int j = g + G * bq;
-        // float4 p + 8 j of the row: K group j / 8, chunk 2 (j % 8) + p / 4
-        const int c = 2 * (j & 7) + (p >> 2);
-        const uint32_t q = quant_pack4<false, true, FAST>(x[i].x, x[i].y,
-            x[i].z, x[i].w, scale, scale, scale, scale, recip, recip, recip,
-            recip, zpf, zpf, zpf, zpf);
-        *(uint32_t *)(rowp + (j >> 3) * 8192 + ((c ^ (r & 15)) << 4)) =
-            q ^ 0x80808080u;
-        if (++bq == S) {
-          bq = 0;
-          ++a;
-        }
-      }
-    };
-    if (scale_is_tame(scale)) // the same for every thread
-      quantize(std::true_type{});
-    else
-      quantize(std::false_type{});
-    __syncthreads();
-  } else {
-    __builtin_amdgcn_s_waitcnt(0x0F70); // this wave's copies have landed
-    __builtin_amdgcn_s_barrier();
   }
   __builtin_amdgcn_sched_barrier(0);
+  // The epilogue's parameters, requested last and first used after the K loop
+  // of the first tiles (a use before that would wait for the weights, which
+  // were requested before them).
+  const int n = ct * 32 + l32;
+  FlightRaw raw = flight_load_params<EPI>(ep, A_OFF, n < N ? n : N - 1);
+  __builtin_amdgcn_sched_barrier(0);
+  FLIGHT_TS(1);
 
-  // ---- K loop: LDS and registers only -----------------------------------------
-  // Lane (row l32, half lh) takes chunk 2 s + lh of its row in step s.  With
-  // s = 8 g + v that is chunk 2 v + lh of K group g, at byte
-  // 8192 g + 256 l32 + ((32 v + 16 lh) ^ (16 (l32 % 16))) of the row tile:
-  // eight lane addresses, one per v, and an immediate per g.
+  // ---- A has landed ------------------------------------------------------------
+  // At most 8 KG memory operations are outstanding: the youngest ones, which
+  // are the parameters and all but a few of the loads of Bp (however many loads
+  // the parameters turned into, the copies of A are older than all of them).
+  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(8 * KG) : "memory");
+  FLIGHT_TS(2);
+  if (A_MODE == 1 || need_rs) {
+    static_for<kFlightMaxTiles>([&](auto tc) {
+      constexpr int t = decltype(tc)::value;
+      if (t < nr) {
+        static_for<8>([&](auto hc) {
+          const int q = wave + decltype(hc)::value * waves;
+          if (q < 8) {
+            // all reads of the piece first: one LDS latency, not KG
+            v4i v[KG];
+#pragma unroll
+            for (int cg = 0; cg < KG; ++cg)
+              v[cg] = *(const v4i *)(sA + ((t * KG + cg) * 8 + q) * 1024 + lane * 16);
+            int32_t sum = 0;
+#pragma unroll
+            for (int cg = 0; cg < KG; ++cg) {
+              if (A_MODE == 1) {
+                v[cg] ^= (v4i){(int)0x80808080, (int)0x80808080, (int)0x80808080,
+                    (int)0x80808080};
+                *(v4i *)(sA + ((t * KG + cg) * 8 + q) * 1024 + lane * 16) = v[cg];
+              }
+              sum += frag_rowsum(v[cg]);
+            }
+            if (need_rs) {
+              // the 16 lanes of a row hold all of its chunks: no other wave
+              // and no other piece adds to this row's sum
+              sum = row16_sum(sum);
+              if ((lane & 15) == 0)
+                s_rs[t * 32 + 4 * q + rl] = sum;
+            }
+          }
+        });
+      }
+    });
+  }
+  FLIGHT_TS(3);
+  lds_sync(); // every wave's rows (and row sums) are in LDS
+  __builtin_amdgcn_sched_barrier(0);
+  FLIGHT_TS(4);
+
   unsigned aaddr[8];
   {
     const unsigned arow = (unsigned)(uintptr_t)(lds_ptr)sA + l32 * 256;
@@ -293,118 +521,347 @@ __global__ __launch_bounds__(kFlightWaves * 64, 1) void k_gemm_i8_flight(
     for (int v = 0; v < 8; ++v)
       aaddr[v] = arow + ((unsigned)(32 * v) ^ xh);
   }
-  const v4i flip4 = {(int)flip, (int)flip, (int)flip, (int)flip};
-  const bool need_rs = ep.need_rowsum;
-  EpiParams epl = ep;
-  if (DQ) {
-    epl.a_scale = &s_scale;
-    epl.a_zp = s_zp;
-    epl.a_zp_len = 1;
-  }
-#pragma unroll 1
-  for (int t = 0; t < nr; ++t) {
-    v16i acc[1][1];
+  const bool q8_lines = EPI == kEpiQ8 && (N & 15) == 0 &&
+                        ((((uintptr_t)ep.out) & 15) == 0);
+  const v16i acc_zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+  auto finish = [&](const v16i &a, const FlightEpi &e, int t)
+                    __attribute__((always_inline)) {
+    uint8_t *const st = stage + (t & 1) * 1024 * waves;
+    if (need_rs) // (the same for every wave)
+      flight_store_tile<EPI, true>(a, e, ep, s_rs + 32 * t, row0 + 32 * t, 32,
+          rn * waves * 32, wave, waves, lane, M, N, 0, st, q8_lines);
+    else
+      flight_store_tile<EPI, false>(a, e, ep, s_rs, row0 + 32 * t, 32,
+          rn * waves * 32, wave, waves, lane, M, N, 0, st, q8_lines);
+  };
+  if (nr == 1) {
+    v16i acc[2] = {acc_zero, acc_zero};
+    flight_kloop<KG, 1>(aaddr, b, acc);
 #pragma unroll
     for (int r = 0; r < 16; ++r)
-      acc[0][0][r] = 0;
-    int32_t rsp[1] = {0};
-    v4i fa[2][G8];
-    auto read_group = [&](auto gc) { // the reads of steps 8 g .. 8 g + 7
-      constexpr int g = decltype(gc)::value;
-      static_for<G8>([&](auto vc) {
-        constexpr int v = decltype(vc)::value;
-        v4i &f = fa[g & 1][v];
-        const unsigned addr = aaddr[v];
-        asm volatile("ds_read_b128 %0, %1 offset:%2"
-                     : "=v"(f)
-                     : "v"(addr), "n"(8192 * g)
-                     : "memory");
-      });
+      acc[0][r] += acc[1][r];
+    FLIGHT_TS(5);
+    flight_params_not_before(raw);
+    const FlightEpi e = flight_epi<EPI>(ep, raw, A_OFF, K, raw.as,
+        ep.a_zp_len > 0 ? (A_OFF ? raw.az : (int32_t)(int8_t)raw.az) : 0);
+    finish(acc[0], e, 0);
+  } else {
+    v16i acc[2] = {acc_zero, acc_zero};
+    // the first two row tiles: the weights are still arriving
+    flight_kloop<KG, 2>(aaddr, b, acc);
+    FLIGHT_TS(5);
+    flight_params_not_before(raw);
+    const FlightEpi e = flight_epi<EPI>(ep, raw, A_OFF, K, raw.as,
+        ep.a_zp_len > 0 ? (A_OFF ? raw.az : (int32_t)(int8_t)raw.az) : 0);
+    finish(acc[0], e, 0);
+    finish(acc[1], e, 1);
+    if (nr == 4) {
+#pragma unroll
+      for (int v = 0; v < 8; ++v)
+        aaddr[v] += 2 * KG * 8192;
+      acc[0] = acc_zero;
+      acc[1] = acc_zero;
+      flight_kloop<KG, 2>(aaddr, b, acc);
+      finish(acc[0], e, 2);
+      finish(acc[1], e, 3);
+    }
+  }
+#ifdef FLIGHT_TIMING
+  FLIGHT_TS(6);
+  asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+  FLIGHT_TS(7);
+  FLIGHT_TS_WRITE;
+#endif
+}
+
+// ---------------------------------------------------------------------------
+// The dynamically quantized layer in one launch.  A block is eight waves; it
+// owns R = 8 << RSH rows of X and 32 * mwaves columns (mwaves <= 4: the waves
+// that multiply; all eight load and quantize X, which is what takes the time,
+// and the last four poll the exchange slots).
+// Thread (row r = tid / TPR, position p = tid % TPR, TPR = 512 / R) takes
+// float4 p + TPR j of its row, j < NJ = (K / 4) / TPR.  Register slot i holds
+// j = ((i / S + share) % G) + G * (i % S) with S = NJ / G: slots 0 .. S-1 are
+// the block's own share of its row region's minimum / maximum, the columns
+// the region's other blocks do not reduce.
+//
+// Order of the memory operations: the rows, the share first (loads complete in
+// order, so the share is there before the rest); [publication]; the epilogue's
+// parameters; then the weights in the waves that multiply and the poll of the
+// slots in the last four waves.  The weights arrive while the blocks wait for
+// one another and quantize.
+// ---------------------------------------------------------------------------
+struct FlightDq {
+  const float *X;            // [M, K] f32
+  unsigned long long *slots; // tagged (launch number, value) slots
+  unsigned epoch;
+  unsigned *failed;
+  unsigned spin_limit;
+  int share_groups; // G: blocks of a row region that split its min / max
+  int mwaves;       // waves that multiply: 32 * mwaves columns per block
+  int act;          // 0 none / Relu by EpiParams::floor, 2 Gelu
+};
+
+template <int KG, int RSH>
+__global__ __launch_bounds__(512, 1) void k_gemm_i8_flight_dq(
+    const int8_t *__restrict__ Bp, int M, int N, EpiParams ep, int regions_n,
+    int bp_tiles, FlightDq dq) {
+  constexpr int KH = 8 * KG, K = 256 * KG;
+  constexpr int WAVES = 8, T = 64 * WAVES;
+  constexpr int R = 8 << RSH;         // rows of the block
+  constexpr int TPR = T / R;          // threads per row: 64, 32 or 16
+  constexpr int NJ = (K / 4) / TPR;   // float4 per thread: KG, 2 KG or 4 KG
+  static_assert(RSH >= 0 && RSH <= 2, "rows");
+  extern __shared__ __attribute__((aligned(1024))) uint8_t sA[]; // one row tile
+  int32_t *const s_rs = (int32_t *)(sA + KG * 8192); // [32]
+  __shared__ float s_lo[WAVES], s_hi[WAVES];
+  __shared__ int s_ok;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int mwaves = dq.mwaves;
+  const int l32 = lane & 31;
+  const int lh = lane >> 5;
+  const int rm = blockIdx.x / regions_n, rn = blockIdx.x % regions_n;
+  const int row0 = rm * R;
+  const bool multiplies = wave < mwaves;
+  const int ct = rn * mwaves + (multiplies ? wave : 0);
+  FLIGHT_TS_DECL;
+  FLIGHT_TS(0);
+
+  typedef float f4 __attribute__((ext_vector_type(4)));
+  const int r = tid / TPR, p = tid % TPR;
+  const bool row_in = row0 + r < M;
+  const f4 *__restrict__ xr =
+      (const f4 *)(dq.X + (int64_t)(row_in ? row0 + r : M - 1) * K) + p;
+  const int G = dq.share_groups, S = NJ / G, share = rn % G;
+  // j of register slot i, as scalar arithmetic
+  int jof[NJ];
+  {
+    int a = 0, bb = 0;
+#pragma unroll
+    for (int i = 0; i < NJ; ++i) {
+      int g = a + share;
+      g = g >= G ? g - G : g;
+      jof[i] = g + G * bb;
+      if (++bb == S) {
+        bb = 0;
+        ++a;
+      }
+    }
+  }
+  // ---- the block's rows, its share of the minimum / maximum first ---------------
+  f4 x[NJ];
+#pragma unroll
+  for (int i = 0; i < NJ; ++i)
+    x[i] = xr[TPR * jof[i]];
+  __builtin_amdgcn_sched_barrier(0);
+  float lo = __builtin_inff(), hi = -__builtin_inff();
+#pragma unroll
+  for (int i = 0; i < NJ; ++i) {
+    if (i < S) {
+      lo = __builtin_fminf(lo, __builtin_fminf(__builtin_fminf(x[i].x, x[i].y),
+                                   __builtin_fminf(x[i].z, x[i].w)));
+      hi = __builtin_fmaxf(hi, __builtin_fmaxf(__builtin_fmaxf(x[i].x, x[i].y),
+                                   __builtin_fmaxf(x[i].z, x[i].w)));
+    }
+  }
+  if (!row_in) { // a copy of the last row, which its own block reduces
+    lo = __builtin_inff();
+    hi = -__builtin_inff();
+  }
+  lo = wave_fold<false>(lo);
+  hi = wave_fold<true>(hi);
+  if (lane == 0) {
+    s_lo[wave] = lo;
+    s_hi[wave] = hi;
+  }
+  if (tid == 0)
+    s_ok = 1;
+  if (tid < 32)
+    s_rs[tid] = 0;
+  lds_sync();
+  // Publishers: the first G blocks of every row region.
+  const int nslots = (int)(gridDim.x / regions_n) * G; // <= 256
+  if (tid == 0 && rn < G) {
+    float bl = s_lo[0], bh = s_hi[0];
+#pragma unroll
+    for (int w = 1; w < WAVES; ++w) {
+      bl = __builtin_fminf(bl, s_lo[w]);
+      bh = __builtin_fmaxf(bh, s_hi[w]);
+    }
+    const unsigned long long tag = (unsigned long long)dq.epoch << 32;
+    const int slot = rm * G + rn;
+    __hip_atomic_store(&dq.slots[2 * slot], tag | __float_as_uint(bl),
+        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(&dq.slots[2 * slot + 1], tag | __float_as_uint(bh),
+        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  FLIGHT_TS(1);
+  __builtin_amdgcn_sched_barrier(0);
+
+  // ---- the epilogue's parameters ------------------------------------------------
+  const int n = ct * 32 + l32;
+  FlightRaw raw = flight_load_params<kEpiF32>(ep, true, n < N ? n : N - 1);
+  const bool need_rs = ep.need_rowsum;
+  lds_sync(); // s_lo / s_hi are reused below
+  __builtin_amdgcn_sched_barrier(0);
+
+  // ---- the weights; the poll ---------------------------------------------------------
+  // The waves that multiply (the first mwaves <= 4) request their weights.  The
+  // last four waves poll: one slot per thread (nslots <= 256), until both
+  // words carry this launch's number; bounded (see k_dql_grid).  Each word was
+  // written by one atomic store and is read by one atomic load, past the
+  // caches that other XCDs do not see.  A polling wave has no weights on their
+  // way, so its answer does not queue behind them.
+  v4i b[KH];
+  bool got = true;
+  if (multiplies) { // (the same for the whole wave)
+    const int ctc = ct < bp_tiles ? ct : bp_tiles - 1;
+    const int8_t *const bp = Bp + (int64_t)ctc * KH * 1024 + lane * 16;
+#pragma unroll
+    for (int s = 0; s < KH; ++s) {
+      b[s] = *(const v4i *)(bp + s * 1024);
+      __builtin_amdgcn_sched_barrier(0); // in this order
+    }
+  } else if (wave >= 4) {
+    const int slot = tid - 256;
+    const bool polls = slot < nslots;
+    const unsigned long long *const slot_p = &dq.slots[2 * (polls ? slot : 0)];
+    unsigned long long w0 = 0, w1 = 0;
+    got = !polls;
+    for (unsigned spin = 0; !got && spin < dq.spin_limit; ++spin) {
+      if (spin)
+        __builtin_amdgcn_s_sleep(1);
+      w0 = __hip_atomic_load(slot_p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      w1 = __hip_atomic_load(slot_p + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      got = (unsigned)(w0 >> 32) == dq.epoch && (unsigned)(w1 >> 32) == dq.epoch;
+    }
+    lo = polls ? __uint_as_float((unsigned)w0) : __builtin_inff();
+    hi = polls ? __uint_as_float((unsigned)w1) : -__builtin_inff();
+    lo = wave_fold<false>(lo);
+    hi = wave_fold<true>(hi);
+    const bool all_ok = __builtin_amdgcn_ballot_w64(!got) == 0;
+    if (lane == 0) {
+      s_lo[wave - 4] = lo;
+      s_hi[wave - 4] = hi;
+      if (!all_ok)
+        s_ok = 0;
+    }
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  FLIGHT_TS(2);
+  lds_sync();
+  if (!s_ok) {
+    // (the loads of the weights still in flight are waited for at the end of
+    // the program like any others)
+    if (tid == 0)
+      __hip_atomic_store(
+          dq.failed, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return;
+  }
+  lo = s_lo[0];
+  hi = s_hi[0];
+#pragma unroll
+  for (int w2 = 1; w2 < 4; ++w2) { // what the four polling waves found
+    lo = __builtin_fminf(lo, s_lo[w2]);
+    hi = __builtin_fmaxf(hi, s_hi[w2]);
+  }
+  FLIGHT_TS(3);
+  float scale, zpf;
+  dynamic_params(lo, hi, scale, zpf);
+
+  // ---- the block's rows as 8-bit values minus 128, into LDS --------------------
+  // float4 c4 = p + TPR j of row r: bytes 4 c4 .. of the row, K group c4 / 64,
+  // chunk (c4 % 64) / 4 at position chunk ^ (r % 16).
+  {
+    const float recip = 1.0f / scale;
+    uint8_t *const rowp = sA + r * 256 + (p & 3) * 4;
+    int32_t sum = 0;
+    auto quantize = [&](auto fast_c) {
+      constexpr int FAST = decltype(fast_c)::value ? 1 : 0;
+#pragma unroll
+      for (int i = 0; i < NJ; ++i) {
+        const int c4 = p + TPR * jof[i];
+        const int c = (c4 & 63) >> 2;
+        const uint32_t q =
+            quant_pack4<false, true, FAST>(x[i].x, x[i].y, x[i].z, x[i].w, scale,
+                scale, scale, scale, recip, recip, recip, recip, zpf, zpf, zpf,
+                zpf) ^
+            0x80808080u;
+        *(uint32_t *)(rowp + (c4 >> 6) * 8192 + ((c ^ (r & 15)) << 4)) = q;
+        sum = __builtin_amdgcn_sdot4((int)q, 0x01010101, sum, false);
+      }
     };
-    read_group(std::integral_constant<int, 0>{});
-    static_for<KG>([&](auto gc) {
-      constexpr int g = decltype(gc)::value;
-      constexpr bool more = g + 1 < KG;
-      if constexpr (more)
-        read_group(std::integral_constant<int, g + 1>{});
-      static_for<G8>([&](auto vc) {
-        constexpr int v = decltype(vc)::value;
-        v4i &f = fa[g & 1][v];
-        // reads complete in order: this one has landed when at most the
-        // later ones of its group, and the next group's, are outstanding
-        asm volatile("s_waitcnt lgkmcnt(%1)"
-                     : "+v"(f)
-                     : "n"(G8 - 1 - v + (more ? G8 : 0))
-                     : "memory");
-        const v4i av = f ^ flip4;
-        if (need_rs)
-          rsp[0] += frag_rowsum(av);
-        acc[0][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
-            av, b[g * G8 + v], acc[0][0], 0, 0, 0);
-      });
-    });
-    gemm_epilogue<1, 1, A_OFF ? 2 : 0, EPI, kAuxThrough>(
-        acc, rsp, row0 + 32 * t, ct * 32, M, N, K, epl);
+    if (scale_is_tame(scale)) // the same for every thread
+      quantize(std::true_type{});
+    else
+      quantize(std::false_type{});
+    if (need_rs) {
+      // the TPR threads of a row are 1, 2 or 4 DPP rows of 16 lanes
+      sum = row16_sum(sum);
+      if ((p & 15) == 0)
+        atomicAdd(&s_rs[r], sum);
+    }
+  }
+  lds_sync();
+  __builtin_amdgcn_sched_barrier(0);
+  FLIGHT_TS(4);
+  if (!multiplies) {
+#ifdef FLIGHT_TIMING
+    asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+#endif
+    return;
+  }
+
+  // ---- K loop ---------------------------------------------------------------------
+  unsigned aaddr[8];
+  {
+    const unsigned arow = (unsigned)(uintptr_t)(lds_ptr)sA + l32 * 256;
+    const unsigned xh = (unsigned)((16 * lh) ^ (16 * (l32 & 15)));
 #pragma unroll
     for (int v = 0; v < 8; ++v)
-      aaddr[v] += KG * 8192;
+      aaddr[v] = arow + ((unsigned)(32 * v) ^ xh);
   }
+  flight_params_not_before(raw);
+  const FlightEpi e =
+      flight_epi<kEpiF32>(ep, raw, true, K, scale, (int32_t)(uint32_t)zpf);
+  v16i accs[2] = {{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0},
+      {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}};
+  flight_kloop<KG, 1>(aaddr, b, accs);
+  v16i acc;
+#pragma unroll
+  for (int r2 = 0; r2 < 16; ++r2)
+    acc[r2] = accs[0][r2] + accs[1][r2];
+  FLIGHT_TS(5);
+  if (need_rs) // (the same for every wave)
+    flight_store_tile<kEpiF32, true>(acc, e, ep, s_rs, row0, R, rn * mwaves * 32,
+        wave, mwaves, lane, M, N, dq.act, nullptr, false);
+  else
+    flight_store_tile<kEpiF32, false>(acc, e, ep, s_rs, row0, R, rn * mwaves * 32,
+        wave, mwaves, lane, M, N, dq.act, nullptr, false);
+#ifdef FLIGHT_TIMING
+  FLIGHT_TS(6);
+  asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+  FLIGHT_TS(7);
+  FLIGHT_TS_WRITE;
+#endif
 }
 
 // A block's LDS beyond the default limit has to be asked for, once per kernel.
 template <typename Kern>
 hipError_t flight_allow_lds(Kern kern) {
-  static const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-      hipFuncAttributeMaxDynamicSharedMemorySize, 4 * kFlightKH * 32 * 32);
+  static const hipError_t e =
+      hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+          hipFuncAttributeMaxDynamicSharedMemorySize, 144 * 1024);
   return e;
 }
 
-template <int KG, bool A_OFF, int EPI>
-hipError_t flight_launch(hipStream_t st, const GemmArgs &g, const EpiParams &ep,
-    uint32_t flip, int nr) {
-  const int ntiles = (int)((g.N + 31) / 32);
-  const int regions_n = (ntiles + kFlightWaves - 1) / kFlightWaves;
-  const int regions_m = (int)((g.M + 32 * nr - 1) / (32 * nr));
-  const int bp_tiles = (int)(round_up(g.N, kGemmBN) / 32);
-  const FlightDq none = {};
-  auto kern = k_gemm_i8_flight<KG, A_OFF, false, EPI>;
-  hipError_t e = flight_allow_lds(kern);
-  if (e != hipSuccess)
-    return e;
-  kern<<<dim3((unsigned)(regions_m * regions_n)), dim3(kFlightWaves * 64),
-      (size_t)nr * KG * 8192, st>>>((const uint8_t *)g.A, g.Bp, (int)g.M,
-      (int)g.N, ep, flip, nr, regions_n, bp_tiles, none);
-  return hipGetLastError();
-}
-
-template <bool A_OFF, int EPI>
-hipError_t flight_launch_kg(hipStream_t st, const GemmArgs &g,
-    const EpiParams &ep, uint32_t flip, int nr) {
-  switch (g.K / 256) {
-  case 2:
-    return flight_launch<2, A_OFF, EPI>(st, g, ep, flip, nr);
-  case 3:
-    return flight_launch<3, A_OFF, EPI>(st, g, ep, flip, nr);
-  case 4:
-    return flight_launch<4, A_OFF, EPI>(st, g, ep, flip, nr);
-  default:
-    return hipErrorInvalidValue;
-  }
-}
-
-template <int KG>
-hipError_t flight_launch_dq(hipStream_t st, const GemmArgs &g,
-    const EpiParams &ep, int regions_m, int regions_n, int bp_tiles,
-    const FlightDq &dq) {
-  auto kern = k_gemm_i8_flight<KG, true, true, kEpiF32>;
-  hipError_t e = flight_allow_lds(kern);
-  if (e != hipSuccess)
-    return e;
-  kern<<<dim3((unsigned)(regions_m * regions_n)), dim3(kFlightWaves * 64),
-      (size_t)KG * 8192, st>>>(nullptr, g.Bp, (int)g.M, (int)g.N, ep, 0u, 1,
-      regions_n, bp_tiles, dq);
-  return hipGetLastError();
-}
+struct FlightShape {
+  int nr, waves; // row tiles per block, column tiles per block
+  int64_t blocks;
+};
 
 int flight_cus() {
   static const int cus = [] {
@@ -418,82 +875,201 @@ int flight_cus() {
   return cus;
 }
 
-bool flight_k_ok(int64_t K) { return K >= 512 && K <= 32 * kFlightKH && K % 256 == 0; }
+bool flight_k_ok(int64_t K) {
+  return K >= 512 && K <= 256 * kFlightMaxKG && K % 256 == 0;
+}
+
+// Among the block shapes that cover the problem with at most one block per
+// CU, the one that brings the fewest bytes into a CU; with equal bytes the one
+// with more waves per block.  staged: the waves go over the rows in LDS once
+// more (uint8 rows, or B carries an offset); four waves share that work.
+FlightShape flight_shape(int64_t M, int64_t N, bool staged) {
+  FlightShape best = {0, 0, 0};
+  int64_t best_bytes = 0;
+  const int cus = flight_cus();
+  for (int nr = 1; nr <= kFlightMaxTiles; nr *= 2)
+    for (int w = staged ? 4 : 1; w <= 4; w *= 2) {
+      const int64_t blocks =
+          ((M + 32 * nr - 1) / (32 * nr)) * ((N + 32 * w - 1) / (32 * w));
+      if (blocks > cus)
+        continue;
+      const int64_t bytes = 32 * nr + 32 * w; // times K
+      if (best.nr == 0 || bytes < best_bytes ||
+          (bytes == best_bytes && w > best.waves)) {
+        best = FlightShape{nr, w, blocks};
+        best_bytes = bytes;
+      }
+    }
+  return best;
+}
+
+bool flight_staged(const GemmArgs &g, int a_mode) {
+  return a_mode == 1 || g.b_unsigned || (g.b_zp != nullptr && g.b_zp_len > 0);
+}
+
+template <int KG, int A_MODE, int EPI>
+hipError_t flight_launch(hipStream_t st, const GemmArgs &g, const EpiParams &ep,
+    const FlightShape &sh) {
+  const int regions_n = (int)((g.N + 32 * sh.waves - 1) / (32 * sh.waves));
+  const int regions_m = (int)((g.M + 32 * sh.nr - 1) / (32 * sh.nr));
+  const int bp_tiles = (int)(round_up(g.N, kGemmBN) / 32);
+  auto kern = k_gemm_i8_flight<KG, A_MODE, EPI>;
+  hipError_t e = flight_allow_lds(kern);
+  if (e != hipSuccess)
+    return e;
+  const size_t lds = (size_t)sh.nr * KG * 8192 + 4 * 32 * kFlightMaxTiles +
+                     2 * 1024 * (size_t)sh.waves;
+  kern<<<dim3((unsigned)(regions_m * regions_n)), dim3(64 * sh.waves), lds, st>>>(
+      (const uint8_t *)g.A, g.Bp, (int)g.M, (int)g.N, ep, sh.nr, regions_n,
+      bp_tiles);
+  return hipGetLastError();
+}
+
+template <int A_MODE, int EPI>
+hipError_t flight_launch_kg(hipStream_t st, const GemmArgs &g,
+    const EpiParams &ep, const FlightShape &sh) {
+  switch (g.K / 256) {
+  case 2:
+    return flight_launch<2, A_MODE, EPI>(st, g, ep, sh);
+  case 3:
+    return flight_launch<3, A_MODE, EPI>(st, g, ep, sh);
+  case 4:
+    return flight_launch<4, A_MODE, EPI>(st, g, ep, sh);
+  default:
+    return hipErrorInvalidValue;
+  }
+}
+
+template <int A_MODE>
+hipError_t flight_launch_epi(hipStream_t st, const GemmArgs &g,
+    const EpiParams &ep, const FlightShape &sh) {
+  switch (g.epi) {
+  case kEpiI32:
+    return flight_launch_kg<A_MODE, kEpiI32>(st, g, ep, sh);
+  case kEpiF32:
+    return flight_launch_kg<A_MODE, kEpiF32>(st, g, ep, sh);
+  default:
+    return flight_launch_kg<A_MODE, kEpiQ8>(st, g, ep, sh);
+  }
+}
+
+// Block shape of the fused layer: R = 8 << rsh rows, 32 * mwaves columns.
+// Among the shapes whose grid is resident at once, the one that brings the
+// fewest bytes into a CU (4 R + 32 mwaves, times K); nothing if there is none.
+struct FlightDqShape {
+  int rsh, mwaves;
+};
+bool flight_dq_shape(int64_t M, int64_t N, FlightDqShape &best) {
+  const int cus = flight_cus() < 256 ? flight_cus() : 256;
+  int64_t best_bytes = 0;
+  bool found = false;
+  for (int rsh = 0; rsh <= 2; ++rsh)
+    for (int w = 1; w <= 4; w *= 2) {
+      const int64_t R = 8 << rsh;
+      if (((M + R - 1) / R) * ((N + 32 * w - 1) / (32 * w)) > cus)
+        continue;
+      const int64_t bytes = 4 * R + 32 * w;
+      if (!found || bytes < best_bytes) {
+        best = FlightDqShape{rsh, w};
+        best_bytes = bytes;
+        found = true;
+      }
+    }
+  return found;
+}
+
+template <int KG, int RSH>
+hipError_t flight_launch_dq(hipStream_t st, const GemmArgs &g,
+    const EpiParams &ep, const FlightDq &dq) {
+  const int regions_n = (int)((g.N + 32 * dq.mwaves - 1) / (32 * dq.mwaves));
+  const int regions_m = (int)((g.M + (8 << RSH) - 1) / (8 << RSH));
+  const int bp_tiles = (int)(round_up(g.N, kGemmBN) / 32);
+  auto kern = k_gemm_i8_flight_dq<KG, RSH>;
+  hipError_t e = flight_allow_lds(kern);
+  if (e != hipSuccess)
+    return e;
+  kern<<<dim3((unsigned)(regions_m * regions_n)), dim3(512),
+      (size_t)KG * 8192 + 128, st>>>(g.Bp, (int)g.M, (int)g.N, ep, regions_n,
+      bp_tiles, dq);
+  return hipGetLastError();
+}
+
+template <int KG>
+hipError_t flight_launch_dq_rows(hipStream_t st, const GemmArgs &g,
+    const EpiParams &ep, int rsh, const FlightDq &dq) {
+  switch (rsh) {
+  case 0:
+    return flight_launch_dq<KG, 0>(st, g, ep, dq);
+  case 1:
+    return flight_launch_dq<KG, 1>(st, g, ep, dq);
+  default:
+    return flight_launch_dq<KG, 2>(st, g, ep, dq);
+  }
+}
 
 } // namespace
 
-// Row tiles per block for this problem: the fewest with which one round of
-// blocks (one block per CU) covers it; 0 if the kernel does not take it.
-int flight_row_tiles(const GemmArgs &g) {
-  if (!flight_k_ok(g.K) || g.M < 1 || g.X || ((((uintptr_t)g.A) & 15) != 0))
-    return 0;
-  const int64_t regions_n = ((g.N + 31) / 32 + kFlightWaves - 1) / kFlightWaves;
-  const int cus = flight_cus();
-  for (int nr = 1; nr <= 4; nr *= 2)
-    if (((g.M + 32 * nr - 1) / (32 * nr)) * regions_n <= cus)
-      return nr;
-  return 0;
+// Whether k_gemm_i8_flight takes this problem (a_mode as in launch_gemm: 0 int8,
+// 1 uint8, 2 stored minus 128).  One zero point per row of A is left to the
+// other kernels.
+bool flight_ok(const GemmArgs &g, int a_mode) {
+  if (!flight_k_ok(g.K) || g.M < 1 || g.X || ((((uintptr_t)g.A) & 15) != 0) ||
+      g.M * g.N >= ((int64_t)1 << 29) || (g.a_zp != nullptr && g.a_zp_len > 1))
+    return false;
+  return flight_shape(g.M, g.N, flight_staged(g, a_mode)).nr > 0;
 }
 
 hipError_t launch_gemm_flight(hipStream_t st, const GemmArgs &g,
     const EpiParams &ep, int a_mode) {
-  const int nr = flight_row_tiles(g);
-  if (nr == 0)
+  if (!flight_ok(g, a_mode))
     return hipErrorInvalidValue;
-  const uint32_t flip = a_mode == 1 ? 0x80808080u : 0u;
-  if (a_mode == 0) {
-    switch (g.epi) {
-    case kEpiI32:
-      return flight_launch_kg<false, kEpiI32>(st, g, ep, flip, nr);
-    case kEpiF32:
-      return flight_launch_kg<false, kEpiF32>(st, g, ep, flip, nr);
-    default:
-      return flight_launch_kg<false, kEpiQ8>(st, g, ep, flip, nr);
-    }
-  }
-  switch (g.epi) {
-  case kEpiI32:
-    return flight_launch_kg<true, kEpiI32>(st, g, ep, flip, nr);
-  case kEpiF32:
-    return flight_launch_kg<true, kEpiF32>(st, g, ep, flip, nr);
+  const bool staged = flight_staged(g, a_mode);
+  const FlightShape sh = flight_shape(g.M, g.N, staged);
+  switch (a_mode) {
+  case 0:
+    return flight_launch_epi<0>(st, g, ep, sh);
+  case 1:
+    return flight_launch_epi<1>(st, g, ep, sh);
   default:
-    return flight_launch_kg<true, kEpiQ8>(st, g, ep, flip, nr);
+    return flight_launch_epi<2>(st, g, ep, sh);
   }
 }
 
-// The fused layer in one launch: 32 rows per block, and every block of the
-// grid resident at once (they wait for one another).
+// The fused layer in one launch: every block of the grid resident at once
+// (they wait for one another).
 bool flight_quantizes_rows(int64_t M, int64_t K, int64_t N, const void *x) {
-  if (!flight_k_ok(K) || M < 1 || ((((uintptr_t)x) & 15) != 0))
+  if (!flight_k_ok(K) || M < 1 || N < 1 || ((((uintptr_t)x) & 15) != 0) ||
+      M * N >= ((int64_t)1 << 29))
     return false;
-  const int64_t regions_n = ((N + 31) / 32 + kFlightWaves - 1) / kFlightWaves;
-  const int cus = flight_cus();
-  return ((M + 31) / 32) * regions_n <= (cus < 256 ? cus : 256);
+  FlightDqShape sh;
+  return flight_dq_shape(M, N, sh);
 }
 
 hipError_t launch_gemm_flight_dq(hipStream_t st, const GemmArgs &g,
     const EpiParams &ep, DqlScratch &scratch) {
-  if (!g.X || g.epi != kEpiF32 || !flight_quantizes_rows(g.M, g.K, g.N, g.X))
+  FlightDqShape sh;
+  if (!g.X || g.epi != kEpiF32 || !flight_quantizes_rows(g.M, g.K, g.N, g.X) ||
+      !flight_dq_shape(g.M, g.N, sh))
     return hipErrorInvalidValue;
-  const int ntiles = (int)((g.N + 31) / 32);
-  const int regions_n = (ntiles + kFlightWaves - 1) / kFlightWaves;
-  const int regions_m = (int)((g.M + 31) / 32);
-  const int bp_tiles = (int)(round_up(g.N, kGemmBN) / 32);
-  if (2 * regions_m * regions_n > 2 * scratch.max_blocks)
+  const int R = 8 << sh.rsh;
+  const int regions_n = (int)((g.N + 32 * sh.mwaves - 1) / (32 * sh.mwaves));
+  const int regions_m = (int)((g.M + R - 1) / R);
+  if (regions_m * regions_n > scratch.max_blocks)
     return hipErrorInvalidValue;
   FlightDq dq = {};
   dq.X = g.X;
-  dq.col_blocks = regions_n;
-  // the largest number of blocks of a row region, a divisor of the K steps,
-  // that can share the region's minimum / maximum between them
-  const int KH = (int)(g.K / 32);
+  dq.act = g.gelu ? 2 : 0;
+  dq.mwaves = sh.mwaves;
+  // the largest number of blocks of a row region, a divisor of the float4s a
+  // thread holds, that can share the region's minimum / maximum between them
+  const int NJ = (int)(g.K / 4) / (512 / R);
   dq.share_groups = 1;
-  for (int d = 1; d <= regions_n && d <= KH; ++d)
-    if (KH % d == 0)
+  for (int d = 1; d <= regions_n && d <= NJ; ++d)
+    if (NJ % d == 0)
       dq.share_groups = d;
   GridExchange ex;
   if (!dql_exchange_begin(st, scratch, ex))
-    return hipErrorNotReady; // another stream's exchange may be running
+    return hipErrorNotReady; // the exchange is off or another stream's runs
   dq.slots = ex.slots;
   dq.epoch = ex.epoch;
   dq.failed = ex.failed;
@@ -501,13 +1077,13 @@ hipError_t launch_gemm_flight_dq(hipStream_t st, const GemmArgs &g,
   hipError_t e;
   switch (g.K / 256) {
   case 2:
-    e = flight_launch_dq<2>(st, g, ep, regions_m, regions_n, bp_tiles, dq);
+    e = flight_launch_dq_rows<2>(st, g, ep, sh.rsh, dq);
     break;
   case 3:
-    e = flight_launch_dq<3>(st, g, ep, regions_m, regions_n, bp_tiles, dq);
+    e = flight_launch_dq_rows<3>(st, g, ep, sh.rsh, dq);
     break;
   default:
-    e = flight_launch_dq<4>(st, g, ep, regions_m, regions_n, bp_tiles, dq);
+    e = flight_launch_dq_rows<4>(st, g, ep, sh.rsh, dq);
     break;
   }
   dql_exchange_end(st, e == hipSuccess);
@@ -516,3 +1092,11 @@ hipError_t launch_gemm_flight_dq(hipStream_t st, const GemmArgs &g,
 
 } // namespace gemm
 } // namespace om
+
+#ifdef FLIGHT_TIMING
+extern "C" int om_dev_flight_ts(void *out, size_t bytes) {
+  (void)hipDeviceSynchronize();
+  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(om::gemm::flight_ts),
+      bytes < sizeof(om::gemm::flight_ts) ? bytes : sizeof(om::gemm::flight_ts));
+}
+#endif

@@ -1418,7 +1418,7 @@ hipError_t gemm_launch_cfg(
   // where a pipelined K loop would pay the memory latency step after step
   // (512 x 1024 x 4096 QLinearMatMul: 8.2 us in 128 x 64 tiles of
   // k_gemm_i8_dma; 128 x 768 x 768: 7.0 us).
-  if ((cfg == kFlight || !(force && force[0])) && flight_row_tiles(g) > 0) {
+  if ((cfg == kFlight || !(force && force[0])) && flight_ok(g, A_MODE)) {
     t_last_kernel = "k_gemm_i8_flight (one round, operands requested at once)";
     return launch_gemm_flight(st, g, ep, A_MODE);
   }
