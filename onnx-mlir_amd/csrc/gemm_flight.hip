@@ -9,37 +9,59 @@
 // launch: 8 us for work that the matrix cores do in under one).  Here a block
 // asks for all of its operands before it waits for any of them: the weights of
 // a wave's 32 columns for all of K go straight into registers (Bp is stored in
-// that order, see gemm_kernels.hip), the block's rows of A for all of K are
-// copied into LDS without passing through registers, and the K loop that
-// follows touches LDS and registers only.  K is limited by the registers (K <=
-// 1024: 128 per lane for the weights) and must be a multiple of 256.
+// that order, see gemm_kernels.hip), the block's rows of A for all of K pass
+// through registers into LDS (uint8 becomes int8 on the way), and the K loop
+// that follows touches LDS and registers only.  K is limited by the registers
+// (K <= 1024: 128 per lane for the weights) and must be a multiple of 256.
 //
 // What bounds such a launch is the path into the CU: it takes in about 64
 // bytes per clock (130 B/ns), and a load instruction is not issued before the
 // ones in front of it have been through.  512 x 1024 x 4096 on 256 CUs is
 // 192 KB per CU however it is tiled -- 1.45 us -- so the launcher picks, among
 // the block shapes that cover the problem in one round, the one with the
-// fewest bytes per block, and the K loop of the first row tile runs while the
-// weights are still arriving.
+// fewest bytes per block.
+//
+// What the compiler must see, and not see (each of these was a measured
+// microsecond):
+//  - every load is an ordinary one in program order; the compiler then puts
+//    a wait for exactly the loads up to the one used in front of each use.
+//    Loads it cannot count (inline asm) make it wait for everything at the
+//    first use of anything, and their destination registers are not safe.
+//  - no flat load (a pointer that went through an integer): while one is
+//    outstanding every wait is for all loads;
+//  - a value loaded from an address that is the same in all lanes is moved
+//    to a scalar register right behind the load, which waits for it: such
+//    loads index with an opaque zero;
+//  - byte loads are widened right behind the load: zero points are loaded as
+//    the aligned word that holds them;
+//  - barriers are s_barrier behind a wait for LDS only (lds_sync): a
+//    workgroup fence waits for the global loads in flight as well;
+//  - branches that only some waves take, with loads in them, merge into a
+//    wait for the shortest count: the multiplying and the polling waves of
+//    the fused kernel run the rest of the kernel in separate branches.
+// One wave per SIMD: vector instructions are not hidden behind anything, a
+// wave issues about one per four clocks, so their number is what a phase
+// costs; between two MFMAs each costs its issue time on top (a wait
+// instruction about eight clocks).
 //
 // k_gemm_i8_flight_dq: the whole dynamically quantized layer in one launch
 // (DynamicQuantizeLinear -> MatMulInteger -> Cast -> Mul,
 // src/Conversion/ONNXToKrnl/Quantization/DynamicQuantizeLinear.cpp:86-158 and
 // src/Conversion/ONNXToKrnl/Math/MatMulInteger.cpp:59-90).  The activation
-// arrives as f32 X[M,K].  A block of w waves owns 4 w rows and 32 w columns.
-// It first loads only its share of its rows (the blocks of a row region split
-// the region's columns between them), reduces it and publishes minimum and
-// maximum in the tagged slots that DynamicQuantizeLinear's one-launch kernel
-// uses; only then does it request the rest of its rows and its weights, which
-// arrive while the blocks wait for one another; then every block reads all
-// slots, derives scale and zero point (every block the same), quantizes its
-// rows into LDS and multiplies.  No block reads more of X than the rows it
-// multiplies.
+// arrives as f32 X[M,K].  A block of eight waves owns 8, 16 or 32 rows and up
+// to 128 columns.  All of its rows are requested at once, its share of them
+// first (the blocks of a row region split the region's columns between them);
+// it reduces the share and publishes minimum and maximum in the tagged slots
+// that DynamicQuantizeLinear's one-launch kernel uses; then it requests its
+// weights, which arrive while the blocks wait for one another; then every
+// block reads all slots, derives scale and zero point (every block the same),
+// quantizes its rows into LDS and multiplies.  No block reads more of X than
+// the rows it multiplies.
 //
 // A in LDS: [row tile of 32][K group of 256 bytes][row][256 bytes]; within a
 // row's 256 bytes the 16-byte chunk c sits at position c ^ (row % 16), so the
 // lanes of an operand read (rows 0..31, the same chunk of each) fall into
-// different banks, and a copy instruction (1 KiB of consecutive LDS) is four
+// different banks, and a staging store (1 KiB of consecutive LDS) is four
 // rows of one K group: 256 contiguous bytes of each row of A.
 
 #include "gemm_common.h"
@@ -60,19 +82,27 @@ __device__ unsigned long long flight_ts[1024 * 10];
 #define FLIGHT_TS_DECL                                                         \
   unsigned long long ts[10] = {};                                              \
   ts[8] = __builtin_readcyclecounter()
+#ifdef FLIGHT_EXP_KCLK
+#define FLIGHT_TS_CYC(i) ts[i] = __builtin_readcyclecounter()
+#define FLIGHT_TS_END
+#else
+#define FLIGHT_TS_CYC(i)
+#define FLIGHT_TS_END ts[9] = __builtin_readcyclecounter()
+#endif
 #define FLIGHT_TS_WRITE                                                        \
-  ts[9] = __builtin_readcyclecounter();                                        \
+  FLIGHT_TS_END;                                                               \
   if (wave == 0 && lane == 0 && blockIdx.x < 1024)                             \
     for (int i_ = 0; i_ < 10; ++i_)                                            \
   flight_ts[blockIdx.x * 10 + i_] = ts[i_]
 #else
 #define FLIGHT_TS(i)
+#define FLIGHT_TS_CYC(i)
 #define FLIGHT_TS_DECL
 #define FLIGHT_TS_WRITE
 #endif
 
 constexpr int kFlightMaxKG = 4;  // K / 256 at most: 128 registers of weights
-constexpr int kFlightMaxTiles = 4;
+constexpr int kFlightMaxTiles = 2;
 
 typedef __attribute__((address_space(3))) void *lds_ptr;
 typedef const __attribute__((address_space(1))) void *glb_ptr;
@@ -178,6 +208,7 @@ __device__ __forceinline__ FlightRaw flight_load_params(
 // otherwise decode them, and wait for them, as early as it can: in front of
 // the K loop, where that wait covers the weights as well).
 __device__ __forceinline__ void flight_params_not_before(FlightRaw &r) {
+  __builtin_amdgcn_sched_barrier(0); // (nor the K loop's last steps behind it)
   asm volatile(""
                : "+v"(r.as), "+v"(r.bs), "+v"(r.ys), "+v"(r.bias), "+v"(r.yz),
                "+v"(r.az), "+v"(r.bz), "+v"(r.cs));
@@ -227,17 +258,20 @@ __device__ __forceinline__ FlightEpi flight_epi(const EpiParams &ep,
 // conversion, store.  Lane (column n = ncol0 + lane % 32, half lh) holds in
 // register r the row 8 (r / 4) + 4 lh + r % 4 of the tile.  Only the first
 // `rows` rows of the tile are the block's.  rs: LDS words with rowsum(A') of
-// the tile's 32 rows (read only if B carries an offset).  Results leave
-// through range-checked buffer stores on a descriptor that covers exactly the
-// M x N output: rows past M fall off its end, columns past N and rows that are
-// not the block's get an offset that is out of range for every row (the
-// hardware checks the sum of the lane's offset and the scalar row offset).
+// the tile's 32 rows (they only matter if B carries an offset: without one
+// they are multiplied by zero, whatever they hold).  Results leave through
+// range-checked buffer stores on a descriptor that covers exactly the M x N
+// output: rows past M fall off its end, columns past N and rows that are not
+// the block's get an offset that is out of range for every row (the hardware
+// checks the sum of the lane's offset and the scalar row offset).
 // act: 0 none / Relu by EpiParams::floor, 2 Gelu.
 // 8-bit results in whole 16-byte pieces (N % 16 == 0, aligned output) pass
 // through `stage` (32 rows x 32 * waves bytes) so that a lane stores 16 bytes
 // of one row and the block's waves together write whole lines; every wave of
 // the block must then call this together.
-template <int EPI, bool RS>
+// (One wave per SIMD: nothing hides the latency of these instructions, so
+// their number is what the epilogue costs.  No branch per element.)
+template <int EPI>
 __device__ __forceinline__ void flight_store_tile(const v16i &acc,
     const FlightEpi &e, const EpiParams &ep, const int32_t *rs, int mrow0,
     int rows, int ncol0_block, int wave, int waves, int lane, int M, int N,
@@ -250,64 +284,84 @@ __device__ __forceinline__ void flight_store_tile(const v16i &acc,
   const uint32_t toff =
       n < N ? ((uint32_t)(mrow0 + 4 * lh) * (uint32_t)N + (uint32_t)n) * (uint32_t)ES
             : 0x80000000u;
-  // rowsum(A') of this lane's rows: four words per group of four registers
-  int32_t rsv[16];
+  // this lane's results before the output conversion
+  // (|rowsum| <= 128 K and |db| < 512 fit 24 bits: a full-rate multiply)
+  uint32_t y[16];
 #pragma unroll
   for (int g = 0; g < 4; ++g) {
-    v4i w = {0, 0, 0, 0};
-    if (RS)
-      w = *(const v4i *)(rs + 8 * g + 4 * lh);
-    rsv[4 * g + 0] = w.x;
-    rsv[4 * g + 1] = w.y;
-    rsv[4 * g + 2] = w.z;
-    rsv[4 * g + 3] = w.w;
+    const v4i w = *(const v4i *)(rs + 8 * g + 4 * lh);
+    y[4 * g + 0] = (uint32_t)acc[4 * g + 0] + e.cj + (uint32_t)__mul24(e.db, w.x);
+    y[4 * g + 1] = (uint32_t)acc[4 * g + 1] + e.cj + (uint32_t)__mul24(e.db, w.y);
+    y[4 * g + 2] = (uint32_t)acc[4 * g + 2] + e.cj + (uint32_t)__mul24(e.db, w.z);
+    y[4 * g + 3] = (uint32_t)acc[4 * g + 3] + e.cj + (uint32_t)__mul24(e.db, w.w);
   }
-  const bool sat = EPI == kEpiQ8 && ep.narrow == kSaturate;
-  const int32_t sat_lo = ep.y_unsigned ? 0 : -128, sat_hi = ep.y_unsigned ? 255 : 127;
+  if (EPI != kEpiQ8) {
+    if (EPI == kEpiF32) {
+      float f[16];
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        f[r] = (float)(int32_t)y[r] * e.sj + e.bj;
+      if (act == 2) { // (the same for every lane)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          y[r] = __float_as_uint(gelu_f32(f[r]));
+      } else {
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          y[r] = __float_as_uint(relu_f32(f[r], ep.floor));
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int rr = 8 * (r >> 2) + (r & 3); // + 4 lh: the row within the tile
+      if (8 * (r >> 2) >= rows) // (the same for every lane) not the block's rows
+        continue;
+      const int voff = (int)(rr + 4 * lh < rows ? toff : 0x80000000u);
+      const int soff = rr * N * ES; // the same for every lane
+      __builtin_amdgcn_raw_buffer_store_b32((int)y[r], rsrc, voff, soff, kAuxThrough);
+    }
+    return;
+  }
+  // 8-bit: wrapping keeps the low byte, which the byte store does by itself;
+  // saturating clamps first
+  const bool sat = ep.narrow == kSaturate;
+  const int32_t sat_lo = !sat ? INT32_MIN : ep.y_unsigned ? 0 : -128;
+  const int32_t sat_hi = !sat ? INT32_MAX : ep.y_unsigned ? 255 : 127;
+  const int32_t sat_hi_v = sat_hi; // (an instruction reads one scalar register)
+  int32_t v[16];
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const float f = (float)(int32_t)y[r] * e.sj;
+    v[r] = (int32_t)((uint32_t)(int32_t)__builtin_rintf(f) + (uint32_t)e.yz);
+    // (one instruction; bounds that do nothing when the result wraps)
+    asm("v_med3_i32 %0, %1, %2, %3" : "=v"(v[r]) : "v"(v[r]), "s"(sat_lo), "v"(sat_hi_v));
+  }
+  if (!q8_lines) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int rr = 8 * (r >> 2) + (r & 3);
+      if (8 * (r >> 2) >= rows)
+        continue;
+      const int voff = (int)(rr + 4 * lh < rows ? toff : 0x80000000u);
+      __builtin_amdgcn_raw_buffer_store_b8((uint8_t)v[r], rsrc, voff, rr * N, 0);
+    }
+    return;
+  }
   const int pitch = 32 * waves;
   uint8_t *const my_stage = stage + 4 * lh * pitch + wave * 32 + l32;
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const int rr = 8 * (r >> 2) + (r & 3); // + 4 lh: the row within the tile
-    if (8 * (r >> 2) >= rows) // (the same for every lane) not the block's rows
-      continue;
-    // |rowsum| <= 128 K and |db| < 512 fit 24 bits: a full-rate multiply
-    uint32_t y = (uint32_t)acc[r] + e.cj;
-    if (RS)
-      y += (uint32_t)__mul24(e.db, rsv[r]);
-    const bool mine = rr + 4 * lh < rows;
-    const int voff = (int)(mine ? toff : 0x80000000u);
-    const int soff = rr * N * ES; // the same for every lane
-    if (EPI == kEpiI32) {
-      __builtin_amdgcn_raw_buffer_store_b32((int)y, rsrc, voff, soff, kAuxThrough);
-    } else if (EPI == kEpiF32) {
-      float f = (float)(int32_t)y * e.sj + e.bj;
-      f = act == 2 ? gelu_f32(f) : relu_f32(f, ep.floor);
-      __builtin_amdgcn_raw_buffer_store_b32(
-          (int)__float_as_uint(f), rsrc, voff, soff, kAuxThrough);
-    } else {
-      const float f = (float)(int32_t)y * e.sj;
-      int32_t v = (int32_t)((uint32_t)(int32_t)__builtin_rintf(f) + (uint32_t)e.yz);
-      if (sat)
-        v = v < sat_lo ? sat_lo : (v > sat_hi ? sat_hi : v);
-      if (q8_lines)
-        my_stage[rr * pitch] = (uint8_t)v;
-      else
-        __builtin_amdgcn_raw_buffer_store_b8((uint8_t)v, rsrc, voff, soff, 0);
-    }
-  }
-  if (EPI == kEpiQ8 && q8_lines) {
-    lds_sync();
-    // lane -> 16 bytes of one row: 2 * waves lanes a row, 32 / waves rows a wave
-    const int row = wave * (32 / waves) + lane / (2 * waves);
-    const int c16 = lane % (2 * waves);
-    const v4i w = *(const v4i *)(stage + row * pitch + c16 * 16);
-    const int col = ncol0_block + c16 * 16;
-    const uint32_t off = (col < N && row < rows)
-                             ? (uint32_t)(mrow0 + row) * (uint32_t)N + (uint32_t)col
-                             : 0x80000000u;
-    __builtin_amdgcn_raw_buffer_store_b128(w, rsrc, (int)off, 0, kAuxThrough);
-  }
+  for (int r = 0; r < 16; ++r)
+    my_stage[(8 * (r >> 2) + (r & 3)) * pitch] = (uint8_t)v[r];
+  lds_sync();
+  // lane -> 16 bytes of one row: 2 * waves lanes a row, 32 / waves rows a wave
+  const int row = wave * (32 / waves) + lane / (2 * waves);
+  const int c16 = lane % (2 * waves);
+  const v4i w = *(const v4i *)(stage + row * pitch + c16 * 16);
+  const int col = ncol0_block + c16 * 16;
+  const uint32_t off = (col < N && row < rows)
+                           ? (uint32_t)(mrow0 + row) * (uint32_t)N + (uint32_t)col
+                           : 0x80000000u;
+  __builtin_amdgcn_raw_buffer_store_b128(w, rsrc, (int)off, 0, kAuxThrough);
 }
 
 // The K loop of one wave: LDS and registers only -- one LDS read and one MFMA a
@@ -356,16 +410,35 @@ __device__ __forceinline__ void flight_kloop(const unsigned (&aaddr)[8],
     constexpr bool more = k + 1 < NB;
     if constexpr (more)
       read_batch(std::integral_constant<int, k + 1>{});
+    // One wait for the batch's operand reads (the next batch's stay
+    // outstanding) and one for its weights: a wait instruction between two
+    // MFMAs costs about eight clocks, a quarter of an MFMA.
+    v4i &f0 = fa[k & 1][0][0], &f1 = fa[k & 1][0][1], &f2 = fa[k & 1][0][2],
+        &f3 = fa[k & 1][0][3];
+    if constexpr (NT == 2) {
+      v4i &g0 = fa[k & 1][1][0], &g1 = fa[k & 1][1][1], &g2 = fa[k & 1][1][2],
+          &g3 = fa[k & 1][1][3];
+      asm volatile("s_waitcnt lgkmcnt(%8)"
+                   : "+v"(f0), "+v"(g0), "+v"(f1), "+v"(g1), "+v"(f2), "+v"(g2),
+                   "+v"(f3), "+v"(g3)
+                   : "n"(more ? BS * NT : 0)
+                   : "memory");
+    } else {
+      asm volatile("s_waitcnt lgkmcnt(%4)"
+                   : "+v"(f0), "+v"(f1), "+v"(f2), "+v"(f3)
+                   : "n"(more ? BS * NT : 0)
+                   : "memory");
+    }
+    // (a use of the batch's last weights: the compiler waits for them here,
+    // and with them for the batch's others, which were requested earlier)
+    const v4i &b_last = b[BS * k + BS - 1];
+    asm volatile("" : : "v"(b_last));
     static_for<BS>([&](auto vc) {
       static_for<NT>([&](auto tc) {
         constexpr int v = decltype(vc)::value, t = decltype(tc)::value;
         constexpr int s = BS * k + v;
         constexpr int c = NT == 2 ? t : (s & 1);
         v4i &f = fa[k & 1][t][v];
-        asm volatile("s_waitcnt lgkmcnt(%1)"
-                     : "+v"(f)
-                     : "n"((BS - 1 - v) * NT + (NT - 1 - t) + (more ? BS * NT : 0))
-                     : "memory");
         acc[c] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f, b[s], acc[c], 0, 0, 0);
       });
     });
@@ -374,23 +447,32 @@ __device__ __forceinline__ void flight_kloop(const unsigned (&aaddr)[8],
 
 // ---------------------------------------------------------------------------
 // KG: K / 256 (a template argument: every loop over K is unrolled and has no
-// branch).  A_MODE: 0 int8 as is, 1 uint8, 2 already stored minus 128.
-// The rows of A are copied into LDS without passing through registers.  When
-// they hold uint8, or when B carries an offset, every wave then goes once over
-// the pieces it copied: uint8 becomes int8 (minus 128) in place, and the row
-// sums of A' are taken -- vector work that is done while the weights are still
-// arriving, so that the K loop stays free of it.
-// Launch: waves = blockDim.x / 64 column tiles side by side, nr row tiles of 32
-// one after the other (1, 2 or 4); LDS nr * KG * 8 KiB + 512 + 2 * waves KiB.
+// branch).  FLIP: A holds uint8 and becomes int8 (minus 128) on its way into
+// LDS; a_off: A' = A - 128 (FLIP, or A was stored that way).
+// A block is WAVES column tiles side by side and NR row tiles of 32 one after
+// the other (1 or 2, 2 NR <= WAVES).  Its rows of A are
+// 8 nr groups of four rows; wave w brings groups w, w + waves, .. (two or four:
+// with the weights, up to 192 registers of operands in flight) through its
+// registers into LDS: uint8 becomes int8 (minus 128) on the
+// way, and the row sums of A' are taken there if B carries an offset -- vector
+// work on data that arrives first, done while the weights are still arriving,
+// so that the K loop stays free of it.
+// Every load is one the compiler sees, in program order A, Bp in order of K,
+// parameters: it puts in front of each use a wait for exactly the loads up to
+// the one used, and the K loop starts while the weights are still arriving.
+// LDS: nr * KG * 8 KiB + 512 + 2 * waves KiB.
 // ---------------------------------------------------------------------------
-template <int KG, int A_MODE, int EPI>
-__global__ __launch_bounds__(256, 1) __attribute__((amdgpu_waves_per_eu(1, 1)))
-void k_gemm_i8_flight(
+template <int KG, bool FLIP, int EPI, int NR, int WAVES>
+__global__ __launch_bounds__(64 * WAVES, 1)
+__attribute__((amdgpu_waves_per_eu(1, 1))) void k_gemm_i8_flight(
     const uint8_t *__restrict__ A, const int8_t *__restrict__ Bp, int M, int N,
-    EpiParams ep, int nr, int regions_n, int bp_tiles) {
+    EpiParams ep, int a_off, int regions_n, int bp_tiles) {
   constexpr int KH = 8 * KG, K = 256 * KG;
-  constexpr bool A_OFF = A_MODE != 0;
+  constexpr int nr = NR, waves = WAVES;
+  constexpr int P = (8 * NR) / WAVES; // groups of four rows a wave stages
   static_assert(KG >= 1 && KG <= kFlightMaxKG, "registers");
+  static_assert(NR <= kFlightMaxTiles && (P == 2 || P == 4), "registers");
+  const bool A_OFF = a_off != 0;
   extern __shared__ __attribute__((aligned(1024))) uint8_t sA[];
   int32_t *const s_rs = (int32_t *)(sA + nr * KG * 8192); // [32 * nr] row sums
   uint8_t *const stage = (uint8_t *)(s_rs + 32 * kFlightMaxTiles);
@@ -398,7 +480,6 @@ void k_gemm_i8_flight(
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int waves = blockDim.x >> 6;
   const int l32 = lane & 31;
   const int lh = lane >> 5;
   const int rm = blockIdx.x / regions_n, rn = blockIdx.x % regions_n;
@@ -409,109 +490,94 @@ void k_gemm_i8_flight(
 
   // ---- everything is requested here ----------------------------------------
   const bool need_rs = ep.need_rowsum;
-  // A piece of 1 KiB of LDS, 16 bytes per lane, is rows 4 q .. 4 q + 3 (q < 8)
-  // of K group cg of row tile t: lane l is position l % 16 of row 4 q + l / 16
-  // and holds the chunk that belongs there.  Wave w handles q = w, w + waves,
-  // ..  Rows past M are copies of the last row and are never stored.
-  // (Spelled out piece by piece rather than as loops, so that the compiler can
-  // count the copies on every path.)
-  // (Buffer loads, not global ones: the compiler takes a global load into LDS
-  // for an access that may touch both memories, and would from then on wait
-  // for every outstanding load at the first use of any.)  The block's rows
-  // start the buffer, so that offsets stay far below 2^31 whatever M is.
+  // Group g of the block is rows 4 g .. 4 g + 3 (of row tile g / 8); for each
+  // K group it is 1 KiB of LDS, 16 bytes per lane: lane l is position l % 16 of
+  // row 4 g + l / 16 and holds the chunk that belongs there.  Rows past M are
+  // copies of the last row and are never stored.
   const int rl = lane >> 4;
-  const int rows_here = M - row0 < 32 * nr ? M - row0 : 32 * nr;
-  const __amdgpu_buffer_rsrc_t arsrc = __builtin_amdgcn_make_buffer_rsrc(
-      (void *)(A + (int64_t)row0 * K), 0, rows_here * K, 0x00020000);
-  static_for<kFlightMaxTiles>([&](auto tc) {
-    constexpr int t = decltype(tc)::value;
-    if (t < nr) {
-      static_for<8>([&](auto hc) {
-        const int q = wave + decltype(hc)::value * waves;
-        if (q < 8) { // (the same for the whole wave)
-          const int r = 4 * q + rl; // row within the tile
-          const int c = (lane & 15) ^ (r & 15);
-          int row = 32 * t + r;
-          row = row < rows_here ? row : rows_here - 1;
-          const int voff = row * K + c * 16;
-          static_for<KG>([&](auto cgc) {
-            constexpr int cg = decltype(cgc)::value;
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(arsrc,
-                (lds_ptr)(sA + ((t * KG + cg) * 8 + q) * 1024), 16, voff,
-                cg * 256, 0, 0); // (an immediate offset would move the LDS side too)
-          });
-        }
-      });
-    }
-  });
-  __builtin_amdgcn_sched_barrier(0);
-  v4i b[KH];
-  {
-    // column tiles past the packed weights (the last region of a ragged N)
-    // read the last tile and are not stored
-    const int ctc = ct < bp_tiles ? ct : bp_tiles - 1;
-    const int8_t *const bp = Bp + (int64_t)ctc * KH * 1024 + lane * 16;
-    // (the last 8 KG memory operations of the wave, in order of K: the K loop
-    // of the first tiles starts while the later ones are still arriving)
+  v4i a[P][KG];
+  auto request_rows = [&](auto hc) __attribute__((always_inline)) {
+    constexpr int h = decltype(hc)::value;
+    const int r = 4 * (wave + h * waves) + rl; // row within the block
+    const int c = (lane & 15) ^ (r & 15);
+    int row = row0 + r;
+    row = row < M ? row : M - 1;
+    const uint8_t *const src = A + (int64_t)row * K + c * 16;
 #pragma unroll
-    for (int s = 0; s < KH; ++s) {
-      b[s] = *(const v4i *)(bp + s * 1024);
+    for (int cg = 0; cg < KG; ++cg) {
+      a[h][cg] = *(const v4i *)(src + cg * 256);
       __builtin_amdgcn_sched_barrier(0); // in this order
     }
-  }
+  };
+  static_for<P>([&](auto hc) { request_rows(hc); });
   __builtin_amdgcn_sched_barrier(0);
+  v4i b[KH];
+  // column tiles past the packed weights (the last region of a ragged N)
+  // read the last tile and are not stored
+  const int ctc = ct < bp_tiles ? ct : bp_tiles - 1;
+  const int8_t *const bp = Bp + (int64_t)ctc * KH * 1024 + lane * 16;
+  auto request_weights = [&](auto from_c, auto to_c) __attribute__((always_inline)) {
+    constexpr int FROM = decltype(from_c)::value, TO = decltype(to_c)::value;
+    static_for<TO - FROM>([&](auto sc) {
+      constexpr int s = FROM + decltype(sc)::value;
+      b[s] = *(const v4i *)(bp + s * 1024);
+      __builtin_amdgcn_sched_barrier(0); // in this order
+    });
+  };
+  // The rows into LDS.
+  auto stage_rows = [&](auto hc) __attribute__((always_inline)) {
+    constexpr int h = decltype(hc)::value;
+    const int g = wave + h * waves;
+    uint8_t *const dst = sA + (g >> 3) * (KG * 8192) + (g & 7) * 1024 + lane * 16;
+    int32_t sum = 0;
+#pragma unroll
+    for (int cg = 0; cg < KG; ++cg) {
+      v4i v = a[h][cg];
+      if (FLIP)
+        v ^= (v4i){(int)0x80808080, (int)0x80808080, (int)0x80808080,
+            (int)0x80808080};
+      *(v4i *)(dst + cg * 8192) = v;
+      if (need_rs) // (the same for every wave)
+        sum += frag_rowsum(v);
+    }
+    if (need_rs) {
+      // the 16 lanes of a row hold all of its chunks: no other wave and no
+      // other group adds to this row's sum
+      sum = row16_sum(sum);
+      if ((lane & 15) == 0)
+        s_rs[4 * g + rl] = sum;
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  // A wave issues a load only when the ones before it have been taken in, so
+  // the requests for the weights take as long as the weights take to arrive,
+  // and the rows, requested first, land halfway through.  They are staged
+  // between the requests, not after them: the K loop can then start as soon
+  // as the last request is out, and follows the weights as they arrive.
+  typedef std::integral_constant<int, 0> c0;
+  typedef std::integral_constant<int, KH / 2> c_half;
+  typedef std::integral_constant<int, 3 * KH / 4> c_3q;
+  typedef std::integral_constant<int, KH> c_all;
+  request_weights(c0{}, c_half{});
+  FLIGHT_TS(1);
+  static_for<P / 2>([&](auto hc) { stage_rows(hc); });
+  FLIGHT_TS(2);
+  request_weights(c_half{}, c_3q{});
+  static_for<P / 2>([&](auto hc) {
+    stage_rows(std::integral_constant<int, P / 2 + decltype(hc)::value>{});
+  });
+  request_weights(c_3q{}, c_all{});
   // The epilogue's parameters, requested last and first used after the K loop
-  // of the first tiles (a use before that would wait for the weights, which
-  // were requested before them).
+  // (a use before that would wait for the weights, which were requested before
+  // them).
   const int n = ct * 32 + l32;
   FlightRaw raw = flight_load_params<EPI>(ep, A_OFF, n < N ? n : N - 1);
   __builtin_amdgcn_sched_barrier(0);
-  FLIGHT_TS(1);
-
-  // ---- A has landed ------------------------------------------------------------
-  // At most 8 KG memory operations are outstanding: the youngest ones, which
-  // are the parameters and all but a few of the loads of Bp (however many loads
-  // the parameters turned into, the copies of A are older than all of them).
-  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(8 * KG) : "memory");
-  FLIGHT_TS(2);
-  if (A_MODE == 1 || need_rs) {
-    static_for<kFlightMaxTiles>([&](auto tc) {
-      constexpr int t = decltype(tc)::value;
-      if (t < nr) {
-        static_for<8>([&](auto hc) {
-          const int q = wave + decltype(hc)::value * waves;
-          if (q < 8) {
-            // all reads of the piece first: one LDS latency, not KG
-            v4i v[KG];
-#pragma unroll
-            for (int cg = 0; cg < KG; ++cg)
-              v[cg] = *(const v4i *)(sA + ((t * KG + cg) * 8 + q) * 1024 + lane * 16);
-            int32_t sum = 0;
-#pragma unroll
-            for (int cg = 0; cg < KG; ++cg) {
-              if (A_MODE == 1) {
-                v[cg] ^= (v4i){(int)0x80808080, (int)0x80808080, (int)0x80808080,
-                    (int)0x80808080};
-                *(v4i *)(sA + ((t * KG + cg) * 8 + q) * 1024 + lane * 16) = v[cg];
-              }
-              sum += frag_rowsum(v[cg]);
-            }
-            if (need_rs) {
-              // the 16 lanes of a row hold all of its chunks: no other wave
-              // and no other piece adds to this row's sum
-              sum = row16_sum(sum);
-              if ((lane & 15) == 0)
-                s_rs[t * 32 + 4 * q + rl] = sum;
-            }
-          }
-        });
-      }
-    });
-  }
   FLIGHT_TS(3);
   lds_sync(); // every wave's rows (and row sums) are in LDS
   __builtin_amdgcn_sched_barrier(0);
   FLIGHT_TS(4);
+  FLIGHT_TS_CYC(8);
 
   unsigned aaddr[8];
   {
@@ -524,48 +590,31 @@ void k_gemm_i8_flight(
   const bool q8_lines = EPI == kEpiQ8 && (N & 15) == 0 &&
                         ((((uintptr_t)ep.out) & 15) == 0);
   const v16i acc_zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-  auto finish = [&](const v16i &a, const FlightEpi &e, int t)
+  auto finish = [&](const v16i &acc, const FlightEpi &e, int t)
                     __attribute__((always_inline)) {
-    uint8_t *const st = stage + (t & 1) * 1024 * waves;
-    if (need_rs) // (the same for every wave)
-      flight_store_tile<EPI, true>(a, e, ep, s_rs + 32 * t, row0 + 32 * t, 32,
-          rn * waves * 32, wave, waves, lane, M, N, 0, st, q8_lines);
-    else
-      flight_store_tile<EPI, false>(a, e, ep, s_rs, row0 + 32 * t, 32,
-          rn * waves * 32, wave, waves, lane, M, N, 0, st, q8_lines);
+    flight_store_tile<EPI>(acc, e, ep, s_rs + 32 * t, row0 + 32 * t, 32,
+        rn * waves * 32, wave, waves, lane, M, N, 0,
+        stage + (t & 1) * 1024 * waves, q8_lines);
   };
-  if (nr == 1) {
-    v16i acc[2] = {acc_zero, acc_zero};
-    flight_kloop<KG, 1>(aaddr, b, acc);
+  auto epi_params = [&]() __attribute__((always_inline)) {
+    flight_params_not_before(raw);
+    return flight_epi<EPI>(ep, raw, A_OFF, K, raw.as,
+        ep.a_zp_len > 0 ? (A_OFF ? raw.az : (int32_t)(int8_t)raw.az) : 0);
+  };
+  v16i acc[2] = {acc_zero, acc_zero};
+  // (the weights are still arriving)
+  flight_kloop<KG, NR>(aaddr, b, acc);
+  if (NR == 1) {
 #pragma unroll
     for (int r = 0; r < 16; ++r)
       acc[0][r] += acc[1][r];
-    FLIGHT_TS(5);
-    flight_params_not_before(raw);
-    const FlightEpi e = flight_epi<EPI>(ep, raw, A_OFF, K, raw.as,
-        ep.a_zp_len > 0 ? (A_OFF ? raw.az : (int32_t)(int8_t)raw.az) : 0);
-    finish(acc[0], e, 0);
-  } else {
-    v16i acc[2] = {acc_zero, acc_zero};
-    // the first two row tiles: the weights are still arriving
-    flight_kloop<KG, 2>(aaddr, b, acc);
-    FLIGHT_TS(5);
-    flight_params_not_before(raw);
-    const FlightEpi e = flight_epi<EPI>(ep, raw, A_OFF, K, raw.as,
-        ep.a_zp_len > 0 ? (A_OFF ? raw.az : (int32_t)(int8_t)raw.az) : 0);
-    finish(acc[0], e, 0);
-    finish(acc[1], e, 1);
-    if (nr == 4) {
-#pragma unroll
-      for (int v = 0; v < 8; ++v)
-        aaddr[v] += 2 * KG * 8192;
-      acc[0] = acc_zero;
-      acc[1] = acc_zero;
-      flight_kloop<KG, 2>(aaddr, b, acc);
-      finish(acc[0], e, 2);
-      finish(acc[1], e, 3);
-    }
   }
+  FLIGHT_TS(5);
+  FLIGHT_TS_CYC(9);
+  const FlightEpi e = epi_params();
+  finish(acc[0], e, 0);
+  if (NR == 2)
+    finish(acc[1], e, 1);
 #ifdef FLIGHT_TIMING
   FLIGHT_TS(6);
   asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
@@ -715,71 +764,38 @@ __global__ __launch_bounds__(512, 1) void k_gemm_i8_flight_dq(
   // written by one atomic store and is read by one atomic load, past the
   // caches that other XCDs do not see.  A polling wave has no weights on their
   // way, so its answer does not queue behind them.
-  v4i b[KH];
-  bool got = true;
-  if (multiplies) { // (the same for the whole wave)
-    const int ctc = ct < bp_tiles ? ct : bp_tiles - 1;
-    const int8_t *const bp = Bp + (int64_t)ctc * KH * 1024 + lane * 16;
+  // The two kinds of waves run the rest of the kernel in separate branches
+  // (with the same barriers): the compiler counts the loads a wave has in
+  // flight per branch, and in common code it would make the multiplying
+  // waves wait for their weights wherever the others have nothing to wait for.
+  float scale = 0.0f, zpf = 0.0f;
+  // Once the poll is over: scale and zero point, the block's rows as 8-bit
+  // values minus 128 into LDS.  float4 c4 = p + TPR j of row r: bytes 4 c4 .. of
+  // the row, K group c4 / 64, chunk (c4 % 64) / 4 at position chunk ^ (r % 16).
+  // False if the exchange gave up.
+  auto rows_to_lds = [&]() __attribute__((always_inline)) {
+    FLIGHT_TS(2);
+    lds_sync();
+    if (!s_ok) {
+      // (the loads of the weights still in flight are waited for at the end of
+      // the program like any others)
+      if (tid == 0)
+        __hip_atomic_store(
+            dq.failed, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      return false;
+    }
+    float xlo = s_lo[0], xhi = s_hi[0];
 #pragma unroll
-    for (int s = 0; s < KH; ++s) {
-      b[s] = *(const v4i *)(bp + s * 1024);
-      __builtin_amdgcn_sched_barrier(0); // in this order
+    for (int w2 = 1; w2 < 4; ++w2) { // what the four polling waves found
+      xlo = __builtin_fminf(xlo, s_lo[w2]);
+      xhi = __builtin_fmaxf(xhi, s_hi[w2]);
     }
-  } else if (wave >= 4) {
-    const int slot = tid - 256;
-    const bool polls = slot < nslots;
-    const unsigned long long *const slot_p = &dq.slots[2 * (polls ? slot : 0)];
-    unsigned long long w0 = 0, w1 = 0;
-    got = !polls;
-    for (unsigned spin = 0; !got && spin < dq.spin_limit; ++spin) {
-      if (spin)
-        __builtin_amdgcn_s_sleep(1);
-      w0 = __hip_atomic_load(slot_p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      w1 = __hip_atomic_load(slot_p + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      got = (unsigned)(w0 >> 32) == dq.epoch && (unsigned)(w1 >> 32) == dq.epoch;
-    }
-    lo = polls ? __uint_as_float((unsigned)w0) : __builtin_inff();
-    hi = polls ? __uint_as_float((unsigned)w1) : -__builtin_inff();
-    lo = wave_fold<false>(lo);
-    hi = wave_fold<true>(hi);
-    const bool all_ok = __builtin_amdgcn_ballot_w64(!got) == 0;
-    if (lane == 0) {
-      s_lo[wave - 4] = lo;
-      s_hi[wave - 4] = hi;
-      if (!all_ok)
-        s_ok = 0;
-    }
-  }
-  __builtin_amdgcn_sched_barrier(0);
-  FLIGHT_TS(2);
-  lds_sync();
-  if (!s_ok) {
-    // (the loads of the weights still in flight are waited for at the end of
-    // the program like any others)
-    if (tid == 0)
-      __hip_atomic_store(
-          dq.failed, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    return;
-  }
-  lo = s_lo[0];
-  hi = s_hi[0];
-#pragma unroll
-  for (int w2 = 1; w2 < 4; ++w2) { // what the four polling waves found
-    lo = __builtin_fminf(lo, s_lo[w2]);
-    hi = __builtin_fmaxf(hi, s_hi[w2]);
-  }
-  FLIGHT_TS(3);
-  float scale, zpf;
-  dynamic_params(lo, hi, scale, zpf);
-
-  // ---- the block's rows as 8-bit values minus 128, into LDS --------------------
-  // float4 c4 = p + TPR j of row r: bytes 4 c4 .. of the row, K group c4 / 64,
-  // chunk (c4 % 64) / 4 at position chunk ^ (r % 16).
-  {
+    FLIGHT_TS(3);
+    dynamic_params(xlo, xhi, scale, zpf);
     const float recip = 1.0f / scale;
     uint8_t *const rowp = sA + r * 256 + (p & 3) * 4;
     int32_t sum = 0;
-    auto quantize = [&](auto fast_c) {
+    auto quantize = [&](auto fast_c) __attribute__((always_inline)) {
       constexpr int FAST = decltype(fast_c)::value ? 1 : 0;
 #pragma unroll
       for (int i = 0; i < NJ; ++i) {
@@ -804,16 +820,56 @@ __global__ __launch_bounds__(512, 1) void k_gemm_i8_flight_dq(
       if ((p & 15) == 0)
         atomicAdd(&s_rs[r], sum);
     }
+    lds_sync();
+    FLIGHT_TS(4);
+    return true;
+  };
+  if (!multiplies) { // (the same for the whole wave)
+    if (wave >= 4) {
+      const int slot = tid - 256;
+      const bool polls = slot < nslots;
+      const unsigned long long *const slot_p = &dq.slots[2 * (polls ? slot : 0)];
+      unsigned long long w0 = 0, w1 = 0;
+      bool got = !polls;
+      for (unsigned spin = 0; !got && spin < dq.spin_limit; ++spin) {
+        if (spin)
+          __builtin_amdgcn_s_sleep(1);
+        w0 = __hip_atomic_load(slot_p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        w1 = __hip_atomic_load(slot_p + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        got = (unsigned)(w0 >> 32) == dq.epoch && (unsigned)(w1 >> 32) == dq.epoch;
+      }
+      lo = polls ? __uint_as_float((unsigned)w0) : __builtin_inff();
+      hi = polls ? __uint_as_float((unsigned)w1) : -__builtin_inff();
+      lo = wave_fold<false>(lo);
+      hi = wave_fold<true>(hi);
+      const bool all_ok = __builtin_amdgcn_ballot_w64(!got) == 0;
+      if (lane == 0) {
+        s_lo[wave - 4] = lo;
+        s_hi[wave - 4] = hi;
+        if (!all_ok)
+          s_ok = 0;
+      }
+    }
+    (void)rows_to_lds();
+    return;
   }
-  lds_sync();
-  __builtin_amdgcn_sched_barrier(0);
-  FLIGHT_TS(4);
-  if (!multiplies) {
+  v4i b[KH];
+  {
+    const int ctc = ct < bp_tiles ? ct : bp_tiles - 1;
+    const int8_t *const bp = Bp + (int64_t)ctc * KH * 1024 + lane * 16;
+#pragma unroll
+    for (int s = 0; s < KH; ++s) {
+      b[s] = *(const v4i *)(bp + s * 1024);
+      __builtin_amdgcn_sched_barrier(0); // in this order
+    }
+  }
+  if (!rows_to_lds()) {
 #ifdef FLIGHT_TIMING
     asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
 #endif
     return;
   }
+  __builtin_amdgcn_sched_barrier(0);
 
   // ---- K loop ---------------------------------------------------------------------
   unsigned aaddr[8];
@@ -824,9 +880,6 @@ __global__ __launch_bounds__(512, 1) void k_gemm_i8_flight_dq(
     for (int v = 0; v < 8; ++v)
       aaddr[v] = arow + ((unsigned)(32 * v) ^ xh);
   }
-  flight_params_not_before(raw);
-  const FlightEpi e =
-      flight_epi<kEpiF32>(ep, raw, true, K, scale, (int32_t)(uint32_t)zpf);
   v16i accs[2] = {{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0},
       {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}};
   flight_kloop<KG, 1>(aaddr, b, accs);
@@ -835,12 +888,11 @@ __global__ __launch_bounds__(512, 1) void k_gemm_i8_flight_dq(
   for (int r2 = 0; r2 < 16; ++r2)
     acc[r2] = accs[0][r2] + accs[1][r2];
   FLIGHT_TS(5);
-  if (need_rs) // (the same for every wave)
-    flight_store_tile<kEpiF32, true>(acc, e, ep, s_rs, row0, R, rn * mwaves * 32,
-        wave, mwaves, lane, M, N, dq.act, nullptr, false);
-  else
-    flight_store_tile<kEpiF32, false>(acc, e, ep, s_rs, row0, R, rn * mwaves * 32,
-        wave, mwaves, lane, M, N, dq.act, nullptr, false);
+  flight_params_not_before(raw);
+  const FlightEpi e =
+      flight_epi<kEpiF32>(ep, raw, true, K, scale, (int32_t)(uint32_t)zpf);
+  flight_store_tile<kEpiF32>(acc, e, ep, s_rs, row0, R, rn * mwaves * 32, wave,
+      mwaves, lane, M, N, dq.act, nullptr, false);
 #ifdef FLIGHT_TIMING
   FLIGHT_TS(6);
   asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
@@ -881,14 +933,14 @@ bool flight_k_ok(int64_t K) {
 
 // Among the block shapes that cover the problem with at most one block per
 // CU, the one that brings the fewest bytes into a CU; with equal bytes the one
-// with more waves per block.  staged: the waves go over the rows in LDS once
-// more (uint8 rows, or B carries an offset); four waves share that work.
-FlightShape flight_shape(int64_t M, int64_t N, bool staged) {
+// with more waves per block.  (2 nr <= waves: a wave stages at most four
+// groups of four rows.)
+FlightShape flight_shape(int64_t M, int64_t N) {
   FlightShape best = {0, 0, 0};
   int64_t best_bytes = 0;
   const int cus = flight_cus();
   for (int nr = 1; nr <= kFlightMaxTiles; nr *= 2)
-    for (int w = staged ? 4 : 1; w <= 4; w *= 2) {
+    for (int w = 2 * nr; w <= 4; w *= 2) {
       const int64_t blocks =
           ((M + 32 * nr - 1) / (32 * nr)) * ((N + 32 * w - 1) / (32 * w));
       if (blocks > cus)
@@ -903,53 +955,59 @@ FlightShape flight_shape(int64_t M, int64_t N, bool staged) {
   return best;
 }
 
-bool flight_staged(const GemmArgs &g, int a_mode) {
-  return a_mode == 1 || g.b_unsigned || (g.b_zp != nullptr && g.b_zp_len > 0);
-}
-
-template <int KG, int A_MODE, int EPI>
+template <int KG, bool FLIP, int EPI, int NR, int WAVES>
 hipError_t flight_launch(hipStream_t st, const GemmArgs &g, const EpiParams &ep,
-    const FlightShape &sh) {
-  const int regions_n = (int)((g.N + 32 * sh.waves - 1) / (32 * sh.waves));
-  const int regions_m = (int)((g.M + 32 * sh.nr - 1) / (32 * sh.nr));
+    int a_mode) {
+  const int regions_n = (int)((g.N + 32 * WAVES - 1) / (32 * WAVES));
+  const int regions_m = (int)((g.M + 32 * NR - 1) / (32 * NR));
   const int bp_tiles = (int)(round_up(g.N, kGemmBN) / 32);
-  auto kern = k_gemm_i8_flight<KG, A_MODE, EPI>;
+  auto kern = k_gemm_i8_flight<KG, FLIP, EPI, NR, WAVES>;
   hipError_t e = flight_allow_lds(kern);
   if (e != hipSuccess)
     return e;
-  const size_t lds = (size_t)sh.nr * KG * 8192 + 4 * 32 * kFlightMaxTiles +
-                     2 * 1024 * (size_t)sh.waves;
-  kern<<<dim3((unsigned)(regions_m * regions_n)), dim3(64 * sh.waves), lds, st>>>(
-      (const uint8_t *)g.A, g.Bp, (int)g.M, (int)g.N, ep, sh.nr, regions_n,
-      bp_tiles);
+  const size_t lds = (size_t)NR * KG * 8192 + 4 * 32 * kFlightMaxTiles +
+                     2 * 1024 * (size_t)WAVES;
+  kern<<<dim3((unsigned)(regions_m * regions_n)), dim3(64 * WAVES), lds, st>>>(
+      (const uint8_t *)g.A, g.Bp, (int)g.M, (int)g.N, ep, a_mode != 0 ? 1 : 0,
+      regions_n, bp_tiles);
   return hipGetLastError();
 }
 
-template <int A_MODE, int EPI>
+template <int KG, bool FLIP, int EPI>
+hipError_t flight_launch_shape(hipStream_t st, const GemmArgs &g,
+    const EpiParams &ep, int a_mode, const FlightShape &sh) {
+  if (sh.nr == 2)
+    return flight_launch<KG, FLIP, EPI, 2, 4>(st, g, ep, a_mode);
+  if (sh.waves == 2)
+    return flight_launch<KG, FLIP, EPI, 1, 2>(st, g, ep, a_mode);
+  return flight_launch<KG, FLIP, EPI, 1, 4>(st, g, ep, a_mode);
+}
+
+template <bool FLIP, int EPI>
 hipError_t flight_launch_kg(hipStream_t st, const GemmArgs &g,
-    const EpiParams &ep, const FlightShape &sh) {
+    const EpiParams &ep, int a_mode, const FlightShape &sh) {
   switch (g.K / 256) {
   case 2:
-    return flight_launch<2, A_MODE, EPI>(st, g, ep, sh);
+    return flight_launch_shape<2, FLIP, EPI>(st, g, ep, a_mode, sh);
   case 3:
-    return flight_launch<3, A_MODE, EPI>(st, g, ep, sh);
+    return flight_launch_shape<3, FLIP, EPI>(st, g, ep, a_mode, sh);
   case 4:
-    return flight_launch<4, A_MODE, EPI>(st, g, ep, sh);
+    return flight_launch_shape<4, FLIP, EPI>(st, g, ep, a_mode, sh);
   default:
     return hipErrorInvalidValue;
   }
 }
 
-template <int A_MODE>
+template <bool FLIP>
 hipError_t flight_launch_epi(hipStream_t st, const GemmArgs &g,
-    const EpiParams &ep, const FlightShape &sh) {
+    const EpiParams &ep, int a_mode, const FlightShape &sh) {
   switch (g.epi) {
   case kEpiI32:
-    return flight_launch_kg<A_MODE, kEpiI32>(st, g, ep, sh);
+    return flight_launch_kg<FLIP, kEpiI32>(st, g, ep, a_mode, sh);
   case kEpiF32:
-    return flight_launch_kg<A_MODE, kEpiF32>(st, g, ep, sh);
+    return flight_launch_kg<FLIP, kEpiF32>(st, g, ep, a_mode, sh);
   default:
-    return flight_launch_kg<A_MODE, kEpiQ8>(st, g, ep, sh);
+    return flight_launch_kg<FLIP, kEpiQ8>(st, g, ep, a_mode, sh);
   }
 }
 
@@ -1016,23 +1074,16 @@ bool flight_ok(const GemmArgs &g, int a_mode) {
   if (!flight_k_ok(g.K) || g.M < 1 || g.X || ((((uintptr_t)g.A) & 15) != 0) ||
       g.M * g.N >= ((int64_t)1 << 29) || (g.a_zp != nullptr && g.a_zp_len > 1))
     return false;
-  return flight_shape(g.M, g.N, flight_staged(g, a_mode)).nr > 0;
+  return flight_shape(g.M, g.N).nr > 0;
 }
 
 hipError_t launch_gemm_flight(hipStream_t st, const GemmArgs &g,
     const EpiParams &ep, int a_mode) {
   if (!flight_ok(g, a_mode))
     return hipErrorInvalidValue;
-  const bool staged = flight_staged(g, a_mode);
-  const FlightShape sh = flight_shape(g.M, g.N, staged);
-  switch (a_mode) {
-  case 0:
-    return flight_launch_epi<0>(st, g, ep, sh);
-  case 1:
-    return flight_launch_epi<1>(st, g, ep, sh);
-  default:
-    return flight_launch_epi<2>(st, g, ep, sh);
-  }
+  const FlightShape sh = flight_shape(g.M, g.N);
+  return a_mode == 1 ? flight_launch_epi<true>(st, g, ep, a_mode, sh)
+                     : flight_launch_epi<false>(st, g, ep, a_mode, sh);
 }
 
 // The fused layer in one launch: every block of the grid resident at once

@@ -694,6 +694,12 @@ __global__ __launch_bounds__(256, MINB) void k_gemm_i8_bs(
   constexpr int YOUNGER = (NST - 2 - AHEAD) * PER_STEP;
   static_assert(YOUNGER < 64 && NST - 2 - AHEAD >= 0 && D >= NST - 2,
       "wait count");
+  // Step 0: the prologue asks for the rows of NST - 1 steps first and for the
+  // weights after them, so the weights of step 0 are followed by those of the
+  // other D - 1 steps only, and the first wait must not let more than that
+  // many operations stand.  (An instantiation with six stages and D = 4 did:
+  // it multiplied with registers whose loads were still in flight.)
+  static_assert(2 * TN * (D - 1) >= YOUNGER, "step 0 would not wait for its weights");
   const v4i flip = {(int)0x80808080, (int)0x80808080, (int)0x80808080,
       (int)0x80808080};
   using O = std::integral_constant<int, 0>;
@@ -1323,9 +1329,12 @@ int choose_tile(int64_t M, int64_t N, int64_t K) {
   const int64_t t128 = tm * ((N + 127) / 128);
   const int64_t t256 = tm * ((N + 255) / 256);
   const int64_t r128 = (t128 + 255) / 256, r256 = (t256 + 255) / 256;
-  if (t256 >= 256 && r256 * 17 < r128 * 10)
+  // (k_gemm_i8_bs only with whole trips of its four-step loop body, K % 256
+  // == 0: the step counts it runs with in production -- K = 2048, 4096, 11008
+  // -- and is validated at.  Other K take the 128 x 128 tiles, a few percent
+  // slower on such shapes.)
+  if (t256 >= 256 && r256 * 17 < r128 * 10 && K % (4 * kGemmBK) == 0)
     return kB128x256;
-  (void)K;
   if (N > 64 && t128 <= 128)
     return kD128x64;
   return kD128x128;
@@ -1360,6 +1369,7 @@ hipError_t gemm_launch_cfg(
       if (EPI != kEpiF32 || !g.dql)
         return hipErrorInvalidValue;
       t_last_kernel = "k_gemm_i8_flight (rows quantized in the kernel)";
+      t_gelu_applied = g.gelu; // this kernel applies it to its results
       return launch_gemm_flight_dq(st, g, ep, *g.dql);
     }
     if constexpr (A_MODE == 2) {

@@ -1885,8 +1885,9 @@ void om_mi355x_DynQuantMatMulDequant(OMTensor *y_t, const OMTensor *x_t,
         if (e == hipSuccess && call.c.dql_gave_up()) {
           fprintf(stderr,
               "om_mi355x: DynQuantMatMulDequant: the blocks of the one-launch "
-              "kernel timed out waiting for one another; redone with separate "
-              "launches, which this thread uses from now on\n");
+              "kernel timed out waiting for one another; redone with two launches "
+              "for the quantization and one for the product, which this thread "
+              "uses from now on\n");
           e = run(false);
         }
       }

@@ -157,3 +157,23 @@ def test_weights_in_registers_kernel_stays_inside_a_ragged_output(rt, oracle, fo
             assert (whole[guard + M * N:] == 0x5A5A5A5A).all(), (M, N, epi, "after")
             assert np.array_equal(whole[guard:guard + M * N].reshape(M, N), want), (M, N, epi)
             buf.free()
+
+
+def test_dispatch_keeps_bs_to_whole_trips(rt, oracle):
+    """k_gemm_i8_bs runs four K steps per trip of its loop; the dispatch gives it
+    only products whose K is a multiple of 256 (the step counts it is validated
+    at).  4096 x 1088 x 4096 -- 17 steps, the launch that once ended a benchmark
+    loop with an illegal memory access (tests/test_bs_address_model.py) -- takes
+    the 128 x 128 tiles of k_gemm_i8_dma instead and matches the oracle; the
+    same product over K = 1024 still takes k_gemm_i8_bs."""
+    rng = np.random.default_rng(1088)
+    A = rng.integers(0, 256, (4096, 1088), dtype=np.uint8)
+    B = rng.integers(-128, 128, (1088, 4096), dtype=np.int8)
+    az = np.uint8(129)
+    print("dispatch test: 4096x1088x4096", flush=True)
+    got = rt.MatMulInteger(A, B, az, None)
+    assert rt.last_gemm_kernel() == "k_gemm_i8_dma (128x128 tiles)", rt.last_gemm_kernel()
+    assert np.array_equal(got, oracle.matmul_integer(A, B, az, None, passes=True))
+    got = rt.MatMulInteger(A[:, :1024], B[:1024], az, None)
+    assert rt.last_gemm_kernel() == "k_gemm_i8_bs (128x256 tiles)", rt.last_gemm_kernel()
+    assert np.array_equal(got, oracle.matmul_integer(np.ascontiguousarray(A[:, :1024]), np.ascontiguousarray(B[:1024]), az, None, passes=True))

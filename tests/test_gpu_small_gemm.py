@@ -33,7 +33,7 @@ def mm(oracle, A, B, a_zp, b_zp):
 
 
 SHAPES = [(65, 512, 100), (128, 768, 768), (200, 1024, 1000), (512, 1024, 4096), (1000, 768, 416),
-          (4096, 768, 768), (97, 768, 33), (3000, 512, 1024)]
+          (2048, 768, 256), (97, 768, 33), (1000, 512, 1024), (256, 1024, 2048)]
 
 
 @pytest.mark.parametrize("M,K,N", SHAPES)
