@@ -73,30 +73,25 @@ namespace gemm {
 namespace {
 
 #ifdef FLIGHT_TIMING
-// Development build: readings of the 100 MHz clock by wave 0 of every block at
-// fixed points, written out when the kernel ends (om_dev_flight_ts reads them).
-__device__ unsigned long long flight_ts[1024 * 10];
+// Measurement build (measure/flight_timeline.py): wave 0 of every block reads
+// the 100 MHz clock at fixed points, slots 0..7, and the cycle counter on entry
+// and at the end, slots 10 and 11; written out when the kernel ends
+// (om_dev_flight_ts reads them).
+constexpr int kFlightTsSlots = 12;
+__device__ unsigned long long flight_ts[1024 * kFlightTsSlots];
 #define FLIGHT_TS(i)                                                           \
   if (wave == 0)                                                               \
   ts[i] = __builtin_amdgcn_s_memrealtime()
 #define FLIGHT_TS_DECL                                                         \
-  unsigned long long ts[10] = {};                                              \
-  ts[8] = __builtin_readcyclecounter()
-#ifdef FLIGHT_EXP_KCLK
-#define FLIGHT_TS_CYC(i) ts[i] = __builtin_readcyclecounter()
-#define FLIGHT_TS_END
-#else
-#define FLIGHT_TS_CYC(i)
-#define FLIGHT_TS_END ts[9] = __builtin_readcyclecounter()
-#endif
+  unsigned long long ts[kFlightTsSlots] = {};                                  \
+  ts[10] = __builtin_readcyclecounter()
 #define FLIGHT_TS_WRITE                                                        \
-  FLIGHT_TS_END;                                                               \
+  ts[11] = __builtin_readcyclecounter();                                       \
   if (wave == 0 && lane == 0 && blockIdx.x < 1024)                             \
-    for (int i_ = 0; i_ < 10; ++i_)                                            \
-  flight_ts[blockIdx.x * 10 + i_] = ts[i_]
+    for (int i_ = 0; i_ < kFlightTsSlots; ++i_)                                \
+  flight_ts[blockIdx.x * kFlightTsSlots + i_] = ts[i_]
 #else
 #define FLIGHT_TS(i)
-#define FLIGHT_TS_CYC(i)
 #define FLIGHT_TS_DECL
 #define FLIGHT_TS_WRITE
 #endif
@@ -577,7 +572,6 @@ __attribute__((amdgpu_waves_per_eu(1, 1))) void k_gemm_i8_flight(
   lds_sync(); // every wave's rows (and row sums) are in LDS
   __builtin_amdgcn_sched_barrier(0);
   FLIGHT_TS(4);
-  FLIGHT_TS_CYC(8);
 
   unsigned aaddr[8];
   {
@@ -610,7 +604,6 @@ __attribute__((amdgpu_waves_per_eu(1, 1))) void k_gemm_i8_flight(
       acc[0][r] += acc[1][r];
   }
   FLIGHT_TS(5);
-  FLIGHT_TS_CYC(9);
   const FlightEpi e = epi_params();
   finish(acc[0], e, 0);
   if (NR == 2)
