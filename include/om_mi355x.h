@@ -116,9 +116,14 @@ void om_mi355x_DynamicQuantizeLinear(
 
 /* DynamicQuantizeLinear for callers that cannot allocate.  This entry point
  * has no counterpart in the reference; it exists for callers that must not
- * reach hipMalloc / hipFree while they run: code under HIP graph capture,
- * tight serving loops, harnesses that forbid allocation.  Same operands and
- * results as om_mi355x_DynamicQuantizeLinear, with these conditions:
+ * reach hipMalloc / hipFree while they run: tight serving loops, harnesses
+ * that forbid allocation, a thread that has a HIP graph capture open on a
+ * stream of its own.  (The call's kernels run on the runtime's stream of the
+ * calling thread, which is private: they are not recorded into the caller's
+ * graph.  Should that stream itself be under capture, the entry point records
+ * its two-launch form, which replays correctly; the one-launch kernel carries
+ * a launch number and would not.)  Same operands and results as
+ * om_mi355x_DynamicQuantizeLinear, with these conditions:
  *  - every tensor's data pointer is GPU memory (om_mi355x_malloc, or a host
  *    buffer declared with om_mi355x_KeepOnDevice); a host tensor is refused
  *    (EINVAL), because staging it could allocate;
@@ -235,14 +240,15 @@ void om_mi355x_free(void *dev_ptr);
 int om_mi355x_memcpy_h2d(void *dst_dev, const void *src_host, size_t bytes);
 int om_mi355x_memcpy_d2h(void *dst_host, const void *src_dev, size_t bytes);
 /* Waits for all work the calling thread has issued; 0, or -1 with the error
- * kept for om_mi355x_last_error().  Takes no tensors, so generated code can
- * reach it as a krnl.call ("krnl.call"(%y) {funcName =
- * "om_mi355x_synchronize", numOfOutput = 1 : si64}: one buffer named as an
- * output keeps the call from being removed as dead, and an argument that a
- * function without parameters never reads is harmless in the C calling
- * conventions of the hosts this runs on); the value returned is then ignored
- * and a failure shows at the next entry point. */
+ * kept for om_mi355x_last_error(). */
 int om_mi355x_synchronize(void);
+/* The same for generated code, which reaches the runtime through krnl.call
+ * and passes every operand as an OMTensor*: "krnl.call"(%y) {funcName =
+ * "om_mi355x_Synchronize", numOfOutput = 1 : si64}.  `anchor` is not read
+ * (naming one buffer as an output keeps the call from being removed as
+ * dead); a failure is kept for om_mi355x_last_error() and shows at the next
+ * entry point. */
+void om_mi355x_Synchronize(OMTensor *anchor);
 
 /* ---- measurement --------------------------------------------------------- */
 /* Brackets subsequent entry-point calls of this thread with HIP events on the

@@ -683,7 +683,8 @@ template <bool SIGNED, bool HAS_ZP, bool RECIP = false>
 __global__ __launch_bounds__(kThreads) void k_quant_general(
     const float *__restrict__ x, uint8_t *__restrict__ y, int64_t channels,
     int64_t inner, const float *__restrict__ scale,
-    const void *__restrict__ zp, int64_t oc_total) {
+    const void *__restrict__ zp, int64_t oc_total, uint32_t flip = 0) {
+  // flip: 0, or 0x80 to store the values minus 128 (see k_quant_flat)
   for (int64_t oc = blockIdx.y; oc < oc_total; oc += gridDim.y) {
     const int64_t c = oc % channels;
     const float s = scale[c];
@@ -693,7 +694,8 @@ __global__ __launch_bounds__(kThreads) void k_quant_general(
     uint8_t *__restrict__ yr = y + oc * inner;
     for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < inner;
          i += (int64_t)gridDim.x * kThreads)
-      yr[i] = (uint8_t)quant_one<SIGNED, HAS_ZP, RECIP ? 2 : 0>(xr[i], s, zpf, r);
+      yr[i] = (uint8_t)(quant_one<SIGNED, HAS_ZP, RECIP ? 2 : 0>(xr[i], s, zpf, r) ^
+                        (flip & 0xFFu));
   }
 }
 
@@ -1973,7 +1975,9 @@ hipError_t quantize_dispatch(hipStream_t st, const float *x, int64_t outer,
             <<<grid, kThreads, 0, st>>>(x, yo, n, scale, zp, flip);
       return hipGetLastError();
     }
-    if (flip != 0)
+    // (values stored minus 128 exist per tensor only: the rows of the fused
+    // layer; misaligned, they take the general kernel below)
+    if (flip != 0 && channels != 1)
       return hipErrorInvalidValue;
     if (channels > 1 && inner == 1 && aligned && n < ((int64_t)1 << 32)) {
       const unsigned grid = (unsigned)(blocks > 0 ? blocks : 1);
@@ -2007,10 +2011,10 @@ hipError_t quantize_dispatch(hipStream_t st, const float *x, int64_t outer,
     dim3 grid((unsigned)gx, (unsigned)gy);
     if (has_zp)
       k_quant_general<SIGNED, true, true>
-          <<<grid, kThreads, 0, st>>>(x, yo, channels, inner, scale, zp, oc);
+          <<<grid, kThreads, 0, st>>>(x, yo, channels, inner, scale, zp, oc, flip);
     else
       k_quant_general<SIGNED, false, true>
-          <<<grid, kThreads, 0, st>>>(x, yo, channels, inner, scale, zp, oc);
+          <<<grid, kThreads, 0, st>>>(x, yo, channels, inner, scale, zp, oc, flip);
     return hipGetLastError();
   }
   if (channels == 1) {
@@ -2040,11 +2044,21 @@ hipError_t quantize_dispatch(hipStream_t st, const float *x, int64_t outer,
             <<<grid, kThreads, 0, st>>>(x, yo, n, scale, zp, flip);
       return hipGetLastError();
     }
-    if (flip != 0)
-      return hipErrorInvalidValue;
     // Misaligned buffers: treat as one long run.
     outer = 1;
     inner = n;
+    if (flip != 0) {
+      // (the rows of the fused layer, stored minus 128: the general kernel)
+      int64_t gx = (n + kThreads - 1) / kThreads;
+      gx = gx > 4096 ? 4096 : gx;
+      if (has_zp)
+        k_quant_general<SIGNED, true><<<dim3((unsigned)gx, 1), kThreads, 0, st>>>(
+            x, yo, 1, n, scale, zp, 1, flip);
+      else
+        k_quant_general<SIGNED, false><<<dim3((unsigned)gx, 1), kThreads, 0, st>>>(
+            x, yo, 1, n, scale, zp, 1, flip);
+      return hipGetLastError();
+    }
   }
   if (flip != 0)
     return hipErrorInvalidValue;

@@ -1701,7 +1701,18 @@ void om_mi355x_DynamicQuantizeLinearNoAlloc(OMTensor *y_t, OMTensor *scale_t,
   s.counter = (unsigned *)(s.partial_max + kNoAllocBlocks);
   s.grid_slots = (unsigned long long *)((char *)s.counter + 256);
   s.max_blocks = kNoAllocBlocks;
-  s.grid_blocks = g_scratch_no_grid[dev]
+  // The one-launch kernel tags its exchange slots with a launch number that
+  // is a kernel argument, and asks another stream whether it is idle: neither
+  // survives being recorded into a graph and replayed.  Should this thread's
+  // stream be under capture, the two-launch form is recorded instead (fill
+  // kernel, minimum / maximum with an arrival counter, quantize), which
+  // carries no such state.
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(c.stream, &capture) != hipSuccess) {
+    (void)hipGetLastError();
+    capture = hipStreamCaptureStatusNone;
+  }
+  s.grid_blocks = (g_scratch_no_grid[dev] || capture != hipStreamCaptureStatusNone)
                       ? 0
                       : std::min(c.dql.grid_blocks, kNoAllocBlocks);
   s.spin_limit = c.dql.spin_limit;
@@ -2096,6 +2107,11 @@ int om_mi355x_synchronize(void) {
   }
   const bool mine_ok = t_ctx.dql_barrier_ok();
   return (noalloc_barrier_ok() && mine_ok) ? 0 : -1;
+}
+
+void om_mi355x_Synchronize(OMTensor *anchor) {
+  (void)anchor;
+  (void)om_mi355x_synchronize();
 }
 
 int om_mi355x_timer_start(void) {

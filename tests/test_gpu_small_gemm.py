@@ -146,3 +146,28 @@ def test_config1_is_one_launch(rt, oracle):
     want = oracle.dequant_epilogue(oracle.matmul_integer(aq, c["B"], a_zp, c["b_zp"]), a_s, c["b_scale"])
     assert same_f32(rt.DynQuantMatMulDequant(c["A"], c["B"], c["b_zp"], c["b_scale"]), want)
     assert rt.last_gemm_kernel() == "k_gemm_i8_flight (rows quantized in the kernel)"
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+def test_fused_layer_takes_an_activation_that_is_not_16_byte_aligned(rt, oracle, mode):
+    """A GPU-resident activation that starts 4 bytes into its buffer (a view):
+    the one-launch kernels want 16-byte rows, so the layer runs as
+    DynamicQuantizeLinear + GEMM, whose quantize pass then stores the rows minus
+    128 with a kernel that takes any alignment -- also when the quotient is
+    computed as x * (1 / scale) (mode 1), where this used to be refused."""
+    M, K, N = 72, 768, 256
+    rng = np.random.default_rng(72 + mode)
+    x = rng.normal(0, 1, (M, K)).astype(np.float32)
+    W = _rand_q(rng, np.int8, (K, N))
+    ws = rng.uniform(1e-3, 1e-2, N).astype(np.float32)
+    buf = rt.DeviceArray.from_numpy(np.concatenate([np.zeros(1, np.float32), x.ravel()]))
+    dx = rt.DeviceArray.__new__(rt.DeviceArray)
+    dx.shape, dx.dtype, dx.ptr, dx.owner = (M, K), np.dtype(np.float32), buf.ptr + 4, buf
+    aq, a_s, a_zp = oracle.dynamic_quantize_linear_mode(x, mode)
+    want = oracle.dequant_epilogue(mm(oracle, aq, W, a_zp, None), a_s, ws)
+    rt.set_quant_mode(mode)
+    got = rt.DynQuantMatMulDequant(dx, W, None, ws)
+    got = got.numpy() if hasattr(got, "numpy") else got
+    assert "flight (rows quantized" not in rt.last_gemm_kernel()
+    assert same_f32(got, want)
+    buf.free()

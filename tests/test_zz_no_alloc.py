@@ -94,3 +94,35 @@ def test_refuses_a_thread_without_a_stream(rt):
     t.start()
     t.join()
     assert len(seen) == 1 and "no stream yet" in seen[0], seen
+
+
+def test_allocates_no_gpu_memory(rt):
+    """Free GPU memory as the driver reports it is the same before and after a
+    run of calls of every size class (the allocating entry point's pool would
+    grow by the temporaries of the largest one)."""
+    import ctypes
+    hip = ctypes.CDLL("libamdhip64.so")
+    free_b, total_b = ctypes.c_size_t(), ctypes.c_size_t()
+
+    def free_bytes():
+        assert hip.hipMemGetInfo(ctypes.byref(free_b), ctypes.byref(total_b)) == 0
+        return free_b.value
+
+    rt.synchronize()
+    rng = np.random.default_rng(3)
+    cases = []
+    for shape in ((4096, 3072), (4096, 768), (257, 1031), (7,)):
+        x = rng.normal(0.0, 1.0, shape).astype(np.float32)
+        cases.append((rt.DeviceArray.from_numpy(x),
+                      (rt.DeviceArray(shape, np.uint8), rt.DeviceArray((), np.float32), rt.DeviceArray((), np.uint8))))
+    rt.synchronize()
+    before = free_bytes()
+    for _ in range(3):
+        for dx, out in cases:
+            rt.DynamicQuantizeLinearNoAlloc(dx, out)
+    rt.synchronize()
+    assert free_bytes() == before
+    for dx, out in cases:
+        dx.free()
+        for o in out:
+            o.free()
