@@ -231,6 +231,37 @@ def qlinear_case(rt, wl, steps, warmup):
     return res
 
 
+def qlinear_ffn_up_case(rt, wl, steps, warmup):
+    """QLinearMatMul at the headline shape (config 4 FFN-up, 4096 x 768 x 3072):
+    uint8 activations with a zero point, symmetric int8 weights (b_zero_point
+    a constant 0, per-tensor scales), uint8 out -- the requantizing epilogue on
+    the kernel that holds the weights in registers."""
+    c = wl.config4("ffn_up")
+    K, N = c["W"].shape
+    M = 4096
+    A = wl.uniform_u8(4, 90, (M, K))
+    ops_ = {"A": A, "a_scale": np.float32(0.0173), "a_zp": np.array(131, np.uint8), "B": c["W"],
+            "b_scale": np.float32(0.004), "b_zp": np.array(0, np.int8), "y_scale": np.float32(0.9),
+            "y_zp": np.array(127, np.uint8)}
+    d = {k: rt.DeviceArray.from_numpy(np.asarray(v)) for k, v in ops_.items()}
+    dY = rt.DeviceArray((M, N), np.uint8)
+    rt.mark_constant(d["B"])
+    rt.mark_constant(d["b_zp"])
+    fn = rt.PreparedCall("om_mi355x_QLinearMatMul", dY, d["A"], d["a_scale"], d["a_zp"], d["B"],
+                         d["b_scale"], d["b_zp"], d["y_scale"], d["y_zp"], rt.WRAP)
+    res = measure(rt, fn, steps, warmup)
+    fn.check()
+    fn.close()
+    rt.unmark_constant(d["b_zp"])
+    ops = 2.0 * M * N * K
+    res.update({"name": "config4 ffn_up QLinearMatMul u8 x i8 -> u8", "M": M, "K": K, "N": N,
+                "kernel": rt.last_gemm_kernel(), "tops": ops / (res["kernel_ms"] * 1e-3) / 1e12,
+                "hbm_bytes_algorithmic": M * K + K * N + M * N})
+    for a in list(d.values()) + [dY]:
+        a.free()
+    return res
+
+
 def fused_case(rt, wl, name, M, K, N, w_i8, w_scale, steps, warmup, X=None, activation=0):
     """DynamicQuantizeLinear -> MatMulInteger -> Cast -> Mul as one call: fp32
     activations in, fp32 out (the chain the quantized models contain);
@@ -436,6 +467,8 @@ def only_mode(rt, wl, what, steps, warmup):
         return {"only": what, **r}
     if what == "config3":
         return {"only": what, **qlinear_case(rt, wl, steps, warmup)}
+    if what == "qlinear_ffn_up":
+        return {"only": what, **qlinear_ffn_up_case(rt, wl, steps, warmup)}
     if what in ("config1", "config1_two_calls"):
         r = config1_cases(rt, wl, steps, warmup, only="fused" if what == "config1" else "separate")
         return {"only": what, **r}
@@ -663,7 +696,7 @@ def main():
                     choices=["copy", "mfma_ceiling", "per_axis_layouts", "gemm_ffn_up", "gemm_qkv", "gemm_out", "gemm_ffn_down",
                              "gemm_prefill_up", "gemm_prefill_down", "fused_ffn_up", "fused_ffn_down",
                              "fused_ffn_up_relu", "fused_ffn_up_gelu",
-                             "decode", "decode4", "decode16", "config1", "config1_two_calls", "config3",
+                             "decode", "decode4", "decode16", "config1", "config1_two_calls", "config3", "qlinear_ffn_up",
                              "quantize_per_axis", "dequantize_per_axis",
                              "quantize_per_tensor", "dequantize_per_tensor", "dynamic_quantize",
                              "quantize_per_axis_ragged", "dequantize_per_axis_ragged",
@@ -729,6 +762,7 @@ def main():
             gemms.append(gemm_case(rt, wl, f"config5 prefill {name}", 2048, k, n, cc["W"], cc["w_scale"],
                                    min(max(MIN_LAUNCHES, args.steps // 10), 500), 2, "f32"))
         gemms.append(qlinear_case(rt, wl, esteps, ewarm))
+        gemms.append(qlinear_ffn_up_case(rt, wl, esteps, ewarm))
         extras["gemm"] = gemms
         extras["headline_rotated"] = rotated_case(rt, wl, M, K, N, c["W"], c["w_scale"], esteps, ewarm)
 

@@ -317,6 +317,10 @@ __global__ __launch_bounds__(WAVES * 64, 1) void k_gemm_i8_wreg(
                         : 0x80000000u;
   const uint32_t tile_pitch = 32u * (uint32_t)N * (uint32_t)ES;
 
+  const bool sat = EPI == kEpiQ8 && ep.narrow == kSaturate;
+  const int32_t sat_lo = !sat ? INT32_MIN : ep.y_unsigned ? 0 : -128;
+  const int32_t sat_hi = !sat ? INT32_MAX : ep.y_unsigned ? 255 : 127;
+
   v16i acc, accp; // the tile being computed, the finished one before it
   // One element of the finished tile: register r.
   auto emit = [&](auto rc) {
@@ -340,13 +344,11 @@ __global__ __launch_bounds__(WAVES * 64, 1) void k_gemm_i8_wreg(
       const float f = (float)(int32_t)y * sj;
       int32_t v =
           (int32_t)((uint32_t)(int32_t)__builtin_rintf(f) + (uint32_t)yz);
-      if (ep.narrow == kSaturate) {
-        const int32_t lo = ep.y_unsigned ? 0 : -128;
-        const int32_t hi = ep.y_unsigned ? 255 : 127;
-        v = v < lo ? lo : (v > hi ? hi : v);
-      }
+      // one instruction, no branch: bounds that do nothing when the result
+      // wraps (the byte store keeps the low byte by itself)
+      asm("v_med3_i32 %0, %1, %2, %3" : "=v"(v) : "v"(v), "s"(sat_lo), "v"(sat_hi));
       __builtin_amdgcn_raw_buffer_store_b8(
-          (unsigned char)(v & 0xFF), out_rsrc, (int)toff, soff, 0);
+          (unsigned char)v, out_rsrc, (int)toff, soff, 0);
     }
   };
 
@@ -472,14 +474,16 @@ hipError_t wreg_launch(hipStream_t st, const GemmArgs &g, const EpiParams &ep) {
 } // namespace
 
 bool wreg_ok(const GemmArgs &g) {
-  const int64_t es = 4;
+  const int64_t es = g.epi == kEpiQ8 ? 1 : 4;
   if (g.M * g.N * es > ((int64_t)1 << 31) ||
       32 * kWregNR * g.N * es >= ((int64_t)1 << 30))
     return false;
   const bool rowsum = g.b_unsigned || (g.b_zp != nullptr && g.b_zp_len > 0);
+  // (8-bit results: 32 bytes of a row per wave and store, whole 32-byte
+  // sectors when the rows are 32 bytes apart at least)
   return g.K == 32 * kWregKH && g.a_zp_len <= 1 && !g.X && !rowsum &&
          ((((uintptr_t)g.A) & 15) == 0) && (g.N * es) % 128 == 0 &&
-         (g.epi == kEpiF32 || g.epi == kEpiI32);
+         (g.epi == kEpiF32 || g.epi == kEpiI32 || g.epi == kEpiQ8);
 }
 
 // One block per CU and round: the kernel pays when its blocks fill at least
@@ -502,6 +506,10 @@ hipError_t launch_gemm_wreg(hipStream_t st, const GemmArgs &g,
 #else
   const bool f32 = g.epi == kEpiF32;
   const int act = !f32 ? 0 : g.relu ? 1 : g.gelu ? 2 : 0;
+  if (g.epi == kEpiQ8)
+    return a_mode == 0   ? wreg_launch<0, kEpiQ8>(st, g, ep)
+           : a_mode == 1 ? wreg_launch<1, kEpiQ8>(st, g, ep)
+                         : wreg_launch<2, kEpiQ8>(st, g, ep);
   switch (a_mode * 4 + (f32 ? act : 3)) {
   case 0:
     return wreg_launch<0, kEpiF32>(st, g, ep);

@@ -119,6 +119,9 @@ struct DevCopy {
   size_t bytes;
 };
 std::unordered_map<const void *, DevCopy> g_const_copies;
+// Zero points in GPU memory that were declared constant and have been read
+// back once: (bytes, whether every one of them is zero).
+std::unordered_map<const void *, std::pair<size_t, bool>> g_const_zero;
 // Packed right-hand sides of constant B, keyed by B's data pointer.
 struct PackedB {
   int8_t *bp;
@@ -1227,6 +1230,46 @@ bool packed_b(Call &call, const View &b, int64_t K, int64_t N,
 // A zero point has one entry, or one per row / column of a matrix (`per`), or
 // -- with batched operands, as [.., M, 1] / [.., 1, N] -- one per row / column
 // of every matrix of its tensor (`per * mats`).
+// Whether a zero point is known to be all zeros: then it stands for no zero
+// point at all (the corrections it enters are multiplied by zero), and for
+// the right-hand side of a product that spares the kernels the row sums of A
+// -- symmetric int8 weights, the common case of QLinearMatMul, whose
+// b_zero_point is a required operand.  Host memory is looked at; GPU memory
+// only if it was declared constant, once (a blocking copy), and remembered
+// until om_mi355x_UnmarkConstant.
+bool zero_point_is_zero(const View &v) {
+  if (v.numel == 0 || v.bytes == 0 || v.bytes > ((size_t)1 << 20))
+    return false;
+  const uint8_t *p = (const uint8_t *)v.data;
+  auto all_zero = [&](const uint8_t *h) {
+    for (size_t i = 0; i < v.bytes; ++i)
+      if (h[i])
+        return false;
+    return true;
+  };
+  void *backing = backed_lookup(v.data);
+  if (!backing && !is_device_ptr(v.data))
+    return all_zero(p);
+  {
+    std::lock_guard<std::mutex> lk(g_mem_mutex);
+    if (!g_constants.count(v.data))
+      return false;
+    auto it = g_const_zero.find(v.data);
+    if (it != g_const_zero.end() && it->second.first == v.bytes)
+      return it->second.second;
+  }
+  std::vector<uint8_t> h(v.bytes);
+  if (hipMemcpy(h.data(), backing ? backing : v.data, v.bytes,
+          hipMemcpyDeviceToHost) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  const bool zero = all_zero(h.data());
+  std::lock_guard<std::mutex> lk(g_mem_mutex);
+  g_const_zero[v.data] = std::make_pair(v.bytes, zero);
+  return zero;
+}
+
 bool zp_len_ok(const View *zp, int64_t per, int64_t mats, const char *op,
     const char *name, int64_t &len) {
   if (!zp) {
@@ -1391,6 +1434,10 @@ void run_matmul(const MatmulSpec &sp) {
   g.colsum = colsum;
   const uint8_t *d_azp = sp.a_zp ? (const uint8_t *)call.in(azp) : nullptr;
   const uint8_t *d_bzp = sp.b_zp ? (const uint8_t *)call.in(bzp) : nullptr;
+  if (d_bzp && !b_uns && zero_point_is_zero(bzp)) {
+    d_bzp = nullptr; // B carries no offset
+    bzl = 0;
+  }
   g.a_zp = d_azp;
   g.a_zp_len = azl;
   g.b_zp = d_bzp;
@@ -1928,6 +1975,7 @@ void om_mi355x_UnmarkConstant(const OMTensor *t) {
   {
     std::lock_guard<std::mutex> lk(g_mem_mutex);
     g_constants.erase(p);
+    g_const_zero.erase(p);
     auto c = g_const_copies.find(p);
     if (c != g_const_copies.end()) {
       drop[0] = c->second.dev;
@@ -2025,6 +2073,7 @@ void om_mi355x_ClearCache(void) {
   }
   g_packed.clear();
   g_constants.clear();
+  g_const_zero.clear();
   for (auto &kv : g_backed)
     (void)hipFree(kv.second.dev);
   g_backed.clear();
@@ -2054,6 +2103,7 @@ void om_mi355x_free(void *p) {
     std::lock_guard<std::mutex> lk(g_mem_mutex);
     g_user_allocs.erase((uintptr_t)p);
     g_constants.erase(p);
+    g_const_zero.erase(p);
     auto it = g_packed.find(p);
     if (it != g_packed.end()) {
       (void)hipFree(it->second.bp);

@@ -932,6 +932,54 @@ def test_weights_in_registers_kernel(rt, oracle, forced, monkeypatch):
     assert np.array_equal(rt.MatMulInteger(A2, B2, az, None), oracle.matmul_integer(A2, B2, az, None))
 
 
+@pytest.mark.parametrize("forced", [True, False])
+def test_weights_in_registers_kernel_requantizes(rt, oracle, forced, monkeypatch):
+    """QLinearMatMul on k_gemm_i8_wreg: K = 768, signed weights whose (required)
+    zero point is all zeros -- a host tensor, or GPU memory declared constant,
+    which the runtime reads once -- so that B carries no offset; uint8 and int8
+    activations and results, wrapping and saturating, shapes with ragged edges
+    (N a multiple of 128: whole lines of 8-bit results), per-column b_scale is
+    not part of the op.  A zero point that is not zero, or not known to be,
+    takes the other kernels and must give the same bits."""
+    if forced:
+        monkeypatch.setenv("OM_MI355X_GEMM_TILE", "4")
+        shapes = [(128, 384), (129, 512), (300, 896), (1000, 384)]
+    else:
+        shapes = [(4096, 3072), (4097, 2304)]
+    rng = np.random.default_rng(76 + forced)
+    K = 768
+    for M, N in shapes:
+        for adt in (np.uint8, np.int8):
+            A, B = _rand_q(rng, adt, (M, K)), _rand_q(rng, np.int8, (K, N))
+            az, yz = _rand_q(rng, adt, ()), _rand_q(rng, adt, ())
+            bz0 = np.zeros((), np.int8)
+            a_s, b_s, y_s = np.float32(0.0173), np.float32(0.004), np.float32(0.08)
+            for mode, omode in ((rt.WRAP, oracle_lib.WRAP), (rt.SATURATE, oracle_lib.SATURATE)):
+                want = oracle.qlinear_matmul(A, a_s, az, B, b_s, bz0, y_s, yz, omode)
+                got = rt.QLinearMatMul(A, a_s, az, B, b_s, bz0, y_s, yz, mode)
+                assert "wreg" in rt.last_gemm_kernel(), (M, N, rt.last_gemm_kernel())
+                assert np.array_equal(got, want), (M, N, adt, mode)
+                assert (want == np.iinfo(adt).max).any() and (want == np.iinfo(adt).min).any() or mode == rt.WRAP
+        # a per-column zero point of zeros is no zero point either
+        got = rt.QLinearMatMul(A, a_s, az, B, b_s, np.zeros(N, np.int8), y_s, yz, rt.SATURATE)
+        assert "wreg" in rt.last_gemm_kernel()
+        assert np.array_equal(got, want)
+        # GPU-resident zero point: only a constant one is looked at
+        dz = rt.DeviceArray.from_numpy(np.zeros((), np.int8))
+        got = rt.QLinearMatMul(A, a_s, az, B, b_s, dz, y_s, yz, rt.SATURATE)
+        assert "wreg" not in rt.last_gemm_kernel() and np.array_equal(got, want)
+        rt.mark_constant(dz)
+        got = rt.QLinearMatMul(A, a_s, az, B, b_s, dz, y_s, yz, rt.SATURATE)
+        assert "wreg" in rt.last_gemm_kernel() and np.array_equal(got, want)
+        rt.unmark_constant(dz)
+        dz.free()
+        # a zero point that is not zero
+        bz = np.array(-3, np.int8)
+        got = rt.QLinearMatMul(A, a_s, az, B, b_s, bz, y_s, yz, rt.SATURATE)
+        assert "wreg" not in rt.last_gemm_kernel()
+        assert np.array_equal(got, oracle.qlinear_matmul(A, a_s, az, B, b_s, bz, y_s, yz, oracle_lib.SATURATE))
+
+
 def test_matmul_random_shapes_around_dispatch_boundaries(rt, oracle):
     """Seeded sweep over shapes that sit on both sides of every dispatch
     condition (M 16/17, 32/33, 64/65, 128/129; K a multiple of 64, of 16, of neither;
