@@ -161,8 +161,11 @@ void om_mi355x_MatMulInteger(OMTensor *y, const OMTensor *a,
  * (src/Conversion/ONNXToKrnl/Math/QLinearMatMul.cpp:26-143).
  * narrow_mode 0 = wrap (what the reference computes: trunci, :134-138),
  *             1 = saturate (what the ONNX specification says).
- * Operand ranks and batch pairing as for om_mi355x_MatMulInteger; scales and
- * y_zp are scalars. */
+ * Operand ranks and batch pairing as for om_mi355x_MatMulInteger; a_scale,
+ * y_scale and y_zp are scalars; b_scale is a scalar or, beyond what the
+ * reference's lowering takes (:53-68 refuses it), one value per column of b
+ * ([N]): column j is then scaled by (a_scale * b_scale[j]) / y_scale, the
+ * reference's expression (:127) with that column's scale. */
 void om_mi355x_QLinearMatMul(OMTensor *y, const OMTensor *a,
     const OMTensor *a_scale, const OMTensor *a_zp, const OMTensor *b,
     const OMTensor *b_scale, const OMTensor *b_zp, const OMTensor *y_scale,

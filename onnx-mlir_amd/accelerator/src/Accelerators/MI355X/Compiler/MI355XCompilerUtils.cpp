@@ -39,6 +39,9 @@ void addPassesMI355X(OwningOpRef<ModuleOp> &module, PassManager &pm,
     // Chains ending in a float scaling become one call each; this has to run
     // while the graph is still in the ONNX dialect and fully shaped.
     if (!mi355xDisableFusion) {
+      // QDQ chains first: what they become is an op the patterns below and
+      // the ONNX-to-Krnl conversion of the accelerator know.
+      pm.addNestedPass<func::FuncOp>(createRecomposeQDQMatMulForMI355XPass());
       pm.addNestedPass<func::FuncOp>(createFuseQuantizedMatMulForMI355XPass());
       pm.addNestedPass<func::FuncOp>(createShapeInferencePass());
       pm.addPass(createCanonicalizerPass());

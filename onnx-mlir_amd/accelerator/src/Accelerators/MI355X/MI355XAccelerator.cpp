@@ -81,6 +81,9 @@ void MI355XAccelerator::registerPasses(int /*optLevel*/) const {
     return onnx_mlir::createFuseQuantizedMatMulForMI355XPass();
   });
   mlir::registerPass([]() -> std::unique_ptr<mlir::Pass> {
+    return onnx_mlir::createRecomposeQDQMatMulForMI355XPass();
+  });
+  mlir::registerPass([]() -> std::unique_ptr<mlir::Pass> {
     return onnx_mlir::createKeepBuffersOnMI355XPass();
   });
 }

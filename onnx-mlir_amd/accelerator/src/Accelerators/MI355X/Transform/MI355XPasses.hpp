@@ -32,6 +32,12 @@ constexpr const char *kMI355XSetQuantMode = "om_mi355x_SetQuantMode";
 /// become one `onnx.Custom` each.
 std::unique_ptr<mlir::Pass> createFuseQuantizedMatMulForMI355XPass();
 
+/// --recompose-qdq-matmul-for-mi355x
+///   DequantizeLinear(a), DequantizeLinear(W) -> MatMul -> QuantizeLinear
+/// becomes onnx.QLinearMatMul, also when W has one scale per output column
+/// (which the runtime's QLinearMatMul takes and the CPU lowering does not).
+std::unique_ptr<mlir::Pass> createRecomposeQDQMatMulForMI355XPass();
+
 /// --keep-buffers-on-mi355x
 /// Runs on Krnl/MemRef IR.  A `memref.alloc` that only MI355X calls touch gets
 /// `om_mi355x_KeepOnDevice` after the allocation and `om_mi355x_Release`

@@ -171,3 +171,37 @@ def test_fused_layer_takes_an_activation_that_is_not_16_byte_aligned(rt, oracle,
     assert "flight (rows quantized" not in rt.last_gemm_kernel()
     assert same_f32(got, want)
     buf.free()
+
+
+def test_qlinear_matmul_with_a_scale_per_column(rt, oracle):
+    """b_scale as one value per column of B (what a QDQ model with per-channel
+    weights recomposes to).  PARITY UNPINNED against the reference, whose
+    lowering refuses this form (QLinearMatMul.cpp:53-68): the expected values
+    are its expression (:127-138) with column j's scale -- f32(acc) * ((a_scale
+    * b_scale[j]) / y_scale), roundEven, + y_zp, narrowed -- over the oracle's
+    exact int32 product, restated here in numpy; with all columns' scales equal
+    that restatement is checked against the oracle's own QLinearMatMul first."""
+    rng = np.random.default_rng(4242)
+
+    def expect(A, a_s, az, B, bs, bz, y_s, yz, saturate):
+        acc = mm(oracle, A, B, az, bz)
+        s = (np.float32(a_s) * bs.astype(np.float32)) / np.float32(y_s)
+        q = np.rint(acc.astype(np.float32) * s[None, :]).astype(np.int64) + int(yz)
+        info = np.iinfo(yz.dtype)
+        if saturate:
+            return np.clip(q, info.min, info.max).astype(yz.dtype)
+        return (q & 0xFF).astype(np.uint8).view(yz.dtype) if yz.dtype == np.int8 else (q & 0xFF).astype(np.uint8)
+
+    for (M, K, N), adt in (((200, 1024, 1000), np.uint8), ((300, 768, 384), np.int8), ((48, 200, 130), np.uint8),
+                            ((1024, 768, 3072), np.uint8)):
+        A, B = _rand_q(rng, adt, (M, K)), _rand_q(rng, np.int8, (K, N))
+        az, yz = _rand_q(rng, adt, ()), _rand_q(rng, adt, ())
+        bz = _rand_q(rng, np.int8, (N,)) if M != 1024 else np.zeros(N, np.int8)
+        a_s, y_s = np.float32(0.0173), np.float32(0.11)
+        same = np.full(N, 0.004, np.float32)
+        for sat, omode, mode in ((False, oracle_lib.WRAP, rt.WRAP), (True, oracle_lib.SATURATE, rt.SATURATE)):
+            assert np.array_equal(expect(A, a_s, az, B, same, bz, y_s, yz, sat),
+                                  oracle.qlinear_matmul(A, a_s, az, B, same[0], bz, y_s, yz, omode))
+            bs = rng.uniform(1e-3, 8e-3, N).astype(np.float32)
+            got = rt.QLinearMatMul(A, a_s, az, B, bs, bz, y_s, yz, mode)
+            assert np.array_equal(got, expect(A, a_s, az, B, bs, bz, y_s, yz, sat)), (M, K, N, sat, rt.last_gemm_kernel())
