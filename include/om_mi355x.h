@@ -206,6 +206,26 @@ void om_mi355x_DynQuantMatMulDequant(OMTensor *y, const OMTensor *x,
     const OMTensor *b, const OMTensor *b_zp, const OMTensor *b_scale,
     const OMTensor *bias, int64_t activation);
 
+/* The same layer in a chain of such layers (FFN-up -> Gelu -> FFN-down).
+ * DynamicQuantizeLinear starts with two reductions over its whole input,
+ * ReduceMin and ReduceMax
+ * (src/Conversion/ONNXToKrnl/Quantization/DynamicQuantizeLinear.cpp:100-110),
+ * before it can quantize any of it; when the input is the result of the layer
+ * before, that layer's kernel can take them over what it stores.
+ *   y_limits: NULL, or f32[2] that receives min(y) and max(y) over all
+ *             elements of y, NaN ignored (what those reductions give; zero
+ *             is not included yet);
+ *   x_limits: NULL, or f32[2] holding min(x) and max(x) in that sense, as an
+ *             earlier call's y_limits received them for this very tensor: the
+ *             call then quantizes x in one pass without looking for them.
+ *             Values that are not x's minimum and maximum give a different
+ *             scale and zero point than DynamicQuantizeLinear(x) would.
+ * Everything else, and every bit of y, as om_mi355x_DynQuantMatMulDequant. */
+void om_mi355x_DynQuantMatMulDequantLimits(OMTensor *y, OMTensor *y_limits,
+    const OMTensor *x, const OMTensor *x_limits, const OMTensor *b,
+    const OMTensor *b_zp, const OMTensor *b_scale, const OMTensor *bias,
+    int64_t activation);
+
 /* ---- residency ---------------------------------------------------------- */
 /* Declares that the host buffer behind `t` never changes for the life of the
  * process (a krnl.global constant: src/Conversion/KrnlToLLVM/KrnlGlobal.cpp

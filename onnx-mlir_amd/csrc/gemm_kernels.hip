@@ -1352,6 +1352,9 @@ thread_local const char *t_last_kernel = "";
 // Whether that kernel applied the onnx.Gelu asked for to its results itself
 // (launch_gemm runs the pass over the output when it did not).
 thread_local bool t_gelu_applied = false;
+// Whether that kernel wrote GemmArgs::y_limits itself (launch_gemm runs the
+// reduction over the output when it did not).
+thread_local bool t_limits_written = false;
 
 template <int A_MODE, int EPI>
 hipError_t gemm_launch_cfg(
@@ -1639,6 +1642,9 @@ hipError_t launch_gemm(hipStream_t s, const GemmArgs &g) {
   ep.narrow = (int)g.narrow;
   const int a_mode = (g.X || g.a_preshifted) ? 2 : (g.a_unsigned ? 1 : 0);
   t_gelu_applied = false;
+  t_limits_written = false;
+  if (g.y_limits && (g.epi != kEpiF32 || !g.dql))
+    return hipErrorInvalidValue;
   hipError_t e;
   switch (a_mode) {
   case 0:
@@ -1659,6 +1665,8 @@ hipError_t launch_gemm(hipStream_t s, const GemmArgs &g) {
         (float *)g.out, n);
     e = hipGetLastError();
   }
+  if (e == hipSuccess && g.y_limits && !t_limits_written)
+    e = launch_minmax_limits(s, *g.dql, (const float *)g.out, g.M * g.N, g.y_limits);
   return e;
 }
 

@@ -64,6 +64,23 @@ hipError_t launch_dynamic_quantize(hipStream_t s, DqlScratch &scratch,
     bool y_shift, int mode = 0);
 constexpr int kQuantReciprocal = 1, kQuantNoZeroPoint = 2;
 
+// Minimum and maximum of a tensor handed from the op that produced it to the
+// DynamicQuantizeLinear that consumes it: limits[0] = min, limits[1] = max
+// over all elements with NaN ignored, zero not yet included (what the
+// reference's two reductions give,
+// src/Conversion/ONNXToKrnl/Quantization/DynamicQuantizeLinear.cpp:100-110).
+struct QuantLimits {
+  const float *limits; // null: not known
+  float *scale_out;    // where the derived scale and zero point go
+  uint8_t *zp_out;
+  int no_zp;           // kQuantNoZeroPoint
+};
+hipError_t launch_quantize_from_limits(hipStream_t s, const float *x, int64_t n,
+    const float *limits, uint8_t *y, float *scale, uint8_t *zp, bool y_shift,
+    int mode = 0);
+hipError_t launch_minmax_limits(hipStream_t s, DqlScratch &scratch,
+    const float *x, int64_t n, float *limits_out);
+
 // The tagged-slot exchange between the blocks of one launch (k_dql_grid, the
 // fused layer of k_gemm_i8_flight).  At most one kernel that uses it may be in
 // flight per process: two of them dispatched at the same time from different
@@ -135,6 +152,15 @@ struct GemmArgs {
   bool y_unsigned;
   NarrowMode narrow;
   void *out;           // i32 / f32 / u8|i8 [M,N]
+  // kEpiF32 only, optional: receives minimum and maximum of `out` (see
+  // QuantLimits) for the DynamicQuantizeLinear that reads it next.  Kernels
+  // that can, reduce them in their epilogue (partial results and arrival
+  // counter in `dql`, which must be set); behind the others a pass over `out`
+  // does.
+  float *y_limits;
+  // With X, optional: minimum and maximum of X as an earlier product's
+  // y_limits gave them; the kernel then does not look for them.
+  const float *x_limits;
 };
 
 hipError_t launch_gemm(hipStream_t s, const GemmArgs &g);

@@ -98,14 +98,34 @@ __device__ __forceinline__ bool wave_all(bool p) {
 constexpr int kUnroll = 4;
 constexpr int kRowUnroll = 8; // rows in flight per thread in the row-walking per-axis kernels
 
+// Scale and zero point of a per-tensor quantize kernel: read from memory, or
+// -- when the caller knows minimum and maximum of x (QuantLimits) -- derived
+// from those as DynamicQuantizeLinear derives them, by every block for itself,
+// and written to where the GEMM that follows reads them by the first block.
+template <bool SIGNED, bool HAS_ZP>
+__device__ __forceinline__ void quant_params(const float *__restrict__ scale_p,
+    const void *__restrict__ zp_p, const QuantLimits &lim, bool first_block,
+    float &s, float &zpf) {
+  if (lim.limits) { // (the same for every thread)
+    dynamic_params(lim.limits[0], lim.limits[1], s, zpf, lim.no_zp != 0);
+    if (first_block && threadIdx.x == 0) {
+      lim.scale_out[0] = s;
+      lim.zp_out[0] = (uint8_t)(uint32_t)zpf;
+    }
+  } else {
+    s = scale_p[0];
+    zpf = HAS_ZP ? load_zp_f32<SIGNED>(zp_p, 0) : 0.0f;
+  }
+}
+
 template <bool SIGNED, bool HAS_ZP>
 __global__ __launch_bounds__(kThreads) void k_quant_flat(
     const float *__restrict__ x, uint8_t *__restrict__ y, int64_t n,
     const float *__restrict__ scale_p, const void *__restrict__ zp_p,
-    uint32_t flip) {
-  const float s = scale_p[0];
+    uint32_t flip, QuantLimits lim) {
+  float s, zpf;
+  quant_params<SIGNED, HAS_ZP>(scale_p, zp_p, lim, blockIdx.x == 0, s, zpf);
   const float r = 1.0f / s;
-  const float zpf = HAS_ZP ? load_zp_f32<SIGNED>(zp_p, 0) : 0.0f;
   const int64_t nvec = n >> 2;
   const f4a *__restrict__ x4 = (const f4a *)x;
   uint32_t *__restrict__ y4 = (uint32_t *)y;
@@ -155,11 +175,12 @@ template <bool SIGNED, bool HAS_ZP>
 __global__ __launch_bounds__(kThreads) void k_quant_tiled(
     const float *__restrict__ x, uint8_t *__restrict__ y, int64_t n,
     const float *__restrict__ scale_p, const void *__restrict__ zp_p,
-    uint32_t flip) {
-  const float s = scale_p[0];
+    uint32_t flip, QuantLimits lim) {
+  float s, zpf;
+  quant_params<SIGNED, HAS_ZP>(
+      scale_p, zp_p, lim, blockIdx.x == 0 && blockIdx.y == 0, s, zpf);
   const float r = 1.0f / s;
   const bool tame = scale_is_tame(s); // the same for every thread
-  const float zpf = HAS_ZP ? load_zp_f32<SIGNED>(zp_p, 0) : 0.0f;
   const int64_t nvec = n >> 2;
   const f4a *__restrict__ x4 = (const f4a *)x;
   uint32_t *__restrict__ y4 = (uint32_t *)y;
@@ -1501,7 +1522,10 @@ __device__ __forceinline__ void block_minmax(float &lo, float &hi) {
 __global__ __launch_bounds__(kThreads) void k_minmax_params(
     const float *__restrict__ x, int64_t n, float *partial_min,
     float *partial_max, unsigned *counter, float *__restrict__ scale_out,
-    uint8_t *__restrict__ zp_out, int no_zp) {
+    uint8_t *__restrict__ zp_out, int no_zp,
+    float *__restrict__ limits_out = nullptr) {
+  // limits_out: minimum and maximum themselves go there (NaN ignored, 0 not
+  // yet included) in place of the parameters derived from them.
   float lo = __builtin_inff(), hi = -__builtin_inff();
   const int64_t nvec = n >> 2;
   const f4a *__restrict__ x4 = (const f4a *)x;
@@ -1584,10 +1608,15 @@ __global__ __launch_bounds__(kThreads) void k_minmax_params(
   }
   block_minmax(lo, hi);
   if (threadIdx.x == 0) {
-    float scale, zpf;
-    dynamic_params(lo, hi, scale, zpf, no_zp != 0);
-    scale_out[0] = scale;
-    zp_out[0] = (uint8_t)(uint32_t)zpf;
+    if (limits_out) {
+      limits_out[0] = lo;
+      limits_out[1] = hi;
+    } else {
+      float scale, zpf;
+      dynamic_params(lo, hi, scale, zpf, no_zp != 0);
+      scale_out[0] = scale;
+      zp_out[0] = (uint8_t)(uint32_t)zpf;
+    }
     __hip_atomic_store(
         counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
@@ -1950,15 +1979,41 @@ unsigned gather_grid(int64_t n) {
   return (unsigned)(blocks > 0 ? blocks : 1);
 }
 
+// Scale and zero point from known limits, as a launch of its own (in front of
+// the quantize kernels that read them from memory).
+__global__ void k_params_from_limits(QuantLimits lim) {
+  float s, zpf;
+  dynamic_params(lim.limits[0], lim.limits[1], s, zpf, lim.no_zp != 0);
+  lim.scale_out[0] = s;
+  lim.zp_out[0] = (uint8_t)(uint32_t)zpf;
+}
+
 template <bool SIGNED>
 hipError_t quantize_dispatch(hipStream_t st, const float *x, int64_t outer,
     int64_t channels, int64_t inner, const float *scale, const void *zp,
-    void *y, uint32_t flip, bool reciprocal = false) {
+    void *y, uint32_t flip, bool reciprocal = false,
+    const QuantLimits *limits = nullptr) {
   const int64_t n = outer * channels * inner;
   if (n == 0)
     return hipSuccess;
   uint8_t *yo = (uint8_t *)y;
   const bool has_zp = zp != nullptr;
+  // Limits of x in place of scale and zero point (per tensor, u8): the two
+  // streaming kernels derive the parameters themselves; in front of any other
+  // kernel a launch of one thread does.
+  QuantLimits lim = {};
+  if (limits) {
+    const bool aligned =
+        ((((uintptr_t)x) & 15) == 0) && ((((uintptr_t)y) & 3) == 0);
+    if (channels == 1 && !reciprocal && aligned && !SIGNED && has_zp) {
+      lim = *limits;
+    } else {
+      k_params_from_limits<<<1, 1, 0, st>>>(*limits);
+      const hipError_t e = hipGetLastError();
+      if (e != hipSuccess)
+        return e;
+    }
+  }
   if (reciprocal) {
     // The reference's fast-math form, x * (1 / scale): a kernel of its own
     // for the per-tensor case, the general kernel for everything else.
@@ -2027,10 +2082,10 @@ hipError_t quantize_dispatch(hipStream_t st, const float *x, int64_t outer,
       const dim3 grid(kTileRun / kThreads, (unsigned)tile_gy);
       if (has_zp)
         k_quant_tiled<SIGNED, true>
-            <<<grid, kThreads, 0, st>>>(x, yo, n, scale, zp, flip);
+            <<<grid, kThreads, 0, st>>>(x, yo, n, scale, zp, flip, lim);
       else
         k_quant_tiled<SIGNED, false>
-            <<<grid, kThreads, 0, st>>>(x, yo, n, scale, zp, flip);
+            <<<grid, kThreads, 0, st>>>(x, yo, n, scale, zp, flip, lim);
       return hipGetLastError();
     }
     if (aligned) {
@@ -2038,10 +2093,10 @@ hipError_t quantize_dispatch(hipStream_t st, const float *x, int64_t outer,
           stream_grid(n >> 2, kThreads * kUnroll, kGridCapQuantFlat);
       if (has_zp)
         k_quant_flat<SIGNED, true>
-            <<<grid, kThreads, 0, st>>>(x, yo, n, scale, zp, flip);
+            <<<grid, kThreads, 0, st>>>(x, yo, n, scale, zp, flip, lim);
       else
         k_quant_flat<SIGNED, false>
-            <<<grid, kThreads, 0, st>>>(x, yo, n, scale, zp, flip);
+            <<<grid, kThreads, 0, st>>>(x, yo, n, scale, zp, flip, lim);
       return hipGetLastError();
     }
     // Misaligned buffers: treat as one long run.
@@ -2398,6 +2453,32 @@ hipError_t launch_dynamic_quantize(hipStream_t s, DqlScratch &scratch,
   // the reference adds: it is an integer in [0, 255]).
   return quantize_dispatch<false>(s, x, 1, 1, n, scale, zp, y,
       y_shift ? 0x80808080u : 0u, (mode & kQuantReciprocal) != 0);
+}
+
+// DynamicQuantizeLinear of a tensor whose minimum and maximum are known:
+// limits[0..1] on the GPU, as launch_minmax_limits or a GEMM's epilogue
+// (GemmArgs::y_limits) wrote them.  One pass over x.
+hipError_t launch_quantize_from_limits(hipStream_t s, const float *x, int64_t n,
+    const float *limits, uint8_t *y, float *scale, uint8_t *zp, bool y_shift,
+    int mode) {
+  QuantLimits lim = {limits, scale, zp, (mode & kQuantNoZeroPoint) ? 1 : 0};
+  if (n == 0) { // scale and zero point are written all the same
+    k_params_from_limits<<<1, 1, 0, s>>>(lim);
+    return hipGetLastError();
+  }
+  return quantize_dispatch<false>(s, x, 1, 1, n, scale, zp, y,
+      y_shift ? 0x80808080u : 0u, (mode & kQuantReciprocal) != 0, &lim);
+}
+
+// Minimum and maximum of x (NaN ignored; +inf / -inf for an empty tensor)
+// into limits_out[0..1]: the first pass of DynamicQuantizeLinear by itself.
+hipError_t launch_minmax_limits(hipStream_t s, DqlScratch &scratch,
+    const float *x, int64_t n, float *limits_out) {
+  const int grid = stream_grid(
+      n >> 2, kThreads * 8, scratch.max_blocks < 512 ? scratch.max_blocks : 512);
+  k_minmax_params<<<grid, kThreads, 0, s>>>(x, n, scratch.partial_min,
+      scratch.partial_max, scratch.counter, nullptr, nullptr, 0, limits_out);
+  return hipGetLastError();
 }
 
 bool dql_exchange_begin(hipStream_t s, DqlScratch &scratch, GridExchange &x) {

@@ -1819,12 +1819,17 @@ void om_mi355x_QLinearMatMul(OMTensor *y, const OMTensor *a,
   run_matmul(sp);
 }
 
-void om_mi355x_DynQuantMatMulDequant(OMTensor *y_t, const OMTensor *x_t,
+} // extern "C"
+
+namespace {
+// The fused layer, with or without the limits of x handed in and those of y
+// handed out (om_mi355x_DynQuantMatMulDequantLimits).
+void dyn_quant_matmul_dequant(const char *op, OMTensor *y_t,
+    OMTensor *ylim_t, const OMTensor *x_t, const OMTensor *xlim_t,
     const OMTensor *b_t, const OMTensor *bzp_t, const OMTensor *bscale_t,
     const OMTensor *bias_t, int64_t activation) {
   const QuantModeScope quant_mode_of_this_op;
-  const char *op = "DynQuantMatMulDequant";
-  View y, x, b, bzp, bs, bias;
+  View y, x, b, bzp, bs, bias, ylim, xlim;
   bool relu, gelu;
   if (!activation_ok(activation, op, relu, gelu))
     return;
@@ -1833,6 +1838,15 @@ void om_mi355x_DynQuantMatMulDequant(OMTensor *y_t, const OMTensor *x_t,
     return;
   if (bzp_t && !view_of(bzp_t, "b_zero_point", bzp))
     return;
+  if ((ylim_t && !view_of(ylim_t, "y_limits", ylim)) ||
+      (xlim_t && !view_of(xlim_t, "x_limits", xlim)))
+    return;
+  if ((ylim_t && (ylim.dtype != OM_MI355X_TYPE_FLOAT || ylim.numel != 2)) ||
+      (xlim_t && (xlim.dtype != OM_MI355X_TYPE_FLOAT || xlim.numel != 2))) {
+    fail(EINVAL, "%s: limits are f32 tensors of two elements (minimum, "
+                 "maximum)", op);
+    return;
+  }
   if (x.dtype != OM_MI355X_TYPE_FLOAT || y.dtype != OM_MI355X_TYPE_FLOAT ||
       !is_q8(b.dtype) || bs.dtype != OM_MI355X_TYPE_FLOAT ||
       (bzp_t && bzp.dtype != b.dtype)) {
@@ -1854,11 +1868,13 @@ void om_mi355x_DynQuantMatMulDequant(OMTensor *y_t, const OMTensor *x_t,
     return;
   if (M == 0 || N == 0)
     return;
-  Call call(t_ctx, "DynQuantMatMulDequant");
+  Call call(t_ctx, op);
   if (!call.ok)
     return;
   const float *dx = (const float *)call.in(x);
+  const float *d_xlim = xlim_t ? (const float *)call.in(xlim, false) : nullptr;
   void *dy = call.out(y); // before the quantization: it decides whether to wait
+  float *d_ylim = ylim_t ? (float *)call.out(ylim) : nullptr;
   const int32_t *colsum = nullptr;
   const int8_t *bp = nullptr;
   if (!call.ok || !packed_b(call, b, K, N, bp, colsum)) {
@@ -1878,12 +1894,19 @@ void om_mi355x_DynQuantMatMulDequant(OMTensor *y_t, const OMTensor *x_t,
     int64_t padded_k = 0;
     GemmArgs g = {};
     g.out = dy;
+    g.y_limits = d_ylim;
+    g.dql = &call.c.dql;
     if (in_kernel) {
       g.X = dx;
-      g.dql = &call.c.dql;
+      g.x_limits = d_xlim;
     } else {
       uint8_t *aq = (uint8_t *)call.temp((size_t)M * K);
-      if (call.ok)
+      if (call.ok && d_xlim)
+        // minimum and maximum are known: one pass, no reduction
+        call.check(launch_quantize_from_limits(call.c.stream, dx, M * K, d_xlim,
+                       aq, call.c.dql_scale, call.c.dql_zp, true, t_quant_mode),
+            "quantize");
+      else if (call.ok)
         run_dql(call, dx, M * K, aq, call.c.dql_scale, call.c.dql_zp, true);
       g.A = aq;
       if (call.ok && gemm_pads_rows(M, K, aq)) {
@@ -1921,7 +1944,10 @@ void om_mi355x_DynQuantMatMulDequant(OMTensor *y_t, const OMTensor *x_t,
     g.gelu = gelu;
     return launch_gemm(call.c.stream, g);
   };
-  const int kind = (call.ok && t_quant_mode == 0 && call.c.dql.grid_blocks >= 0)
+  // (known limits of x: the kernels that quantize rows themselves do not
+  // take them yet)
+  const int kind = (call.ok && t_quant_mode == 0 && call.c.dql.grid_blocks >= 0 &&
+                       !d_xlim)
                        ? gemm_quantizes_rows(M, K, N, dx)
                        : 0;
   // Blocks that wait for one another (more rows than one block quantizes for
@@ -1942,10 +1968,10 @@ void om_mi355x_DynQuantMatMulDequant(OMTensor *y_t, const OMTensor *x_t,
         e = hipStreamSynchronize(call.c.stream);
         if (e == hipSuccess && call.c.dql_gave_up()) {
           fprintf(stderr,
-              "om_mi355x: DynQuantMatMulDequant: the blocks of the one-launch "
+              "om_mi355x: %s: the blocks of the one-launch "
               "kernel timed out waiting for one another; redone with two launches "
               "for the quantization and one for the product, which this thread "
-              "uses from now on\n");
+              "uses from now on\n", op);
           e = run(false);
         }
       }
@@ -1954,6 +1980,24 @@ void om_mi355x_DynQuantMatMulDequant(OMTensor *y_t, const OMTensor *x_t,
       call.check(e, op);
   }
   call.finish();
+}
+} // namespace
+
+extern "C" {
+
+void om_mi355x_DynQuantMatMulDequant(OMTensor *y_t, const OMTensor *x_t,
+    const OMTensor *b_t, const OMTensor *bzp_t, const OMTensor *bscale_t,
+    const OMTensor *bias_t, int64_t activation) {
+  dyn_quant_matmul_dequant("DynQuantMatMulDequant", y_t, nullptr, x_t, nullptr,
+      b_t, bzp_t, bscale_t, bias_t, activation);
+}
+
+void om_mi355x_DynQuantMatMulDequantLimits(OMTensor *y_t, OMTensor *ylim_t,
+    const OMTensor *x_t, const OMTensor *xlim_t, const OMTensor *b_t,
+    const OMTensor *bzp_t, const OMTensor *bscale_t, const OMTensor *bias_t,
+    int64_t activation) {
+  dyn_quant_matmul_dequant("DynQuantMatMulDequantLimits", y_t, ylim_t, x_t,
+      xlim_t, b_t, bzp_t, bscale_t, bias_t, activation);
 }
 
 // ---------------------------------------------------------------------------

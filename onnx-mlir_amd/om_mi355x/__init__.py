@@ -94,6 +94,7 @@ def _declare(lib, shim):
         "om_mi355x_MatMulIntegerDequant": [P, P, P, P, P, P, P, P, I64],
         "om_mi355x_QLinearMatMul": [P, P, P, P, P, P, P, P, P, I64],
         "om_mi355x_DynQuantMatMulDequant": [P, P, P, P, P, P, I64],
+        "om_mi355x_DynQuantMatMulDequantLimits": [P, P, P, P, P, P, P, P, I64],
         "om_mi355x_MarkConstant": [P],
         "om_mi355x_UnmarkConstant": [P],
         "om_mi355x_KeepOnDevice": [P],
@@ -520,6 +521,30 @@ def DynQuantMatMulDequant(x: Tensor, b: Tensor, b_zero_point: Optional[Tensor],
         _lib.om_mi355x_DynQuantMatMulDequant(hy, hx, hb, hbz, hbs, hbias, int(activation))
     _check()
     return y
+
+
+def DynQuantMatMulDequantLimits(x: Tensor, b: Tensor, b_zero_point: Optional[Tensor],
+                                b_scale: Tensor, bias: Optional[Tensor] = None,
+                                out: Optional[Tensor] = None, activation: int = ACTIVATION_NONE,
+                                x_limits: Optional[Tensor] = None, y_limits: Optional[Tensor] = None,
+                                want_limits: bool = True):
+    """om_mi355x_DynQuantMatMulDequantLimits: returns (y, y_limits); y_limits is
+    None when want_limits is false and none were passed in."""
+    load()
+    x, b, b_scale = _host(x), _host(b), _host(b_scale, np.float32)
+    bz = None if b_zero_point is None else _host(b_zero_point)
+    bias = None if bias is None else _host(bias, np.float32)
+    xl = None if x_limits is None else _host(x_limits, np.float32)
+    y = out if out is not None else _like(x, _mm_shape(x, b), np.float32)
+    yl = y_limits
+    if yl is None and want_limits:
+        yl = _like(x, (2,), np.float32)
+    with _OMT(y) as hy, _OMT(yl) as hyl, _OMT(x) as hx, _OMT(xl) as hxl, _OMT(b) as hb, \
+            _OMT(bz) as hbz, _OMT(b_scale) as hbs, _OMT(bias) as hbias:
+        _emit_quant_mode()
+        _lib.om_mi355x_DynQuantMatMulDequantLimits(hy, hyl, hx, hxl, hb, hbz, hbs, hbias, int(activation))
+    _check()
+    return y, yl
 
 
 class PreparedCall:

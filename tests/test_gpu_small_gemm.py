@@ -205,3 +205,81 @@ def test_qlinear_matmul_with_a_scale_per_column(rt, oracle):
             bs = rng.uniform(1e-3, 8e-3, N).astype(np.float32)
             got = rt.QLinearMatMul(A, a_s, az, B, bs, bz, y_s, yz, mode)
             assert np.array_equal(got, expect(A, a_s, az, B, bs, bz, y_s, yz, sat)), (M, K, N, sat, rt.last_gemm_kernel())
+
+
+def _limits(a):
+    a = np.asarray(a, np.float32)
+    return np.array([np.fmin.reduce(a, axis=None), np.fmax.reduce(a, axis=None)], np.float32)
+
+
+@pytest.mark.parametrize("M,K,N,N2", [(128, 768, 3072, 768), (4096, 768, 3072, 768), (16, 4096, 1024, 512),
+                                      (33, 200, 130, 70), (300, 768, 1000, 416), (2, 64, 8, 5)])
+def test_chain_of_layers_hands_the_limits_on(rt, oracle, M, K, N, N2):
+    """om_mi355x_DynQuantMatMulDequantLimits: y_limits of a layer is minimum and
+    maximum of its result (NaN ignored), bit for bit what numpy finds in it,
+    whatever kernel produced y (in its epilogue, or a pass over y behind it) and
+    with bias, Relu or Gelu applied; a second layer given them as x_limits
+    returns exactly what it returns without them, and what the oracle's chain of
+    the separate ops gives.  Host and GPU-resident tensors."""
+    rng = np.random.default_rng(M + N)
+    x = rng.normal(0, 1, (M, K)).astype(np.float32)
+    W1, W2 = _rand_q(rng, np.int8, (K, N)), _rand_q(rng, np.int8, (N, N2))
+    s1 = rng.uniform(1e-3, 1e-2, N).astype(np.float32)
+    s2 = rng.uniform(1e-3, 1e-2, N2).astype(np.float32)
+    bias = rng.normal(0, 1, N).astype(np.float32)
+    for act in (0, 1, 2):
+        h_plain = rt.DynQuantMatMulDequant(x, W1, None, s1, bias, activation=act)
+        h, hl = rt.DynQuantMatMulDequantLimits(x, W1, None, s1, bias, activation=act)
+        assert same_f32(h, h_plain), (act, rt.last_gemm_kernel())
+        assert same_f32(hl, _limits(h)), (act, hl, _limits(h), rt.last_gemm_kernel())
+        y_plain = rt.DynQuantMatMulDequant(h, W2, None, s2)
+        y, yl = rt.DynQuantMatMulDequantLimits(h, W2, None, s2, x_limits=hl)
+        assert same_f32(y, y_plain), act
+        assert same_f32(yl, _limits(y))
+        if act != 2:  # (the oracle's Gelu differs from the kernel's in the last bits)
+            aq, a_s, a_zp = oracle.dynamic_quantize_linear(h)
+            assert same_f32(y, oracle.dequant_epilogue(mm(oracle, aq, W2, a_zp, None), a_s, s2))
+    # GPU-resident, the limits never leave the GPU
+    dx, dW1, dW2, ds1, ds2 = (rt.DeviceArray.from_numpy(v) for v in (x, W1, W2, s1, s2))
+    dh, dhl = rt.DeviceArray((M, N), np.float32), rt.DeviceArray((2,), np.float32)
+    dy = rt.DeviceArray((M, N2), np.float32)
+    for _ in range(3):
+        rt.DynQuantMatMulDequantLimits(dx, dW1, None, ds1, None, out=dh, activation=1, y_limits=dhl)
+        rt.DynQuantMatMulDequantLimits(dh, dW2, None, ds2, None, out=dy, x_limits=dhl, want_limits=False)
+    rt.synchronize()
+    h = rt.DynQuantMatMulDequant(x, W1, None, s1, None, activation=1)
+    assert same_f32(dh.numpy(), h) and same_f32(dhl.numpy(), _limits(h))
+    assert same_f32(dy.numpy(), rt.DynQuantMatMulDequant(h, W2, None, s2))
+    for d in (dx, dW1, dW2, ds1, ds2, dh, dhl, dy):
+        d.free()
+
+
+def test_limits_with_nan_infinities_and_the_other_quotient(rt, oracle):
+    """NaN in the result is ignored by the limits (as the reductions of
+    DynamicQuantizeLinear ignore it), infinities are not; limits handed to a
+    layer under SetQuantMode(1) and (2) give what that mode gives without them;
+    limits of the wrong size are refused."""
+    rng = np.random.default_rng(99)
+    M, K, N = 70, 320, 96
+    x = rng.normal(0, 1, (M, K)).astype(np.float32)
+    W = _rand_q(rng, np.int8, (K, N))
+    s = rng.uniform(1e-3, 1e-2, N).astype(np.float32)
+    bias = rng.normal(0, 1, N).astype(np.float32)
+    bias[5], bias[9] = np.nan, np.inf
+    h, hl = rt.DynQuantMatMulDequantLimits(x, W, None, s, bias)
+    assert np.isnan(h[:, 5]).all() and same_f32(hl, _limits(h)) and hl[1] == np.inf
+    bias[9] = 1.0
+    h, hl = rt.DynQuantMatMulDequantLimits(x, W, None, s, bias)
+    assert np.isfinite(hl).all() and same_f32(hl, _limits(h))
+    W2 = _rand_q(rng, np.int8, (N, 40))
+    s2 = rng.uniform(1e-3, 1e-2, 40).astype(np.float32)
+    h = np.nan_to_num(h, nan=0.25)
+    hl = _limits(h)
+    for mode in (1, 2, 3):
+        rt.set_quant_mode(mode)
+        want = rt.DynQuantMatMulDequant(h, W2, None, s2)
+        rt.set_quant_mode(mode)
+        got, _ = rt.DynQuantMatMulDequantLimits(h, W2, None, s2, x_limits=hl, want_limits=False)
+        assert same_f32(got, want), mode
+    with pytest.raises(rt.RuntimeError_, match="limits"):
+        rt.DynQuantMatMulDequantLimits(h, W2, None, s2, x_limits=np.zeros(3, np.float32))
