@@ -57,7 +57,17 @@ __device__ __forceinline__ void lds_barrier() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
+// Where a kernel with the f32 epilogue leaves minimum and maximum of what it
+// stored (GemmArgs::y_limits): `out`, null when not asked for; one partial
+// pair per block; an arrival counter that is zero between launches.
+struct LimitsOut {
+  float *out;
+  float *part_min, *part_max;
+  unsigned *counter;
+};
+
 struct EpiParams {
+  LimitsOut limits;
   const void *a_zp;
   int64_t a_zp_len;
   const void *b_zp;
@@ -77,6 +87,72 @@ struct EpiParams {
   bool y_unsigned;
   int narrow;
 };
+
+// Called once by every thread of a block of `nwaves` waves (the waves that are
+// still running, in uniform control flow) with the minimum and maximum of the
+// elements it stored, NaN ignored (+inf / -inf if it stored none).  The block's
+// pair goes to its slot; the block that arrives last folds all slots and
+// writes L.out[0..1] (the scheme of DynamicQuantizeLinear's reduction kernel:
+// partials as device-scope atomic stores, a ticket drawn after they have been
+// acknowledged, the counter put back to zero by the last block).
+// lds: 2 * nwaves + 1 words nobody else uses any more; sync: a barrier of the
+// calling waves that orders LDS.
+template <typename Sync>
+__device__ __forceinline__ void block_publish_limits(float lo, float hi,
+    const LimitsOut &L, float *lds, int wave, int lane, int nwaves, Sync sync) {
+  lo = wave_min(lo);
+  hi = wave_max(hi);
+  if (lane == 0) {
+    lds[wave] = lo;
+    lds[nwaves + wave] = hi;
+  }
+  sync();
+  if (wave == 0 && lane == 0) {
+    for (int w = 1; w < nwaves; ++w) {
+      lo = __builtin_fminf(lo, lds[w]);
+      hi = __builtin_fmaxf(hi, lds[nwaves + w]);
+    }
+    __hip_atomic_store(&L.part_min[blockIdx.x], lo, __ATOMIC_RELAXED,
+        __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(&L.part_max[blockIdx.x], hi, __ATOMIC_RELAXED,
+        __HIP_MEMORY_SCOPE_AGENT);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): both stores acknowledged
+    const unsigned ticket = __hip_atomic_fetch_add(
+        L.counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    lds[2 * nwaves] = ticket == gridDim.x - 1 ? 1.0f : 0.0f;
+  }
+  sync();
+  if (lds[2 * nwaves] == 0.0f)
+    return;
+  // the last block to arrive
+  lo = __builtin_inff();
+  hi = -__builtin_inff();
+  for (unsigned i = wave * 64 + lane; i < gridDim.x; i += nwaves * 64) {
+    lo = __builtin_fminf(lo, __hip_atomic_load(&L.part_min[i], __ATOMIC_RELAXED,
+                                 __HIP_MEMORY_SCOPE_AGENT));
+    hi = __builtin_fmaxf(hi, __hip_atomic_load(&L.part_max[i], __ATOMIC_RELAXED,
+                                 __HIP_MEMORY_SCOPE_AGENT));
+  }
+  lo = wave_min(lo);
+  hi = wave_max(hi);
+  sync(); // (everyone has read the flag)
+  if (lane == 0) {
+    lds[wave] = lo;
+    lds[nwaves + wave] = hi;
+  }
+  sync();
+  if (wave == 0 && lane == 0) {
+    for (int w = 1; w < nwaves; ++w) {
+      lo = __builtin_fminf(lo, lds[w]);
+      hi = __builtin_fmaxf(hi, lds[nwaves + w]);
+    }
+    L.out[0] = lo;
+    L.out[1] = hi;
+    __hip_atomic_store(L.counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
 
 // onnx.Relu as the reference lowers it: max(0, x) with the maximum that
 // returns the other operand for a NaN

@@ -270,7 +270,9 @@ template <int EPI>
 __device__ __forceinline__ void flight_store_tile(const v16i &acc,
     const FlightEpi &e, const EpiParams &ep, const int32_t *rs, int mrow0,
     int rows, int ncol0_block, int wave, int waves, int lane, int M, int N,
-    int act, uint8_t *stage, bool q8_lines) {
+    int act, uint8_t *stage, bool q8_lines, float &lim_lo, float &lim_hi) {
+  // lim_lo / lim_hi: running minimum and maximum of the f32 results this lane
+  // has stored (only kept when the caller asked for them, ep.limits.out)
   constexpr int ES = (EPI == kEpiQ8) ? 1 : 4;
   const int l32 = lane & 31, lh = lane >> 5;
   const int n = ncol0_block + wave * 32 + l32;
@@ -304,6 +306,18 @@ __device__ __forceinline__ void flight_store_tile(const v16i &acc,
 #pragma unroll
         for (int r = 0; r < 16; ++r)
           y[r] = __float_as_uint(relu_f32(f[r], ep.floor));
+      }
+      if (ep.limits.out != nullptr) { // (the same for every lane)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          if (8 * (r >> 2) >= rows)
+            continue;
+          // rows of the tile that are not the block's count as NaN: ignored
+          const bool mine = 8 * (r >> 2) + (r & 3) + 4 * lh < rows;
+          const float v = mine ? __uint_as_float(y[r]) : __builtin_nanf("");
+          lim_lo = __builtin_fminf(lim_lo, v);
+          lim_hi = __builtin_fmaxf(lim_hi, v);
+        }
       }
     }
 #pragma unroll
@@ -443,7 +457,8 @@ __device__ __forceinline__ void flight_kloop(const unsigned (&aaddr)[8],
 // ---------------------------------------------------------------------------
 // KG: K / 256 (a template argument: every loop over K is unrolled and has no
 // branch).  FLIP: A holds uint8 and becomes int8 (minus 128) on its way into
-// LDS; a_off: A' = A - 128 (FLIP, or A was stored that way).
+// LDS; flags: bit 0, A' = A - 128 (FLIP, or A was stored that way); bit 1,
+// onnx.Gelu on the f32 result.
 // A block is WAVES column tiles side by side and NR row tiles of 32 one after
 // the other (1 or 2, 2 NR <= WAVES).  Its rows of A are
 // 8 nr groups of four rows; wave w brings groups w, w + waves, .. (two or four:
@@ -461,13 +476,14 @@ template <int KG, bool FLIP, int EPI, int NR, int WAVES>
 __global__ __launch_bounds__(64 * WAVES, 1)
 __attribute__((amdgpu_waves_per_eu(1, 1))) void k_gemm_i8_flight(
     const uint8_t *__restrict__ A, const int8_t *__restrict__ Bp, int M, int N,
-    EpiParams ep, int a_off, int regions_n, int bp_tiles) {
+    EpiParams ep, int flags, int regions_n, int bp_tiles) {
   constexpr int KH = 8 * KG, K = 256 * KG;
   constexpr int nr = NR, waves = WAVES;
   constexpr int P = (8 * NR) / WAVES; // groups of four rows a wave stages
   static_assert(KG >= 1 && KG <= kFlightMaxKG, "registers");
   static_assert(NR <= kFlightMaxTiles && (P == 2 || P == 4), "registers");
-  const bool A_OFF = a_off != 0;
+  const bool A_OFF = (flags & 1) != 0; // flags: 1 a_off, 2 onnx.Gelu on the f32 result
+  const int act = (flags & 2) ? 2 : 0;
   extern __shared__ __attribute__((aligned(1024))) uint8_t sA[];
   int32_t *const s_rs = (int32_t *)(sA + nr * KG * 8192); // [32 * nr] row sums
   uint8_t *const stage = (uint8_t *)(s_rs + 32 * kFlightMaxTiles);
@@ -584,11 +600,12 @@ __attribute__((amdgpu_waves_per_eu(1, 1))) void k_gemm_i8_flight(
   const bool q8_lines = EPI == kEpiQ8 && (N & 15) == 0 &&
                         ((((uintptr_t)ep.out) & 15) == 0);
   const v16i acc_zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+  float lim_lo = __builtin_inff(), lim_hi = -__builtin_inff();
   auto finish = [&](const v16i &acc, const FlightEpi &e, int t)
                     __attribute__((always_inline)) {
     flight_store_tile<EPI>(acc, e, ep, s_rs + 32 * t, row0 + 32 * t, 32,
-        rn * waves * 32, wave, waves, lane, M, N, 0,
-        stage + (t & 1) * 1024 * waves, q8_lines);
+        rn * waves * 32, wave, waves, lane, M, N, act,
+        stage + (t & 1) * 1024 * waves, q8_lines, lim_lo, lim_hi);
   };
   auto epi_params = [&]() __attribute__((always_inline)) {
     flight_params_not_before(raw);
@@ -608,6 +625,16 @@ __attribute__((amdgpu_waves_per_eu(1, 1))) void k_gemm_i8_flight(
   finish(acc[0], e, 0);
   if (NR == 2)
     finish(acc[1], e, 1);
+  if (EPI == kEpiF32 && ep.limits.out != nullptr) { // (the same for every wave)
+    // rows past M are copies of the last row; columns past N are nobody's
+    if (n >= N) {
+      lim_lo = __builtin_inff();
+      lim_hi = -__builtin_inff();
+    }
+    lds_sync(); // (the staging area is free)
+    block_publish_limits(lim_lo, lim_hi, ep.limits, (float *)stage, wave, lane,
+        waves, [] { lds_sync(); });
+  }
 #ifdef FLIGHT_TIMING
   FLIGHT_TS(6);
   asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
@@ -884,8 +911,20 @@ __global__ __launch_bounds__(512, 1) void k_gemm_i8_flight_dq(
   flight_params_not_before(raw);
   const FlightEpi e =
       flight_epi<kEpiF32>(ep, raw, true, K, scale, (int32_t)(uint32_t)zpf);
+  float lim_lo = __builtin_inff(), lim_hi = -__builtin_inff();
   flight_store_tile<kEpiF32>(acc, e, ep, s_rs, row0, R, rn * mwaves * 32, wave,
-      mwaves, lane, M, N, dq.act, nullptr, false);
+      mwaves, lane, M, N, dq.act, nullptr, false, lim_lo, lim_hi);
+  if (ep.limits.out != nullptr) { // (the same for every wave)
+    // Rows past M are copies of the last row; columns past N are nobody's.
+    // Only the multiplying waves are still running: the barrier counts them.
+    if (n >= N) {
+      lim_lo = __builtin_inff();
+      lim_hi = -__builtin_inff();
+    }
+    lds_sync(); // (the row sums have been read)
+    block_publish_limits(lim_lo, lim_hi, ep.limits, (float *)s_rs, wave, lane,
+        mwaves, [] { lds_sync(); });
+  }
 #ifdef FLIGHT_TIMING
   FLIGHT_TS(6);
   asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
@@ -961,8 +1000,9 @@ hipError_t flight_launch(hipStream_t st, const GemmArgs &g, const EpiParams &ep,
   const size_t lds = (size_t)NR * KG * 8192 + 4 * 32 * kFlightMaxTiles +
                      2 * 1024 * (size_t)WAVES;
   kern<<<dim3((unsigned)(regions_m * regions_n)), dim3(64 * WAVES), lds, st>>>(
-      (const uint8_t *)g.A, g.Bp, (int)g.M, (int)g.N, ep, a_mode != 0 ? 1 : 0,
-      regions_n, bp_tiles);
+      (const uint8_t *)g.A, g.Bp, (int)g.M, (int)g.N, ep,
+      (a_mode != 0 ? 1 : 0) | (EPI == kEpiF32 && g.gelu ? 2 : 0), regions_n,
+      bp_tiles);
   return hipGetLastError();
 }
 

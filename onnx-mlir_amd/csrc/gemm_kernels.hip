@@ -1373,6 +1373,7 @@ hipError_t gemm_launch_cfg(
         return hipErrorInvalidValue;
       t_last_kernel = "k_gemm_i8_flight (rows quantized in the kernel)";
       t_gelu_applied = g.gelu; // this kernel applies it to its results
+      t_limits_written = ep.limits.out != nullptr; // and reduces their limits
       return launch_gemm_flight_dq(st, g, ep, *g.dql);
     }
     if constexpr (A_MODE == 2) {
@@ -1433,6 +1434,8 @@ hipError_t gemm_launch_cfg(
   // k_gemm_i8_dma; 128 x 768 x 768: 7.0 us).
   if ((cfg == kFlight || !(force && force[0])) && flight_ok(g, A_MODE)) {
     t_last_kernel = "k_gemm_i8_flight (one round, operands requested at once)";
+    t_gelu_applied = EPI == kEpiF32 && g.gelu; // this kernel applies it itself
+    t_limits_written = EPI == kEpiF32 && ep.limits.out != nullptr;
     return launch_gemm_flight(st, g, ep, A_MODE);
   }
   // Weights in registers: K = 768 (the projections of a BERT-base layer)
@@ -1441,7 +1444,11 @@ hipError_t gemm_launch_cfg(
   if (wreg_ok(g) && (cfg == kW128x384 || (!forced && wreg_pays(g.M, g.N)))) {
     t_last_kernel = "k_gemm_i8_wreg (weights in registers, 128x384 blocks)";
     t_gelu_applied = g.epi == kEpiF32 && g.gelu; // this kernel applies it to its results
-    return launch_gemm_wreg(st, g, ep, A_MODE);
+    EpiParams epw = ep;
+    if (((g.M + 127) / 128) * ((g.N + 383) / 384) > kDqlMaxBlocks)
+      epw.limits = LimitsOut{}; // more blocks than partial slots: a pass over y
+    t_limits_written = EPI == kEpiF32 && epw.limits.out != nullptr;
+    return launch_gemm_wreg(st, g, epw, A_MODE);
   }
   switch (cfg) {
   case kB128x256: {
@@ -1635,6 +1642,10 @@ hipError_t launch_gemm(hipStream_t s, const GemmArgs &g) {
   ep.y_zp = g.y_zp;
   ep.bias = g.epi == kEpiF32 ? g.bias : nullptr;
   ep.bias_len = g.bias_len;
+  ep.limits = LimitsOut{};
+  if (g.y_limits) // (slot [4] of the counters: [0] is DynamicQuantizeLinear's)
+    ep.limits = LimitsOut{g.y_limits, g.dql->partial_min, g.dql->partial_max,
+        g.dql->counter + 4};
   ep.floor = relu_floor(g.epi == kEpiF32 && g.relu);
   ep.out = g.out;
   ep.b_unsigned = g.b_unsigned;

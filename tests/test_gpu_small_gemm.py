@@ -165,8 +165,11 @@ def test_fused_layer_takes_an_activation_that_is_not_16_byte_aligned(rt, oracle,
     dx.shape, dx.dtype, dx.ptr, dx.owner = (M, K), np.dtype(np.float32), buf.ptr + 4, buf
     aq, a_s, a_zp = oracle.dynamic_quantize_linear_mode(x, mode)
     want = oracle.dequant_epilogue(mm(oracle, aq, W, a_zp, None), a_s, ws)
-    rt.set_quant_mode(mode)
-    got = rt.DynQuantMatMulDequant(dx, W, None, ws)
+    rt.set_quant_mode(mode)  # (what a model compiled with that option emits in front of each op)
+    try:
+        got = rt.DynQuantMatMulDequant(dx, W, None, ws)
+    finally:
+        rt.set_quant_mode(0)
     got = got.numpy() if hasattr(got, "numpy") else got
     assert "flight (rows quantized" not in rt.last_gemm_kernel()
     assert same_f32(got, want)
@@ -275,11 +278,15 @@ def test_limits_with_nan_infinities_and_the_other_quotient(rt, oracle):
     s2 = rng.uniform(1e-3, 1e-2, 40).astype(np.float32)
     h = np.nan_to_num(h, nan=0.25)
     hl = _limits(h)
-    for mode in (1, 2, 3):
-        rt.set_quant_mode(mode)
-        want = rt.DynQuantMatMulDequant(h, W2, None, s2)
-        rt.set_quant_mode(mode)
-        got, _ = rt.DynQuantMatMulDequantLimits(h, W2, None, s2, x_limits=hl, want_limits=False)
-        assert same_f32(got, want), mode
+    try:
+        for mode in (1, 2, 3):
+            rt.set_quant_mode(mode)
+            want = rt.DynQuantMatMulDequant(h, W2, None, s2)
+            got, _ = rt.DynQuantMatMulDequantLimits(h, W2, None, s2, x_limits=hl, want_limits=False)
+            assert same_f32(got, want), mode
+            aq, a_s, a_zp = oracle.dynamic_quantize_linear_mode(h, mode)
+            assert same_f32(got, oracle.dequant_epilogue(mm(oracle, aq, W2, a_zp, None), a_s, s2)), mode
+    finally:
+        rt.set_quant_mode(0)
     with pytest.raises(rt.RuntimeError_, match="limits"):
         rt.DynQuantMatMulDequantLimits(h, W2, None, s2, x_limits=np.zeros(3, np.float32))
