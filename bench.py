@@ -207,6 +207,74 @@ def decode_case(rt, wl, M, steps, warmup):
     return res
 
 
+def chain_case(rt, wl, M, steps, warmup, limits):
+    """Config 4's feed-forward block as two dynamically quantized layers in a
+    row, FFN-up -> Gelu -> FFN-down, GPU-resident: two calls of
+    om_mi355x_DynQuantMatMulDequant, or (limits) of
+    om_mi355x_DynQuantMatMulDequantLimits with the first call's y_limits handed
+    to the second as x_limits, so that the second layer's
+    DynamicQuantizeLinear is one pass over its input."""
+    up, down = wl.config4("ffn_up"), wl.config4("ffn_down")
+    K, N = up["W"].shape
+    N2 = down["W"].shape[1]
+    dX = rt.DeviceArray.from_numpy(wl.normal_f32(4, 70, (M, K)))
+    dW1, dS1 = rt.DeviceArray.from_numpy(up["W"]), rt.DeviceArray.from_numpy(up["w_scale"])
+    dW2, dS2 = rt.DeviceArray.from_numpy(down["W"]), rt.DeviceArray.from_numpy(down["w_scale"])
+    dH, dY = rt.DeviceArray((M, N), np.float32), rt.DeviceArray((M, N2), np.float32)
+    dL = rt.DeviceArray((2,), np.float32)
+    rt.mark_constant(dW1)
+    rt.mark_constant(dW2)
+    if limits:
+        f1 = rt.PreparedCall("om_mi355x_DynQuantMatMulDequantLimits", dH, dL, dX, None, dW1, None, dS1, None, 2)
+        f2 = rt.PreparedCall("om_mi355x_DynQuantMatMulDequantLimits", dY, None, dH, dL, dW2, None, dS2, None, 0)
+    else:
+        f1 = rt.PreparedCall("om_mi355x_DynQuantMatMulDequant", dH, dX, dW1, None, dS1, None, 2)
+        f2 = rt.PreparedCall("om_mi355x_DynQuantMatMulDequant", dY, dH, dW2, None, dS2, None, 0)
+
+    def fn():
+        f1()
+        f2()
+
+    res = measure(rt, fn, steps, warmup)
+    f1.check()
+    f2.check()
+    f1.close()
+    f2.close()
+    ops = 2.0 * M * N * K + 2.0 * M * N2 * N
+    res.update({"name": f"config4 M={M} ffn_up -> Gelu -> ffn_down, " +
+                        ("limits handed on" if limits else "two plain calls"),
+                "M": M, "K": K, "N": N, "N2": N2, "kernel": rt.last_gemm_kernel(),
+                "tops": ops / (res["kernel_ms"] * 1e-3) / 1e12})
+    for d in (dX, dW1, dS1, dW2, dS2, dH, dY, dL):
+        d.free()
+    return res
+
+
+def decode_limits_case(rt, wl, M, steps, warmup):
+    """A decode step whose activation comes with its minimum and maximum (from
+    the layer before): om_mi355x_DynQuantMatMulDequantLimits with x_limits."""
+    c = wl.config5("up", M=M)
+    K, N = c["W"].shape
+    x = c["X"]
+    dX = rt.DeviceArray.from_numpy(x)
+    dL = rt.DeviceArray.from_numpy(np.array([x.min(), x.max()], np.float32))
+    dW, dS = rt.DeviceArray.from_numpy(c["W"]), rt.DeviceArray.from_numpy(c["w_scale"])
+    dY = rt.DeviceArray((M, N), np.float32)
+    rt.mark_constant(dW)
+    fn = rt.PreparedCall("om_mi355x_DynQuantMatMulDequantLimits", dY, None, dX, dL, dW, None, dS, None, 0)
+    res = measure(rt, fn, steps, warmup)
+    fn.check()
+    fn.close()
+    nbytes = K * N + M * K + 4 * M * N
+    res.update({"name": f"config5 decode M={M}, limits of x known", "M": M, "K": K, "N": N,
+                "kernel": rt.last_gemm_kernel(),
+                "gbs": nbytes / (res["kernel_ms"] * 1e-3) / 1e9, "bytes": nbytes,
+                "hbm_frac": nbytes / (res["kernel_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS})
+    for d in (dX, dL, dW, dS, dY):
+        d.free()
+    return res
+
+
 def qlinear_case(rt, wl, steps, warmup):
     """Config 3: QLinearMatMul, uint8 x uint8 -> uint8 with both zero points
     non-zero (row sums of A and the per-row correction are part of the step)."""
@@ -467,6 +535,11 @@ def only_mode(rt, wl, what, steps, warmup):
         return {"only": what, **r}
     if what == "config3":
         return {"only": what, **qlinear_case(rt, wl, steps, warmup)}
+    if what in ("chain", "chain_limits", "chain128", "chain128_limits"):
+        return {"only": what, **chain_case(rt, wl, 128 if "128" in what else 4096, steps, warmup,
+                                           what.endswith("limits"))}
+    if what == "decode16_limits":
+        return {"only": what, **decode_limits_case(rt, wl, 16, steps, warmup)}
     if what == "qlinear_ffn_up":
         return {"only": what, **qlinear_ffn_up_case(rt, wl, steps, warmup)}
     if what in ("config1", "config1_two_calls"):
@@ -696,7 +769,7 @@ def main():
                     choices=["copy", "mfma_ceiling", "per_axis_layouts", "gemm_ffn_up", "gemm_qkv", "gemm_out", "gemm_ffn_down",
                              "gemm_prefill_up", "gemm_prefill_down", "fused_ffn_up", "fused_ffn_down",
                              "fused_ffn_up_relu", "fused_ffn_up_gelu",
-                             "decode", "decode4", "decode16", "config1", "config1_two_calls", "config3", "qlinear_ffn_up",
+                             "decode", "decode4", "decode16", "config1", "config1_two_calls", "config3", "qlinear_ffn_up", "chain", "chain_limits", "chain128", "chain128_limits", "decode16_limits",
                              "quantize_per_axis", "dequantize_per_axis",
                              "quantize_per_tensor", "dequantize_per_tensor", "dynamic_quantize",
                              "quantize_per_axis_ragged", "dequantize_per_axis_ragged",

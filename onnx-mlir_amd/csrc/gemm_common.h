@@ -68,6 +68,10 @@ struct LimitsOut {
 
 struct EpiParams {
   LimitsOut limits;
+  // Kernels that quantize an f32 activation themselves (GemmArgs::X): its
+  // minimum and maximum when the caller knows them (GemmArgs::x_limits), so
+  // that they are not looked for; null otherwise.
+  const float *x_limits;
   const void *a_zp;
   int64_t a_zp_len;
   const void *b_zp;

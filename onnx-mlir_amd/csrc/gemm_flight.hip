@@ -751,9 +751,12 @@ __global__ __launch_bounds__(512, 1) void k_gemm_i8_flight_dq(
   if (tid < 32)
     s_rs[tid] = 0;
   lds_sync();
+  // The caller knows minimum and maximum of X (from the layer before): nothing
+  // is published and nobody polls.
+  const bool known = ep.x_limits != nullptr;
   // Publishers: the first G blocks of every row region.
   const int nslots = (int)(gridDim.x / regions_n) * G; // <= 256
-  if (tid == 0 && rn < G) {
+  if (tid == 0 && rn < G && !known) {
     float bl = s_lo[0], bh = s_hi[0];
 #pragma unroll
     for (int w = 1; w < WAVES; ++w) {
@@ -810,6 +813,10 @@ __global__ __launch_bounds__(512, 1) void k_gemm_i8_flight_dq(
       xlo = __builtin_fminf(xlo, s_lo[w2]);
       xhi = __builtin_fmaxf(xhi, s_hi[w2]);
     }
+    if (known) {
+      xlo = ep.x_limits[0];
+      xhi = ep.x_limits[1];
+    }
     FLIGHT_TS(3);
     dynamic_params(xlo, xhi, scale, zpf);
     const float recip = 1.0f / scale;
@@ -845,7 +852,7 @@ __global__ __launch_bounds__(512, 1) void k_gemm_i8_flight_dq(
     return true;
   };
   if (!multiplies) { // (the same for the whole wave)
-    if (wave >= 4) {
+    if (wave >= 4 && !known) {
       const int slot = tid - 256;
       const bool polls = slot < nslots;
       const unsigned long long *const slot_p = &dq.slots[2 * (polls ? slot : 0)];
@@ -1151,8 +1158,11 @@ hipError_t launch_gemm_flight_dq(hipStream_t st, const GemmArgs &g,
   for (int d = 1; d <= regions_n && d <= NJ; ++d)
     if (NJ % d == 0)
       dq.share_groups = d;
-  GridExchange ex;
-  if (!dql_exchange_begin(st, scratch, ex))
+  // (minimum and maximum of X known: the blocks do not wait for one another,
+  // and the kernel is like any other)
+  const bool exchanges = ep.x_limits == nullptr;
+  GridExchange ex = {};
+  if (exchanges && !dql_exchange_begin(st, scratch, ex))
     return hipErrorNotReady; // the exchange is off or another stream's runs
   dq.slots = ex.slots;
   dq.epoch = ex.epoch;
@@ -1170,7 +1180,8 @@ hipError_t launch_gemm_flight_dq(hipStream_t st, const GemmArgs &g,
     e = flight_launch_dq_rows<4>(st, g, ep, sh.rsh, dq);
     break;
   }
-  dql_exchange_end(st, e == hipSuccess);
+  if (exchanges)
+    dql_exchange_end(st, e == hipSuccess);
   return e;
 }
 

@@ -1012,19 +1012,24 @@ __global__ __launch_bounds__(512) void k_gemm_i8_skinny_bp(
       hi = __builtin_fmaxf(__builtin_fmaxf(hi, v[j].x),
           __builtin_fmaxf(__builtin_fmaxf(v[j].y, v[j].z), v[j].w));
     }
-    lo = wave_min(lo);
-    hi = wave_max(hi);
-    if (lane == 0) {
-      s_lo[wave] = lo;
-      s_hi[wave] = hi;
-    }
-    __syncthreads();
-    lo = s_lo[0];
-    hi = s_hi[0];
+    if (ep.x_limits) { // (the same for every thread) known from the layer before
+      lo = ep.x_limits[0];
+      hi = ep.x_limits[1];
+    } else {
+      lo = wave_min(lo);
+      hi = wave_max(hi);
+      if (lane == 0) {
+        s_lo[wave] = lo;
+        s_hi[wave] = hi;
+      }
+      __syncthreads();
+      lo = s_lo[0];
+      hi = s_hi[0];
 #pragma unroll
-    for (int w = 1; w < WAVES; ++w) {
-      lo = __builtin_fminf(lo, s_lo[w]);
-      hi = __builtin_fmaxf(hi, s_hi[w]);
+      for (int w = 1; w < WAVES; ++w) {
+        lo = __builtin_fminf(lo, s_lo[w]);
+        hi = __builtin_fmaxf(hi, s_hi[w]);
+      }
     }
     float zpf;
     dynamic_params(lo, hi, dq_scale, zpf);
@@ -1444,11 +1449,7 @@ hipError_t gemm_launch_cfg(
   if (wreg_ok(g) && (cfg == kW128x384 || (!forced && wreg_pays(g.M, g.N)))) {
     t_last_kernel = "k_gemm_i8_wreg (weights in registers, 128x384 blocks)";
     t_gelu_applied = g.epi == kEpiF32 && g.gelu; // this kernel applies it to its results
-    EpiParams epw = ep;
-    if (((g.M + 127) / 128) * ((g.N + 383) / 384) > kDqlMaxBlocks)
-      epw.limits = LimitsOut{}; // more blocks than partial slots: a pass over y
-    t_limits_written = EPI == kEpiF32 && epw.limits.out != nullptr;
-    return launch_gemm_wreg(st, g, epw, A_MODE);
+    return launch_gemm_wreg(st, g, ep, A_MODE); // (limits of y: by a pass over it)
   }
   switch (cfg) {
   case kB128x256: {
@@ -1642,6 +1643,7 @@ hipError_t launch_gemm(hipStream_t s, const GemmArgs &g) {
   ep.y_zp = g.y_zp;
   ep.bias = g.epi == kEpiF32 ? g.bias : nullptr;
   ep.bias_len = g.bias_len;
+  ep.x_limits = g.X ? g.x_limits : nullptr;
   ep.limits = LimitsOut{};
   if (g.y_limits) // (slot [4] of the counters: [0] is DynamicQuantizeLinear's)
     ep.limits = LimitsOut{g.y_limits, g.dql->partial_min, g.dql->partial_max,

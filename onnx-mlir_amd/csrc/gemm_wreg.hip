@@ -81,8 +81,7 @@ constexpr int wreg_younger(int s, int pf, int fix_ops, int fix_read, int fix_wri
   return x;
 }
 
-template <int KH, int WAVES, int NR, int A_MODE, int EPI, bool STREAM, int ACT,
-    bool LIM = false>
+template <int KH, int WAVES, int NR, int A_MODE, int EPI, bool STREAM, int ACT>
 __global__ __launch_bounds__(WAVES * 64, 1) void k_gemm_i8_wreg(
     const uint8_t *__restrict__ A, const int8_t *__restrict__ Bp, int M, int N,
     EpiParams ep, int regions_m, int regions_n, int bp_tiles) {
@@ -322,9 +321,6 @@ __global__ __launch_bounds__(WAVES * 64, 1) void k_gemm_i8_wreg(
   const int32_t sat_lo = !sat ? INT32_MIN : ep.y_unsigned ? 0 : -128;
   const int32_t sat_hi = !sat ? INT32_MAX : ep.y_unsigned ? 255 : 127;
 
-  // minimum and maximum of the f32 results this lane stores (EpiParams::limits)
-  float lim_lo = __builtin_inff(), lim_hi = -__builtin_inff();
-
   v16i acc, accp; // the tile being computed, the finished one before it
   // One element of the finished tile: register r.
   auto emit = [&](auto rc) {
@@ -342,12 +338,6 @@ __global__ __launch_bounds__(WAVES * 64, 1) void k_gemm_i8_wreg(
         f = relu_f32(f, 0.0f);
       else if (ACT == 2)
         f = gelu_f32(f);
-      // (LIM, a template argument: the two instructions an element cost 2 %
-      // of the kernel, the loop has no slot to spare)
-      if (LIM) {
-        lim_lo = __builtin_fminf(lim_lo, f);
-        lim_hi = __builtin_fmaxf(lim_hi, f);
-      }
       __builtin_amdgcn_raw_buffer_store_b32(
           (int)__float_as_uint(f), out_rsrc, (int)toff, soff, kAux);
     } else {
@@ -454,17 +444,6 @@ __global__ __launch_bounds__(WAVES * 64, 1) void k_gemm_i8_wreg(
   // the last tile
   static_for<16>([&](auto rc) { emit(rc); });
   asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory"); // reads past the last tile
-  if (EPI == kEpiF32 && LIM) {
-    // Rows past M are copies of the last row and change neither limit; the
-    // columns past N are nobody's.
-    if (n >= N) {
-      lim_lo = __builtin_inff();
-      lim_hi = -__builtin_inff();
-    }
-    __syncthreads(); // every wave is done with the tiles in LDS
-    block_publish_limits(lim_lo, lim_hi, ep.limits, (float *)sA, wave, lane,
-        WAVES, [] { __syncthreads(); });
-  }
 #ifdef WREG_TIMING
   WREG_TS(2 + NR);
   asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
@@ -486,15 +465,13 @@ hipError_t wreg_launch(hipStream_t st, const GemmArgs &g, const EpiParams &ep) {
   const int ntiles = (int)((g.N + 31) / 32);
   const int regions_n = (ntiles + kWregWaves - 1) / kWregWaves;
   const int bp_tiles = (int)(round_up(g.N, kGemmBN) / 32);
-  const dim3 grid((unsigned)(regions_m * regions_n)), block(kWregWaves * 64);
-  if (EPI == kEpiF32 && ep.limits.out != nullptr)
-    k_gemm_i8_wreg<kWregKH, kWregWaves, kWregNR, A_MODE, EPI, true, ACT,
-        EPI == kEpiF32><<<grid, block, 0, st>>>((const uint8_t *)g.A, g.Bp, M, N,
-        ep, regions_m, regions_n, bp_tiles);
-  else
-    k_gemm_i8_wreg<kWregKH, kWregWaves, kWregNR, A_MODE, EPI, true, ACT>
-        <<<grid, block, 0, st>>>((const uint8_t *)g.A, g.Bp, M, N, ep,
-            regions_m, regions_n, bp_tiles);
+  // (Minimum and maximum of the results, EpiParams::limits, are not taken
+  // here: the kernel has no two registers to spare -- with them the compiler
+  // spills a dozen of the weights' and the launch takes 26 us instead of 16;
+  // kept in LDS by atomics 20 us -- so a pass over y takes them.)
+  k_gemm_i8_wreg<kWregKH, kWregWaves, kWregNR, A_MODE, EPI, true, ACT>
+      <<<dim3((unsigned)(regions_m * regions_n)), dim3(kWregWaves * 64), 0, st>>>(
+          (const uint8_t *)g.A, g.Bp, M, N, ep, regions_m, regions_n, bp_tiles);
   return hipGetLastError();
 }
 

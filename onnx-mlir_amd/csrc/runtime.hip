@@ -1944,17 +1944,15 @@ void dyn_quant_matmul_dequant(const char *op, OMTensor *y_t,
     g.gelu = gelu;
     return launch_gemm(call.c.stream, g);
   };
-  // (known limits of x: the kernels that quantize rows themselves do not
-  // take them yet)
-  const int kind = (call.ok && t_quant_mode == 0 && call.c.dql.grid_blocks >= 0 &&
-                       !d_xlim)
+  const int kind = (call.ok && t_quant_mode == 0 && call.c.dql.grid_blocks >= 0)
                        ? gemm_quantizes_rows(M, K, N, dx)
                        : 0;
   // Blocks that wait for one another (more rows than one block quantizes for
-  // itself) raise the same flag as DynamicQuantizeLinear's one-launch kernel
-  // when they give up; checked like that kernel's.
-  const bool exchanges = kind == 2;
-  const bool in_kernel = kind == 1 || (kind == 2 && call.c.dql.grid_blocks > 0);
+  // itself, and limits of x that are not known) raise the same flag as
+  // DynamicQuantizeLinear's one-launch kernel when they give up; checked like
+  // that kernel's.
+  const bool exchanges = kind == 2 && !d_xlim;
+  const bool in_kernel = kind == 1 || (kind == 2 && (d_xlim || call.c.dql.grid_blocks > 0));
   hipError_t e = hipSuccess;
   if (call.ok) {
     e = run(in_kernel);

@@ -216,7 +216,9 @@ def _limits(a):
 
 
 @pytest.mark.parametrize("M,K,N,N2", [(128, 768, 3072, 768), (4096, 768, 3072, 768), (16, 4096, 1024, 512),
-                                      (33, 200, 130, 70), (300, 768, 1000, 416), (2, 64, 8, 5)])
+                                      (33, 200, 130, 70), (300, 768, 1000, 416), (2, 64, 8, 5),
+                                      # second layer quantized inside its kernel: one round of blocks; every block for itself
+                                      (128, 768, 1024, 768), (200, 512, 768, 1000), (8, 1024, 2048, 512), (16, 512, 2048, 11008)])
 def test_chain_of_layers_hands_the_limits_on(rt, oracle, M, K, N, N2):
     """om_mi355x_DynQuantMatMulDequantLimits: y_limits of a layer is minimum and
     maximum of its result (NaN ignored), bit for bit what numpy finds in it,
@@ -236,8 +238,10 @@ def test_chain_of_layers_hands_the_limits_on(rt, oracle, M, K, N, N2):
         assert same_f32(h, h_plain), (act, rt.last_gemm_kernel())
         assert same_f32(hl, _limits(h)), (act, hl, _limits(h), rt.last_gemm_kernel())
         y_plain = rt.DynQuantMatMulDequant(h, W2, None, s2)
+        kernel = rt.last_gemm_kernel()
         y, yl = rt.DynQuantMatMulDequantLimits(h, W2, None, s2, x_limits=hl)
-        assert same_f32(y, y_plain), act
+        assert rt.last_gemm_kernel() == kernel  # (known limits do not change the kernel)
+        assert same_f32(y, y_plain), (act, kernel)
         assert same_f32(yl, _limits(y))
         if act != 2:  # (the oracle's Gelu differs from the kernel's in the last bits)
             aq, a_s, a_zp = oracle.dynamic_quantize_linear(h)
