@@ -615,6 +615,12 @@ __attribute__((amdgpu_waves_per_eu(1, 1))) void k_gemm_i8_flight(
   v16i acc[2] = {acc_zero, acc_zero};
   // (the weights are still arriving)
   flight_kloop<KG, NR>(aaddr, b, acc);
+  // (A use of every weight register behind the loop: without it the compiler
+  // hands a step's registers to the operand reads of the steps after it, and
+  // the loop runs a tenth slower.)
+#pragma unroll
+  for (int s = 0; s < KH; ++s)
+    asm volatile("" : : "v"(b[s]));
   if (NR == 1) {
 #pragma unroll
     for (int r = 0; r < 16; ++r)
