@@ -23,7 +23,11 @@
 // the conversion and the store of the finished tile's 16 elements per lane are
 // spread, one per K step, between the MFMAs of the next tile (two accumulator
 // sets), so the matrix cores do not wait for the epilogue and the output is
-// written in a steady stream instead of in a burst at the end.
+// written in a steady stream instead of in a burst at the end.  32-bit results
+// go straight to memory, a 128-byte line per row and wave.  8-bit results are
+// first gathered in LDS, the whole 32 x (32 WAVES) tile of the block, and
+// leave one K loop later in 16-byte pieces of whole lines, one store per
+// wave and tile.
 //
 // A tile in LDS: row r at r * K, its 16-byte chunk c at position
 // c ^ (r % 16): the lanes of an operand read (16 rows at a time, the same
@@ -34,7 +38,7 @@
 // Order of a wave's memory operations, which the explicit waits count on
 // (operations complete in the order they were issued): per-column parameters,
 // the copy of row tile 0 (CPT instructions), the loads of Bp (KH), the copies
-// of tiles 1..NR-1; later only stores, 16 per tile.  "Tile u has landed" = at
+// of tiles 1..NR-1; later only stores, 16 per tile (one for 8-bit results).  "Tile u has landed" = at
 // most [what was issued after its copies] operations are outstanding.  Every
 // block copies and computes all NR tiles (rows past M are copies of the last
 // row and are not stored), so the counts hold for every block.
@@ -59,25 +63,47 @@ __device__ unsigned long long wreg_ts[16 * 16];
 // waits for them in tile t, at K step WAIT_STEP: the copies of the tiles after
 // that, the loads of Bp issued in tile 0 (one per step), the stores of the
 // tiles before t (16 each) and those of tile t so far (one per step from
-// EPI_FIRST on).
-template <int KH, int CPT, int NR, int B_FIRST, int WAIT_STEP, int EPI_FIRST>
+// EPI_FIRST on).  STAGED (8-bit results, gathered in LDS): one store per
+// tile, issued in the tile's last step, after the wait.
+template <int KH, int CPT, int NR, int B_FIRST, int WAIT_STEP, int EPI_FIRST, bool STAGED>
 struct WregNeed {
   static constexpr int at(int t) {
     const int b_late = KH - B_FIRST;
     const int b_seen = t > 0 ? b_late : (WAIT_STEP < b_late ? WAIT_STEP : b_late);
     const int here = WAIT_STEP - EPI_FIRST < 16 ? WAIT_STEP - EPI_FIRST : 16;
-    return CPT * (NR - 2 - t) + b_seen + (t > 0 ? 16 * (t - 1) + here : 0);
+    const int stores = t == 0 ? 0 : STAGED ? t - 1 : 16 * (t - 1) + here;
+    return CPT * (NR - 2 - t) + b_seen + stores;
   }
 };
+// LDS operations issued between the steps `from` (after its operand read) and
+// `to` (before its operand read) of a tile other than the block's first by
+// the staged epilogue: one write per step from epi_first on, 16 in all, each
+// at the end of its step.
+constexpr int wreg_staged_writes(int from, int to, int epi_first) {
+  int x = 0;
+  for (int j = from; j < to; ++j)
+    if (j >= epi_first && j < epi_first + 16)
+      ++x;
+  return x;
+}
 // LDS operations issued after the read for step s when step s waits for it:
-// the pf reads ahead of it, and the fix-up's fix_ops reads (issued in step
-// fix_read) and as many writes (step fix_write) while they are among those.
-constexpr int wreg_younger(int s, int pf, int fix_ops, int fix_read, int fix_write) {
+// the pf reads ahead of it, the fix-up's fix_ops reads (issued in step
+// fix_read) and as many writes (step fix_write) while they are among those,
+// and, with `staged` (the staged epilogue, in a tile that has a finished one
+// to store), its writes of the pf steps before and its read of the gathered
+// tile, issued in step flush_read.
+constexpr int wreg_younger(int s, int pf, int fix_ops, int fix_read, int fix_write,
+    bool staged, int epi_first, int flush_read) {
   int x = pf;
   if (s >= fix_read && s < fix_read + pf)
     x += fix_ops;
   if (s >= fix_write && s < fix_write + pf)
     x += fix_ops;
+  if (staged) {
+    x += wreg_staged_writes(s - pf, s, epi_first);
+    if (s >= flush_read && s < flush_read + pf)
+      x += 1;
+  }
   return x;
 }
 
@@ -108,10 +134,24 @@ __global__ __launch_bounds__(WAVES * 64, 1) void k_gemm_i8_wreg(
                     kFixWrite + PF <= KH - PF && kFixRead >= kEpiFirst,
       "shape");
   constexpr int kWaitStep = FIX ? kFixRead : KH - PF;
-  using Need = WregNeed<KH, CPT, NR, kBFirst, kWaitStep, kEpiFirst>;
+  // 8-bit results are gathered in LDS, a 32 x (32 WAVES) tile of the block at
+  // a time, and leave in whole 128-byte lines, 16 bytes a lane: a wave's own
+  // part of a row is 32 bytes, and the memory system takes as long over a
+  // 32-byte piece as over a line.  Two tiles: one is being filled (one byte
+  // a lane and K step) while the one before it is read back and stored.
+  constexpr bool STAGED = (EPI == kEpiQ8);
+  constexpr int kStagePitch = 32 * WAVES + 16; // rows 4 apart: different banks
+  constexpr int kStageBytes = 32 * kStagePitch;
+  constexpr int kStageAt = (NR + 1) * TILE_BYTES;
+  constexpr int kFlushRead = KH - PF;   // step: behind the tile's barrier
+  static_assert(!STAGED || (kEpiFirst + 16 <= kFlushRead && (32 * WAVES) % 16 == 0 &&
+                               kStageAt + 2 * kStageBytes <= 160 * 1024),
+      "staged epilogue");
+  using Need = WregNeed<KH, CPT, NR, kBFirst, kWaitStep, kEpiFirst, STAGED>;
   static_assert(kBFirst + CPT * (NR - 1) <= 63 && Need::at(NR - 2) <= 63, "counter");
   // (+ one spare tile: the reads that run ahead of the last tile's last steps)
-  __shared__ __attribute__((aligned(1024))) uint8_t sA[(NR + 1) * TILE_BYTES];
+  __shared__ __attribute__((aligned(1024)))
+  uint8_t sA[(NR + 1) * TILE_BYTES + (STAGED ? 2 * kStageBytes : 0)];
 
 #ifdef WREG_TIMING
   unsigned long long ts[16] = {};
@@ -171,9 +211,14 @@ __global__ __launch_bounds__(WAVES * 64, 1) void k_gemm_i8_wreg(
 
   // ---- copies of A into LDS, loads of Bp into registers --------------------
   typedef __attribute__((address_space(3))) void *lds_ptr;
-  typedef const __attribute__((address_space(1))) void *glb_ptr;
   // Copy instruction j of a tile fills LDS chunks [64 j, 64 j + 64): chunk q is
   // position q % CPR of row q / CPR and holds chunk (q % CPR) ^ (row % 16).
+  // (A buffer load, not a global one: the compiler takes a global load into
+  // LDS for an operation that may complete out of order with everything else
+  // and from then on waits for ALL outstanding memory operations wherever it
+  // waits for one, which the loads of Bp in tile 0 make it do.)
+  const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint8_t *>(A), 0, (int)((uint32_t)M * (uint32_t)K), 0x00020000);
   auto copy_tile = [&](int t) {
 #pragma unroll
     for (int jj = 0; jj < CPT; ++jj) {
@@ -182,9 +227,9 @@ __global__ __launch_bounds__(WAVES * 64, 1) void k_gemm_i8_wreg(
       const int c = (q % CPR) ^ (r & 15);
       int row = row0 + t * 32 + r;
       row = row < M ? row : M - 1; // rows past M: never stored
-      __builtin_amdgcn_global_load_lds(
-          (glb_ptr)(A + (int64_t)row * K + c * 16),
-          (lds_ptr)(sA + t * TILE_BYTES + (wave * CPT + jj) * 1024), 16, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc,
+          (lds_ptr)(sA + t * TILE_BYTES + (wave * CPT + jj) * 1024), 16,
+          (int)((uint32_t)row * (uint32_t)K + (uint32_t)(c * 16)), 0, 0, 0);
     }
   };
   copy_tile(0);
@@ -316,10 +361,41 @@ __global__ __launch_bounds__(WAVES * 64, 1) void k_gemm_i8_wreg(
                               (uint32_t)ES
                         : 0x80000000u;
   const uint32_t tile_pitch = 32u * (uint32_t)N * (uint32_t)ES;
+  // Staged: where the lane puts its bytes (row 4 * lh of the tile being
+  // filled, its own column), and what it stores of a gathered tile: piece
+  // idx % (2 WAVES) of row idx / (2 WAVES), idx = its number in the block.
+  unsigned saddr = (unsigned)(uintptr_t)(lds_ptr)sA + kStageAt +
+                   4 * lh * kStagePitch + wave * 32 + l32;
+  int stage_row0 = row0 * N; // offset of the gathered tile's first row
+  auto flush_read = [&](v4i &dst, int buf) {
+    // (the lane's number is read again here rather than kept in a register)
+    const int idx = wave * 64 + (int)__builtin_amdgcn_mbcnt_hi(
+                                    ~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+    const int frow = idx / (2 * WAVES);
+    const int fch = idx - frow * (2 * WAVES);
+    const unsigned addr = (unsigned)(uintptr_t)(lds_ptr)sA + kStageAt +
+                          buf * kStageBytes + frow * kStagePitch + fch * 16;
+    asm volatile("ds_read_b128 %0, %1" : "=v"(dst) : "v"(addr) : "memory");
+  };
+  auto flush_store = [&](const v4i &src) {
+    const int idx = wave * 64 + (int)__builtin_amdgcn_mbcnt_hi(
+                                    ~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+    const int frow = idx / (2 * WAVES);
+    const int fch = idx - frow * (2 * WAVES);
+    const int col = rn * (32 * WAVES) + fch * 16;
+    const uint32_t off =
+        col < N ? (uint32_t)(stage_row0 + frow * N + col) : 0x80000000u;
+    __builtin_amdgcn_raw_buffer_store_b128(
+        src, out_rsrc, (int)off, 0, STREAM ? kAuxThrough : 0);
+  };
 
   const bool sat = EPI == kEpiQ8 && ep.narrow == kSaturate;
   const int32_t sat_lo = !sat ? INT32_MIN : ep.y_unsigned ? 0 : -128;
-  const int32_t sat_hi = !sat ? INT32_MAX : ep.y_unsigned ? 255 : 127;
+  int32_t sat_hi = !sat ? INT32_MAX : ep.y_unsigned ? 255 : 127;
+  // (kept in a vector register: the clamp takes one scalar operand, and the
+  // compiler would otherwise move the other one over before every element)
+  if (EPI == kEpiQ8)
+    asm volatile("v_mov_b32 %0, %1" : "=v"(sat_hi) : "s"(sat_hi));
 
   v16i acc, accp; // the tile being computed, the finished one before it
   // One element of the finished tile: register r.
@@ -346,9 +422,14 @@ __global__ __launch_bounds__(WAVES * 64, 1) void k_gemm_i8_wreg(
           (int32_t)((uint32_t)(int32_t)__builtin_rintf(f) + (uint32_t)yz);
       // one instruction, no branch: bounds that do nothing when the result
       // wraps (the byte store keeps the low byte by itself)
-      asm("v_med3_i32 %0, %1, %2, %3" : "=v"(v) : "v"(v), "s"(sat_lo), "v"(sat_hi));
-      __builtin_amdgcn_raw_buffer_store_b8(
-          (unsigned char)v, out_rsrc, (int)toff, soff, 0);
+      // (named here: asm operands alone do not capture)
+      const int32_t lo = sat_lo, hi = sat_hi;
+      const unsigned at = saddr;
+      asm("v_med3_i32 %0, %1, %2, %3" : "=v"(v) : "v"(v), "s"(lo), "v"(hi));
+      asm volatile("ds_write_b8 %0, %1 offset:%2"
+                   :
+                   : "v"(at), "v"(v), "n"(row * kStagePitch)
+                   : "memory");
     }
   };
 
@@ -365,21 +446,33 @@ __global__ __launch_bounds__(WAVES * 64, 1) void k_gemm_i8_wreg(
   // and issues the remaining loads of Bp.
   auto tile = [&](auto firstc, int t) {
     constexpr bool FIRST = decltype(firstc)::value;
+    constexpr bool ST = STAGED && !FIRST; // a finished tile passes through LDS
+    v4i gathered;
     static_for<KH>([&](auto sc) {
       constexpr int s2 = decltype(sc)::value;
       if constexpr (FIX && s2 == kFixRead) {
         next_tile_landed(t);
         fix_read(std::integral_constant<int, TILE_BYTES>{});
       }
-      if constexpr (FIX && s2 == kFixWrite) // reads issued since: kFixWrite - kFixRead
+      if constexpr (FIX && s2 == kFixWrite) // operations issued since the reads
         fix_write(std::integral_constant<int, TILE_BYTES>{},
-            std::integral_constant<int, kFixWrite - kFixRead>{});
+            std::integral_constant<int,
+                kFixWrite - kFixRead +
+                    (ST ? wreg_staged_writes(kFixRead, kFixWrite, kEpiFirst) : 0)>{});
       if constexpr (s2 == KH - PF) {
-        if (FIX) // the fix-up's writes are done: reads issued since them
-          asm volatile("s_waitcnt lgkmcnt(%0)" : : "n"(KH - PF - kFixWrite) : "memory");
+        if (FIX) // the fix-up's writes are done: operations issued since them
+          asm volatile("s_waitcnt lgkmcnt(%0)"
+                       :
+                       : "n"(KH - PF - kFixWrite +
+                             (ST ? wreg_staged_writes(kFixWrite, KH - PF, kEpiFirst) : 0))
+                       : "memory");
         else
           next_tile_landed(t);
+        // (the bytes of the finished tile were written before the operand read
+        // that step s2 - 1 waited for: every wave's are in LDS behind the barrier)
         __builtin_amdgcn_s_barrier();
+        if constexpr (ST)
+          flush_read(gathered, (t - 1) & 1);
       }
 #ifndef WREG_ABL_NO_LDS
       aread(std::integral_constant<int, s2 + PF>{});
@@ -388,7 +481,8 @@ __global__ __launch_bounds__(WAVES * 64, 1) void k_gemm_i8_wreg(
         v4i &f = fa[s2 % NB];
         asm volatile("s_waitcnt lgkmcnt(%1)"
                      : "+v"(f)
-                     : "n"(wreg_younger(s2, PF, FIX ? CPT : 0, kFixRead, kFixWrite))
+                     : "n"(wreg_younger(s2, PF, FIX ? CPT : 0, kFixRead, kFixWrite, ST,
+                         kEpiFirst, kFlushRead))
                      : "memory");
       }
 #ifdef WREG_ABL_NO_MFMA
@@ -412,6 +506,15 @@ __global__ __launch_bounds__(WAVES * 64, 1) void k_gemm_i8_wreg(
 #ifndef WREG_ABL_NO_EPI
       if constexpr (!FIRST && s2 >= kEpiFirst && s2 < kEpiFirst + 16)
         emit(std::integral_constant<int, s2 - kEpiFirst>{});
+      if constexpr (ST && s2 == KH - 1) {
+        // the operand reads of the steps since are younger than the read of
+        // the gathered tile
+        asm volatile("s_waitcnt lgkmcnt(%1)"
+                     : "+v"(gathered)
+                     : "n"(KH - kFlushRead)
+                     : "memory");
+        flush_store(gathered);
+      }
 #endif
       __builtin_amdgcn_sched_barrier(0);
     });
@@ -419,11 +522,19 @@ __global__ __launch_bounds__(WAVES * 64, 1) void k_gemm_i8_wreg(
     // reads and the output rows move on.  (fa is indexed by the step within
     // the tile: KH is a multiple of NB, so the ring carries over.)
     accp = acc;
-    if constexpr (!FIRST)
+    if constexpr (!FIRST) {
       toff += tile_pitch;
-#pragma unroll
-    for (int v = 0; v < 8; ++v)
-      aaddr[v] += TILE_BYTES;
+      if (STAGED) { // the other staging tile, the next 32 rows
+        saddr += ((t - 1) & 1) ? -kStageBytes : kStageBytes;
+        stage_row0 += 32 * N;
+      }
+    }
+    // (in place: written as plain additions the compiler keeps the eight
+    // addresses of tile 0 and makes eight more per tile from them)
+    static_for<8>([&](auto vc) {
+      unsigned &a = aaddr[decltype(vc)::value];
+      asm volatile("v_add_u32_e32 %0, %1, %0" : "+v"(a) : "n"(TILE_BYTES));
+    });
     own += TILE_BYTES;
     __builtin_amdgcn_sched_barrier(0);
   };
@@ -444,6 +555,13 @@ __global__ __launch_bounds__(WAVES * 64, 1) void k_gemm_i8_wreg(
   // the last tile
   static_for<16>([&](auto rc) { emit(rc); });
   asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory"); // reads past the last tile
+  if (STAGED) {
+    v4i gathered;
+    __builtin_amdgcn_s_barrier();
+    flush_read(gathered, (NR - 1) & 1);
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(gathered) : : "memory");
+    flush_store(gathered);
+  }
 #ifdef WREG_TIMING
   WREG_TS(2 + NR);
   asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
@@ -480,13 +598,13 @@ hipError_t wreg_launch(hipStream_t st, const GemmArgs &g, const EpiParams &ep) {
 bool wreg_ok(const GemmArgs &g) {
   const int64_t es = g.epi == kEpiQ8 ? 1 : 4;
   if (g.M * g.N * es > ((int64_t)1 << 31) ||
-      32 * kWregNR * g.N * es >= ((int64_t)1 << 30))
+      32 * kWregNR * g.N * es >= ((int64_t)1 << 30) || g.M * g.K >= ((int64_t)1 << 32))
     return false;
   const bool rowsum = g.b_unsigned || (g.b_zp != nullptr && g.b_zp_len > 0);
-  // (8-bit results: 32 bytes of a row per wave and store, whole 32-byte
-  // sectors when the rows are 32 bytes apart at least)
+  // (8-bit results leave in 16-byte pieces of whole 128-byte lines)
   return g.K == 32 * kWregKH && g.a_zp_len <= 1 && !g.X && !rowsum &&
          ((((uintptr_t)g.A) & 15) == 0) && (g.N * es) % 128 == 0 &&
+         (g.epi != kEpiQ8 || (((uintptr_t)g.out) & 15) == 0) &&
          (g.epi == kEpiF32 || g.epi == kEpiI32 || g.epi == kEpiQ8);
 }
 

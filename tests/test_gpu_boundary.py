@@ -129,7 +129,7 @@ def test_weights_in_registers_kernel_stays_inside_a_ragged_output(rt, oracle, fo
     the remainder M % 32 is."""
     if forced:
         monkeypatch.setenv("OM_MI355X_GEMM_TILE", "4")
-        shapes = [(17, 32), (30, 64), (129, 416), (131, 384), (300, 800), (1000, 416)]
+        shapes = [(17, 32), (30, 64), (129, 416), (131, 384), (300, 800), (1000, 416), (333, 896)]
     else:
         shapes = [(4001, 2304), (4065, 3072), (4095, 3072)]
     rng = np.random.default_rng(4242 + forced)
@@ -157,6 +157,22 @@ def test_weights_in_registers_kernel_stays_inside_a_ragged_output(rt, oracle, fo
             assert (whole[guard + M * N:] == 0x5A5A5A5A).all(), (M, N, epi, "after")
             assert np.array_equal(whole[guard:guard + M * N].reshape(M, N), want), (M, N, epi)
             buf.free()
+        if N % 128:
+            continue
+        # 8-bit results, gathered in LDS and stored 16 bytes a lane
+        bz0 = np.zeros((), np.int8)
+        a_s, b_s, y_s, yz = np.float32(0.0173), np.float32(0.004), np.float32(0.08), np.uint8(131)
+        want = oracle.qlinear_matmul(A, a_s, az, B, b_s, bz0, y_s, yz, oracle_lib.SATURATE)
+        buf = rt.DeviceArray.from_numpy(np.full(guard + M * N + guard, 0x5A, np.uint8))
+        y = rt.DeviceArray.view_of(buf, guard, (M, N))
+        rt.QLinearMatMul(A, a_s, az, B, b_s, bz0, y_s, yz, rt.SATURATE, out=y)
+        assert "wreg" in rt.last_gemm_kernel(), (M, N, rt.last_gemm_kernel())
+        rt.synchronize()
+        whole = buf.numpy()
+        assert (whole[:guard] == 0x5A).all(), (M, N, "q8", "before")
+        assert (whole[guard + M * N:] == 0x5A).all(), (M, N, "q8", "after")
+        assert np.array_equal(whole[guard:guard + M * N].reshape(M, N), want), (M, N, "q8")
+        buf.free()
 
 
 def test_dispatch_keeps_bs_to_whole_trips(rt, oracle):
