@@ -1449,7 +1449,9 @@ hipError_t gemm_launch_cfg(
   if (wreg_ok(g) && (cfg == kW128x384 || (!forced && wreg_pays(g.M, g.N)))) {
     t_last_kernel = "k_gemm_i8_wreg (weights in registers, 128x384 blocks)";
     t_gelu_applied = g.epi == kEpiF32 && g.gelu; // this kernel applies it to its results
-    return launch_gemm_wreg(st, g, ep, A_MODE); // (limits of y: by a pass over it)
+    // (the limits of y: in the kernel for the f32 results of a fused layer)
+    t_limits_written = A_MODE == 2 && EPI == kEpiF32 && ep.limits.out != nullptr;
+    return launch_gemm_wreg(st, g, ep, A_MODE);
   }
   switch (cfg) {
   case kB128x256: {

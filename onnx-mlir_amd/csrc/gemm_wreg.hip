@@ -107,7 +107,10 @@ constexpr int wreg_younger(int s, int pf, int fix_ops, int fix_read, int fix_wri
   return x;
 }
 
-template <int KH, int WAVES, int NR, int A_MODE, int EPI, bool STREAM, int ACT>
+// LIM: minimum and maximum of the (f32) results are kept per lane while they
+// are stored and reduced over the grid when the block ends (EpiParams::limits).
+template <int KH, int WAVES, int NR, int A_MODE, int EPI, bool STREAM, int ACT,
+    bool LIM = false>
 __global__ __launch_bounds__(WAVES * 64, 1) void k_gemm_i8_wreg(
     const uint8_t *__restrict__ A, const int8_t *__restrict__ Bp, int M, int N,
     EpiParams ep, int regions_m, int regions_n, int bp_tiles) {
@@ -397,6 +400,10 @@ __global__ __launch_bounds__(WAVES * 64, 1) void k_gemm_i8_wreg(
   if (EPI == kEpiQ8)
     asm volatile("v_mov_b32 %0, %1" : "=v"(sat_hi) : "s"(sat_hi));
 
+  static_assert(!LIM || EPI == kEpiF32, "limits of f32 results");
+  // (rows past M are copies of row M - 1, whose results they repeat: they
+  // change neither limit; the lanes of a column past N are taken out at the end)
+  float lim_lo = __builtin_inff(), lim_hi = -__builtin_inff();
   v16i acc, accp; // the tile being computed, the finished one before it
   // One element of the finished tile: register r.
   auto emit = [&](auto rc) {
@@ -414,6 +421,16 @@ __global__ __launch_bounds__(WAVES * 64, 1) void k_gemm_i8_wreg(
         f = relu_f32(f, 0.0f);
       else if (ACT == 2)
         f = gelu_f32(f);
+      if (LIM) {
+        // A NaN is ignored (the instructions return their other operand), as
+        // DynamicQuantizeLinear's reductions ignore it.  Written as
+        // instructions in place: the compiler moves minnum / maxnum calls to
+        // the end of the tile and keeps the tile's sixteen results until then.
+        float &lo = lim_lo, &hi = lim_hi;
+        asm volatile("v_min_f32 %0, %0, %2\n\tv_max_f32 %1, %1, %2"
+                     : "+v"(lo), "+v"(hi)
+                     : "v"(f));
+      }
       __builtin_amdgcn_raw_buffer_store_b32(
           (int)__float_as_uint(f), out_rsrc, (int)toff, soff, kAux);
     } else {
@@ -562,6 +579,17 @@ __global__ __launch_bounds__(WAVES * 64, 1) void k_gemm_i8_wreg(
     asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(gathered) : : "memory");
     flush_store(gathered);
   }
+  if constexpr (LIM) {
+    if (n >= N) {
+      lim_lo = __builtin_inff();
+      lim_hi = -__builtin_inff();
+    }
+    // (the tiles in LDS are not read any more; behind a barrier their place
+    // is free)
+    __syncthreads();
+    block_publish_limits(lim_lo, lim_hi, ep.limits, (float *)sA, wave, lane, WAVES,
+        [] { __syncthreads(); });
+  }
 #ifdef WREG_TIMING
   WREG_TS(2 + NR);
   asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
@@ -583,10 +611,17 @@ hipError_t wreg_launch(hipStream_t st, const GemmArgs &g, const EpiParams &ep) {
   const int ntiles = (int)((g.N + 31) / 32);
   const int regions_n = (ntiles + kWregWaves - 1) / kWregWaves;
   const int bp_tiles = (int)(round_up(g.N, kGemmBN) / 32);
-  // (Minimum and maximum of the results, EpiParams::limits, are not taken
-  // here: the kernel has no two registers to spare -- with them the compiler
-  // spills a dozen of the weights' and the launch takes 26 us instead of 16;
-  // kept in LDS by atomics 20 us -- so a pass over y takes them.)
+  // Minimum and maximum of the results (EpiParams::limits) are taken in the
+  // kernel for the f32 results of a fused layer (its activations arrive
+  // stored minus 128: A_MODE 2); elsewhere a pass over y takes them.
+  if constexpr (A_MODE == 2 && EPI == kEpiF32) {
+    if (ep.limits.out != nullptr) {
+      k_gemm_i8_wreg<kWregKH, kWregWaves, kWregNR, A_MODE, EPI, true, ACT, true>
+          <<<dim3((unsigned)(regions_m * regions_n)), dim3(kWregWaves * 64), 0, st>>>(
+              (const uint8_t *)g.A, g.Bp, M, N, ep, regions_m, regions_n, bp_tiles);
+      return hipGetLastError();
+    }
+  }
   k_gemm_i8_wreg<kWregKH, kWregWaves, kWregNR, A_MODE, EPI, true, ACT>
       <<<dim3((unsigned)(regions_m * regions_n)), dim3(kWregWaves * 64), 0, st>>>(
           (const uint8_t *)g.A, g.Bp, M, N, ep, regions_m, regions_n, bp_tiles);
