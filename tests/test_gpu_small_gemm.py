@@ -216,6 +216,8 @@ def _limits(a):
 
 
 @pytest.mark.parametrize("M,K,N,N2", [(128, 768, 3072, 768), (4096, 768, 3072, 768), (16, 4096, 1024, 512),
+                                      # ragged rows and a last column tile past N in the weights-in-registers kernel
+                                      (2945, 768, 3040, 416),
                                       (33, 200, 130, 70), (300, 768, 1000, 416), (2, 64, 8, 5),
                                       # second layer quantized inside its kernel: one round of blocks; every block for itself
                                       (128, 768, 1024, 768), (200, 512, 768, 1000), (8, 1024, 2048, 512), (16, 512, 2048, 11008)])
