@@ -123,30 +123,39 @@ __global__ __launch_bounds__(kThreads) void k_quant_flat(
     const float *__restrict__ x, uint8_t *__restrict__ y, int64_t n,
     const float *__restrict__ scale_p, const void *__restrict__ zp_p,
     uint32_t flip, QuantLimits lim) {
-  float s, zpf;
-  quant_params<SIGNED, HAS_ZP>(scale_p, zp_p, lim, blockIdx.x == 0, s, zpf);
-  const float r = 1.0f / s;
   const int64_t nvec = n >> 2;
   const f4a *__restrict__ x4 = (const f4a *)x;
   uint32_t *__restrict__ y4 = (uint32_t *)y;
   const int64_t step = (int64_t)gridDim.x * (kThreads * kUnroll);
+  const int64_t base0 = (int64_t)blockIdx.x * (kThreads * kUnroll);
+  // The block's first vectors are requested before scale and zero point are
+  // (no branch around them: one past the end is the last one again, and is
+  // not stored): the parameters first would put a memory round trip of their
+  // own in front of the data's.
+  f4a v[kUnroll];
+  auto request = [&](int64_t base) {
+#pragma unroll
+    for (int j = 0; j < kUnroll; ++j) {
+      const int64_t idx = base + j * kThreads + threadIdx.x;
+      v[j] = __builtin_nontemporal_load(&x4[idx < nvec ? idx : nvec - 1]);
+    }
+  };
+  if (base0 < nvec) // (the same for the whole block; implies nvec > 0)
+    request(base0);
+  __builtin_amdgcn_sched_barrier(0);
+  float s, zpf;
+  quant_params<SIGNED, HAS_ZP>(scale_p, zp_p, lim, blockIdx.x == 0, s, zpf);
+  const float r = 1.0f / s;
   auto body = [&](auto fast_c) {
     constexpr bool FAST = decltype(fast_c)::value;
-    for (int64_t base = (int64_t)blockIdx.x * (kThreads * kUnroll);
-         base < nvec; base += step) {
-      f4a v[kUnroll];
-      int64_t idx[kUnroll];
+    for (int64_t base = base0; base < nvec; base += step) {
+      if (base != base0)
+        request(base);
 #pragma unroll
       for (int j = 0; j < kUnroll; ++j) {
-        idx[j] = base + j * kThreads + threadIdx.x;
-        if (idx[j] < nvec)
-          v[j] = __builtin_nontemporal_load(&x4[idx[j]]);
-      }
-#pragma unroll
-      for (int j = 0; j < kUnroll; ++j) {
-        if (idx[j] < nvec)
-          q_store(&y4[idx[j]],
-              quant_four<SIGNED, HAS_ZP, FAST>(v[j], s, r, zpf, flip));
+        const int64_t idx = base + j * kThreads + threadIdx.x;
+        if (idx < nvec)
+          q_store(&y4[idx], quant_four<SIGNED, HAS_ZP, FAST>(v[j], s, r, zpf, flip));
       }
     }
   };
@@ -176,23 +185,29 @@ __global__ __launch_bounds__(kThreads) void k_quant_tiled(
     const float *__restrict__ x, uint8_t *__restrict__ y, int64_t n,
     const float *__restrict__ scale_p, const void *__restrict__ zp_p,
     uint32_t flip, QuantLimits lim) {
+  const int64_t nvec = n >> 2; // >= 1: the kernel is for large tensors
+  const f4a *__restrict__ x4 = (const f4a *)x;
+  uint32_t *__restrict__ y4 = (uint32_t *)y;
+  const int64_t first = (int64_t)blockIdx.y * kTileRows * kTileRun +
+                        (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  // The vectors are requested before scale and zero point are, and without a
+  // branch around any of them (one past the end is the last one again, and is
+  // not stored): a block lives for one memory round trip, and parameters
+  // loaded first -- a scalar load that the zero point's load waits for, and a
+  // wait for that one -- made it two and a half (83 % of HBM peak against
+  // 88 % for the per-axis kernel, which asks for its rows first).
+  f4a v[kTileRows];
+#pragma unroll
+  for (int j = 0; j < kTileRows; ++j) {
+    const int64_t idx = first + (int64_t)j * kTileRun;
+    v[j] = __builtin_nontemporal_load(&x4[idx < nvec ? idx : nvec - 1]);
+  }
+  __builtin_amdgcn_sched_barrier(0);
   float s, zpf;
   quant_params<SIGNED, HAS_ZP>(
       scale_p, zp_p, lim, blockIdx.x == 0 && blockIdx.y == 0, s, zpf);
   const float r = 1.0f / s;
   const bool tame = scale_is_tame(s); // the same for every thread
-  const int64_t nvec = n >> 2;
-  const f4a *__restrict__ x4 = (const f4a *)x;
-  uint32_t *__restrict__ y4 = (uint32_t *)y;
-  const int64_t first = (int64_t)blockIdx.y * kTileRows * kTileRun +
-                        (int64_t)blockIdx.x * kThreads + threadIdx.x;
-  f4a v[kTileRows];
-#pragma unroll
-  for (int j = 0; j < kTileRows; ++j) {
-    const int64_t idx = first + (int64_t)j * kTileRun;
-    if (idx < nvec)
-      v[j] = __builtin_nontemporal_load(&x4[idx]);
-  }
   auto store = [&](auto fast_c) {
     constexpr bool FAST = decltype(fast_c)::value;
 #pragma unroll
