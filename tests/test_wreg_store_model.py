@@ -157,3 +157,59 @@ def test_lgkm_counts_follow_from_the_order_of_a_step(staged, fix):
             got = wreg_younger(s, PF, 2 if fix else 0, FIX_READ, FIX_WRITE, st, EPI_FIRST, FLUSH_READ)
             assert got == want, (staged, fix, first, s, got, want)
             assert got <= 15  # the counter's range
+
+
+# ---------------------------------------------------------------------------
+# vmcnt: "tile t + 1 has landed" = at most Need::at(t) operations outstanding
+# ---------------------------------------------------------------------------
+CPT, B_FIRST = KH // WAVES, 8
+
+
+def wreg_need(t, wait_step, staged):
+    """The kernel's WregNeed<...>::at(t)."""
+    b_late = KH - B_FIRST
+    b_seen = b_late if t > 0 else min(wait_step, b_late)
+    here = min(wait_step - EPI_FIRST, 16)
+    stores = 0 if t == 0 else (t - 1 if staged else 16 * (t - 1) + here)
+    return CPT * (NR - 2 - t) + b_seen + stores
+
+
+def wave_memory_ops(wait_step, staged):
+    """A wave's vector-memory operations in program order, as (kind, tile)
+    tuples, with ("wait", t) where tile t waits for tile t + 1."""
+    ops = [("param", 0)] * 8
+    ops += [("copy", 0)] * CPT
+    ops += [("b", 0)] * B_FIRST
+    for t in range(1, NR):
+        ops += [("copy", t)] * CPT
+    for t in range(NR):
+        for s in range(KH):
+            if s == wait_step and t < NR - 1:
+                ops.append(("wait", t))
+            if t == 0 and s + B_FIRST < KH:
+                ops.append(("b", 0))            # behind the step's MFMA
+            if t > 0 and not staged and EPI_FIRST <= s < EPI_FIRST + 16:
+                ops.append(("store", t - 1))
+            if t > 0 and staged and s == KH - 1:
+                ops.append(("store", t - 1))
+    return ops
+
+
+@pytest.mark.parametrize("staged", [False, True])
+@pytest.mark.parametrize("fix", [False, True])
+def test_vmcnt_counts_follow_from_the_order_of_the_loop(staged, fix):
+    wait_step = FIX_READ if fix else KH - PF
+    ops = wave_memory_ops(wait_step, staged)
+    for t in range(NR - 1):
+        at = ops.index(("wait", t))
+        last_copy = max(i for i, o in enumerate(ops[:at]) if o == ("copy", t + 1))
+        younger = sum(1 for o in ops[last_copy + 1:at] if o[0] != "wait")
+        assert wreg_need(t, wait_step, staged) == younger, (staged, fix, t)
+        assert younger <= 63  # the counter's range
+    # the first wait of the kernel, before the loop: tile 0's copies have landed
+    # when at most the first loads of Bp and the copies of the other tiles,
+    # which were issued behind them, are outstanding
+    prologue = 8 + CPT + B_FIRST + CPT * (NR - 1)   # everything issued before the loop
+    last_copy0 = max(i for i, o in enumerate(ops[:prologue]) if o == ("copy", 0))
+    assert len(ops[last_copy0 + 1:prologue]) == B_FIRST + CPT * (NR - 1)  # the kernel's constant
+    assert all(o[0] in ("b", "copy") for o in ops[last_copy0 + 1:prologue])
