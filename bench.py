@@ -822,6 +822,10 @@ def main():
                     fused.append(fused_case(rt, wl, f"config4 {name} fused layer, Gelu", 4096, k, n, cc["W"],
                                             cc["w_scale"], esteps, ewarm, activation=2))
         extras["fused"] = fused
+        # the feed-forward block as two fused layers in a row, without and with
+        # the first layer's limits handed to the second
+        extras["ffn_block"] = {"plain": chain_case(rt, wl, 4096, esteps, ewarm, False),
+                               "limits": chain_case(rt, wl, 4096, esteps, ewarm, True)}
     if "gemm" in groups:
         gemms = []
         for name, (k, n) in wl.CONFIG4_SHAPES.items():
@@ -905,7 +909,8 @@ def main():
         line["detail_file"] = "gpurun_out/bench_detail.json"
     except OSError:
         line["detail_file"] = None
-    line["extras"] = for_line(extras)
+    # (the feed-forward block's pair is in the summary and in the detail file)
+    line["extras"] = for_line({k: v for k, v in extras.items() if k != "ffn_block"})
     line["configs"] = config_summary(main_res, extras)
     print(json.dumps(sig(line), separators=(",", ":")))
 
