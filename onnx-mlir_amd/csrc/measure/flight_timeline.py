@@ -36,6 +36,9 @@ def main():
     ap.add_argument("--case", choices=("fused", "f32", "q8"), default="fused")
     ap.add_argument("--shape", default="128x768x768")
     ap.add_argument("--launches", type=int, default=2000)
+    ap.add_argument("--operands", choices=("random", "constant"), default="random",
+                    help="constant: every byte of both operands the same small value (the matrix cores "
+                         "draw less power on such data, see measure/mfma_ceiling.hip)")
     args = ap.parse_args()
     M, K, N = (int(v) for v in args.shape.split("x"))
     rt.LIB_PATH = os.path.join(HERE, "libom_mi355x.so")
@@ -53,6 +56,8 @@ def main():
     elif args.case == "q8":
         A = rng.integers(0, 256, (M, K), dtype=np.uint8)
         Bu = rng.integers(0, 256, (K, N), dtype=np.uint8)
+        if args.operands == "constant":
+            A[:], Bu[:] = 129, 121
         d = [rt.DeviceArray.from_numpy(np.asarray(x)) for x in
              (A, np.float32(0.01), np.uint8(128), Bu, np.float32(0.005), np.uint8(120), np.float32(0.5), np.uint8(0))]
         rt.mark_constant(d[3])
